@@ -1,0 +1,209 @@
+"""Pins for the oracle's LunarLander: constants algebra, reset invariants, reward/done decision table."""
+import ctypes as C
+import math
+
+import numpy as np
+
+H, W = 400.0 / 30.0, 20.0
+BOD, JNT, EDG, META = 8, 56, 91, 188
+
+
+def fresh(orc, seed=5, env=0):
+    row = np.zeros(192, np.float32)
+    orc.orc_ll_reset(row, orc.orc_ll_combined_seed(seed, env))
+    return row
+
+
+def step(orc, row, action, env=0):
+    r, d = np.zeros(1, np.float32), np.zeros(1, np.float32)
+    contacts = np.zeros(72, np.float32)
+    n = C.c_int(0)
+    orc.orc_ll_step(row, env, action, r, d, contacts.ctypes.data, C.addressof(n))
+    return float(r[0]), float(d[0]), contacts, n.value
+
+
+def test_reset_invariants(orc):
+    row = fresh(orc)
+    assert row[90] == 2 and row[187] == 10                    # joint / edge counts
+    b = row[BOD:BOD + 39].reshape(3, 13)
+    np.testing.assert_allclose(b[0, :3], [10.0, H, 0.0], rtol=1e-7)
+    np.testing.assert_allclose(b[1, :2], [10 - 20 / 30, H - 10 / 30 - 18 / 30], rtol=1e-6)
+    np.testing.assert_allclose(b[2, :2], [10 + 20 / 30, H - 10 / 30 - 18 / 30], rtol=1e-6)
+    assert (np.abs(b[:, 3:5]) <= 4.0).all() and (b[:, 3:5] == b[0, 3:5]).all()
+    np.testing.assert_allclose(b[:, 9:12], [[5, .2, .5], [.2, 5, 50], [.2, 5, 50]], rtol=1e-6)
+    assert list(b[:, 12]) == [0, 1, 2]
+    e = row[EDG:EDG + 60].reshape(10, 6)
+    np.testing.assert_allclose(e[:, 0], np.arange(10) * 2.0)
+    np.testing.assert_allclose(e[:, 2], np.arange(1, 11) * 2.0)
+    np.testing.assert_array_equal(e[:-1, 3], e[1:, 1])         # polyline is continuous
+    assert (e[3:7, 1] == np.float32(H / 4)).all() and (e[2:7, 3] == np.float32(H / 4)).all()  # flat helipad
+    assert (e[:, 1] >= 0).all() and (e[:, 1] <= H / 2).all()
+    np.testing.assert_allclose(np.hypot(e[:, 4], e[:, 5]), 1.0, atol=1e-6)
+    j = row[JNT:JNT + 34].reshape(2, 17)
+    np.testing.assert_allclose(j[0, :10], [0, 0, 1, -20 / 30, -10 / 30, 0, 8 / 30, 0, 0.4, 0.9], rtol=1e-6)
+    np.testing.assert_allclose(j[1, :10], [0, 0, 2, 20 / 30, -10 / 30, 0, 8 / 30, 0, -0.9, -0.4], rtol=1e-6)
+    assert (j[:, 12] == 400).all() and (j[:, 13] == 40).all() and (j[:, 14] == 5).all()
+    # observation algebra from the constants: y_n = (H - (H/4 + (18/30)/30)) / (H/2)
+    y_n = (H - (H / 4 + 18 / 30 / 30)) / (H / 2)
+    obs = row[:8]
+    np.testing.assert_allclose(obs, [0, y_n, b[0, 3] * 10 / 50, b[0, 4] * (H / 2) / 50, 0, 0, 0, 0],
+                               rtol=1e-6, atol=1e-7)
+    shaping = -100 * math.hypot(obs[0], obs[1]) - 100 * math.hypot(obs[2], obs[3])
+    assert abs(row[META + 2] - shaping) < 1e-3 and row[META] == 0 and row[META + 3] == 0
+    # different env / seed -> different terrain and velocity; same -> identical
+    assert not np.array_equal(fresh(orc, 5, 1), row) and np.array_equal(fresh(orc, 5, 0), row)
+    assert orc.orc_ll_combined_seed(3, 4) == (3 * 2654435761 + 5 * 12345)
+
+
+def test_gravity_only_noop_steps(orc):
+    # the reference's own "gravity only" parity idea: 20 no-op steps, lander in free flight
+    row = fresh(orc)
+    vy0, y0, vx0 = row[BOD + 4], row[BOD + 1], row[BOD + 3]
+    for k in range(1, 21):
+        r, d, _, n = step(orc, row, 0)
+        assert n == 0 and d == 0.0 and row[META] == k
+    # the legs (4% of the mass each) swing in on their springs, so the hull only approximately free-falls
+    assert abs(row[BOD + 4] - (vy0 - 10 * 0.02 * 20)) < 0.3
+    assert abs(row[BOD + 3] - vx0) < 0.3
+    # whole-system linear momentum follows gravity exactly
+    m = np.array([5.0, 0.2, 0.2])
+    b = row[BOD:BOD + 39].reshape(3, 13)
+    np.testing.assert_allclose((m * b[:, 4]).sum() / m.sum(), vy0 - 4.0, atol=2e-3)
+    np.testing.assert_allclose((m * b[:, 3]).sum() / m.sum(), vx0, atol=2e-3)
+    # joints hold the legs on: anchors coincide to within slop-ish tolerance
+    for leg, ax in ((1, -20 / 30), (2, 20 / 30)):
+        a = b[0]
+        wa = (a[0] + ax * math.cos(a[2]) + 10 / 30 * math.sin(a[2]), a[1] + ax * math.sin(a[2]) - 10 / 30 * math.cos(a[2]))
+        l = b[leg]
+        wb = (l[0] - 8 / 30 * math.sin(l[2]), l[1] + 8 / 30 * math.cos(l[2]))
+        assert math.hypot(wa[0] - wb[0], wa[1] - wb[1]) < 0.02
+    # legs end up inside their angular limits
+    assert 0.35 < b[1, 2] - b[0, 2] < 0.95 and -0.95 < b[2, 2] - b[0, 2] < -0.35
+
+
+def test_reward_is_shaping_difference_minus_fuel(orc):
+    for action, fuel in ((0, 0.0), (2, 0.30), (1, 0.03), (3, 0.03)):
+        row = fresh(orc, 9)
+        prev = float(row[META + 2])
+        r, d, _, _ = step(orc, row, action)
+        o = row[:8]
+        sh = (-100 * math.hypot(o[0], o[1]) - 100 * math.hypot(o[2], o[3]) - 100 * abs(o[4])
+              + 10 * o[6] + 10 * o[7])
+        assert abs(r - (sh - prev - fuel)) < 2e-3 and abs(row[META + 2] - sh) < 1e-3
+        np.testing.assert_allclose(o[:2], [(row[BOD] - 10) / 10, (row[BOD + 1] - (H / 4 + 0.02)) / (H / 2)], rtol=1e-5, atol=1e-7)
+        np.testing.assert_allclose(o[2:6], [row[BOD + 3] * 10 / 50, row[BOD + 4] * (H / 2) / 50, row[BOD + 2], 20 * row[BOD + 5] / 50], rtol=1e-5, atol=1e-7)
+
+
+def test_main_engine_pushes_up_side_engines_turn(orc):
+    base = fresh(orc, 11)
+    rows = {a: base.copy() for a in range(4)}
+    for a, row in rows.items():
+        step(orc, row, a)
+    assert rows[2][BOD + 4] > rows[0][BOD + 4] + 0.2           # main engine: ~13*(4/30)/5 upward
+    assert abs((rows[2][BOD + 4] - rows[0][BOD + 4]) - 13 * (4 / 30) / 5) < 0.25
+    assert rows[1][BOD + 5] * rows[3][BOD + 5] < 0              # side engines spin opposite ways
+    # at angle 0: o_x = -(3 d_y + dir * 12/30) * (-1), impulse_x = -0.6 * o_x, dv_x = impulse_x / 5
+    assert abs((rows[1][BOD + 3] - rows[0][BOD + 3]) - (-0.6 * 0.4 / 5)) < 0.02
+    assert abs((rows[3][BOD + 3] - rows[0][BOD + 3]) - (+0.6 * 0.4 / 5)) < 0.02
+
+
+def test_dispersion_stream_depends_on_env_and_step(orc):
+    a, b = fresh(orc, 11), fresh(orc, 11)
+    step(orc, a, 2, env=0); step(orc, b, 2, env=1)
+    assert a[BOD + 3] != b[BOD + 3]
+    c = fresh(orc, 11)
+    c[META] = 5
+    step(orc, c, 2, env=0)
+    assert a[BOD + 3] != c[BOD + 3]
+
+
+def place(orc, x=10.0, y=None, vy=0.0, vx=0.0, angle=0.0):
+    """Lander (with legs attached at rest pose) moved rigidly; helipad terrain is flat at H/4."""
+    row = fresh(orc, 21)
+    b = row[BOD:BOD + 39].reshape(3, 13)
+    dy = (y if y is not None else b[0, 1]) - b[0, 1]
+    dx = x - b[0, 0]
+    b[:, 0] += dx; b[:, 1] += dy
+    b[:, 3] = vx; b[:, 4] = vy
+    b[0, 2] = angle
+    obs0 = np.zeros(8, np.float32)
+    return row
+
+
+def test_termination_table(orc):
+    # out of bounds: |x_norm| >= 1 -> reward == -100 exactly, done
+    row = place(orc, x=20.5)
+    r, d, _, _ = step(orc, row, 0)
+    assert (r, d) == (-100.0, 1.0) and row[META + 3] == 1.0
+    # done rows are frozen: reward 0, done 1, state untouched
+    snap = row.copy()
+    r, d, _, _ = step(orc, row, 2)
+    assert (r, d) == (0.0, 1.0) and np.array_equal(snap, row)
+    # hull touching the ground -> -100
+    row = place(orc, y=H / 4 + 0.2, vy=-1.0)
+    r, d, c, n = step(orc, row, 0)
+    assert n > 0 and 0 in c[:n * 9:9] and (r, d) == (-100.0, 1.0)
+    # step limit: the 1000th step ends the episode without touching the reward
+    row = fresh(orc, 21); row[META] = 999
+    r, d, _, _ = step(orc, row, 0)
+    assert d == 1.0 and abs(r) < 50 and row[META] == 1000
+    row = fresh(orc, 21); row[META] = 998
+    assert step(orc, row, 0)[1] == 0.0
+
+
+def test_landing_at_rest_bonus(orc):
+    # The at-rest branch is exercised with every body made static (inverse mass 0), which the
+    # integrator and both solvers leave untouched, standing on the pad with the hull clear of it.
+    def standing(vx=0.0, omega=0.0, lift=0.0):
+        row = place(orc, y=H / 4 + 1.195 + lift)
+        b = row[BOD:BOD + 39].reshape(3, 13)
+        b[:, 10:12] = 0.0
+        b[0, 3] = vx; b[0, 5] = omega
+        return row
+    row = standing()
+    prev = float(row[META + 2])
+    r, d, c, n = step(orc, row, 0)
+    o = row[:8]
+    assert n > 0 and 0 not in c[:n * 9:9]                   # only leg contacts
+    assert o[6] == 1.0 and o[7] == 1.0 and d == 1.0
+    sh = -100 * math.hypot(o[0], o[1]) + 20.0
+    assert abs(r - (sh - prev + 100.0)) < 1e-3              # bonus is ADDED to the shaping delta
+    # moving or spinning at or above the 0.01 thresholds: no bonus, episode continues
+    for kw in (dict(vx=0.011), dict(omega=-0.011)):
+        row = standing(**kw)
+        prev = float(row[META + 2])
+        r, d, _, _ = step(orc, row, 0)
+        assert d == 0.0 and abs(r - (float(row[META + 2]) - prev)) < 1e-3
+    # legs 0.025 above the pad (tolerance is 0.01): no leg contact, no bonus
+    row = standing(lift=0.03)
+    r, d, _, _ = step(orc, row, 0)
+    assert d == 0.0 and row[6] == 0.0
+
+
+def test_resting_contact_keeps_hull_off_the_ground(orc):
+    # drop onto the pad from 1.2 units: legs take the load, the hull never touches, no termination
+    row = place(orc, y=H / 4 + 1.4, vy=-0.2)
+    for _ in range(300):
+        r, d, c, n = step(orc, row, 0)
+        assert d == 0.0 and 0 not in c[:n * 9:9]
+    assert row[6] == 1.0 and row[7] == 1.0 and row[BOD + 1] > H / 4 + 0.5
+
+
+def test_batch_matches_single(orc):
+    n = 33
+    s = np.zeros((n, 192), np.float32)
+    orc.orc_ll_reset_batch(s, n, 77)
+    singles = np.stack([fresh(orc, 77, i) for i in range(n)])
+    np.testing.assert_array_equal(s, singles)
+    acts = (np.arange(n) % 4).astype(np.float32)
+    r, d, o = np.zeros(n, np.float32), np.zeros(n, np.float32), np.zeros((n, 8), np.float32)
+    for _ in range(5):
+        orc.orc_ll_step_batch(s, acts, r, d, o, n, 4)
+        for i in range(n):
+            step(orc, singles[i], int(acts[i]), env=i)
+    np.testing.assert_array_equal(s, singles)
+    np.testing.assert_array_equal(o, s[:, :8])
+    dn = np.zeros(n, np.float32); dn[3] = 1
+    s2 = s.copy()
+    orc.orc_ll_selective_reset_batch(s2, dn, n, 78)
+    assert np.array_equal(s2[np.arange(n) != 3], s[np.arange(n) != 3]) and s2[3, META] == 0
