@@ -1,0 +1,184 @@
+/*
+ * libmrl_hip.so -- C ABI of the MI355X (gfx950) rollout / PPO-update path for mojo-rl.
+ *
+ * Every entry point replaces one interface of the reference (cited per function as
+ * file:line under the reference tree).  Conventions:
+ *   - all data pointers are DEVICE pointers to fp32 buffers in the reference's own
+ *     layouts (row-major, obs at offset 0 of each env row, rollout buffers time-major);
+ *   - the caller owns every buffer; the library owns only its mrl_ctx;
+ *   - every call only enqueues work on the context's stream (no synchronisation),
+ *     like DeviceContext.enqueue_function in the reference;
+ *   - return value 0 = success; non-zero = failure, text in mrl_last_error()
+ *     (thread-local).  A Mojo shim turns non-zero into `raise Error(...)`.
+ */
+#ifndef MRL_H
+#define MRL_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mrl_ctx mrl_ctx;
+
+enum {
+    MRL_OK = 0,
+    MRL_E_ARG = -1,      /* bad argument (null pointer, size, unknown id) */
+    MRL_E_HIP = -2,      /* a HIP runtime call failed */
+    MRL_E_UNSUPPORTED = -3
+};
+
+enum mrl_env_id {
+    MRL_ENV_CARTPOLE = 0,    /* envs/cartpole.mojo:120 CartPoleEnv */
+    MRL_ENV_PENDULUM = 1,    /* envs/pendulum/pendulum_v2.mojo:57 PendulumV2 */
+    MRL_ENV_LUNARLANDER = 2, /* envs/lunar_lander/lunar_lander_v2.mojo:123 LunarLanderV2 */
+    MRL_ENV_BIPEDAL = 3,     /* envs/bipedal_walker/bipedal_walker_v2.mojo:103 BipedalWalkerV2 */
+    MRL_ENV_HALFCHEETAH = 4  /* envs/half_cheetah/cheetah_planar_v2.mojo:91 HalfCheetahPlanarV2 */
+};
+
+/* layer kinds of an MLP description; deep_rl/model/{linear,linear_relu,linear_tanh,stochastic_actor}.mojo */
+enum mrl_layer_kind {
+    MRL_LINEAR = 0,
+    MRL_LINEAR_RELU = 1,
+    MRL_LINEAR_TANH = 2,
+    MRL_STOCHASTIC_ACTOR = 3 /* out_dim = action_dim; output is [mean | clamped log_std] */
+};
+
+typedef struct {
+    int32_t kind;    /* mrl_layer_kind */
+    int32_t in_dim;
+    int32_t out_dim;
+} mrl_layer;
+
+#define MRL_MAX_LAYERS 8
+
+/* Seq2[...] nest flattened to its leaf layers; deep_rl/model/sequential.mojo:867-953 (seq()) */
+typedef struct {
+    int32_t n_layers;
+    mrl_layer layers[MRL_MAX_LAYERS];
+} mrl_mlp_desc;
+
+/* ------------------------------------------------------------------ library / context */
+
+int mrl_version(void);
+const char *mrl_last_error(void);
+
+/* hip_stream: a hipStream_t, or NULL for the default stream.  Replaces the DeviceContext
+ * argument every reference GPU method takes (one in-order stream). */
+int mrl_ctx_create(void *hip_stream, mrl_ctx **out);
+int mrl_ctx_destroy(mrl_ctx *ctx);
+/* blocks until the context's stream has drained; DeviceContext.synchronize() */
+int mrl_ctx_synchronize(mrl_ctx *ctx);
+
+/* ------------------------------------------------------------------ environments
+ * GPUDiscreteEnv / GPUContinuousEnv, core/env_traits.mojo:230-397:
+ *   comptime STATE_SIZE / OBS_DIM / NUM_ACTIONS / ACTION_DIM   -> mrl_env_dims
+ *   reset_kernel_gpu[B,S](ctx, states, rng_seed)               -> mrl_env_reset
+ *   selective_reset_kernel_gpu[B,S](ctx, states, dones, seed)  -> mrl_env_selective_reset
+ *   step_kernel_gpu[B,S,O](ctx, states, actions, rewards,
+ *                          dones, obs, rng_seed)               -> mrl_env_step
+ * states [batch, STATE_SIZE]; actions [batch] (discrete, stored as fp32) or
+ * [batch, ACTION_DIM]; rewards, dones [batch]; obs [batch, OBS_DIM].
+ * num_actions is 0 for continuous-only envs, action_dim 0 for discrete-only ones. */
+int mrl_env_dims(int env_id, int *state_size, int *obs_dim, int *num_actions, int *action_dim);
+int mrl_env_reset(mrl_ctx *ctx, int env_id, int batch, float *states, uint64_t seed);
+int mrl_env_selective_reset(mrl_ctx *ctx, int env_id, int batch, float *states, float *dones,
+                            uint64_t seed);
+int mrl_env_step(mrl_ctx *ctx, int env_id, int batch, float *states, const float *actions,
+                 float *rewards, float *dones, float *obs, uint64_t seed);
+/* step, then re-initialise rows that finished with the selective-reset protocol, then write
+ * obs from the (possibly fresh) row: the sequence step_kernel_gpu -> selective_reset_kernel_gpu
+ * -> _extract_obs_from_state_kernel of deep_agents/ppo/ppo.mojo:2148-2285 in one launch.
+ * rewards/dones report the step that just happened. */
+int mrl_env_step_autoreset(mrl_ctx *ctx, int env_id, int batch, float *states, const float *actions,
+                           float *rewards, float *dones, float *obs, uint64_t step_seed,
+                           uint64_t reset_seed);
+
+/* ------------------------------------------------------------------ MLP
+ * Model.forward_gpu_no_cache_ws / forward_gpu_ws / backward_gpu_ws,
+ * deep_rl/model/model.mojo:200-273; Seq2 chaining deep_rl/model/sequential.mojo:537-848.
+ * params [L0|L1|...], each [W (in x out, row-major) | b] (+ log_std for the actor head);
+ * cache (nullable) blocked per layer [batch x CACHE_i]; backward OVERWRITES grads.
+ * No workspace argument: intermediates stay on chip. */
+int mrl_mlp_param_size(const mrl_mlp_desc *desc);
+int mrl_mlp_cache_size(const mrl_mlp_desc *desc); /* floats per sample */
+int mrl_mlp_out_dim(const mrl_mlp_desc *desc);
+int mrl_mlp_forward(mrl_ctx *ctx, const mrl_mlp_desc *desc, int batch, const float *in,
+                    const float *params, float *out, float *cache);
+int mrl_mlp_backward(mrl_ctx *ctx, const mrl_mlp_desc *desc, int batch, const float *grad_out,
+                     const float *params, const float *cache, float *grads, float *grad_in);
+
+/* ------------------------------------------------------------------ PPO pieces */
+
+/* _sample_actions_kernel, deep_agents/ppo/ppo.mojo:4064-4123 */
+int mrl_sample_categorical(mrl_ctx *ctx, const float *logits, int n, int num_actions, uint32_t seed,
+                           float *actions, float *log_probs);
+/* _sample_continuous_actions_kernel, deep_agents/ppo/kernels.mojo:12-98 */
+int mrl_sample_gaussian(mrl_ctx *ctx, const float *actor_out, int n, int action_dim, uint32_t seed,
+                        float *actions, float *log_probs);
+/* host GAE loop of train_gpu, deep_agents/ppo/ppo.mojo:2317-2353 (time-major, idx = t*N + env) */
+int mrl_gae(mrl_ctx *ctx, int T, int N, const float *rewards, const float *values,
+            const float *dones, const float *bootstrap, double gamma, double lam, float *adv,
+            float *ret);
+/* (x - mean) / (sqrt(var + 1e-8) + 1e-8) in place: ppo.mojo:2356-2371, :2478-2511 + :637-653,
+ * kernels.mojo:507-599 */
+int mrl_normalize_advantages(mrl_ctx *ctx, float *x, int n);
+/* ppo_gather_minibatch_kernel ppo.mojo:135-191 / kernels.mojo:161-226: rows of the rollout
+ * buffers picked by int32 indices */
+int mrl_gather_minibatch(mrl_ctx *ctx, const int32_t *indices, int mb, int obs_dim, int act_dim,
+                         const float *r_obs, const float *r_actions, const float *r_adv,
+                         const float *r_ret, const float *r_logp, const float *r_values,
+                         float *mb_obs, float *mb_actions, float *mb_adv, float *mb_ret,
+                         float *mb_logp, float *mb_values);
+/* ppo_actor_grad_with_kl_kernel, ppo.mojo:285-378 */
+int mrl_ppo_actor_grad_discrete(mrl_ctx *ctx, const float *logits, const float *old_log_probs,
+                                const float *advantages, const float *actions, int mb,
+                                int num_actions, float clip_eps, float entropy_coef,
+                                float *grad_logits, float *kl);
+/* ppo_continuous_actor_grad_kernel, kernels.mojo:230-412 */
+int mrl_ppo_actor_grad_gaussian(mrl_ctx *ctx, const float *actor_out, const float *old_log_probs,
+                                const float *advantages, const float *actions, int mb,
+                                int action_dim, float clip_eps, float entropy_coef, float *grad_out,
+                                float *kl);
+/* convention 0: ppo.mojo:538-633 (2*c_v*(V-R)/MB); convention 1: kernels.mojo:416-486 ((V-R)/MB) */
+int mrl_ppo_critic_grad(mrl_ctx *ctx, const float *values, const float *old_values,
+                        const float *returns, int mb, int convention, int clipped, float value_coef,
+                        float clip_eps, float *grad_values);
+/* gradient_norm_kernel + reduce + apply, ppo.mojo:382-534 / kernels.mojo:603-805; in place */
+int mrl_clip_grad_norm(mrl_ctx *ctx, float *grads, int n, float max_norm);
+/* Adam.step_gpu, deep_rl/optimizer/adam.mojo:52-105, :162-247.  t is the optimiser's step count
+ * AFTER the increment (1 on the first call); state is [n, 2] interleaved (m, v). */
+int mrl_adam_step(mrl_ctx *ctx, float *params, const float *grads, float *state, int n, int t,
+                  double lr, double beta1, double beta2, double eps);
+/* clamp_log_std_params_kernel, kernels.mojo:842-873 */
+int mrl_clamp_log_std(mrl_ctx *ctx, float *params, int offset, int action_dim);
+
+/* ------------------------------------------------------------------ fused rollout step
+ * One time step of train_gpu's collection loop for a discrete-action env
+ * (deep_agents/ppo/ppo.mojo:2069-2285): actor + critic forward on obs, categorical
+ * sampling, store of (obs, action, log_prob, value) into rollout row t, env step with
+ * auto-reset, store of (reward, done), episode accounting.  The rollout buffers are the
+ * reference's time-major ones ([T*N, ...], row = t*N + env); ep_return / ep_length are
+ * the per-env accumulators of deep_rl/gpu/rl_kernels.mojo:103-227; finished episodes are
+ * appended to done_returns / done_lengths (capacity done_cap) through the counter
+ * done_count instead of being copied to the host every step. */
+typedef struct {
+    int32_t env_id, n_envs, obs_dim, num_actions;
+    float *states, *obs;                     /* [N, STATE_SIZE], [N, OBS] current observation */
+    const float *actor_params, *critic_params;
+    mrl_mlp_desc actor, critic;
+    float *r_obs, *r_actions, *r_log_probs, *r_values, *r_rewards, *r_dones; /* rollout buffers */
+    float *ep_return, *ep_length;            /* [N] */
+    float *done_returns, *done_lengths;      /* [done_cap] */
+    int32_t *done_count;                     /* [1] */
+    int32_t done_cap;
+} mrl_rollout;
+
+int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_seed,
+                     uint64_t step_seed, uint64_t reset_seed);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,16 @@
+"""MI355X-native rollout / PPO-update path for mojo-rl, behind the reference's own interfaces.
+
+The compute lives in libmrl_hip.so (hand-written gfx950 kernels, C ABI in include/mrl.h);
+this package is the host-side mirror of the reference's env / model / optimizer traits.
+Importing it loads the library and fails loudly if it is missing.
+"""
+from . import _lib
+from ._lib import MrlError, LINEAR, LINEAR_RELU, LINEAR_TANH, STOCHASTIC_ACTOR
+
+_lib.lib()  # load now: a missing or unloadable HIP library is an import error, not a fallback
+
+from .context import DeviceContext  # noqa: E402
+from .envs import CartPoleEnv, PendulumV2, LunarLanderV2  # noqa: E402
+
+__all__ = ["DeviceContext", "CartPoleEnv", "PendulumV2", "LunarLanderV2", "MrlError",
+           "LINEAR", "LINEAR_RELU", "LINEAR_TANH", "STOCHASTIC_ACTOR"]

@@ -1,0 +1,53 @@
+"""DeviceContext: the one in-order stream every reference GPU method takes as `ctx`.
+
+Mirrors the subset of Mojo's gpu.host.DeviceContext that the rollout / update path uses
+(enqueue_create_buffer, enqueue_memset, synchronize); buffers are torch tensors on the GPU.
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise _lib.MrlError("device buffer expected, got a %s tensor" % t.device)
+    if not t.is_contiguous():
+        raise _lib.MrlError("device buffers must be contiguous")
+    return t.data_ptr()
+
+
+class DeviceContext:
+    def __init__(self, device="cuda:0", stream=None):
+        if not torch.cuda.is_available():
+            raise _lib.MrlError("no GPU visible: the MI355X path has no CPU fallback")
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        self.stream = stream if stream is not None else torch.cuda.current_stream(self.device)
+        handle = C.c_void_p()
+        _lib.call("mrl_ctx_create", C.c_void_p(self.stream.cuda_stream), C.byref(handle))
+        self.handle = handle
+
+    def enqueue_create_buffer(self, n, dtype=torch.float32):
+        return torch.empty(n, dtype=dtype, device=self.device)
+
+    def enqueue_memset(self, buf, value):
+        with torch.cuda.stream(self.stream):
+            buf.fill_(value)
+
+    def synchronize(self):
+        _lib.call("mrl_ctx_synchronize", self.handle)
+
+    def close(self):
+        if self.handle:
+            _lib.call("mrl_ctx_destroy", self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,61 @@
+// Context lifetime and error reporting of libmrl_hip.so.
+#include "mrl_host.hpp"
+#include "env_lunar.hpp"
+
+namespace mrl {
+
+static thread_local char g_error[512] = "";
+
+int set_error(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+}  // namespace mrl
+
+extern "C" {
+
+int mrl_version(void) { return 100; }
+
+const char *mrl_last_error(void) { return mrl::g_error; }
+
+int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
+    MRL_CHECK_ARG(out != nullptr, "mrl_ctx_create: out is NULL");
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0)
+        return mrl::set_error(MRL_E_HIP, "mrl_ctx_create: no HIP device (%s)", hipGetErrorString(e));
+    mrl_ctx *c = new mrl_ctx();
+    c->stream = (hipStream_t)hip_stream;
+    MRL_CHECK_HIP(hipGetDevice(&c->device));
+    c->ll_shapes = nullptr;
+    c->reduce_scratch = nullptr;
+    c->reduce_scratch_floats = 4096;
+    MRL_CHECK_HIP(hipMalloc(&c->ll_shapes, sizeof(mrl::ll::Shapes)));
+    mrl::ll::Shapes sh = mrl::ll::make_shapes();
+    MRL_CHECK_HIP(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));
+    MRL_CHECK_HIP(hipMalloc(&c->reduce_scratch, sizeof(float) * c->reduce_scratch_floats));
+    *out = c;
+    return MRL_OK;
+}
+
+int mrl_ctx_destroy(mrl_ctx *ctx) {
+    if (!ctx) return MRL_OK;
+    hipStreamSynchronize(ctx->stream);
+    for (auto &kv : ctx->cartpole_steps) hipFree(kv.second.steps);
+    if (ctx->ll_shapes) hipFree(ctx->ll_shapes);
+    if (ctx->reduce_scratch) hipFree(ctx->reduce_scratch);
+    delete ctx;
+    return MRL_OK;
+}
+
+int mrl_ctx_synchronize(mrl_ctx *ctx) {
+    MRL_CHECK_ARG(ctx != nullptr, "mrl_ctx_synchronize: ctx is NULL");
+    MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    return MRL_OK;
+}
+
+}  // extern "C"

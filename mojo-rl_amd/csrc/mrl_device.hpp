@@ -1,0 +1,72 @@
+// Device-side helpers shared by the gfx950 kernels: numeric conventions and random streams.
+//
+// Numeric conventions (they are what make results reproducible against a CPU statement
+// of the same arithmetic):
+//   * every translation unit is built with -ffp-contract=off: a*b+c is two roundings
+//     unless fmaf() is written out;
+//   * fp32 sin/cos of an fp32 angle are the correctly rounded values, computed through
+//     the fp64 routine and rounded once;
+//   * fp32 divide and sqrt are IEEE (hipcc default for gfx9).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define MRL_DEV __device__ __forceinline__
+
+namespace mrl {
+
+MRL_DEV float sin32(float x) { return (float)::sin((double)x); }
+MRL_DEV float cos32(float x) { return (float)::cos((double)x); }
+MRL_DEV void sincos32(float x, float &s, float &c) {
+    double ds, dc;
+    ::sincos((double)x, &ds, &dc);
+    s = (float)ds;
+    c = (float)dc;
+}
+
+// deep_rl/gpu/random.mojo:11-43
+MRL_DEV uint32_t xorshift32(uint32_t x) {
+    x ^= x << 13;
+    x ^= x >> 17;
+    x ^= x << 5;
+    return x;
+}
+MRL_DEV float random_uniform(uint32_t &state) {
+    state = xorshift32(state);
+    return (float)state / (float)0xFFFFFFFFu;
+}
+MRL_DEV float random_range(uint32_t &state, float lo, float hi) {
+    float u = random_uniform(state);
+    return lo + u * (hi - lo);
+}
+
+// Philox4x32-10 (Random123).  key = (seed lo, hi); counter = (offset lo, hi, 0, 0) + call;
+// uniform = float(x & 0x7fffffff) * 4.6566127342e-10f  -- the stream layout of
+// random.philox.Random(seed, offset).step_uniform() that the reference draws from.
+struct Uniform4 { float v[4]; };
+
+MRL_DEV Uniform4 philox_uniform4(uint64_t seed, uint64_t offset, uint64_t call_index) {
+    uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+    uint64_t lo = offset + call_index;
+    uint32_t c0 = (uint32_t)lo, c1 = (uint32_t)(lo >> 32), c2 = (lo < offset) ? 1u : 0u, c3 = 0u;
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+        uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+        uint32_t n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        uint32_t n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    Uniform4 u;
+    u.v[0] = (float)(c0 & 0x7FFFFFFFu) * 4.6566127342e-10f;
+    u.v[1] = (float)(c1 & 0x7FFFFFFFu) * 4.6566127342e-10f;
+    u.v[2] = (float)(c2 & 0x7FFFFFFFu) * 4.6566127342e-10f;
+    u.v[3] = (float)(c3 & 0x7FFFFFFFu) * 4.6566127342e-10f;
+    return u;
+}
+
+}  // namespace mrl

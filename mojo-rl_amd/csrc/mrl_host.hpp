@@ -1,0 +1,45 @@
+// Host-side plumbing shared by the translation units of libmrl_hip.so: the context object,
+// the thread-local error string and launch helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include <unordered_map>
+#include "../../include/mrl.h"
+
+struct mrl_ctx {
+    hipStream_t stream;
+    int device;
+    // CartPole keeps its per-env step counter (truncation at 500) outside the [B,4] state rows;
+    // one int32[batch] array per states pointer, created on first use, freed with the context.
+    struct Side { int32_t *steps; int batch; };
+    std::unordered_map<const void *, Side> cartpole_steps;
+    // device copy of the shape tables (filled at context creation)
+    float *ll_shapes;
+    // scratch for two-pass reductions (grad-norm partial sums, advantage statistics)
+    float *reduce_scratch;
+    int reduce_scratch_floats;
+};
+
+namespace mrl {
+
+int set_error(int code, const char *fmt, ...);
+
+inline int grid_for(long n, int block) { return (int)((n + block - 1) / block); }
+
+}  // namespace mrl
+
+#define MRL_CHECK_ARG(cond, ...)                                   \
+    do {                                                           \
+        if (!(cond)) return mrl::set_error(MRL_E_ARG, __VA_ARGS__); \
+    } while (0)
+
+#define MRL_CHECK_HIP(expr)                                                              \
+    do {                                                                                 \
+        hipError_t _e = (expr);                                                          \
+        if (_e != hipSuccess)                                                            \
+            return mrl::set_error(MRL_E_HIP, "%s failed: %s", #expr, hipGetErrorString(_e)); \
+    } while (0)
+
+#define MRL_CHECK_LAUNCH() MRL_CHECK_HIP(hipGetLastError())

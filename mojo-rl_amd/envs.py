@@ -1,0 +1,77 @@
+"""Batched environments behind the reference's GPUDiscreteEnv / GPUContinuousEnv traits.
+
+core/env_traits.mojo:230-397 declares, per environment type, the compile-time constants
+STATE_SIZE / OBS_DIM / NUM_ACTIONS / ACTION_DIM and three static methods
+    step_kernel_gpu[BATCH, STATE_SIZE, OBS_DIM](ctx, states, actions, rewards, dones, obs, rng_seed)
+    reset_kernel_gpu[BATCH, STATE_SIZE](ctx, states, rng_seed)
+    selective_reset_kernel_gpu[BATCH, STATE_SIZE](ctx, states, dones, rng_seed)
+over flat fp32 device buffers.  The classes below keep those names and argument meanings; the
+compile-time BATCH becomes the leading size of the buffers.  All calls only enqueue.
+"""
+from . import _lib
+from .context import _ptr
+
+
+class _GPUEnv:
+    ENV_ID = -1
+    STATE_SIZE = 0
+    OBS_DIM = 0
+    NUM_ACTIONS = 0   # discrete envs
+    ACTION_DIM = 0    # continuous envs
+
+    @classmethod
+    def _batch(cls, states):
+        n = states.numel()
+        if n % cls.STATE_SIZE:
+            raise _lib.MrlError("states buffer of %d floats is not a multiple of STATE_SIZE=%d"
+                                % (n, cls.STATE_SIZE))
+        return n // cls.STATE_SIZE
+
+    @classmethod
+    def _check(cls, batch, actions=None, rewards=None, dones=None, obs=None):
+        aw = cls.ACTION_DIM if cls.ACTION_DIM else 1
+        for name, t, want in (("actions", actions, batch * aw), ("rewards", rewards, batch),
+                              ("dones", dones, batch), ("obs", obs, batch * cls.OBS_DIM)):
+            if t is not None and t.numel() != want:
+                raise _lib.MrlError("%s buffer holds %d floats, expected %d" % (name, t.numel(), want))
+
+    @classmethod
+    def step_kernel_gpu(cls, ctx, states, actions, rewards, dones, obs, rng_seed=0):
+        b = cls._batch(states)
+        cls._check(b, actions, rewards, dones, obs)
+        _lib.call("mrl_env_step", ctx.handle, cls.ENV_ID, b, _ptr(states), _ptr(actions),
+                  _ptr(rewards), _ptr(dones), _ptr(obs), int(rng_seed) & (2**64 - 1))
+
+    @classmethod
+    def reset_kernel_gpu(cls, ctx, states, rng_seed=0):
+        _lib.call("mrl_env_reset", ctx.handle, cls.ENV_ID, cls._batch(states), _ptr(states),
+                  int(rng_seed) & (2**64 - 1))
+
+    @classmethod
+    def selective_reset_kernel_gpu(cls, ctx, states, dones, rng_seed):
+        b = cls._batch(states)
+        cls._check(b, dones=dones)
+        _lib.call("mrl_env_selective_reset", ctx.handle, cls.ENV_ID, b, _ptr(states), _ptr(dones),
+                  int(rng_seed) & (2**64 - 1))
+
+    @classmethod
+    def step_autoreset_kernel_gpu(cls, ctx, states, actions, rewards, dones, obs, step_seed=0,
+                                  reset_seed=0):
+        """step_kernel_gpu, selective_reset_kernel_gpu and the obs extraction in one launch."""
+        b = cls._batch(states)
+        cls._check(b, actions, rewards, dones, obs)
+        _lib.call("mrl_env_step_autoreset", ctx.handle, cls.ENV_ID, b, _ptr(states), _ptr(actions),
+                  _ptr(rewards), _ptr(dones), _ptr(obs), int(step_seed) & (2**64 - 1),
+                  int(reset_seed) & (2**64 - 1))
+
+
+class CartPoleEnv(_GPUEnv):           # envs/cartpole.mojo:120
+    ENV_ID, STATE_SIZE, OBS_DIM, NUM_ACTIONS = _lib.ENV_CARTPOLE, 4, 4, 2
+
+
+class PendulumV2(_GPUEnv):            # envs/pendulum/pendulum_v2.mojo:57
+    ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_PENDULUM, 8, 3, 1
+
+
+class LunarLanderV2(_GPUEnv):         # envs/lunar_lander/lunar_lander_v2.mojo:123
+    ENV_ID, STATE_SIZE, OBS_DIM, NUM_ACTIONS = _lib.ENV_LUNARLANDER, 192, 8, 4

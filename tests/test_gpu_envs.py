@@ -1,0 +1,230 @@
+"""GPU parity: env kernels (through the C ABI) against the CPU oracle on identical seeded inputs.
+
+Bar: per-step fp32 state and observations within 1e-5 relative (1e-6 absolute); reward and done
+flags exact over the first 64 steps.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-5, 1e-6
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ctx(mrl):
+    return mrl.DeviceContext("cuda:0")
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def close(a, b):
+    np.testing.assert_allclose(a, b, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("batch", [1, 63, 4096])
+def test_cartpole_rollout_parity(mrl, orc, ctx, batch):
+    say("cartpole batch", batch)
+    E = mrl.CartPoleEnv
+    s_h = np.zeros((batch, 4), np.float32); st_h = np.zeros(batch, np.int32)
+    orc.orc_cartpole_reset_batch(s_h, st_h, batch, 12345)
+    s = torch.zeros(batch * 4, device="cuda")
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch, batch * 4))
+    E.reset_kernel_gpu(ctx, s, 0)
+    ctx.synchronize()
+    np.testing.assert_array_equal(s.cpu().numpy().reshape(batch, 4), s_h)
+    rng = np.random.default_rng(0)
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 4), np.float32)
+    for t in range(64):
+        act = rng.integers(0, 2, batch).astype(np.float32)
+        a.copy_(dev(act))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_cartpole_step_batch(s_h, st_h, act, r_h, d_h, o_h, batch)
+        ctx.synchronize()
+        close(s.cpu().numpy().reshape(batch, 4), s_h)
+        close(o.cpu().numpy().reshape(batch, 4), o_h)
+        np.testing.assert_array_equal(r.cpu().numpy(), r_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        seed = 1000 + t
+        E.selective_reset_kernel_gpu(ctx, s, d, seed)
+        orc.orc_cartpole_selective_reset_batch(s_h, st_h, d_h, batch, seed)
+        ctx.synchronize()
+        np.testing.assert_array_equal(s.cpu().numpy().reshape(batch, 4), s_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+
+
+def test_cartpole_truncation_counter(mrl, orc, ctx):
+    # always push towards the centre: the pole survives past 500 steps only by truncation
+    batch = 8
+    E = mrl.CartPoleEnv
+    s = torch.zeros(batch * 4, device="cuda")
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch, batch * 4))
+    E.reset_kernel_gpu(ctx, s, 0)
+    s_h = np.zeros((batch, 4), np.float32); st_h = np.zeros(batch, np.int32)
+    orc.orc_cartpole_reset_batch(s_h, st_h, batch, 12345)
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 4), np.float32)
+    saw_trunc = False
+    for t in range(520):
+        act = (s_h[:, 2] + 0.5 * s_h[:, 3] > 0).astype(np.float32)   # bang-bang on the angle
+        a.copy_(dev(act))
+        E.step_kernel_gpu(ctx, s, a, r, d, o)
+        orc.orc_cartpole_step_batch(s_h, st_h, act, r_h, d_h, o_h, batch)
+        ctx.synchronize()
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        np.testing.assert_array_equal(r.cpu().numpy(), r_h)
+        saw_trunc |= bool(((d_h > 0.5) & (r_h > 0.5)).any())
+        E.selective_reset_kernel_gpu(ctx, s, d, t)
+        orc.orc_cartpole_selective_reset_batch(s_h, st_h, d_h, batch, t)
+    assert saw_trunc
+
+
+@pytest.mark.parametrize("batch", [1, 257, 16384])
+def test_pendulum_rollout_parity(mrl, orc, ctx, batch):
+    say("pendulum batch", batch)
+    E = mrl.PendulumV2
+    s_h = np.zeros((batch, 8), np.float32)
+    orc.orc_pendulum_reset_batch(s_h, batch, 42)
+    s = torch.zeros(batch * 8, device="cuda")
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch, batch * 3))
+    E.reset_kernel_gpu(ctx, s, 42)
+    ctx.synchronize()
+    close(s.cpu().numpy().reshape(batch, 8), s_h)
+    rng = np.random.default_rng(1)
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 3), np.float32)
+    s_h[:, 4] = 150; s[4::8] = 150                        # so the 200-step truncation falls inside the test
+    for t in range(64):
+        act = rng.uniform(-1.3, 1.3, batch).astype(np.float32)
+        a.copy_(dev(act))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_pendulum_step_batch(s_h, act, r_h, d_h, o_h, batch)
+        ctx.synchronize()
+        close(s.cpu().numpy().reshape(batch, 8), s_h)
+        close(o.cpu().numpy().reshape(batch, 3), o_h)
+        close(r.cpu().numpy(), r_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        s_h[:] = s.cpu().numpy().reshape(batch, 8)        # re-synchronise: per-step parity, not drift
+        E.selective_reset_kernel_gpu(ctx, s, d, 7 + t)
+        orc.orc_pendulum_selective_reset_batch(s_h, d_h, batch, 7 + t)
+        ctx.synchronize()
+        close(s.cpu().numpy().reshape(batch, 8), s_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        s_h[:] = s.cpu().numpy().reshape(batch, 8)
+
+
+def ll_policy(rng, obs, t):
+    """A seeded stand-in policy that fires engines often enough to exercise every action."""
+    a = rng.integers(0, 4, obs.shape[0])
+    a[obs[:, 3] < -0.3] = 2                                 # falling fast: main engine
+    return a.astype(np.float32)
+
+
+@pytest.mark.parametrize("batch,seed", [(1, 3), (65, 4), (8192, 5)])
+def test_lunar_lander_rollout_parity(mrl, orc, ctx, batch, seed):
+    say("lunar batch", batch)
+    E = mrl.LunarLanderV2
+    s_h = np.zeros((batch, 192), np.float32)
+    orc.orc_ll_reset_batch(s_h, batch, seed)
+    s = torch.full((batch * 192,), 7.0, device="cuda")     # garbage: reset must write every float
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch, batch * 8))
+    E.reset_kernel_gpu(ctx, s, seed)
+    ctx.synchronize()
+    close(s.cpu().numpy().reshape(batch, 192), s_h)
+    s_h[:] = s.cpu().numpy().reshape(batch, 192)
+    rng = np.random.default_rng(seed)
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 8), np.float32)
+    n_done = 0
+    for t in range(64):
+        act = ll_policy(rng, s_h[:, :8], t)
+        a.copy_(dev(act))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_ll_step_batch(s_h, act, r_h, d_h, o_h, batch, 8)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 192)
+        close(sg, s_h)
+        close(o.cpu().numpy().reshape(batch, 8), o_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        np.testing.assert_array_equal(r.cpu().numpy(), r_h)   # reward exact
+        n_done += int(d_h.sum())
+        s_h[:] = sg
+    say("  finished rows seen:", n_done)
+
+
+def test_lunar_lander_contacts_and_reset_cycle(mrl, orc, ctx):
+    # start low over the pad so that contacts, crashes and landings all occur within 64 steps
+    batch = 2048
+    E = mrl.LunarLanderV2
+    s_h = np.zeros((batch, 192), np.float32)
+    orc.orc_ll_reset_batch(s_h, batch, 11)
+    rng = np.random.default_rng(11)
+    b = s_h[:, 8:47].reshape(batch, 3, 13)
+    drop = rng.uniform(7.5, 9.4, batch).astype(np.float32)
+    b[:, :, 1] -= drop[:, None]
+    b[:, :, 0] += rng.uniform(-6, 6, batch).astype(np.float32)[:, None]
+    b[:, 0, 2] = rng.uniform(-0.4, 0.4, batch).astype(np.float32)
+    s = dev(s_h.reshape(-1))
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch, batch * 8))
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 8), np.float32)
+    crashes = lands = 0
+    for t in range(64):
+        act = rng.integers(0, 4, batch).astype(np.float32)
+        a.copy_(dev(act))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_ll_step_batch(s_h, act, r_h, d_h, o_h, batch, 8)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 192)
+        close(sg, s_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        np.testing.assert_array_equal(r.cpu().numpy(), r_h)
+        crashes += int((r_h == -100).sum()); lands += int((o_h[:, 6] + o_h[:, 7] > 0).sum())
+        s_h[:] = sg
+        E.selective_reset_kernel_gpu(ctx, s, d, 900 + t)
+        orc.orc_ll_selective_reset_batch(s_h, d_h, batch, 900 + t)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 192)
+        close(sg, s_h)
+        s_h[:] = sg
+    say("  crashes", crashes, "leg-contact observations", lands)
+    assert crashes > 50 and lands > 500
+
+
+def test_lunar_lander_autoreset_equals_step_then_selective_reset(mrl, ctx):
+    batch = 1000
+    E = mrl.LunarLanderV2
+    s1 = torch.zeros(batch * 192, device="cuda")
+    E.reset_kernel_gpu(ctx, s1, 21)
+    s1.view(batch, 192)[:, 188] = torch.randint(990, 1000, (batch,), device="cuda").float()  # near the step limit
+    s2 = s1.clone()
+    bufs = lambda: tuple(torch.zeros(n, device="cuda") for n in (batch, batch, batch * 8))
+    r1, d1, o1 = bufs(); r2, d2, o2 = bufs()
+    a = torch.randint(0, 4, (batch,), device="cuda").float()
+    for t in range(12):
+        E.step_kernel_gpu(ctx, s1, a, r1, d1, o1, t)
+        E.selective_reset_kernel_gpu(ctx, s1, d1, 50 + t)
+        E.step_autoreset_kernel_gpu(ctx, s2, a, r2, d2, o2, t, 50 + t)
+        ctx.synchronize()
+        assert torch.equal(s1, s2) and torch.equal(r1, r2) and torch.equal(d1, d2)
+        assert torch.equal(o2.view(batch, 8), s2.view(batch, 192)[:, :8])
+    assert d1.sum() >= 0
+
+
+def test_env_argument_errors(mrl, ctx):
+    s = torch.zeros(10, device="cuda")
+    with pytest.raises(mrl.MrlError):
+        mrl.LunarLanderV2.reset_kernel_gpu(ctx, s, 0)            # not a multiple of STATE_SIZE
+    s = torch.zeros(192, device="cuda")
+    with pytest.raises(mrl.MrlError):
+        mrl.LunarLanderV2.step_kernel_gpu(ctx, s, torch.zeros(2, device="cuda"), torch.zeros(1, device="cuda"),
+                                          torch.zeros(1, device="cuda"), torch.zeros(8, device="cuda"))
+    with pytest.raises(mrl.MrlError):
+        mrl.LunarLanderV2.reset_kernel_gpu(ctx, torch.zeros(192), 0)  # host tensor
+    empty = torch.zeros(0, device="cuda")
+    mrl.LunarLanderV2.reset_kernel_gpu(ctx, empty, 0)            # empty batch is a no-op
