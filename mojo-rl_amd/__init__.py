@@ -11,6 +11,10 @@ _lib.lib()  # load now: a missing or unloadable HIP library is an import error, 
 
 from .context import DeviceContext  # noqa: E402
 from .envs import CartPoleEnv, PendulumV2, LunarLanderV2  # noqa: E402
+from .model import Model, Linear, LinearReLU, LinearTanh, StochasticActor, seq  # noqa: E402
+from .optimizer import Adam  # noqa: E402
+from . import ppo  # noqa: E402
 
-__all__ = ["DeviceContext", "CartPoleEnv", "PendulumV2", "LunarLanderV2", "MrlError",
+__all__ = ["DeviceContext", "CartPoleEnv", "PendulumV2", "LunarLanderV2", "MrlError", "Model",
+           "Linear", "LinearReLU", "LinearTanh", "StochasticActor", "seq", "Adam", "ppo",
            "LINEAR", "LINEAR_RELU", "LINEAR_TANH", "STOCHASTIC_ACTOR"]

@@ -34,6 +34,10 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     c->ll_shapes = nullptr;
     c->reduce_scratch = nullptr;
     c->reduce_scratch_floats = 4096;
+    c->mlp_ws = nullptr;
+    c->mlp_ws_floats = 0;
+    c->rollout_ws = nullptr;
+    c->rollout_ws_floats = 0;
     MRL_CHECK_HIP(hipMalloc(&c->ll_shapes, sizeof(mrl::ll::Shapes)));
     mrl::ll::Shapes sh = mrl::ll::make_shapes();
     MRL_CHECK_HIP(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));
@@ -48,6 +52,8 @@ int mrl_ctx_destroy(mrl_ctx *ctx) {
     for (auto &kv : ctx->cartpole_steps) hipFree(kv.second.steps);
     if (ctx->ll_shapes) hipFree(ctx->ll_shapes);
     if (ctx->reduce_scratch) hipFree(ctx->reduce_scratch);
+    if (ctx->mlp_ws) hipFree(ctx->mlp_ws);
+    if (ctx->rollout_ws) hipFree(ctx->rollout_ws);
     delete ctx;
     return MRL_OK;
 }

@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <algorithm>
 #include <unordered_map>
 #include "../../include/mrl.h"
 
@@ -20,6 +21,13 @@ struct mrl_ctx {
     // scratch for two-pass reductions (grad-norm partial sums, advantage statistics)
     float *reduce_scratch;
     int reduce_scratch_floats;
+    // MLP workspace: activations between layers and split-batch partial gradients; grown on demand
+    float *mlp_ws;
+    size_t mlp_ws_floats;
+    // per-step temporaries of the fused rollout step (logits, values, actions, log-probs,
+    // rewards, dones for n_envs), grown on demand
+    float *rollout_ws;
+    size_t rollout_ws_floats;
 };
 
 namespace mrl {

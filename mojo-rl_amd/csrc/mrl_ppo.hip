@@ -1,0 +1,544 @@
+// PPO elementwise and reduction kernels: samplers, GAE, advantage normalisation, minibatch
+// gather, loss gradients, global-norm clipping, Adam.  All are HBM-bound: one pass over the
+// data, coalesced, reductions by wavefront shuffles and one small second stage.
+#include "mrl_host.hpp"
+#include "mrl_device.hpp"
+
+namespace mrl {
+
+constexpr int TPB = 256;
+
+MRL_DEV float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// block sum, result valid in every lane of wavefront 0 (and in thread 0)
+MRL_DEV float block_sum(float v, float *smem) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    float r = 0.0f;
+    if (w == 0) {
+        r = (lane < (int)(blockDim.x >> 6)) ? smem[lane] : 0.0f;
+        r = wave_sum(r);
+    }
+    __syncthreads();
+    return r;
+}
+
+// ---------------------------------------------------------------- samplers
+
+// deep_agents/ppo/ppo.mojo:4064-4123
+__global__ __launch_bounds__(TPB) void sample_categorical_kernel(const float *__restrict__ logits,
+                                                                 int n, int A, uint32_t seed,
+                                                                 float *__restrict__ actions,
+                                                                 float *__restrict__ log_probs) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float *l = logits + (long)i * A;
+    uint32_t rng = seed ^ ((uint32_t)i * 2654435761u);
+    rng = xorshift32(rng);
+    float max_logit = l[0];
+    for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
+    float sum_exp = 0.0f;
+    for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
+    float u = random_uniform(rng);
+    float cumsum = 0.0f;
+    int sel = 0;
+    for (int a = 0; a < A; ++a) {
+        float prob = expf(l[a] - max_logit) / sum_exp;
+        cumsum = cumsum + prob;
+        if (u < cumsum) { sel = a; break; }
+    }
+    actions[i] = (float)sel;
+    float p = expf(l[sel] - max_logit) / sum_exp;
+    log_probs[i] = logf(p + 1e-8f);
+}
+
+// deep_agents/ppo/kernels.mojo:12-98
+__global__ __launch_bounds__(TPB) void sample_gaussian_kernel(const float *__restrict__ actor_out,
+                                                              int n, int A, uint32_t seed,
+                                                              float *__restrict__ actions,
+                                                              float *__restrict__ log_probs) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
+    float total = 0.0f;
+    for (int j = 0; j < A; ++j) {
+        float mean = actor_out[(long)i * 2 * A + j];
+        float log_std = actor_out[(long)i * 2 * A + A + j];
+        if (log_std < -5.0f) log_std = -5.0f;
+        else if (log_std > 2.0f) log_std = 2.0f;
+        Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j), 0, 0);
+        float u1 = rv.v[0] + 1e-8f;
+        float mag = sqrtf(-2.0f * logf(u1));
+        float noise = mag * cosf(rv.v[1] * (float)6.283185307179586);
+        float std = expf(log_std);
+        float action = mean + std * noise;
+        actions[(long)i * A + j] = action;
+        float an = (action - mean) / (std + EPS);
+        float lg = -0.5f * (LOG_2PI + 2.0f * log_std + an * an);
+        total = total + lg;
+    }
+    log_probs[i] = total;
+}
+
+// ---------------------------------------------------------------- GAE
+// One lane per env scans t = T-1 .. 0; index t*N + env makes every step of the scan a
+// coalesced row access.  deep_agents/ppo/ppo.mojo:2317-2353
+__global__ __launch_bounds__(TPB) void gae_kernel(int T, int N, const float *__restrict__ rewards,
+                                                  const float *__restrict__ values,
+                                                  const float *__restrict__ dones,
+                                                  const float *__restrict__ bootstrap, float gamma,
+                                                  float decay, float *__restrict__ adv,
+                                                  float *__restrict__ ret) {
+    int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= N) return;
+    float gae = 0.0f;
+    float next_val = bootstrap[e];
+    for (int t = T - 1; t >= 0; --t) {
+        long idx = (long)t * N + e;
+        float v = values[idx];
+        float nv = next_val;
+        if (dones[idx] > 0.5f) { nv = 0.0f; gae = 0.0f; }
+        float delta = rewards[idx] + gamma * nv - v;
+        gae = delta + decay * gae;
+        adv[idx] = gae;
+        ret[idx] = gae + v;
+        next_val = v;
+    }
+}
+
+// ---------------------------------------------------------------- advantage normalisation
+// pass 1: per-block sums -> scratch[0..nb); pass 2: mean; pass 3: per-block sum of squared
+// deviations; pass 4: (x - mean) / (sqrt(var + 1e-8) + 1e-8).  Two-pass variance like the
+// reference (ppo.mojo:2356-2371), with fp32 sums taken blockwise.
+__global__ __launch_bounds__(TPB) void partial_sum_kernel(const float *__restrict__ x, int n,
+                                                          const float *__restrict__ mean_ptr,
+                                                          float *__restrict__ out) {
+    __shared__ float smem[4];
+    const float mean = mean_ptr ? *mean_ptr : 0.0f;
+    float s = 0.0f;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        float d = x[i] - mean;
+        s += mean_ptr ? d * d : x[i];
+    }
+    s = block_sum(s, smem);
+    if (threadIdx.x == 0) out[blockIdx.x] = s;
+}
+
+// out[0] = sum(in[0..nb)) / n
+__global__ __launch_bounds__(TPB) void finish_mean_kernel(const float *__restrict__ in, int nb, int n,
+                                                          float *__restrict__ out) {
+    __shared__ float smem[4];
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < nb; i += blockDim.x) s += in[i];
+    s = block_sum(s, smem);
+    if (threadIdx.x == 0) out[0] = s / (float)n;
+}
+
+__global__ __launch_bounds__(TPB) void normalize_apply_kernel(float *__restrict__ x, int n,
+                                                              const float *__restrict__ stats) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float mean = stats[0], variance = stats[1];
+    const float std = sqrtf(variance + 1e-8f);
+    x[i] = (x[i] - mean) / (std + 1e-8f);
+}
+
+// ---------------------------------------------------------------- gather
+__global__ __launch_bounds__(TPB) void gather_kernel(const int32_t *__restrict__ idx, int mb, int obs_dim,
+                                                     int act_dim, const float *r_obs, const float *r_act,
+                                                     const float *r_adv, const float *r_ret,
+                                                     const float *r_logp, const float *r_val,
+                                                     float *mb_obs, float *mb_act, float *mb_adv,
+                                                     float *mb_ret, float *mb_logp, float *mb_val) {
+    // one lane per output float of the widest array (obs): consecutive lanes copy consecutive words
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int w = obs_dim;
+    if (i >= (long)mb * w) return;
+    int b = (int)(i / w), c = (int)(i - (long)b * w);
+    long src = idx[b];
+    mb_obs[i] = r_obs[src * obs_dim + c];
+    if (c < act_dim) mb_act[(long)b * act_dim + c] = r_act[src * act_dim + c];
+    if (c == 0) {
+        mb_adv[b] = r_adv[src];
+        mb_ret[b] = r_ret[src];
+        mb_logp[b] = r_logp[src];
+        mb_val[b] = r_val[src];
+    }
+}
+
+// ---------------------------------------------------------------- loss gradients
+
+// deep_agents/ppo/ppo.mojo:285-378
+__global__ __launch_bounds__(TPB) void actor_grad_discrete_kernel(
+    const float *__restrict__ logits, const float *__restrict__ old_logp,
+    const float *__restrict__ adv, const float *__restrict__ actions, int mb, int A, float clip_eps,
+    float ent_coef, float *__restrict__ grad_logits, float *__restrict__ kl) {
+    int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= mb) return;
+    const float *l = logits + (long)b * A;
+    int action = (int)actions[b];
+    float advantage = adv[b];
+    float max_logit = l[0];
+    for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
+    float sum_exp = 0.0f;
+    for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
+    float p_action = 0.0f;
+    for (int a = 0; a < A; ++a) {
+        float p = expf(l[a] - max_logit) / sum_exp;
+        if (a == action) p_action = p;
+    }
+    float new_logp = logf(p_action + 1e-8f);
+    float old = old_logp[b];
+    kl[b] = old - new_logp;
+    float ratio = expf(new_logp - old);
+    bool clipped = (ratio < 1.0f - clip_eps) || (ratio > 1.0f + clip_eps);
+    for (int a = 0; a < A; ++a) {
+        float g = 0.0f;
+        if (!clipped) {
+            float p = expf(l[a] - max_logit) / sum_exp;
+            float d_log_prob = (a == action) ? 1.0f - p : -p;
+            float log_prob_ent = logf(p + 1e-8f);
+            float d_entropy = -p * (1.0f + log_prob_ent);
+            g = (-advantage * ratio * d_log_prob - ent_coef * d_entropy) / (float)mb;
+        }
+        grad_logits[(long)b * A + a] = g;
+    }
+}
+
+// deep_agents/ppo/kernels.mojo:230-412
+__global__ __launch_bounds__(TPB) void actor_grad_gaussian_kernel(
+    const float *__restrict__ actor_out, const float *__restrict__ old_logp,
+    const float *__restrict__ adv, const float *__restrict__ actions, int mb, int A, float clip_eps,
+    float ent_coef, float *__restrict__ grad_out, float *__restrict__ kl_out) {
+    int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= mb) return;
+    const float eps = 1e-6f, log_2pi = (float)1.8378770664093453;
+    const float *o = actor_out + (long)b * 2 * A;
+    const float *act = actions + (long)b * A;
+    float advantage = adv[b], old_log_prob = old_logp[b];
+    float new_log_prob = 0.0f;
+    for (int j = 0; j < A; ++j) {
+        float log_std = o[A + j];
+        if (log_std < -5.0f) log_std = -5.0f;
+        else if (log_std > 2.0f) log_std = 2.0f;
+        float std = expf(log_std);
+        float an = (act[j] - o[j]) / (std + eps);
+        float lg = -0.5f * (log_2pi + 2.0f * log_std + an * an);
+        new_log_prob = new_log_prob + lg;
+    }
+    float diff = new_log_prob - old_log_prob;
+    if (diff > 20.0f) diff = 20.0f;
+    else if (diff < -20.0f) diff = -20.0f;
+    float ratio = expf(diff);
+    float kl = (ratio - 1.0f) - diff;
+    if (kl < 0.0f) kl = 0.0f;
+    else if (kl > 100.0f) kl = 100.0f;
+    kl_out[b] = kl;
+    float clipped_ratio = ratio;
+    if (clipped_ratio < 1.0f - clip_eps) clipped_ratio = 1.0f - clip_eps;
+    else if (clipped_ratio > 1.0f + clip_eps) clipped_ratio = 1.0f + clip_eps;
+    bool is_clipped = clipped_ratio * advantage < ratio * advantage;
+    float *g = grad_out + (long)b * 2 * A;
+    for (int j = 0; j < A; ++j) {
+        float gm = 0.0f, gs = 0.0f;
+        if (!is_clipped) {
+            float log_std = o[A + j];
+            if (log_std < -5.0f) log_std = -5.0f;
+            else if (log_std > 2.0f) log_std = 2.0f;
+            float std = expf(log_std);
+            float an = (act[j] - o[j]) / (std + eps);
+            float d_mean = an / (std + eps);
+            float d_log_std = an * an - 1.0f;
+            gm = (-advantage * ratio * d_mean) / (float)mb;
+            gs = (-advantage * ratio * d_log_std - ent_coef * 1.0f) / (float)mb;
+            if (gm > 10.0f) gm = 10.0f;
+            else if (gm < -10.0f) gm = -10.0f;
+            if (gs > 10.0f) gs = 10.0f;
+            else if (gs < -10.0f) gs = -10.0f;
+        }
+        g[j] = gm;
+        g[A + j] = gs;
+    }
+}
+
+// ppo.mojo:538-633 (convention 0) and kernels.mojo:416-486 (convention 1)
+__global__ __launch_bounds__(TPB) void critic_grad_kernel(const float *__restrict__ values,
+                                                          const float *__restrict__ old_values,
+                                                          const float *__restrict__ returns, int mb,
+                                                          int convention, int clipped,
+                                                          float value_coef, float clip_eps,
+                                                          float *__restrict__ grad) {
+    int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= mb) return;
+    float v = values[b], ret = returns[b];
+    float out;
+    if (convention == 0) {
+        if (!clipped) {
+            out = 2.0f * value_coef * (v - ret) / (float)mb;
+        } else {
+            float v_old = old_values[b];
+            float v_diff = v - v_old;
+            float v_clipped;
+            if (v_diff > clip_eps) v_clipped = v_old + clip_eps;
+            else if (v_diff < -clip_eps) v_clipped = v_old - clip_eps;
+            else v_clipped = v;
+            float loss_unclipped = (v - ret) * (v - ret);
+            float loss_clipped = (v_clipped - ret) * (v_clipped - ret);
+            float g;
+            if (loss_unclipped > loss_clipped) g = 2.0f * (v - ret);
+            else if (v_diff > clip_eps || v_diff < -clip_eps) g = 0.0f;
+            else g = 2.0f * (v - ret);
+            out = value_coef * g / (float)mb;
+        }
+    } else {
+        if (!clipped) {
+            out = (v - ret) / (float)mb;
+        } else {
+            float old_value = old_values[b];
+            float d = v - old_value;
+            float mn = d < clip_eps ? d : clip_eps;
+            float mx = mn > -clip_eps ? mn : -clip_eps;
+            float value_clipped = old_value + mx;
+            float loss_unclipped = (v - ret) * (v - ret);
+            float loss_clipped = (value_clipped - ret) * (value_clipped - ret);
+            if (loss_clipped > loss_unclipped) {
+                float clip_sign = 1.0f;
+                if (v - old_value > clip_eps) clip_sign = 0.0f;
+                else if (v - old_value < -clip_eps) clip_sign = 0.0f;
+                out = clip_sign * (value_clipped - ret) / (float)mb;
+            } else {
+                out = (v - ret) / (float)mb;
+            }
+        }
+    }
+    grad[b] = out;
+}
+
+// ---------------------------------------------------------------- clip by global norm
+__global__ __launch_bounds__(TPB) void sq_partial_kernel(const float *__restrict__ g, int n,
+                                                         float *__restrict__ out) {
+    __shared__ float smem[4];
+    float s = 0.0f;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        s += g[i] * g[i];
+    s = block_sum(s, smem);
+    if (threadIdx.x == 0) out[blockIdx.x] = s;
+}
+
+// every block re-reduces the (few) partial sums, then scales its slice: no single-block stage
+__global__ __launch_bounds__(TPB) void clip_apply_kernel(float *__restrict__ g, int n,
+                                                         const float *__restrict__ partial, int nb,
+                                                         float max_norm) {
+    __shared__ float smem[4];
+    __shared__ float scale_s;
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < nb; i += blockDim.x) s += partial[i];
+    s = block_sum(s, smem);
+    if (threadIdx.x == 0) {
+        float norm = sqrtf(s);
+        float scale = 1.0f;
+        if (norm > max_norm) scale = max_norm / (norm + 1e-8f);
+        scale_s = scale;
+    }
+    __syncthreads();
+    const float scale = scale_s;
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) g[i] = g[i] * scale;
+}
+
+// ---------------------------------------------------------------- Adam
+// deep_rl/optimizer/adam.mojo:52-105; state interleaved (m, v) per parameter -> one 8-byte access
+__global__ __launch_bounds__(TPB) void adam_kernel(float *__restrict__ p, const float *__restrict__ g,
+                                                   float2 *__restrict__ state, int n, float lr,
+                                                   float beta1, float beta2, float omb1, float omb2,
+                                                   float eps, float bc1, float bc2) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float gi = g[i];
+    float2 mv = state[i];
+    float m_new = beta1 * mv.x + omb1 * gi;
+    float v_new = beta2 * mv.y + omb2 * gi * gi;
+    state[i] = make_float2(m_new, v_new);
+    float m_hat = m_new / bc1, v_hat = v_new / bc2;
+    p[i] = p[i] - lr * m_hat / (sqrtf(v_hat) + eps);
+}
+
+__global__ void clamp_log_std_kernel(float *params, int offset, int A) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= A) return;
+    float v = params[offset + i];
+    if (v < -5.0f) params[offset + i] = -5.0f;
+    else if (v > 2.0f) params[offset + i] = 2.0f;
+}
+
+}  // namespace mrl
+
+using namespace mrl;
+
+extern "C" {
+
+int mrl_sample_categorical(mrl_ctx *ctx, const float *logits, int n, int num_actions, uint32_t seed,
+                           float *actions, float *log_probs) {
+    MRL_CHECK_ARG(ctx, "mrl_sample_categorical: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0 && num_actions > 0, "mrl_sample_categorical: bad sizes");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(logits && actions && log_probs, "mrl_sample_categorical: NULL buffer");
+    hipLaunchKernelGGL(sample_categorical_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream,
+                       logits, n, num_actions, seed, actions, log_probs);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_sample_gaussian(mrl_ctx *ctx, const float *actor_out, int n, int action_dim, uint32_t seed,
+                        float *actions, float *log_probs) {
+    MRL_CHECK_ARG(ctx, "mrl_sample_gaussian: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0 && action_dim > 0, "mrl_sample_gaussian: bad sizes");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(actor_out && actions && log_probs, "mrl_sample_gaussian: NULL buffer");
+    hipLaunchKernelGGL(sample_gaussian_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream,
+                       actor_out, n, action_dim, seed, actions, log_probs);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_gae(mrl_ctx *ctx, int T, int N, const float *rewards, const float *values,
+            const float *dones, const float *bootstrap, double gamma, double lam, float *adv,
+            float *ret) {
+    MRL_CHECK_ARG(ctx, "mrl_gae: ctx is NULL");
+    MRL_CHECK_ARG(T >= 0 && N >= 0, "mrl_gae: negative size");
+    if (T == 0 || N == 0) return MRL_OK;
+    MRL_CHECK_ARG(rewards && values && dones && bootstrap && adv && ret, "mrl_gae: NULL buffer");
+    hipLaunchKernelGGL(gae_kernel, dim3(grid_for(N, 64)), dim3(64), 0, ctx->stream, T, N, rewards,
+                       values, dones, bootstrap, (float)gamma, (float)(gamma * lam), adv, ret);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_normalize_advantages(mrl_ctx *ctx, float *x, int n) {
+    MRL_CHECK_ARG(ctx, "mrl_normalize_advantages: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0, "mrl_normalize_advantages: negative size");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(x, "mrl_normalize_advantages: NULL buffer");
+    int nb = std::min(1024, grid_for(n, TPB));
+    float *part = ctx->reduce_scratch;         // [0, nb)
+    float *stats = ctx->reduce_scratch + 2048;  // mean, variance
+    hipLaunchKernelGGL(partial_sum_kernel, dim3(nb), dim3(TPB), 0, ctx->stream, x, n, (const float *)nullptr, part);
+    hipLaunchKernelGGL(finish_mean_kernel, dim3(1), dim3(TPB), 0, ctx->stream, part, nb, n, stats);
+    hipLaunchKernelGGL(partial_sum_kernel, dim3(nb), dim3(TPB), 0, ctx->stream, x, n, (const float *)stats, part);
+    hipLaunchKernelGGL(finish_mean_kernel, dim3(1), dim3(TPB), 0, ctx->stream, part, nb, n, stats + 1);
+    hipLaunchKernelGGL(normalize_apply_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream, x, n, stats);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_gather_minibatch(mrl_ctx *ctx, const int32_t *indices, int mb, int obs_dim, int act_dim,
+                         const float *r_obs, const float *r_actions, const float *r_adv,
+                         const float *r_ret, const float *r_logp, const float *r_values,
+                         float *mb_obs, float *mb_actions, float *mb_adv, float *mb_ret,
+                         float *mb_logp, float *mb_values) {
+    MRL_CHECK_ARG(ctx, "mrl_gather_minibatch: ctx is NULL");
+    MRL_CHECK_ARG(mb >= 0 && obs_dim > 0 && act_dim > 0 && act_dim <= obs_dim,
+                  "mrl_gather_minibatch: bad sizes (need 0 < act_dim <= obs_dim)");
+    if (mb == 0) return MRL_OK;
+    MRL_CHECK_ARG(indices && r_obs && r_actions && r_adv && r_ret && r_logp && r_values && mb_obs &&
+                      mb_actions && mb_adv && mb_ret && mb_logp && mb_values,
+                  "mrl_gather_minibatch: NULL buffer");
+    hipLaunchKernelGGL(gather_kernel, dim3(grid_for((long)mb * obs_dim, TPB)), dim3(TPB), 0, ctx->stream,
+                       indices, mb, obs_dim, act_dim, r_obs, r_actions, r_adv, r_ret, r_logp, r_values,
+                       mb_obs, mb_actions, mb_adv, mb_ret, mb_logp, mb_values);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_ppo_actor_grad_discrete(mrl_ctx *ctx, const float *logits, const float *old_log_probs,
+                                const float *advantages, const float *actions, int mb,
+                                int num_actions, float clip_eps, float entropy_coef,
+                                float *grad_logits, float *kl) {
+    MRL_CHECK_ARG(ctx, "mrl_ppo_actor_grad_discrete: ctx is NULL");
+    MRL_CHECK_ARG(mb >= 0 && num_actions > 0, "mrl_ppo_actor_grad_discrete: bad sizes");
+    if (mb == 0) return MRL_OK;
+    MRL_CHECK_ARG(logits && old_log_probs && advantages && actions && grad_logits && kl,
+                  "mrl_ppo_actor_grad_discrete: NULL buffer");
+    hipLaunchKernelGGL(actor_grad_discrete_kernel, dim3(grid_for(mb, TPB)), dim3(TPB), 0, ctx->stream,
+                       logits, old_log_probs, advantages, actions, mb, num_actions, clip_eps,
+                       entropy_coef, grad_logits, kl);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_ppo_actor_grad_gaussian(mrl_ctx *ctx, const float *actor_out, const float *old_log_probs,
+                                const float *advantages, const float *actions, int mb,
+                                int action_dim, float clip_eps, float entropy_coef, float *grad_out,
+                                float *kl) {
+    MRL_CHECK_ARG(ctx, "mrl_ppo_actor_grad_gaussian: ctx is NULL");
+    MRL_CHECK_ARG(mb >= 0 && action_dim > 0, "mrl_ppo_actor_grad_gaussian: bad sizes");
+    if (mb == 0) return MRL_OK;
+    MRL_CHECK_ARG(actor_out && old_log_probs && advantages && actions && grad_out && kl,
+                  "mrl_ppo_actor_grad_gaussian: NULL buffer");
+    hipLaunchKernelGGL(actor_grad_gaussian_kernel, dim3(grid_for(mb, TPB)), dim3(TPB), 0, ctx->stream,
+                       actor_out, old_log_probs, advantages, actions, mb, action_dim, clip_eps,
+                       entropy_coef, grad_out, kl);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_ppo_critic_grad(mrl_ctx *ctx, const float *values, const float *old_values,
+                        const float *returns, int mb, int convention, int clipped, float value_coef,
+                        float clip_eps, float *grad_values) {
+    MRL_CHECK_ARG(ctx, "mrl_ppo_critic_grad: ctx is NULL");
+    MRL_CHECK_ARG(mb >= 0 && (convention == 0 || convention == 1), "mrl_ppo_critic_grad: bad arguments");
+    if (mb == 0) return MRL_OK;
+    MRL_CHECK_ARG(values && returns && grad_values && (!clipped || old_values),
+                  "mrl_ppo_critic_grad: NULL buffer");
+    hipLaunchKernelGGL(critic_grad_kernel, dim3(grid_for(mb, TPB)), dim3(TPB), 0, ctx->stream, values,
+                       old_values, returns, mb, convention, clipped, value_coef, clip_eps, grad_values);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_clip_grad_norm(mrl_ctx *ctx, float *grads, int n, float max_norm) {
+    MRL_CHECK_ARG(ctx, "mrl_clip_grad_norm: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0, "mrl_clip_grad_norm: negative size");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(grads, "mrl_clip_grad_norm: NULL buffer");
+    int nb = std::min(256, grid_for(n, TPB));
+    float *part = ctx->reduce_scratch + 1024;
+    hipLaunchKernelGGL(sq_partial_kernel, dim3(nb), dim3(TPB), 0, ctx->stream, grads, n, part);
+    hipLaunchKernelGGL(clip_apply_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream, grads, n,
+                       part, nb, max_norm);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_adam_step(mrl_ctx *ctx, float *params, const float *grads, float *state, int n, int t,
+                  double lr, double beta1, double beta2, double eps) {
+    MRL_CHECK_ARG(ctx, "mrl_adam_step: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0 && t >= 1, "mrl_adam_step: need n >= 0 and step count t >= 1");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(params && grads && state, "mrl_adam_step: NULL buffer");
+    // bias corrections in fp64 then rounded, as the host code of the reference does
+    float bc1 = (float)(1.0 - pow(beta1, (double)t));
+    float bc2 = (float)(1.0 - pow(beta2, (double)t));
+    hipLaunchKernelGGL(adam_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream, params, grads,
+                       reinterpret_cast<float2 *>(state), n, (float)lr, (float)beta1, (float)beta2,
+                       (float)(1.0 - beta1), (float)(1.0 - beta2), (float)eps, bc1, bc2);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_clamp_log_std(mrl_ctx *ctx, float *params, int offset, int action_dim) {
+    MRL_CHECK_ARG(ctx && params, "mrl_clamp_log_std: NULL argument");
+    MRL_CHECK_ARG(offset >= 0 && action_dim > 0, "mrl_clamp_log_std: bad sizes");
+    hipLaunchKernelGGL(clamp_log_std_kernel, dim3(grid_for(action_dim, 64)), dim3(64), 0, ctx->stream,
+                       params, offset, action_dim);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,121 @@
+// One time step of the PPO collection loop (deep_agents/ppo/ppo.mojo:2069-2285) without any
+// host round trip: policy + value forward, categorical sampling, rollout stores, env step with
+// auto-reset, episode accounting.  Finished episodes are appended to a device-side list through
+// a counter instead of being copied to the host after every step.
+#include "mrl_host.hpp"
+#include "mrl_device.hpp"
+
+namespace mrl {
+
+// sampling (ppo.mojo:4064-4123) fused with _store_pre_step_kernel (ppo.mojo:662-690):
+// rollout row t gets obs, action, log-prob and value; `actions` feeds the env step.
+__global__ __launch_bounds__(256) void sample_store_kernel(
+    const float *__restrict__ logits, const float *__restrict__ values, const float *__restrict__ obs,
+    int n, int A, int obs_dim, uint32_t seed, float *__restrict__ actions, float *__restrict__ r_obs,
+    float *__restrict__ r_actions, float *__restrict__ r_logp, float *__restrict__ r_values) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float *l = logits + (long)i * A;
+    uint32_t rng = seed ^ ((uint32_t)i * 2654435761u);
+    rng = xorshift32(rng);
+    float max_logit = l[0];
+    for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
+    float sum_exp = 0.0f;
+    for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
+    float u = random_uniform(rng);
+    float cumsum = 0.0f;
+    int sel = 0;
+    for (int a = 0; a < A; ++a) {
+        float prob = expf(l[a] - max_logit) / sum_exp;
+        cumsum = cumsum + prob;
+        if (u < cumsum) { sel = a; break; }
+    }
+    float p = expf(l[sel] - max_logit) / sum_exp;
+    actions[i] = (float)sel;
+    r_actions[i] = (float)sel;
+    r_logp[i] = logf(p + 1e-8f);
+    r_values[i] = values[i];
+    for (int k = 0; k < obs_dim; ++k) r_obs[(long)i * obs_dim + k] = obs[(long)i * obs_dim + k];
+}
+
+// _store_post_step_kernel (ppo.mojo:692-708) + accumulate_rewards / increment_steps /
+// extract_completed_episodes (deep_rl/gpu/rl_kernels.mojo:103-200) in one pass
+__global__ __launch_bounds__(256) void post_store_kernel(
+    const float *__restrict__ rewards, const float *__restrict__ dones, int n,
+    float *__restrict__ r_rewards, float *__restrict__ r_dones, float *__restrict__ ep_return,
+    float *__restrict__ ep_length, float *__restrict__ done_returns, float *__restrict__ done_lengths,
+    int32_t *__restrict__ done_count, int done_cap) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float r = rewards[i], d = dones[i];
+    r_rewards[i] = r;
+    r_dones[i] = d;
+    float er = ep_return[i] + r;
+    float el = ep_length[i] + 1.0f;
+    if (d > 0.5f) {
+        int slot = atomicAdd(done_count, 1);
+        if (slot < done_cap) {
+            done_returns[slot] = er;
+            done_lengths[slot] = el;
+        }
+        er = 0.0f;
+        el = 0.0f;
+    }
+    ep_return[i] = er;
+    ep_length[i] = el;
+}
+
+}  // namespace mrl
+
+using namespace mrl;
+
+extern "C" {
+
+int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_seed,
+                     uint64_t step_seed, uint64_t reset_seed) {
+    MRL_CHECK_ARG(ctx && r, "mrl_rollout_step: NULL argument");
+    MRL_CHECK_ARG(r->n_envs > 0 && t >= 0, "mrl_rollout_step: bad sizes");
+    MRL_CHECK_ARG(r->states && r->obs && r->actor_params && r->critic_params && r->r_obs &&
+                      r->r_actions && r->r_log_probs && r->r_values && r->r_rewards && r->r_dones &&
+                      r->ep_return && r->ep_length && r->done_returns && r->done_lengths && r->done_count,
+                  "mrl_rollout_step: NULL buffer in descriptor");
+    int ss, od, na, ad;
+    int rc = mrl_env_dims(r->env_id, &ss, &od, &na, &ad);
+    if (rc) return rc;
+    MRL_CHECK_ARG(na > 0 && na == r->num_actions && od == r->obs_dim,
+                  "mrl_rollout_step: descriptor does not match a discrete-action env");
+    MRL_CHECK_ARG(mrl_mlp_out_dim(&r->actor) == na && mrl_mlp_out_dim(&r->critic) == 1,
+                  "mrl_rollout_step: actor must end in num_actions logits, critic in 1 value");
+    const int N = r->n_envs;
+    const size_t need = (size_t)N * (na + 5);
+    if (ctx->rollout_ws_floats < need) {
+        MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+        if (ctx->rollout_ws) MRL_CHECK_HIP(hipFree(ctx->rollout_ws));
+        ctx->rollout_ws = nullptr;
+        ctx->rollout_ws_floats = 0;
+        MRL_CHECK_HIP(hipMalloc(&ctx->rollout_ws, sizeof(float) * need));
+        ctx->rollout_ws_floats = need;
+    }
+    float *logits = ctx->rollout_ws, *values = logits + (size_t)N * na, *actions = values + N;
+    float *rewards = actions + N, *dones = rewards + N;
+
+    rc = mrl_mlp_forward(ctx, &r->actor, N, r->obs, r->actor_params, logits, nullptr);
+    if (rc) return rc;
+    rc = mrl_mlp_forward(ctx, &r->critic, N, r->obs, r->critic_params, values, nullptr);
+    if (rc) return rc;
+    const size_t row = (size_t)t * N;
+    hipLaunchKernelGGL(sample_store_kernel, dim3(grid_for(N, 256)), dim3(256), 0, ctx->stream, logits,
+                       values, r->obs, N, na, od, sample_seed, actions, r->r_obs + row * od,
+                       r->r_actions + row, r->r_log_probs + row, r->r_values + row);
+    MRL_CHECK_LAUNCH();
+    rc = mrl_env_step_autoreset(ctx, r->env_id, N, r->states, actions, rewards, dones, r->obs, step_seed,
+                                reset_seed);
+    if (rc) return rc;
+    hipLaunchKernelGGL(post_store_kernel, dim3(grid_for(N, 256)), dim3(256), 0, ctx->stream, rewards,
+                       dones, N, r->r_rewards + row, r->r_dones + row, r->ep_return, r->ep_length,
+                       r->done_returns, r->done_lengths, r->done_count, r->done_cap);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,120 @@
+"""GPU parity: MLP forward / backward through the C ABI against the CPU oracle (serial fp32 loops
+of the reference layers) and a torch fp32 reference.  Bar: outputs and gradients within 1e-4
+relative (floor 1e-5 absolute, scaled by the magnitude of the tensor)."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+RELU, TANH, LIN, ACTOR = 1, 2, 0, 3
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def ctx(mrl):
+    return mrl.DeviceContext("cuda:0")
+
+
+def mk(mrl, spec):
+    f = {RELU: mrl.LinearReLU, TANH: mrl.LinearTanh, LIN: mrl.Linear, ACTOR: mrl.StochasticActor}
+    return mrl.seq(*[f[k](i, o) for k, i, o in spec])
+
+
+def close(got, want, what):
+    scale = max(1.0, float(np.abs(want).max()))
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5 * scale, err_msg=what)
+
+
+CASES = [
+    ("lunar actor", [(RELU, 8, 256), (RELU, 256, 256), (LIN, 256, 4)], 300),
+    ("lunar critic", [(RELU, 8, 256), (RELU, 256, 256), (LIN, 256, 1)], 257),
+    ("cartpole actor", [(RELU, 4, 64), (RELU, 64, 64), (LIN, 64, 2)], 129),
+    ("pendulum actor", [(TANH, 3, 64), (TANH, 64, 64), (ACTOR, 64, 1)], 200),
+    ("cheetah actor", [(TANH, 17, 256), (TANH, 256, 256), (ACTOR, 256, 6)], 96),
+    ("bipedal critic", [(TANH, 24, 256), (TANH, 256, 256), (LIN, 256, 1)], 64),
+    ("odd sizes", [(RELU, 5, 33), (TANH, 33, 70), (LIN, 70, 3)], 37),
+    ("single layer", [(LIN, 7, 5)], 1),
+]
+
+
+@pytest.mark.parametrize("name,spec,batch", CASES, ids=[c[0] for c in CASES])
+def test_forward_backward_parity(mrl, orc, orcmod, ctx, name, spec, batch):
+    say("mlp case", name, batch)
+    rng = np.random.default_rng(abs(hash(name)) % 2**31)
+    model = mk(mrl, spec)
+    ls = orcmod.layers(spec)
+    P, CS, OD = model.PARAM_SIZE, model.CACHE_SIZE, model.OUT_DIM
+    assert P == orc.orc_mlp_param_size(ls, len(spec)) and CS == orc.orc_mlp_cache_size(ls, len(spec))
+    fan = np.sqrt(2.0 / spec[0][1])
+    params = rng.uniform(-fan, fan, P).astype(np.float32) * 0.7
+    x = rng.normal(size=(batch, spec[0][1])).astype(np.float32)
+    go = rng.normal(size=(batch, OD)).astype(np.float32)
+
+    out_h = np.zeros((batch, OD), np.float32); cache_h = np.zeros(batch * CS, np.float32)
+    orc.orc_mlp_forward(ls, len(spec), batch, x, params, out_h, cache_h.ctypes.data)
+    grads_h = np.zeros(P, np.float32); gin_h = np.zeros_like(x)
+    orc.orc_mlp_backward(ls, len(spec), batch, go, params, cache_h, grads_h, gin_h.ctypes.data)
+
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    p_d, x_d, go_d = d(params), d(x.reshape(-1)), d(go.reshape(-1))
+    out_d = torch.full((batch * OD,), 9.0, device="cuda"); out_nc = torch.full((batch * OD,), 9.0, device="cuda")
+    cache_d = torch.full((batch * CS,), 9.0, device="cuda")
+    grads_d = torch.full((P,), 9.0, device="cuda"); gin_d = torch.full((x.size,), 9.0, device="cuda")
+    model.forward_gpu_no_cache_ws(ctx, out_nc, x_d, p_d)
+    model.forward_gpu_ws(ctx, out_d, x_d, p_d, cache_d)
+    model.backward_gpu_ws(ctx, gin_d, go_d, p_d, cache_d, grads_d)     # overwrites the 9.0s
+    ctx.synchronize()
+    close(out_d.cpu().numpy().reshape(batch, OD), out_h, "forward")
+    assert torch.equal(out_d, out_nc)
+    close(cache_d.cpu().numpy(), cache_h, "cache")
+    close(grads_d.cpu().numpy(), grads_h, "param grads")
+    close(gin_d.cpu().numpy().reshape(x.shape), gin_h, "input grads")
+    # backward without grad_input (what the PPO update asks for on the first layer)
+    grads2 = torch.zeros(P, device="cuda")
+    model.backward_gpu_ws(ctx, None, go_d, p_d, cache_d, grads2)
+    ctx.synchronize()
+    assert torch.equal(grads2, grads_d)
+
+
+def test_forward_matches_torch_fp32_at_update_size(mrl, ctx):
+    # minibatch of 4096 rows through the 256-wide nets against torch fp32 matmuls
+    torch.manual_seed(0)
+    model = mk(mrl, [(RELU, 8, 256), (RELU, 256, 256), (LIN, 256, 4)])
+    B = 4096
+    p = (torch.rand(model.PARAM_SIZE, device="cuda") - 0.5) * 0.2
+    x = torch.randn(B, 8, device="cuda")
+    W0, b0 = p[:2048].view(8, 256), p[2048:2304]
+    W1, b1 = p[2304:2304 + 65536].view(256, 256), p[67840:68096]
+    W2, b2 = p[68096:68096 + 1024].view(256, 4), p[69120:69124]
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    h1 = torch.relu(x @ W0 + b0); h2 = torch.relu(h1 @ W1 + b1); want = h2 @ W2 + b2
+    out = torch.zeros(B * 4, device="cuda"); cache = torch.zeros(B * model.CACHE_SIZE, device="cuda")
+    model.forward_gpu_ws(ctx, out, x.reshape(-1), p, cache)
+    go = torch.randn(B, 4, device="cuda")
+    grads = torch.zeros(model.PARAM_SIZE, device="cuda")
+    model.backward_gpu_ws(ctx, None, go.reshape(-1), p, cache, grads)
+    ctx.synchronize()
+    torch.testing.assert_close(out.view(B, 4), want, rtol=1e-4, atol=1e-5)
+    m2 = go @ W2.T * (h2 > 0); m1 = m2 @ W1.T * (h1 > 0)
+    want_g = torch.cat([(x.T @ m1).reshape(-1), m1.sum(0), (h1.T @ m2).reshape(-1), m2.sum(0),
+                        (h2.T @ go).reshape(-1), go.sum(0)])
+    torch.backends.cuda.matmul.allow_tf32 = prev
+    torch.testing.assert_close(grads, want_g, rtol=1e-4, atol=1e-4 * float(want_g.abs().max()))
+
+
+def test_mlp_argument_errors(mrl, ctx):
+    model = mk(mrl, [(RELU, 8, 16), (LIN, 16, 2)])
+    p = torch.zeros(model.PARAM_SIZE, device="cuda")
+    with pytest.raises(mrl.MrlError):
+        model.forward_gpu_no_cache_ws(ctx, torch.zeros(4, device="cuda"), torch.zeros(9, device="cuda"), p)
+    with pytest.raises(mrl.MrlError):
+        model.forward_gpu_no_cache_ws(ctx, torch.zeros(1, device="cuda"), torch.zeros(8, device="cuda"), p)
+    with pytest.raises(mrl.MrlError):
+        mrl.seq(mrl.LinearReLU(8, 16), mrl.Linear(15, 2))       # dims do not chain
+    model.forward_gpu_no_cache_ws(ctx, torch.zeros(0, device="cuda"), torch.zeros(0, device="cuda"), p)
