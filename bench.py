@@ -1,0 +1,168 @@
+#!/usr/bin/env python3
+"""Headline benchmark: LunarLander 8192-env rollout (policy + value forward, sampling, env step
+with auto-reset, rollout stores) and the PPO update, on one MI355X.
+
+One "step" = one collection step over all 8192 envs.  `value` = env-steps/s including the policy
+forward, inputs resident in HBM.  The PPO update throughput (samples/s) is reported beside it in
+the same JSON line, with the roofline figures of the dominant kernel (device time measured live
+with HIP events on the launch stream) and the CPU baseline (the oracle's C restatement of the
+reference's CPU path, timed on this box's host cores on a bounded sample).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+N_ENVS, HIDDEN, OBS, NA = 8192, 256, 8, 4
+ENV_STEP_BYTES = 672                  # algorithmic HBM bytes per LunarLander env-step (live fields)
+FWD_FLOPS = 2 * ((OBS * HIDDEN + HIDDEN * HIDDEN + HIDDEN * NA) + (OBS * HIDDEN + HIDDEN * HIDDEN + HIDDEN * 1))
+HBM_PEAK_GBS, MFMA_FP32_PEAK_TFLOPS = 8000.0, 157.3
+
+
+def cpu_baseline(np, n_envs=2048, steps=60):
+    """Oracle (C restatement of the reference CPU path): env step + policy/value forward + sampling,
+    single thread, on a bounded sample of the same workload."""
+    from oracle import orc
+    o = orc.load()
+    spec_a = [(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, NA)]
+    spec_c = [(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, 1)]
+    la, lc = orc.layers(spec_a), orc.layers(spec_c)
+    rng = np.random.default_rng(0)
+    pa = rng.uniform(-0.1, 0.1, o.orc_mlp_param_size(la, 3)).astype(np.float32)
+    pc = rng.uniform(-0.1, 0.1, o.orc_mlp_param_size(lc, 3)).astype(np.float32)
+    s = np.zeros((n_envs, 192), np.float32)
+    o.orc_ll_reset_batch(s, n_envs, 1)
+    obs = np.ascontiguousarray(s[:, :8])
+    logits, values = np.zeros((n_envs, NA), np.float32), np.zeros((n_envs, 1), np.float32)
+    a, lp = np.zeros(n_envs, np.float32), np.zeros(n_envs, np.float32)
+    r, d = np.zeros(n_envs, np.float32), np.zeros(n_envs, np.float32)
+    t0 = time.perf_counter()
+    for t in range(steps):
+        o.orc_mlp_forward(la, 3, n_envs, obs, pa, logits, None)
+        o.orc_mlp_forward(lc, 3, n_envs, obs, pc, values, None)
+        o.orc_sample_categorical(logits, n_envs, NA, 100 + t, a, lp)
+        o.orc_ll_step_batch(s, a, r, d, obs, n_envs, 1)
+        o.orc_ll_selective_reset_batch(s, d, n_envs, 500 + t)
+        obs[:] = s[:, :8]
+    dt = time.perf_counter() - t0
+    return {"value": n_envs * steps / dt, "unit": "env-steps/s", "cores": 1, "kind": "port",
+            "sample": "%d envs x %d collection steps (env step + actor/critic forward + sampling), "
+                      "single thread, %.1f s" % (n_envs, steps, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--update-minibatches", type=int, default=200,
+                    help="minibatches of 4096 timed for the PPO-update figure")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one MI355X; --gpus %d is not supported "
+                 "(no collective or multi-GPU path is part of it)" % args.gpus)
+
+    import numpy as np
+    import torch
+    mrl = importlib.import_module("mojo-rl_amd")
+    ctx = mrl.DeviceContext("cuda:0")
+    E = mrl.LunarLanderV2
+    actor = mrl.seq(mrl.LinearReLU(OBS, HIDDEN), mrl.LinearReLU(HIDDEN, HIDDEN), mrl.Linear(HIDDEN, NA))
+    critic = mrl.seq(mrl.LinearReLU(OBS, HIDDEN), mrl.LinearReLU(HIDDEN, HIDDEN), mrl.Linear(HIDDEN, 1))
+    T = max(args.steps, 1)
+    rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N_ENVS, T, done_cap=4 * N_ENVS + 64 * T)
+    g = torch.Generator(device="cuda").manual_seed(0x5EED + 2)
+    # reference init: Xavier over the flat vector with the network's in/out dims (initializers.mojo:69-76)
+    bound_a, bound_c = (2.0 / (OBS + NA)) ** 0.5, (2.0 / (OBS + 1)) ** 0.5
+    rb.actor_params = (torch.rand(actor.PARAM_SIZE, device="cuda", generator=g) * 2 - 1) * bound_a * 0.1
+    rb.critic_params = (torch.rand(critic.PARAM_SIZE, device="cuda", generator=g) * 2 - 1) * bound_c * 0.1
+    E.reset_kernel_gpu(ctx, rb.states, 0x5EED + 2)
+    rb.obs.copy_(rb.states.view(N_ENVS, E.STATE_SIZE)[:, :OBS].reshape(-1))
+    desc = rb.descriptor()
+
+    for w in range(args.warmup):
+        mrl.ppo.rollout_step(ctx, desc, w % T, 7 + w, 0, 9000 + w)
+    ctx.synchronize()
+    rb.done_count.zero_()
+    ctx.synchronize()
+
+    # ---- timed region: exactly `steps` collection steps
+    ctx.profile_begin(8 * T + 16)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(T):
+        mrl.ppo.rollout_step(ctx, desc, t, 1000 + t, 0, 50000 + t)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    phases = ctx.profile_end()
+    env_steps_per_s = N_ENVS * T / dt
+    episodes = int(rb.done_count.item())
+
+    ph_us = {k: (1e3 * v[0] / max(v[1], 1)) for k, v in phases.items()}
+    fwd_us, env_us = ph_us["policy_fwd"], ph_us["env_step"]
+    fwd_tflops = FWD_FLOPS * N_ENVS / (fwd_us * 1e-6) / 1e12
+    env_gbs = ENV_STEP_BYTES * N_ENVS / (env_us * 1e-6) / 1e9
+    if fwd_us >= env_us:
+        roofline = {"kernel": "linear_fwd_kernel (actor+critic forward, 6 launches)", "bound": "mfma",
+                    "achieved": fwd_tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": fwd_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": None,
+                    "avg_launch_us": fwd_us}
+    else:
+        roofline = {"kernel": "ll_step_kernel<autoreset>", "bound": "hbm", "achieved": env_gbs,
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": env_gbs / HBM_PEAK_GBS,
+                    "traffic": None, "avg_launch_us": env_us}
+
+    # ---- PPO update on the collected batch (minibatch 4096, reference defaults)
+    MB = 4096
+    upd = mrl.ppo.DiscreteUpdate(ctx, rb, MB, mrl.Adam(lr=3e-4), mrl.Adam(lr=1e-3), target_kl=0.0)
+    upd.compute_advantages()
+    total = N_ENVS * T
+    n_mb = max(1, min(args.update_minibatches, total // MB))
+    perm = torch.randperm(total, device="cuda", generator=g).to(torch.int32)
+    for k in range(3):
+        upd.minibatch_step(perm[k * MB:(k + 1) * MB])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for k in range(n_mb):
+        upd.minibatch_step(perm[k * MB:(k + 1) * MB])
+    torch.cuda.synchronize()
+    dtu = time.perf_counter() - t1
+    update_sps = n_mb * MB / dtu
+    t2 = time.perf_counter()
+    upd.compute_advantages()
+    torch.cuda.synchronize()
+    gae_ms = (time.perf_counter() - t2) * 1e3
+
+    out = {
+        "metric": "env-steps/s incl. policy fwd on 1 MI355X; PPO update samples/s",
+        "value": env_steps_per_s, "unit": "env-steps/s", "n_gpus": 1, "steps": T, "warmup": args.warmup,
+        "ms_per_step": 1e3 * dt / T, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "LunarLander-v2 discrete, 8192 envs, policy 8-256-256-4 + value 8-256-256-1 "
+                               "(BASELINE.json configs[2]); update: minibatch 4096, clip 0.2, Adam",
+                   "n_envs": N_ENVS, "rollout_steps": T, "minibatch": MB},
+        "ppo_update_samples_per_s": update_sps,
+        "ppo_update": {"minibatches_timed": n_mb, "ms_per_minibatch": 1e3 * dtu / n_mb,
+                       "gae_plus_normalise_ms": gae_ms},
+        "episodes_finished": episodes,
+        "phase_us_per_step": ph_us,
+        "kernels": {"policy_fwd_TFLOPs": fwd_tflops, "env_step_GBs": env_gbs,
+                    "env_step_frac_hbm": env_gbs / HBM_PEAK_GBS,
+                    "policy_fwd_frac_mfma": fwd_tflops / MFMA_FP32_PEAK_TFLOPS},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(np)
+    ctx.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -71,6 +71,21 @@ int mrl_ctx_destroy(mrl_ctx *ctx);
 /* blocks until the context's stream has drained; DeviceContext.synchronize() */
 int mrl_ctx_synchronize(mrl_ctx *ctx);
 
+/* Device-time accounting per phase, the counterpart of the perf_counter_ns phase timers that
+ * train_gpu prints (deep_agents/ppo/ppo.mojo:2062-2067, :2777-2838) measured with HIP events on
+ * the context's stream instead of host enqueue times.  mrl_profile_begin arms it (at most
+ * max_marks phase boundaries are recorded); mrl_profile_end synchronises, adds up the time of
+ * each phase id (MRL_PHASE_*) into total_ms[n_phases] / counts[n_phases] and disarms it. */
+enum {
+    MRL_PHASE_POLICY_FWD = 0, /* actor + critic forward of a rollout step */
+    MRL_PHASE_SAMPLE = 1,     /* sampling + pre-step stores */
+    MRL_PHASE_ENV = 2,        /* env step (+ auto-reset) */
+    MRL_PHASE_POST = 3,       /* post-step stores and episode accounting */
+    MRL_PHASE_COUNT = 4
+};
+int mrl_profile_begin(mrl_ctx *ctx, int max_marks);
+int mrl_profile_end(mrl_ctx *ctx, int n_phases, double *total_ms, int *counts);
+
 /* ------------------------------------------------------------------ environments
  * GPUDiscreteEnv / GPUContinuousEnv, core/env_traits.mojo:230-397:
  *   comptime STATE_SIZE / OBS_DIM / NUM_ACTIONS / ACTION_DIM   -> mrl_env_dims

@@ -6,6 +6,10 @@ is no CPU or eager fallback.  torch is used for device memory and the stream onl
 import ctypes as C
 import os
 
+# torch first: streams and device memory come from torch, so the library must bind to the HIP
+# runtime that torch has already loaded into the process (one runtime per process, first one wins).
+import torch  # noqa: F401
+
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libmrl_hip.so")
 
@@ -48,6 +52,8 @@ SIGNATURES = {
     "mrl_ctx_create": [P, C.POINTER(P)],
     "mrl_ctx_destroy": [P],
     "mrl_ctx_synchronize": [P],
+    "mrl_profile_begin": [P, I],
+    "mrl_profile_end": [P, I, C.POINTER(D), C.POINTER(I)],
     "mrl_env_dims": [I, C.POINTER(I), C.POINTER(I), C.POINTER(I), C.POINTER(I)],
     "mrl_env_reset": [P, I, I, P, U64],
     "mrl_env_selective_reset": [P, I, I, P, P, U64],

@@ -41,6 +41,20 @@ class DeviceContext:
     def synchronize(self):
         _lib.call("mrl_ctx_synchronize", self.handle)
 
+    PHASES = ("policy_fwd", "sample_store", "env_step", "post_store")
+
+    def profile_begin(self, max_marks=8192):
+        """Arm per-phase device timing (HIP events on this context's stream)."""
+        _lib.call("mrl_profile_begin", self.handle, max_marks)
+
+    def profile_end(self):
+        """Synchronise and return {phase: (total_ms, launches)}."""
+        n = len(self.PHASES)
+        ms = (C.c_double * n)()
+        cnt = (C.c_int * n)()
+        _lib.call("mrl_profile_end", self.handle, n, ms, cnt)
+        return {p: (ms[i], cnt[i]) for i, p in enumerate(self.PHASES)}
+
     def close(self):
         if self.handle:
             _lib.call("mrl_ctx_destroy", self.handle)

@@ -38,6 +38,8 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     c->mlp_ws_floats = 0;
     c->rollout_ws = nullptr;
     c->rollout_ws_floats = 0;
+    c->profiling = false;
+    c->prof_used = 0;
     MRL_CHECK_HIP(hipMalloc(&c->ll_shapes, sizeof(mrl::ll::Shapes)));
     mrl::ll::Shapes sh = mrl::ll::make_shapes();
     MRL_CHECK_HIP(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));
@@ -54,6 +56,7 @@ int mrl_ctx_destroy(mrl_ctx *ctx) {
     if (ctx->reduce_scratch) hipFree(ctx->reduce_scratch);
     if (ctx->mlp_ws) hipFree(ctx->mlp_ws);
     if (ctx->rollout_ws) hipFree(ctx->rollout_ws);
+    for (hipEvent_t e : ctx->prof_events) hipEventDestroy(e);
     delete ctx;
     return MRL_OK;
 }
@@ -61,6 +64,36 @@ int mrl_ctx_destroy(mrl_ctx *ctx) {
 int mrl_ctx_synchronize(mrl_ctx *ctx) {
     MRL_CHECK_ARG(ctx != nullptr, "mrl_ctx_synchronize: ctx is NULL");
     MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    return MRL_OK;
+}
+
+int mrl_profile_begin(mrl_ctx *ctx, int max_marks) {
+    MRL_CHECK_ARG(ctx != nullptr && max_marks > 0, "mrl_profile_begin: bad arguments");
+    while ((int)ctx->prof_events.size() < max_marks) {
+        hipEvent_t e;
+        MRL_CHECK_HIP(hipEventCreate(&e));
+        ctx->prof_events.push_back(e);
+    }
+    ctx->prof_tags.assign(ctx->prof_events.size(), -1);
+    ctx->prof_used = 0;
+    ctx->profiling = true;
+    return MRL_OK;
+}
+
+int mrl_profile_end(mrl_ctx *ctx, int n_phases, double *total_ms, int *counts) {
+    MRL_CHECK_ARG(ctx && total_ms && counts && n_phases > 0, "mrl_profile_end: bad arguments");
+    ctx->profiling = false;
+    MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    for (int i = 0; i < n_phases; ++i) { total_ms[i] = 0.0; counts[i] = 0; }
+    for (size_t i = 1; i < ctx->prof_used; ++i) {
+        int tag = ctx->prof_tags[i];
+        if (tag < 0 || tag >= n_phases) continue;
+        float ms = 0.0f;
+        MRL_CHECK_HIP(hipEventElapsedTime(&ms, ctx->prof_events[i - 1], ctx->prof_events[i]));
+        total_ms[tag] += ms;
+        counts[tag] += 1;
+    }
+    ctx->prof_used = 0;
     return MRL_OK;
 }
 

@@ -7,6 +7,7 @@
 #include <stdarg.h>
 #include <algorithm>
 #include <unordered_map>
+#include <vector>
 #include "../../include/mrl.h"
 
 struct mrl_ctx {
@@ -28,6 +29,11 @@ struct mrl_ctx {
     // rewards, dones for n_envs), grown on demand
     float *rollout_ws;
     size_t rollout_ws_floats;
+    // phase timing: events recorded on `stream` at phase boundaries while armed
+    bool profiling;
+    std::vector<hipEvent_t> prof_events;
+    std::vector<int> prof_tags;
+    size_t prof_used;
 };
 
 namespace mrl {
@@ -35,6 +41,13 @@ namespace mrl {
 int set_error(int code, const char *fmt, ...);
 
 inline int grid_for(long n, int block) { return (int)((n + block - 1) / block); }
+
+// records a phase boundary: the time since the previous mark is charged to `tag` (tag < 0: start)
+inline void profile_mark(mrl_ctx *ctx, int tag) {
+    if (!ctx->profiling || ctx->prof_used >= ctx->prof_events.size()) return;
+    if (hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream) != hipSuccess) return;
+    ctx->prof_tags[ctx->prof_used++] = tag;
+}
 
 }  // namespace mrl
 

@@ -99,22 +99,27 @@ int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_
     float *logits = ctx->rollout_ws, *values = logits + (size_t)N * na, *actions = values + N;
     float *rewards = actions + N, *dones = rewards + N;
 
+    profile_mark(ctx, -1);
     rc = mrl_mlp_forward(ctx, &r->actor, N, r->obs, r->actor_params, logits, nullptr);
     if (rc) return rc;
     rc = mrl_mlp_forward(ctx, &r->critic, N, r->obs, r->critic_params, values, nullptr);
     if (rc) return rc;
+    profile_mark(ctx, MRL_PHASE_POLICY_FWD);
     const size_t row = (size_t)t * N;
     hipLaunchKernelGGL(sample_store_kernel, dim3(grid_for(N, 256)), dim3(256), 0, ctx->stream, logits,
                        values, r->obs, N, na, od, sample_seed, actions, r->r_obs + row * od,
                        r->r_actions + row, r->r_log_probs + row, r->r_values + row);
     MRL_CHECK_LAUNCH();
+    profile_mark(ctx, MRL_PHASE_SAMPLE);
     rc = mrl_env_step_autoreset(ctx, r->env_id, N, r->states, actions, rewards, dones, r->obs, step_seed,
                                 reset_seed);
     if (rc) return rc;
+    profile_mark(ctx, MRL_PHASE_ENV);
     hipLaunchKernelGGL(post_store_kernel, dim3(grid_for(N, 256)), dim3(256), 0, ctx->stream, rewards,
                        dones, N, r->r_rewards + row, r->r_dones + row, r->ep_return, r->ep_length,
                        r->done_returns, r->done_lengths, r->done_count, r->done_cap);
     MRL_CHECK_LAUNCH();
+    profile_mark(ctx, MRL_PHASE_POST);
     return MRL_OK;
 }
 

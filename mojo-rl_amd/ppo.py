@@ -122,3 +122,76 @@ def rollout_step(ctx, desc, t, sample_seed, step_seed=0, reset_seed=0):
     """One pass of train_gpu's inner loop body (ppo.mojo:2069-2285), enqueue only."""
     _lib.call("mrl_rollout_step", ctx.handle, C.byref(desc), t, int(sample_seed) & 0xFFFFFFFF,
               int(step_seed) & (2**64 - 1), int(reset_seed) & (2**64 - 1))
+
+
+class DiscreteUpdate:
+    """Phases 2 and 3 of DeepPPOAgent.train_gpu (deep_agents/ppo/ppo.mojo:2296-2727) on device
+    buffers: bootstrap value, GAE, advantage normalisation, then epochs of shuffled minibatches,
+    each running actor forward / loss gradient / backward / clip / Adam and the same for the
+    critic.  Nothing is copied to the host inside an epoch; the mean KL of the last minibatch is
+    read once per epoch for the early-stop test."""
+
+    def __init__(self, ctx, rb, minibatch, actor_opt, critic_opt, gamma=0.99, gae_lambda=0.95,
+                 clip_epsilon=0.2, entropy_coef=0.01, value_loss_coef=0.5, max_grad_norm=0.5,
+                 clip_value=True, normalize_advantages=True, norm_adv_per_minibatch=True,
+                 target_kl=0.015):
+        self.ctx, self.rb, self.mb = ctx, rb, minibatch
+        self.actor_opt, self.critic_opt = actor_opt, critic_opt
+        self.gamma, self.gae_lambda = gamma, gae_lambda
+        self.clip_epsilon, self.entropy_coef, self.value_loss_coef = clip_epsilon, entropy_coef, value_loss_coef
+        self.max_grad_norm, self.clip_value = max_grad_norm, clip_value
+        self.normalize_advantages, self.norm_adv_per_minibatch = normalize_advantages, norm_adv_per_minibatch
+        self.target_kl = target_kl
+        dev = ctx.device
+        z = lambda n: torch.zeros(n, device=dev)
+        total = rb.n_envs * rb.rollout_len
+        obs_dim, na = rb.env.OBS_DIM, rb.env.NUM_ACTIONS
+        self.total = total
+        self.advantages, self.returns, self.bootstrap = z(total), z(total), z(rb.n_envs)
+        self.mb_obs, self.mb_actions = z(minibatch * obs_dim), z(minibatch)
+        self.mb_adv, self.mb_ret, self.mb_logp, self.mb_val = z(minibatch), z(minibatch), z(minibatch), z(minibatch)
+        self.logits, self.values = z(minibatch * na), z(minibatch)
+        self.g_logits, self.g_values, self.kl = z(minibatch * na), z(minibatch), z(minibatch)
+        self.actor_cache = z(minibatch * rb.actor.CACHE_SIZE)
+        self.critic_cache = z(minibatch * rb.critic.CACHE_SIZE)
+        self.actor_grads, self.critic_grads = z(rb.actor.PARAM_SIZE), z(rb.critic.PARAM_SIZE)
+        self.actor_state, self.critic_state = z(2 * rb.actor.PARAM_SIZE), z(2 * rb.critic.PARAM_SIZE)
+
+    def compute_advantages(self):
+        rb, ctx = self.rb, self.ctx
+        rb.critic.forward_gpu_no_cache_ws(ctx, self.bootstrap, rb.obs, rb.critic_params)
+        compute_gae(ctx, rb.r_rewards, rb.r_values, rb.r_dones, self.bootstrap, self.gamma,
+                    self.gae_lambda, self.advantages, self.returns)
+        if self.normalize_advantages:
+            normalize_advantages(ctx, self.advantages)
+
+    def minibatch_step(self, indices):
+        rb, ctx = self.rb, self.ctx
+        gather_minibatch(ctx, indices,
+                         (rb.r_obs, rb.r_actions, self.advantages, self.returns, rb.r_log_probs, rb.r_values),
+                         (self.mb_obs, self.mb_actions, self.mb_adv, self.mb_ret, self.mb_logp, self.mb_val),
+                         rb.env.OBS_DIM, 1)
+        if self.norm_adv_per_minibatch:
+            normalize_advantages(ctx, self.mb_adv)
+        rb.actor.forward_gpu_ws(ctx, self.logits, self.mb_obs, rb.actor_params, self.actor_cache)
+        ppo_actor_grad_with_kl(ctx, self.g_logits, self.kl, self.logits, self.mb_logp, self.mb_adv,
+                               self.mb_actions, self.clip_epsilon, self.entropy_coef)
+        rb.actor.backward_gpu_ws(ctx, None, self.g_logits, rb.actor_params, self.actor_cache, self.actor_grads)
+        if self.max_grad_norm > 0.0:
+            clip_grad_norm(ctx, self.actor_grads, self.max_grad_norm)
+        self.actor_opt.step_gpu(ctx, rb.actor_params, self.actor_grads, self.actor_state)
+        rb.critic.forward_gpu_ws(ctx, self.values, self.mb_obs, rb.critic_params, self.critic_cache)
+        ppo_critic_grad(ctx, self.g_values, self.values, self.mb_ret, self.value_loss_coef,
+                        self.mb_val if self.clip_value else None, self.clip_epsilon)
+        rb.critic.backward_gpu_ws(ctx, None, self.g_values, rb.critic_params, self.critic_cache, self.critic_grads)
+        if self.max_grad_norm > 0.0:
+            clip_grad_norm(ctx, self.critic_grads, self.max_grad_norm)
+        self.critic_opt.step_gpu(ctx, rb.critic_params, self.critic_grads, self.critic_state)
+
+    def run_epoch(self, permutation):
+        """permutation: int32 device tensor over the T*N samples; only whole minibatches are used
+        (ppo.mojo:2438).  Returns the mean KL of the epoch's last minibatch."""
+        n_mb = self.total // self.mb
+        for k in range(n_mb):
+            self.minibatch_step(permutation[k * self.mb:(k + 1) * self.mb])
+        return float(self.kl.mean().item()) if self.target_kl > 0.0 else 0.0
