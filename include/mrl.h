@@ -178,6 +178,16 @@ int mrl_clamp_log_std(mrl_ctx *ctx, float *params, int offset, int action_dim);
  * the per-env accumulators of deep_rl/gpu/rl_kernels.mojo:103-227; finished episodes are
  * appended to done_returns / done_lengths (capacity done_cap) through the counter
  * done_count instead of being copied to the host every step. */
+/* Policy half of a collection step for a discrete-action agent, one launch when both nets are
+ * IN -> H -> H -> out with H in {64, 256} and ReLU or tanh hidden layers (layer by layer
+ * otherwise): actor + critic forward (Model.forward_gpu_no_cache_ws, ppo.mojo:2073-2090),
+ * _sample_actions_kernel (ppo.mojo:4064-4123) and _store_pre_step_kernel (ppo.mojo:662-690).
+ * actions [n] feeds the env step; r_* are the rollout rows of this time step. */
+int mrl_policy_step_discrete(mrl_ctx *ctx, const mrl_mlp_desc *actor, const mrl_mlp_desc *critic, int n,
+                             const float *obs, const float *actor_params, const float *critic_params,
+                             uint32_t seed, float *actions, float *r_obs, float *r_actions,
+                             float *r_log_probs, float *r_values);
+
 typedef struct {
     int32_t env_id, n_envs, obs_dim, num_actions;
     float *states, *obs;                     /* [N, STATE_SIZE], [N, OBS] current observation */

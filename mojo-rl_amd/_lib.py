@@ -75,6 +75,7 @@ SIGNATURES = {
     "mrl_clip_grad_norm": [P, P, I, F],
     "mrl_adam_step": [P, P, P, P, I, I, D, D, D, D],
     "mrl_clamp_log_std": [P, P, I, I],
+    "mrl_policy_step_discrete": [P, DP, DP, I, P, P, P, U32, P, P, P, P, P],
     "mrl_rollout_step": [P, RP, I, U32, U64, U64],
 }
 _SPECIAL = {"mrl_version": (C.c_int, []), "mrl_last_error": (C.c_char_p, [])}

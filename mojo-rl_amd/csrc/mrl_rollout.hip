@@ -7,6 +7,10 @@
 
 namespace mrl {
 
+int launch_policy_discrete(mrl_ctx *ctx, const mrl_mlp_desc &a, const mrl_mlp_desc &c, const float *obs,
+                           int n, const float *ap, const float *cp, uint32_t seed, float *actions,
+                           float *r_obs, float *r_actions, float *r_logp, float *r_values);
+
 // sampling (ppo.mojo:4064-4123) fused with _store_pre_step_kernel (ppo.mojo:662-690):
 // rollout row t gets obs, action, log-prob and value; `actions` feeds the env step.
 __global__ __launch_bounds__(256) void sample_store_kernel(
@@ -71,6 +75,56 @@ using namespace mrl;
 
 extern "C" {
 
+// layer-by-layer fallback needs logits/values temporaries
+static int ensure_rollout_ws(mrl_ctx *ctx, size_t need) {
+    if (ctx->rollout_ws_floats < need) {
+        MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+        if (ctx->rollout_ws) MRL_CHECK_HIP(hipFree(ctx->rollout_ws));
+        ctx->rollout_ws = nullptr;
+        ctx->rollout_ws_floats = 0;
+        MRL_CHECK_HIP(hipMalloc(&ctx->rollout_ws, sizeof(float) * need));
+        ctx->rollout_ws_floats = need;
+    }
+    return MRL_OK;
+}
+
+int mrl_policy_step_discrete(mrl_ctx *ctx, const mrl_mlp_desc *actor, const mrl_mlp_desc *critic, int n,
+                             const float *obs, const float *actor_params, const float *critic_params,
+                             uint32_t seed, float *actions, float *r_obs, float *r_actions,
+                             float *r_log_probs, float *r_values) {
+    MRL_CHECK_ARG(ctx && actor && critic, "mrl_policy_step_discrete: NULL argument");
+    MRL_CHECK_ARG(n >= 0, "mrl_policy_step_discrete: negative n");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(obs && actor_params && critic_params && actions && r_obs && r_actions && r_log_probs &&
+                      r_values, "mrl_policy_step_discrete: NULL buffer");
+    const int na = mrl_mlp_out_dim(actor), nv = mrl_mlp_out_dim(critic);
+    MRL_CHECK_ARG(na > 0 && nv == 1, "mrl_policy_step_discrete: actor must end in logits, critic in 1 value");
+    MRL_CHECK_ARG(actor->layers[0].in_dim == critic->layers[0].in_dim,
+                  "mrl_policy_step_discrete: actor and critic read different observation widths");
+    const int od = actor->layers[0].in_dim;
+    profile_mark(ctx, -1);
+    int rc = launch_policy_discrete(ctx, *actor, *critic, obs, n, actor_params, critic_params, seed,
+                                    actions, r_obs, r_actions, r_log_probs, r_values);
+    if (rc == MRL_OK) {
+        profile_mark(ctx, MRL_PHASE_POLICY_FWD);
+        return MRL_OK;
+    }
+    if (rc != MRL_E_UNSUPPORTED) return rc;
+    rc = ensure_rollout_ws(ctx, (size_t)n * (na + 5));
+    if (rc) return rc;
+    float *logits = ctx->rollout_ws, *values = logits + (size_t)n * na;
+    rc = mrl_mlp_forward(ctx, actor, n, obs, actor_params, logits, nullptr);
+    if (rc) return rc;
+    rc = mrl_mlp_forward(ctx, critic, n, obs, critic_params, values, nullptr);
+    if (rc) return rc;
+    profile_mark(ctx, MRL_PHASE_POLICY_FWD);
+    hipLaunchKernelGGL(sample_store_kernel, dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream, logits,
+                       values, obs, n, na, od, seed, actions, r_obs, r_actions, r_log_probs, r_values);
+    MRL_CHECK_LAUNCH();
+    profile_mark(ctx, MRL_PHASE_SAMPLE);
+    return MRL_OK;
+}
+
 int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_seed,
                      uint64_t step_seed, uint64_t reset_seed) {
     MRL_CHECK_ARG(ctx && r, "mrl_rollout_step: NULL argument");
@@ -84,33 +138,21 @@ int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_
     if (rc) return rc;
     MRL_CHECK_ARG(na > 0 && na == r->num_actions && od == r->obs_dim,
                   "mrl_rollout_step: descriptor does not match a discrete-action env");
-    MRL_CHECK_ARG(mrl_mlp_out_dim(&r->actor) == na && mrl_mlp_out_dim(&r->critic) == 1,
-                  "mrl_rollout_step: actor must end in num_actions logits, critic in 1 value");
+    MRL_CHECK_ARG(mrl_mlp_out_dim(&r->actor) == na && r->actor.layers[0].in_dim == od,
+                  "mrl_rollout_step: actor must map obs_dim to num_actions logits");
     const int N = r->n_envs;
-    const size_t need = (size_t)N * (na + 5);
-    if (ctx->rollout_ws_floats < need) {
-        MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
-        if (ctx->rollout_ws) MRL_CHECK_HIP(hipFree(ctx->rollout_ws));
-        ctx->rollout_ws = nullptr;
-        ctx->rollout_ws_floats = 0;
-        MRL_CHECK_HIP(hipMalloc(&ctx->rollout_ws, sizeof(float) * need));
-        ctx->rollout_ws_floats = need;
-    }
-    float *logits = ctx->rollout_ws, *values = logits + (size_t)N * na, *actions = values + N;
+    rc = ensure_rollout_ws(ctx, (size_t)N * (na + 5));
+    if (rc) return rc;
+    // [logits N*na | values N] are used by the layer-by-layer policy path; the tail holds the
+    // step's actions, rewards and dones
+    float *actions = ctx->rollout_ws + (size_t)N * (na + 1);
     float *rewards = actions + N, *dones = rewards + N;
-
-    profile_mark(ctx, -1);
-    rc = mrl_mlp_forward(ctx, &r->actor, N, r->obs, r->actor_params, logits, nullptr);
-    if (rc) return rc;
-    rc = mrl_mlp_forward(ctx, &r->critic, N, r->obs, r->critic_params, values, nullptr);
-    if (rc) return rc;
-    profile_mark(ctx, MRL_PHASE_POLICY_FWD);
     const size_t row = (size_t)t * N;
-    hipLaunchKernelGGL(sample_store_kernel, dim3(grid_for(N, 256)), dim3(256), 0, ctx->stream, logits,
-                       values, r->obs, N, na, od, sample_seed, actions, r->r_obs + row * od,
-                       r->r_actions + row, r->r_log_probs + row, r->r_values + row);
-    MRL_CHECK_LAUNCH();
-    profile_mark(ctx, MRL_PHASE_SAMPLE);
+    rc = mrl_policy_step_discrete(ctx, &r->actor, &r->critic, N, r->obs, r->actor_params,
+                                  r->critic_params, sample_seed, actions, r->r_obs + row * od,
+                                  r->r_actions + row, r->r_log_probs + row, r->r_values + row);
+    if (rc) return rc;
+    profile_mark(ctx, -1);
     rc = mrl_env_step_autoreset(ctx, r->env_id, N, r->states, actions, rewards, dones, r->obs, step_seed,
                                 reset_seed);
     if (rc) return rc;
