@@ -1,6 +1,7 @@
 // Context lifetime and error reporting of libmrl_hip.so.
 #include "mrl_host.hpp"
 #include "env_lunar.hpp"
+#include "env_walkers.hpp"
 
 namespace mrl {
 
@@ -43,6 +44,15 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     MRL_CHECK_HIP(hipMalloc(&c->ll_shapes, sizeof(mrl::ll::Shapes)));
     mrl::ll::Shapes sh = mrl::ll::make_shapes();
     MRL_CHECK_HIP(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));
+    c->bw_shapes = c->hc_shapes = nullptr;
+    {
+        mrl::bw::Shapes bs = mrl::bw::make_shapes();
+        MRL_CHECK_HIP(hipMalloc(&c->bw_shapes, sizeof(bs)));
+        MRL_CHECK_HIP(hipMemcpy(c->bw_shapes, &bs, sizeof(bs), hipMemcpyHostToDevice));
+        mrl::hc::Shapes hs = mrl::hc::make_shapes();
+        MRL_CHECK_HIP(hipMalloc(&c->hc_shapes, sizeof(hs)));
+        MRL_CHECK_HIP(hipMemcpy(c->hc_shapes, &hs, sizeof(hs), hipMemcpyHostToDevice));
+    }
     MRL_CHECK_HIP(hipMalloc(&c->reduce_scratch, sizeof(float) * c->reduce_scratch_floats));
     *out = c;
     return MRL_OK;
@@ -53,6 +63,8 @@ int mrl_ctx_destroy(mrl_ctx *ctx) {
     hipStreamSynchronize(ctx->stream);
     for (auto &kv : ctx->cartpole_steps) hipFree(kv.second.steps);
     if (ctx->ll_shapes) hipFree(ctx->ll_shapes);
+    if (ctx->bw_shapes) hipFree(ctx->bw_shapes);
+    if (ctx->hc_shapes) hipFree(ctx->hc_shapes);
     if (ctx->reduce_scratch) hipFree(ctx->reduce_scratch);
     if (ctx->mlp_ws) hipFree(ctx->mlp_ws);
     if (ctx->rollout_ws) hipFree(ctx->rollout_ws);

@@ -9,16 +9,19 @@
 #include "mrl_host.hpp"
 #include "env_classic.hpp"
 #include "env_lunar.hpp"
+#include "env_walkers.hpp"
 
 namespace mrl {
 
-constexpr int EPB = 64;  // envs per block == wavefront size
 
 // ---------------------------------------------------------------- CartPole / Pendulum
 
+// autoreset: a finished env is re-initialised with the selective-reset stream before its state and
+// observation are written; rewards / dones still report the step that ended the episode
 __global__ __launch_bounds__(256) void cartpole_step_kernel(float *states, int32_t *steps,
                                                             const float *actions, float *rewards,
-                                                            float *dones, float *obs, int batch) {
+                                                            float *dones, float *obs, int batch,
+                                                            int autoreset, uint32_t reset_seed) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= batch) return;
     float4 v = reinterpret_cast<const float4 *>(states)[i];
@@ -26,6 +29,7 @@ __global__ __launch_bounds__(256) void cartpole_step_kernel(float *states, int32
     int32_t st = steps[i];
     float r, d;
     cartpole::step(s, st, (int)actions[i], r, d);
+    if (autoreset && d > 0.5f) cartpole::reset(s, st, i, reset_seed);
     float4 o = make_float4(s[0], s[1], s[2], s[3]);
     reinterpret_cast<float4 *>(states)[i] = o;
     reinterpret_cast<float4 *>(obs)[i] = o;
@@ -53,7 +57,8 @@ __global__ __launch_bounds__(256) void cartpole_reset_kernel(float *states, int3
 
 __global__ __launch_bounds__(256) void pendulum_step_kernel(float *states, const float *actions,
                                                             float *rewards, float *dones,
-                                                            float *obs, int batch) {
+                                                            float *obs, int batch, int autoreset,
+                                                            uint64_t reset_seed) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= batch) return;
     float4 *row = reinterpret_cast<float4 *>(states) + 2 * (size_t)i;
@@ -61,6 +66,7 @@ __global__ __launch_bounds__(256) void pendulum_step_kernel(float *states, const
     float s[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
     float r, d;
     pendulum::step(s, actions[i], r, d);
+    if (autoreset && d > 0.5f) pendulum::reset(s, i, reset_seed);
     row[0] = make_float4(s[0], s[1], s[2], s[3]);
     row[1] = make_float4(s[4], s[5], s[6], s[7]);
     obs[3 * (size_t)i + 0] = s[0];
@@ -85,97 +91,170 @@ __global__ __launch_bounds__(256) void pendulum_reset_kernel(float *states, floa
     if (selective) dones[i] = 0.0f;
 }
 
-// ---------------------------------------------------------------- LunarLander
+// ---------------------------------------------------------------- physics2d envs
+// Per-env traits of the LDS-staged kernels.  EPB = env rows per workgroup (one wavefront; with
+// 32 rows the upper half of the lanes only helps with the copies), DYN_END = first float of the
+// row that a step never writes (everything before it, plus the metadata, is copied back).
 
-constexpr int LL_STRIDE = ll::STATE + 1;              // 193: odd => conflict-free lane access
-constexpr int LL_CSTRIDE = 8 * CONTACT_SIZE + 1;      // 73
-constexpr int LL_DYN = ll::L::JOINTS_OFF;             // [0, 56): obs + bodies + forces
-
-MRL_DEV void stage_in(float *lds, const float *g, int nenv, int lane) {
-    // rows are 192 floats = 48 float4, never straddled by a 16-byte load
-    const float4 *src = reinterpret_cast<const float4 *>(g);
-    const int total4 = nenv * (ll::STATE / 4);
-    for (int i = lane; i < total4; i += EPB) {
-        float4 v = src[i];
-        int f = i * 4;
-        int r = f / ll::STATE, c = f - r * ll::STATE;
-        float *d = lds + r * LL_STRIDE + c;
-        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+struct LunarLander {
+    using L = ll::L;
+    static constexpr int STATE = ll::STATE, OBS = ll::OBS, ACT_W = 1, EPB = 64;
+    static constexpr int DYN_END = L::JOINTS_OFF, NSHAPE = 3 * SHAPE_SIZE;
+    static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
+                             float &r, float &d) {
+        ll::step_row(row, cts, shapes, env, (int)a[0], r, d);
     }
-}
-
-MRL_DEV void stage_out_range(const float *lds, float *g, int nenv, int lane, int c0, int c1,
-                             const int *row_flag, int want_flag) {
-    const int w = c1 - c0;
-    const int total = nenv * w;
-    for (int i = lane; i < total; i += EPB) {
-        int r = i / w, c = c0 + (i - r * w);
-        if (row_flag == nullptr || row_flag[r] == want_flag) g[(size_t)r * ll::STATE + c] = lds[r * LL_STRIDE + c];
+    static MRL_DEV void reset(float *row, uint64_t seed, int env) {
+        ll::reset_row(row, ll::combined_seed(seed, env));
     }
-}
+};
 
-// AUTORESET = false: GPUDiscreteEnv.step_kernel_gpu.  AUTORESET = true: step, then rows that
+struct BipedalWalker {
+    using L = bw::L;
+    static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 32;
+    static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = bw::NSHAPE_FLOATS;
+    static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
+                             float &r, float &d) {
+        bw::step_row(row, cts, shapes, env, a, r, d);
+    }
+    static MRL_DEV void reset(float *row, uint64_t seed, int env) { bw::reset_row(row, walker_seed(seed, env)); }
+};
+
+struct HalfCheetah {
+    using L = hc::L;
+    static constexpr int STATE = hc::STATE, OBS = hc::OBS, ACT_W = hc::ACT, EPB = 64;
+    static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = hc::NSHAPE_FLOATS;
+    static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
+                             float &r, float &d) {
+        hc::step_row(row, cts, shapes, env, a, r, d);
+    }
+    static MRL_DEV void reset(float *row, uint64_t seed, int env) { hc::reset_row(row, walker_seed(seed, env)); }
+};
+
+constexpr int WAVE = 64;
+
+template <class E>
+struct Stage {
+    static constexpr int STRIDE = E::STATE | 1;                            // odd => conflict-free lane access
+    static constexpr int CSTRIDE = (E::L::MAX_CONTACTS * CONTACT_SIZE) | 1;
+
+    static MRL_DEV void in(float *lds, const float *g, int nenv, int lane) {
+        if (E::STATE % 4 == 0) {   // rows are whole float4s, never straddled by a 16-byte load
+            const float4 *src = reinterpret_cast<const float4 *>(g);
+            const int total4 = nenv * (E::STATE / 4);
+            for (int i = lane; i < total4; i += WAVE) {
+                float4 v = src[i];
+                int f = i * 4;
+                int r = f / E::STATE, c = f - r * E::STATE;
+                float *d = lds + r * STRIDE + c;
+                d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+            }
+        } else {
+            const int total = nenv * E::STATE;
+            for (int i = lane; i < total; i += WAVE) {
+                int r = i / E::STATE, c = i - r * E::STATE;
+                lds[r * STRIDE + c] = g[i];
+            }
+        }
+    }
+
+    static MRL_DEV void out(const float *lds, float *g, int nenv, int lane, int c0, int c1,
+                            const int *row_flag) {
+        const int w = c1 - c0;
+        const int total = nenv * w;
+        for (int i = lane; i < total; i += WAVE) {
+            int r = i / w, c = c0 + (i - r * w);
+            if (row_flag == nullptr || row_flag[r]) g[(size_t)r * E::STATE + c] = lds[r * STRIDE + c];
+        }
+    }
+};
+
+// AUTORESET = false: step_kernel_gpu of the trait.  AUTORESET = true: step, then rows that
 // finished are re-initialised in place (selective reset) before the observation is copied out.
-template <bool AUTORESET>
-__global__ __launch_bounds__(EPB) void ll_step_kernel(float *states, const float *actions,
-                                                      float *rewards, float *dones, float *obs,
-                                                      const float *shapes_g, int batch,
-                                                      uint64_t reset_seed) {
-    __shared__ float rows[EPB * LL_STRIDE];
-    __shared__ float cts[EPB * LL_CSTRIDE];
-    __shared__ float shapes[3 * SHAPE_SIZE];
-    __shared__ int was_reset[EPB];
+template <class E, bool AUTORESET>
+__global__ __launch_bounds__(WAVE) void phys_step_kernel(float *states, const float *actions,
+                                                         float *rewards, float *dones, float *obs,
+                                                         const float *shapes_g, int batch,
+                                                         uint64_t reset_seed) {
+    using S = Stage<E>;
+    __shared__ float rows[E::EPB * S::STRIDE];
+    __shared__ float cts[E::EPB * S::CSTRIDE];
+    __shared__ float shapes[E::NSHAPE];
+    __shared__ int was_reset[E::EPB];
     const int lane = threadIdx.x;
-    const int env0 = blockIdx.x * EPB;
-    const int nenv = min(EPB, batch - env0);
-    float *gbase = states + (size_t)env0 * ll::STATE;
+    const int env0 = blockIdx.x * E::EPB;
+    const int nenv = min(E::EPB, batch - env0);
+    float *gbase = states + (size_t)env0 * E::STATE;
 
-    stage_in(rows, gbase, nenv, lane);
-    if (lane < 3 * SHAPE_SIZE) shapes[lane] = shapes_g[lane];
-    was_reset[lane] = 0;
+    S::in(rows, gbase, nenv, lane);
+    for (int i = lane; i < E::NSHAPE; i += WAVE) shapes[i] = shapes_g[i];
+    if (lane < E::EPB) was_reset[lane] = 0;
     __syncthreads();
 
     if (lane < nenv) {
         const int env = env0 + lane;
-        float *row = rows + lane * LL_STRIDE;
+        float *row = rows + lane * S::STRIDE;
         float r, d;
-        ll::step_row(row, cts + lane * LL_CSTRIDE, shapes, env, (int)actions[env], r, d);
+        E::step(row, cts + lane * S::CSTRIDE, shapes, env, actions + (size_t)env * E::ACT_W, r, d);
         rewards[env] = r;
         dones[env] = d;
         if (AUTORESET && d > 0.5f) {
-            ll::reset_row(row, ll::combined_seed(reset_seed, env));
+            E::reset(row, reset_seed, env);
             was_reset[lane] = 1;
         }
     }
     __syncthreads();
 
-    // observation out: [nenv, 8] contiguous
-    for (int i = lane; i < nenv * ll::OBS; i += EPB) {
-        int r = i >> 3, c = i & 7;
-        obs[(size_t)env0 * ll::OBS + i] = rows[r * LL_STRIDE + c];
+    for (int i = lane; i < nenv * E::OBS; i += WAVE) {   // observation out: [nenv, OBS] contiguous
+        int r = i / E::OBS, c = i - r * E::OBS;
+        obs[(size_t)env0 * E::OBS + i] = rows[r * S::STRIDE + c];
     }
-    stage_out_range(rows, gbase, nenv, lane, 0, LL_DYN, nullptr, 0);
-    stage_out_range(rows, gbase, nenv, lane, ll::L::META_OFF, ll::STATE, nullptr, 0);
-    if (AUTORESET) stage_out_range(rows, gbase, nenv, lane, LL_DYN, ll::L::META_OFF, was_reset, 1);
+    S::out(rows, gbase, nenv, lane, 0, E::DYN_END, nullptr);
+    S::out(rows, gbase, nenv, lane, E::L::META_OFF, E::STATE, nullptr);
+    if (AUTORESET) S::out(rows, gbase, nenv, lane, E::DYN_END, E::L::META_OFF, was_reset);
 }
 
-__global__ __launch_bounds__(EPB) void ll_reset_kernel(float *states, const float *dones, int batch,
-                                                       uint64_t seed, int selective) {
-    __shared__ float rows[EPB * LL_STRIDE];
-    __shared__ int was_reset[EPB];
+template <class E>
+__global__ __launch_bounds__(WAVE) void phys_reset_kernel(float *states, const float *dones, int batch,
+                                                          uint64_t seed, int selective) {
+    using S = Stage<E>;
+    __shared__ float rows[E::EPB * S::STRIDE];
+    __shared__ int was_reset[E::EPB];
     const int lane = threadIdx.x;
-    const int env0 = blockIdx.x * EPB;
-    const int nenv = min(EPB, batch - env0);
-    was_reset[lane] = 0;
+    const int env0 = blockIdx.x * E::EPB;
+    const int nenv = min(E::EPB, batch - env0);
+    if (lane < E::EPB) was_reset[lane] = 0;
     if (lane < nenv) {
         const int env = env0 + lane;
         if (!selective || dones[env] > 0.5f) {
-            ll::reset_row(rows + lane * LL_STRIDE, ll::combined_seed(seed, env));
+            E::reset(rows + lane * S::STRIDE, seed, env);
             was_reset[lane] = 1;
         }
     }
     __syncthreads();
-    stage_out_range(rows, states + (size_t)env0 * ll::STATE, nenv, lane, 0, ll::STATE, was_reset, 1);
+    S::out(rows, states + (size_t)env0 * E::STATE, nenv, lane, 0, E::STATE, was_reset);
+}
+
+template <class E>
+static int launch_phys_reset(mrl_ctx *ctx, int batch, float *states, const float *dones, uint64_t seed,
+                             int selective) {
+    hipLaunchKernelGGL(phys_reset_kernel<E>, dim3(grid_for(batch, E::EPB)), dim3(WAVE), 0, ctx->stream,
+                       states, dones, batch, seed, selective);
+    return MRL_OK;
+}
+
+template <class E>
+static int launch_phys_step(mrl_ctx *ctx, int batch, float *states, const float *actions, float *rewards,
+                            float *dones, float *obs, const float *shapes, bool autoreset,
+                            uint64_t reset_seed) {
+    dim3 grid(grid_for(batch, E::EPB));
+    if (autoreset)
+        hipLaunchKernelGGL((phys_step_kernel<E, true>), grid, dim3(WAVE), 0, ctx->stream, states, actions,
+                           rewards, dones, obs, shapes, batch, reset_seed);
+    else
+        hipLaunchKernelGGL((phys_step_kernel<E, false>), grid, dim3(WAVE), 0, ctx->stream, states, actions,
+                           rewards, dones, obs, shapes, batch, reset_seed);
+    return MRL_OK;
 }
 
 static int cartpole_side(mrl_ctx *ctx, const float *states, int batch, int32_t **out) {
@@ -209,6 +288,8 @@ int mrl_env_dims(int env_id, int *state_size, int *obs_dim, int *num_actions, in
         case MRL_ENV_CARTPOLE: s = 4; o = 4; na = 2; ad = 0; break;
         case MRL_ENV_PENDULUM: s = 8; o = 3; na = 0; ad = 1; break;
         case MRL_ENV_LUNARLANDER: s = ll::STATE; o = ll::OBS; na = 4; ad = 0; break;
+        case MRL_ENV_BIPEDAL: s = bw::STATE; o = bw::OBS; na = 0; ad = bw::ACT; break;
+        case MRL_ENV_HALFCHEETAH: s = hc::STATE; o = hc::OBS; na = 0; ad = hc::ACT; break;
         default: return set_error(MRL_E_UNSUPPORTED, "mrl_env_dims: env_id %d is not built", env_id);
     }
     if (state_size) *state_size = s;
@@ -241,10 +322,9 @@ static int env_reset_impl(mrl_ctx *ctx, int env_id, int batch, float *states, fl
             hipLaunchKernelGGL(pendulum_reset_kernel, dim3(grid_for(batch, 256)), dim3(256), 0,
                                ctx->stream, states, dones, batch, seed, selective);
             break;
-        case MRL_ENV_LUNARLANDER:
-            hipLaunchKernelGGL(ll_reset_kernel, dim3(grid_for(batch, EPB)), dim3(EPB), 0,
-                               ctx->stream, states, dones, batch, seed, selective);
-            break;
+        case MRL_ENV_LUNARLANDER: launch_phys_reset<LunarLander>(ctx, batch, states, dones, seed, selective); break;
+        case MRL_ENV_BIPEDAL: launch_phys_reset<BipedalWalker>(ctx, batch, states, dones, seed, selective); break;
+        case MRL_ENV_HALFCHEETAH: launch_phys_reset<HalfCheetah>(ctx, batch, states, dones, seed, selective); break;
         default:
             return set_error(MRL_E_UNSUPPORTED, "mrl_env_reset: env_id %d is not built", env_id);
     }
@@ -275,25 +355,26 @@ static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, con
             int rc = cartpole_side(ctx, states, batch, &steps);
             if (rc) return rc;
             hipLaunchKernelGGL(cartpole_step_kernel, dim3(grid_for(batch, 256)), dim3(256), 0,
-                               ctx->stream, states, steps, actions, rewards, dones, obs, batch);
-            MRL_CHECK_LAUNCH();
-            if (autoreset) return set_error(MRL_E_UNSUPPORTED, "autoreset: LunarLander only for now");
+                               ctx->stream, states, steps, actions, rewards, dones, obs, batch,
+                               autoreset ? 1 : 0, (uint32_t)reset_seed);
             break;
         }
         case MRL_ENV_PENDULUM:
-            if (autoreset) return set_error(MRL_E_UNSUPPORTED, "autoreset: LunarLander only for now");
             hipLaunchKernelGGL(pendulum_step_kernel, dim3(grid_for(batch, 256)), dim3(256), 0,
-                               ctx->stream, states, actions, rewards, dones, obs, batch);
+                               ctx->stream, states, actions, rewards, dones, obs, batch,
+                               autoreset ? 1 : 0, reset_seed);
             break;
         case MRL_ENV_LUNARLANDER:
-            if (autoreset)
-                hipLaunchKernelGGL(ll_step_kernel<true>, dim3(grid_for(batch, EPB)), dim3(EPB), 0,
-                                   ctx->stream, states, actions, rewards, dones, obs, ctx->ll_shapes,
-                                   batch, reset_seed);
-            else
-                hipLaunchKernelGGL(ll_step_kernel<false>, dim3(grid_for(batch, EPB)), dim3(EPB), 0,
-                                   ctx->stream, states, actions, rewards, dones, obs, ctx->ll_shapes,
-                                   batch, reset_seed);
+            launch_phys_step<LunarLander>(ctx, batch, states, actions, rewards, dones, obs, ctx->ll_shapes,
+                                          autoreset, reset_seed);
+            break;
+        case MRL_ENV_BIPEDAL:
+            launch_phys_step<BipedalWalker>(ctx, batch, states, actions, rewards, dones, obs, ctx->bw_shapes,
+                                            autoreset, reset_seed);
+            break;
+        case MRL_ENV_HALFCHEETAH:
+            launch_phys_step<HalfCheetah>(ctx, batch, states, actions, rewards, dones, obs, ctx->hc_shapes,
+                                          autoreset, reset_seed);
             break;
         default:
             return set_error(MRL_E_UNSUPPORTED, "mrl_env_step: env_id %d is not built", env_id);

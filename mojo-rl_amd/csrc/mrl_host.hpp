@@ -18,7 +18,7 @@ struct mrl_ctx {
     struct Side { int32_t *steps; int batch; };
     std::unordered_map<const void *, Side> cartpole_steps;
     // device copy of the shape tables (filled at context creation)
-    float *ll_shapes;
+    float *ll_shapes, *bw_shapes, *hc_shapes;
     // scratch for two-pass reductions (grad-norm partial sums, advantage statistics)
     float *reduce_scratch;
     int reduce_scratch_floats;

@@ -75,3 +75,11 @@ class PendulumV2(_GPUEnv):            # envs/pendulum/pendulum_v2.mojo:57
 
 class LunarLanderV2(_GPUEnv):         # envs/lunar_lander/lunar_lander_v2.mojo:123
     ENV_ID, STATE_SIZE, OBS_DIM, NUM_ACTIONS = _lib.ENV_LUNARLANDER, 192, 8, 4
+
+
+class BipedalWalkerV2(_GPUEnv):       # envs/bipedal_walker/bipedal_walker_v2.mojo:103
+    ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_BIPEDAL, 950, 24, 4
+
+
+class HalfCheetahPlanarV2(_GPUEnv):   # envs/half_cheetah/cheetah_planar_v2.mojo:91
+    ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_HALFCHEETAH, 253, 17, 6

@@ -119,6 +119,25 @@ void orc_ll_selective_reset_batch(float *states, const float *dones, int batch, 
 void orc_ll_step_batch(float *states, const float *actions, float *rewards, float *dones,
                        float *obs, int batch, int n_threads);
 
+/* ---------------------------------------- BipedalWalker / HalfCheetah --- */
+#define ORC_BW_STATE 950
+#define ORC_HC_STATE 253
+void orc_bw_layout(orc_layout *L);
+void orc_bw_shapes(float *shapes /* 5*20 */);
+void orc_bw_reset(float *row, uint64_t combined_seed);
+void orc_bw_step(float *row, const float action[4], float *reward, float *done);
+/* dones == NULL: reset every env; otherwise only rows with dones > 0.5 (flags are left as they are) */
+void orc_bw_reset_batch(float *states, const float *dones, int batch, uint64_t seed);
+void orc_bw_step_batch(float *states, const float *actions, float *rewards, float *dones, float *obs,
+                       int batch, int n_threads);
+void orc_hc_layout(orc_layout *L);
+void orc_hc_shapes(float *shapes /* 7*20 */);
+void orc_hc_reset(float *row, uint64_t combined_seed);
+void orc_hc_step(float *row, const float action[6], float *reward, float *done);
+void orc_hc_reset_batch(float *states, const float *dones, int batch, uint64_t seed);
+void orc_hc_step_batch(float *states, const float *actions, float *rewards, float *dones, float *obs,
+                       int batch, int n_threads);
+
 /* ------------------------------------------------------------- MLP/NN --- */
 enum { ORC_LINEAR = 0, ORC_LINEAR_RELU = 1, ORC_LINEAR_TANH = 2, ORC_STOCHASTIC_ACTOR = 3 };
 typedef struct { int kind, in_dim, out_dim; } orc_layer; /* out_dim = action_dim for actor head */

@@ -78,6 +78,18 @@ def load():
         "orc_ll_reset_batch": (None, [f32p, C.c_int, C.c_uint64]),
         "orc_ll_selective_reset_batch": (None, [f32p, f32p, C.c_int, C.c_uint64]),
         "orc_ll_step_batch": (None, [f32p, f32p, f32p, f32p, f32p, C.c_int, C.c_int]),
+        "orc_bw_layout": (None, [LP]),
+        "orc_bw_shapes": (None, [f32p]),
+        "orc_bw_reset": (None, [f32p, C.c_uint64]),
+        "orc_bw_step": (None, [f32p, f32p, f32p, f32p]),
+        "orc_bw_reset_batch": (None, [f32p, C.c_void_p, C.c_int, C.c_uint64]),
+        "orc_bw_step_batch": (None, [f32p, f32p, f32p, f32p, f32p, C.c_int, C.c_int]),
+        "orc_hc_layout": (None, [LP]),
+        "orc_hc_shapes": (None, [f32p]),
+        "orc_hc_reset": (None, [f32p, C.c_uint64]),
+        "orc_hc_step": (None, [f32p, f32p, f32p, f32p]),
+        "orc_hc_reset_batch": (None, [f32p, C.c_void_p, C.c_int, C.c_uint64]),
+        "orc_hc_step_batch": (None, [f32p, f32p, f32p, f32p, f32p, C.c_int, C.c_int]),
         "orc_mlp_param_size": (C.c_int, [YP, C.c_int]),
         "orc_mlp_cache_size": (C.c_int, [YP, C.c_int]),
         "orc_mlp_forward": (None, [YP, C.c_int, C.c_int, f32p, f32p, f32p, C.c_void_p]),

