@@ -64,6 +64,9 @@ def main():
     ap.add_argument("--update-minibatches", type=int, default=200,
                     help="minibatches of 4096 timed for the PPO-update figure")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 64 MiB read + 64 MiB write elementwise kernel 10 times, the "
+                         "known-size reference for scaling FETCH_SIZE / WRITE_SIZE counter readings")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one MI355X; --gpus %d is not supported "
@@ -158,6 +161,14 @@ def main():
                     "policy_fwd_frac_mfma": fwd_tflops / MFMA_FP32_PEAK_TFLOPS},
         "roofline": roofline,
     }
+    if args.copy_calibration:
+        src = torch.ones(16 * 1024 * 1024, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        out["copy_calibration"] = {"kernel": "at::native::vectorized_elementwise_kernel (add scalar)",
+                                   "bytes_read": src.numel() * 4, "bytes_written": dst.numel() * 4, "launches": 10}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(np)
     ctx.close()
