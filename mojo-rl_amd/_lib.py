@@ -11,7 +11,8 @@ import os
 import torch  # noqa: F401
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libmrl_hip.so")
+# MRL_HIP_LIB points at an alternative build of the same library (e.g. an instrumented one)
+LIB_PATH = os.environ.get("MRL_HIP_LIB") or os.path.join(HERE, "libmrl_hip.so")
 
 MAX_LAYERS = 8
 LINEAR, LINEAR_RELU, LINEAR_TANH, STOCHASTIC_ACTOR = 0, 1, 2, 3

@@ -11,7 +11,7 @@
 // Philox(seed = env + 12345, offset = step_count), reset seed
 // Int(f32(seed)) * 2654435761 + (env + 1) * 12345.
 #pragma once
-#include "physics2d.hpp"
+#include "physics2d_reg.hpp"
 
 namespace mrl {
 namespace ll {
@@ -175,6 +175,69 @@ MRL_DEV void reset_row(float *row, uint64_t cseed) {
     row[L::META_OFF + META_PREV_SHAPING] = shaping(obs);
 }
 
+// Same row as reset_row, written by the 64 lanes of one wavefront together: the 13 Philox draws,
+// the 11 smoothed heights and the 10 edges each go to their own lane, the row is zero-filled in
+// stripes, and bodies / joints / counters are set by separate lanes.  Every value is computed by
+// the same expressions as in reset_row, so the result is bit-identical; only who computes it
+// differs.  All lanes of the wavefront must call this with the same `row`.
+MRL_DEV void reset_row_wave(float *row, uint64_t cseed, int lane) {
+    for (int k = lane; k < STATE; k += 64) row[k] = 0.0f;
+    // lane 0: velocity draw; lanes 1..12: terrain draws 0..11 of the second stream
+    Uniform4 u = philox_uniform4(lane == 0 ? cseed : cseed + 1000ull, 0,
+                                 lane == 0 ? 0ull : (uint64_t)((lane - 1) & 15));
+    const double raw = (double)u.v[0] * (H_UNITS / 2.0);       // lanes 1..12: raw[lane - 1]
+    const double raw_m = __shfl(raw, (lane + 63) & 63, 64);     // raw[lane - 2]
+    const double raw_p = __shfl(raw, (lane + 1) & 63, 64);      // raw[lane]
+    const int c = lane - 1;                                      // chunk index on lanes 1..11
+    double sm;
+    if (c == 0) sm = (raw + raw + raw_p) / 3.0;
+    else if (c == TERRAIN_CHUNKS - 1) sm = (raw_m + raw + raw) / 3.0;
+    else sm = (raw_m + raw + raw_p) / 3.0;
+    float h = (float)sm;
+    if (c >= TERRAIN_CHUNKS / 2 - 2 && c < TERRAIN_CHUNKS / 2 + 3) h = (float)HELIPAD_Y;
+    const float h_next = __shfl(h, (lane + 1) & 63, 64);
+    if (c >= 0 && c < TERRAIN_CHUNKS - 1) {                      // edge c from heights c, c + 1
+        const double x_spacing = W_UNITS / (double)(TERRAIN_CHUNKS - 1);
+        double x0 = 0.0 + (double)c * x_spacing, y0 = (double)h;
+        double x1 = 0.0 + (double)(c + 1) * x_spacing, y1 = (double)h_next;
+        double dx = x1 - x0, dy = y1 - y0;
+        double length = ::sqrt(dx * dx + dy * dy);
+        double nx = -dy / length, ny = dx / length;
+        if (ny < 0) { nx = -nx; ny = -ny; }
+        float *E = row + L::EDGES_OFF + c * 6;
+        E[0] = (float)x0; E[1] = (float)y0; E[2] = (float)x1; E[3] = (float)y1;
+        E[4] = (float)nx; E[5] = (float)ny;
+    }
+    const float u0 = __shfl(u.v[0], 0, 64), u1 = __shfl(u.v[1], 0, 64);
+    const double init_x = HELIPAD_X, init_y = H_UNITS;
+    const double init_vx = (((double)u0 * 2.0 - 1.0) * 1000.0) * DT / LANDER_MASS;
+    const double init_vy = (((double)u1 * 2.0 - 1.0) * 1000.0) * DT / LANDER_MASS;
+    const double leg_y = init_y - (10.0 / SCALE) - LEG_DOWN;
+    float *B = row + L::BODIES_OFF;
+    float *J = row + L::JOINTS_OFF;
+    if (lane == 16) set_body(B, init_x, init_y, init_vx, init_vy, LANDER_MASS, LANDER_INERTIA, 0);
+    if (lane == 17) set_body(B + BODY_SIZE, init_x - LEG_AWAY, leg_y, init_vx, init_vy, LEG_MASS, LEG_INERTIA, 1);
+    if (lane == 18) set_body(B + 2 * BODY_SIZE, init_x + LEG_AWAY, leg_y, init_vx, init_vy, LEG_MASS, LEG_INERTIA, 2);
+    if (lane == 19) set_joint(J, 1, -LEG_AWAY, -10.0 / SCALE, 0.0, LEG_H, 0.4, 0.9);
+    if (lane == 20) set_joint(J + JOINT_SIZE, 2, LEG_AWAY, -10.0 / SCALE, 0.0, LEG_H, -0.9, -0.4);
+    if (lane == 21) {
+        row[L::EDGE_COUNT_OFF] = (float)(TERRAIN_CHUNKS - 1);
+        row[L::JOINT_COUNT_OFF] = 2.0f;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (lane == 0) {
+        float obs[8];
+        observe(row, obs);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) row[k] = obs[k];
+        row[L::META_OFF + META_PREV_SHAPING] = shaping(obs);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 MRL_DEV void apply_engines(float *row, int env, int step_count, double m_power, double s_power,
                            double direction) {
     if (m_power == 0.0 && s_power == 0.0) return;
@@ -235,21 +298,8 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
     const float gx = (float)0.0, gy = (float)-10.0, dt = (float)DT;
     const float friction = (float)0.1, restitution = (float)0.0;
     const float baumgarte = (float)0.2, slop = (float)0.005;
-    integrate_velocities<L>(row, gx, gy, dt);
-    int n = edge_detect<L>(row, shapes, contacts);
-    JointAnchors<L> an;
-    joint_anchors_all<L>(row, an);
-    for (int it = 0; it < 6; ++it) {
-        contact_solve_velocity<L>(row, contacts, n, friction, restitution);
-        joint_solve_velocity<L>(row, an, dt);
-    }
-    integrate_positions<L>(row, dt);
-    for (int it = 0; it < 2; ++it) {
-        contact_solve_position<L>(row, contacts, n, baumgarte, slop);
-        joint_solve_position<L>(row, baumgarte, slop);
-    }
-#pragma unroll
-    for (int k = 0; k < 9; ++k) row[L::FORCES_OFF + k] = 0.0f;
+    const int n = reg_physics_substep<L, false>(row, shapes, contacts, gx, gy, dt, friction, restitution,
+                                                baumgarte, slop, 6, 2);
 
     step_count += 1;
     float obs[8];

@@ -107,6 +107,10 @@ struct LunarLander {
     static MRL_DEV void reset(float *row, uint64_t seed, int env) {
         ll::reset_row(row, ll::combined_seed(seed, env));
     }
+    static constexpr bool WAVE_RESET = true;
+    static MRL_DEV void reset_wave(float *row, uint64_t seed, int env, int lane) {
+        ll::reset_row_wave(row, ll::combined_seed(seed, env), lane);
+    }
 };
 
 struct BipedalWalker {
@@ -118,6 +122,8 @@ struct BipedalWalker {
         bw::step_row(row, cts, shapes, env, a, r, d);
     }
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { bw::reset_row(row, walker_seed(seed, env)); }
+    static constexpr bool WAVE_RESET = false;
+    static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
 };
 
 struct HalfCheetah {
@@ -129,9 +135,12 @@ struct HalfCheetah {
         hc::step_row(row, cts, shapes, env, a, r, d);
     }
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { hc::reset_row(row, walker_seed(seed, env)); }
+    static constexpr bool WAVE_RESET = false;
+    static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
 };
 
-constexpr int WAVE = 64;
+constexpr int WAVE = 64;    // the compute phase runs on one wavefront, one lane per env
+constexpr int BLOCK = 256;  // all four wavefronts of the workgroup move the rows between HBM and LDS
 
 template <class E>
 struct Stage {
@@ -142,7 +151,7 @@ struct Stage {
         if (E::STATE % 4 == 0) {   // rows are whole float4s, never straddled by a 16-byte load
             const float4 *src = reinterpret_cast<const float4 *>(g);
             const int total4 = nenv * (E::STATE / 4);
-            for (int i = lane; i < total4; i += WAVE) {
+            for (int i = lane; i < total4; i += BLOCK) {
                 float4 v = src[i];
                 int f = i * 4;
                 int r = f / E::STATE, c = f - r * E::STATE;
@@ -151,7 +160,7 @@ struct Stage {
             }
         } else {
             const int total = nenv * E::STATE;
-            for (int i = lane; i < total; i += WAVE) {
+            for (int i = lane; i < total; i += BLOCK) {
                 int r = i / E::STATE, c = i - r * E::STATE;
                 lds[r * STRIDE + c] = g[i];
             }
@@ -162,83 +171,102 @@ struct Stage {
                             const int *row_flag) {
         const int w = c1 - c0;
         const int total = nenv * w;
-        for (int i = lane; i < total; i += WAVE) {
+        for (int i = lane; i < total; i += BLOCK) {
             int r = i / w, c = c0 + (i - r * w);
             if (row_flag == nullptr || row_flag[r]) g[(size_t)r * E::STATE + c] = lds[r * STRIDE + c];
         }
     }
 };
 
+// Resets the rows whose bit is set in `mask` (lanes of wavefront 0).  A handful of rows -- the
+// usual case inside a step -- are rebuilt one after the other by all 64 lanes together; many rows
+// (a full reset) are rebuilt by their own lanes in parallel.
+template <class E>
+MRL_DEV void reset_rows(float *rows, int *was_reset, unsigned long long mask, uint64_t seed, int env0,
+                        int lane) {
+    using S = Stage<E>;
+    if (E::WAVE_RESET && __popcll(mask) <= 8) {
+        while (mask) {
+            const int src = __ffsll((long long)mask) - 1;
+            mask &= mask - 1;
+            E::reset_wave(rows + src * S::STRIDE, seed, env0 + src, lane);
+            if (lane == 0) was_reset[src] = 1;
+        }
+    } else if ((mask >> lane) & 1ull) {
+        E::reset(rows + lane * S::STRIDE, seed, env0 + lane);
+        was_reset[lane] = 1;
+    }
+}
+
 // AUTORESET = false: step_kernel_gpu of the trait.  AUTORESET = true: step, then rows that
 // finished are re-initialised in place (selective reset) before the observation is copied out.
 template <class E, bool AUTORESET>
-__global__ __launch_bounds__(WAVE) void phys_step_kernel(float *states, const float *actions,
-                                                         float *rewards, float *dones, float *obs,
-                                                         const float *shapes_g, int batch,
-                                                         uint64_t reset_seed) {
+__global__ __launch_bounds__(BLOCK) void phys_step_kernel(float *states, const float *actions,
+                                                          float *rewards, float *dones, float *obs,
+                                                          const float *shapes_g, int batch,
+                                                          uint64_t reset_seed) {
     using S = Stage<E>;
     __shared__ float rows[E::EPB * S::STRIDE];
     __shared__ float cts[E::EPB * S::CSTRIDE];
     __shared__ float shapes[E::NSHAPE];
     __shared__ int was_reset[E::EPB];
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x;
     const int env0 = blockIdx.x * E::EPB;
     const int nenv = min(E::EPB, batch - env0);
     float *gbase = states + (size_t)env0 * E::STATE;
 
-    S::in(rows, gbase, nenv, lane);
-    for (int i = lane; i < E::NSHAPE; i += WAVE) shapes[i] = shapes_g[i];
-    if (lane < E::EPB) was_reset[lane] = 0;
+    S::in(rows, gbase, nenv, tid);
+    for (int i = tid; i < E::NSHAPE; i += BLOCK) shapes[i] = shapes_g[i];
+    if (tid < E::EPB) was_reset[tid] = 0;
     __syncthreads();
 
-    if (lane < nenv) {
-        const int env = env0 + lane;
-        float *row = rows + lane * S::STRIDE;
-        float r, d;
-        E::step(row, cts + lane * S::CSTRIDE, shapes, env, actions + (size_t)env * E::ACT_W, r, d);
-        rewards[env] = r;
-        dones[env] = d;
-        if (AUTORESET && d > 0.5f) {
-            E::reset(row, reset_seed, env);
-            was_reset[lane] = 1;
+    if (tid < WAVE) {
+        bool finished = false;
+        if (tid < nenv) {
+            const int env = env0 + tid;
+            float r, d;
+            E::step(rows + tid * S::STRIDE, cts + tid * S::CSTRIDE, shapes, env,
+                    actions + (size_t)env * E::ACT_W, r, d);
+            rewards[env] = r;
+            dones[env] = d;
+            finished = d > 0.5f;
         }
+        if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, tid);
     }
     __syncthreads();
 
-    for (int i = lane; i < nenv * E::OBS; i += WAVE) {   // observation out: [nenv, OBS] contiguous
+    for (int i = tid; i < nenv * E::OBS; i += BLOCK) {   // observation out: [nenv, OBS] contiguous
         int r = i / E::OBS, c = i - r * E::OBS;
         obs[(size_t)env0 * E::OBS + i] = rows[r * S::STRIDE + c];
     }
-    S::out(rows, gbase, nenv, lane, 0, E::DYN_END, nullptr);
-    S::out(rows, gbase, nenv, lane, E::L::META_OFF, E::STATE, nullptr);
-    if (AUTORESET) S::out(rows, gbase, nenv, lane, E::DYN_END, E::L::META_OFF, was_reset);
+    S::out(rows, gbase, nenv, tid, 0, E::DYN_END, nullptr);
+    S::out(rows, gbase, nenv, tid, E::L::META_OFF, E::STATE, nullptr);
+    if (AUTORESET) S::out(rows, gbase, nenv, tid, E::DYN_END, E::L::META_OFF, was_reset);
 }
 
 template <class E>
-__global__ __launch_bounds__(WAVE) void phys_reset_kernel(float *states, const float *dones, int batch,
-                                                          uint64_t seed, int selective) {
+__global__ __launch_bounds__(BLOCK) void phys_reset_kernel(float *states, const float *dones, int batch,
+                                                           uint64_t seed, int selective) {
     using S = Stage<E>;
     __shared__ float rows[E::EPB * S::STRIDE];
     __shared__ int was_reset[E::EPB];
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x;
     const int env0 = blockIdx.x * E::EPB;
     const int nenv = min(E::EPB, batch - env0);
-    if (lane < E::EPB) was_reset[lane] = 0;
-    if (lane < nenv) {
-        const int env = env0 + lane;
-        if (!selective || dones[env] > 0.5f) {
-            E::reset(rows + lane * S::STRIDE, seed, env);
-            was_reset[lane] = 1;
-        }
+    if (tid < E::EPB) was_reset[tid] = 0;
+    __syncthreads();
+    if (tid < WAVE) {
+        const bool want = tid < nenv && (!selective || dones[env0 + tid] > 0.5f);
+        reset_rows<E>(rows, was_reset, __ballot(want), seed, env0, tid);
     }
     __syncthreads();
-    S::out(rows, states + (size_t)env0 * E::STATE, nenv, lane, 0, E::STATE, was_reset);
+    S::out(rows, states + (size_t)env0 * E::STATE, nenv, tid, 0, E::STATE, was_reset);
 }
 
 template <class E>
 static int launch_phys_reset(mrl_ctx *ctx, int batch, float *states, const float *dones, uint64_t seed,
                              int selective) {
-    hipLaunchKernelGGL(phys_reset_kernel<E>, dim3(grid_for(batch, E::EPB)), dim3(WAVE), 0, ctx->stream,
+    hipLaunchKernelGGL(phys_reset_kernel<E>, dim3(grid_for(batch, E::EPB)), dim3(BLOCK), 0, ctx->stream,
                        states, dones, batch, seed, selective);
     return MRL_OK;
 }
@@ -249,10 +277,10 @@ static int launch_phys_step(mrl_ctx *ctx, int batch, float *states, const float 
                             uint64_t reset_seed) {
     dim3 grid(grid_for(batch, E::EPB));
     if (autoreset)
-        hipLaunchKernelGGL((phys_step_kernel<E, true>), grid, dim3(WAVE), 0, ctx->stream, states, actions,
+        hipLaunchKernelGGL((phys_step_kernel<E, true>), grid, dim3(BLOCK), 0, ctx->stream, states, actions,
                            rewards, dones, obs, shapes, batch, reset_seed);
     else
-        hipLaunchKernelGGL((phys_step_kernel<E, false>), grid, dim3(WAVE), 0, ctx->stream, states, actions,
+        hipLaunchKernelGGL((phys_step_kernel<E, false>), grid, dim3(BLOCK), 0, ctx->stream, states, actions,
                            rewards, dones, obs, shapes, batch, reset_seed);
     return MRL_OK;
 }

@@ -92,12 +92,57 @@ MRL_DEV void put_contact(float *c, int body, float px, float py, float nx, float
     c[C_DEPTH] = depth; c[C_JN] = 0.0f; c[C_JT] = 0.0f;
 }
 
-// vertex / circle against the row's terrain polyline; contacts in (body, vertex, edge) order
+// One vertex against one terrain edge whose x range it already passed.
+MRL_DEV void vertex_edge_test(const float *E, int b, float world_x, float world_y, float *contacts,
+                              int &count, int max_contacts) {
+    float e_x0 = E[0], e_x1 = E[2];
+    float e_y0 = E[1], e_y1 = E[3], e_nx = E[4], e_ny = E[5];
+    float edge_dx = e_x1 - e_x0, edge_dy = e_y1 - e_y0;
+    float edge_len_sq = edge_dx * edge_dx + edge_dy * edge_dy;
+    if (edge_len_sq < 1e-6f) return;
+    float t = ((world_x - e_x0) * edge_dx + (world_y - e_y0) * edge_dy) / edge_len_sq;
+    if (t < 0.0f) t = 0.0f;
+    if (t > 1.0f) t = 1.0f;
+    float closest_x = e_x0 + t * edge_dx, closest_y = e_y0 + t * edge_dy;
+    float dist_x = world_x - closest_x, dist_y = world_y - closest_y;
+    float penetration = -(dist_x * e_nx + dist_y * e_ny);
+    if (penetration > 0.0f && count < max_contacts) {
+        put_contact(contacts + count * CONTACT_SIZE, b, world_x, world_y, e_nx, e_ny, penetration);
+        count += 1;
+    }
+}
+
+// true when the vertex passes the x-range pre-check of collision/edge_terrain.mojo:236-249
+MRL_DEV bool edge_x_pass(float e_x0, float e_x1, float world_x) {
+    const float margin = 0.1f;
+    float x_min = e_x0 - margin, x_max = e_x1 + margin;
+    if (e_x0 > e_x1) { x_min = e_x1 - margin; x_max = e_x0 + margin; }
+    return !(world_x < x_min || world_x > x_max);
+}
+
+// vertex / circle against the row's terrain polyline; contacts in (body, vertex, edge) order.
+//
+// The x-range pre-check rejects almost every (vertex, edge) pair, but which pairs survive differs
+// from lane to lane, so a plain loop over the edges makes the wavefront run the full test for the
+// union of all lanes' survivors.  Instead each lane first collects its survivors of up to 32 edges
+// in a bit mask (cheap, no divergence), then all lanes walk their own masks together: the
+// wavefront runs the full test max-over-lanes(popcount) times.  Edges are visited in ascending
+// order per lane, so the contact list is the same.
 template <class L>
 MRL_DEV int edge_detect(const float *row, const float *shapes, float *contacts) {
     int count = 0;
-    const int n_edges = (int)row[L::EDGE_COUNT_OFF];
+    int n_edges = (int)row[L::EDGE_COUNT_OFF];
     const float *edges = row + L::EDGES_OFF;
+    constexpr bool SMALL = L::MAX_EDGES <= 16;     // edge x ranges fit in registers
+    constexpr int NR = SMALL ? L::MAX_EDGES : 1;
+    float ex0[NR], ex1[NR];
+    if (SMALL) {
+#pragma unroll
+        for (int e = 0; e < NR; ++e) {
+            ex0[e] = edges[e * 6];
+            ex1[e] = edges[e * 6 + 2];
+        }
+    }
     for (int b = 0; b < L::NUM_BODIES; ++b) {
         const float *B = row + L::BODIES_OFF + b * BODY_SIZE;
         float body_x = B[IDX_X], body_y = B[IDX_Y];
@@ -112,27 +157,31 @@ MRL_DEV int edge_detect(const float *row, const float *shapes, float *contacts) 
                 float local_x = S[2 + v * 2], local_y = S[3 + v * 2];
                 float world_x = body_x + local_x * cos_a - local_y * sin_a;
                 float world_y = body_y + local_x * sin_a + local_y * cos_a;
-                for (int e = 0; e < n_edges; ++e) {
-                    const float *E = edges + e * 6;
-                    float e_x0 = E[0], e_x1 = E[2];
-                    const float margin = 0.1f;
-                    float x_min = e_x0 - margin, x_max = e_x1 + margin;
-                    if (e_x0 > e_x1) { x_min = e_x1 - margin; x_max = e_x0 + margin; }
-                    if (world_x < x_min || world_x > x_max) continue;
-                    float e_y0 = E[1], e_y1 = E[3], e_nx = E[4], e_ny = E[5];
-                    float edge_dx = e_x1 - e_x0, edge_dy = e_y1 - e_y0;
-                    float edge_len_sq = edge_dx * edge_dx + edge_dy * edge_dy;
-                    if (edge_len_sq < 1e-6f) continue;
-                    float t = ((world_x - e_x0) * edge_dx + (world_y - e_y0) * edge_dy) / edge_len_sq;
-                    if (t < 0.0f) t = 0.0f;
-                    if (t > 1.0f) t = 1.0f;
-                    float closest_x = e_x0 + t * edge_dx, closest_y = e_y0 + t * edge_dy;
-                    float dist_x = world_x - closest_x, dist_y = world_y - closest_y;
-                    float penetration = -(dist_x * e_nx + dist_y * e_ny);
-                    if (penetration > 0.0f && count < L::MAX_CONTACTS) {
-                        put_contact(contacts + count * CONTACT_SIZE, b, world_x, world_y, e_nx, e_ny,
-                                    penetration);
-                        count += 1;
+                if (SMALL) {
+                    unsigned mask = 0;
+#pragma unroll
+                    for (int e = 0; e < NR; ++e)
+                        if (e < n_edges && edge_x_pass(ex0[e], ex1[e], world_x)) mask |= 1u << e;
+                    while (mask) {
+                        const int e = __ffs((int)mask) - 1;
+                        mask &= mask - 1;
+                        vertex_edge_test(edges + e * 6, b, world_x, world_y, contacts, count,
+                                         L::MAX_CONTACTS);
+                    }
+                } else {
+                    for (int e0 = 0; e0 < n_edges; e0 += 32) {
+                        const int m = min(32, n_edges - e0);
+                        unsigned mask = 0;
+                        for (int k = 0; k < m; ++k) {
+                            const float *E = edges + (e0 + k) * 6;
+                            if (edge_x_pass(E[0], E[2], world_x)) mask |= 1u << k;
+                        }
+                        while (mask) {
+                            const int e = e0 + __ffs((int)mask) - 1;
+                            mask &= mask - 1;
+                            vertex_edge_test(edges + e * 6, b, world_x, world_y, contacts, count,
+                                             L::MAX_CONTACTS);
+                        }
                     }
                 }
             }
