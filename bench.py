@@ -56,6 +56,23 @@ def cpu_baseline(np, n_envs=2048, steps=60):
                       "single thread, %.1f s" % (n_envs, steps, dt)}
 
 
+def measured_traffic():
+    """HBM bytes per launch by kernel name, from the committed counter summary
+    (profiles/bench_lunarlander8192_hbm_traffic.md: FETCH_SIZE / WRITE_SIZE readings of two
+    rocprofv3 --pmc runs of this script, already scaled by the copy-kernel calibration).
+    Empty when the file is absent."""
+    path = os.path.join(ROOT, "profiles", "bench_lunarlander8192_hbm_traffic.md")
+    out = {}
+    if not os.path.exists(path):
+        return out
+    with open(path) as f:
+        for line in f:
+            cells = [c.strip() for c in line.strip().strip("|").split("|")]
+            if len(cells) == 6 and cells[4].isdigit():
+                out[cells[0].replace("void ", "")] = int(cells[4])
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -81,11 +98,10 @@ def main():
     critic = mrl.seq(mrl.LinearReLU(OBS, HIDDEN), mrl.LinearReLU(HIDDEN, HIDDEN), mrl.Linear(HIDDEN, 1))
     T = max(args.steps, 1)
     rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N_ENVS, T, done_cap=4 * N_ENVS + 64 * T)
-    g = torch.Generator(device="cuda").manual_seed(0x5EED + 2)
     # reference init: Xavier over the flat vector with the network's in/out dims (initializers.mojo:69-76)
-    bound_a, bound_c = (2.0 / (OBS + NA)) ** 0.5, (2.0 / (OBS + 1)) ** 0.5
-    rb.actor_params = (torch.rand(actor.PARAM_SIZE, device="cuda", generator=g) * 2 - 1) * bound_a * 0.1
-    rb.critic_params = (torch.rand(critic.PARAM_SIZE, device="cuda", generator=g) * 2 - 1) * bound_c * 0.1
+    anet = mrl.Network(ctx, actor, mrl.Adam(lr=3e-4), mrl.Xavier(seed=0x5EED + 2))
+    cnet = mrl.Network(ctx, critic, mrl.Adam(lr=1e-3), mrl.Xavier(seed=0x5EED + 3))
+    rb.actor_params, rb.critic_params = anet.params, cnet.params
     E.reset_kernel_gpu(ctx, rb.states, 0x5EED + 2)
     rb.obs.copy_(rb.states.view(N_ENVS, E.STATE_SIZE)[:, :OBS].reshape(-1))
     desc = rb.descriptor()
@@ -112,23 +128,27 @@ def main():
     fwd_us, env_us = ph_us["policy_fwd"], ph_us["env_step"]
     fwd_tflops = FWD_FLOPS * N_ENVS / (fwd_us * 1e-6) / 1e12
     env_gbs = ENV_STEP_BYTES * N_ENVS / (env_us * 1e-6) / 1e9
+    traffic = measured_traffic()
     if fwd_us >= env_us:
-        roofline = {"kernel": "linear_fwd_kernel (actor+critic forward, 6 launches)", "bound": "mfma",
+        name = "mrl::policy_kernel<256, 1, false>"
+        roofline = {"kernel": name + " (actor + critic forward, sampling, stores)", "bound": "mfma",
                     "achieved": fwd_tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": fwd_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": None,
+                    "frac": fwd_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": traffic.get(name),
                     "avg_launch_us": fwd_us}
     else:
-        roofline = {"kernel": "ll_step_kernel<autoreset>", "bound": "hbm", "achieved": env_gbs,
+        name = "mrl::phys_step_kernel<mrl::LunarLander, true>"
+        roofline = {"kernel": name + " (env step + auto-reset)", "bound": "hbm", "achieved": env_gbs,
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": env_gbs / HBM_PEAK_GBS,
-                    "traffic": None, "avg_launch_us": env_us}
+                    "traffic": traffic.get(name), "avg_launch_us": env_us}
 
     # ---- PPO update on the collected batch (minibatch 4096, reference defaults)
     MB = 4096
-    upd = mrl.ppo.DiscreteUpdate(ctx, rb, MB, mrl.Adam(lr=3e-4), mrl.Adam(lr=1e-3), target_kl=0.0)
+    upd = mrl.ppo.DiscreteUpdate(ctx, rb, MB, anet.optimizer, cnet.optimizer, target_kl=0.0)
     upd.compute_advantages()
     total = N_ENVS * T
     n_mb = max(1, min(args.update_minibatches, total // MB))
-    perm = torch.randperm(total, device="cuda", generator=g).to(torch.int32)
+    perm = upd.indices
+    mrl.ppo.permutation(ctx, perm, 0x5EED)
     for k in range(3):
         upd.minibatch_step(perm[k * MB:(k + 1) * MB])
     torch.cuda.synchronize()

@@ -139,6 +139,23 @@ int mrl_gae(mrl_ctx *ctx, int T, int N, const float *rewards, const float *value
 /* (x - mean) / (sqrt(var + 1e-8) + 1e-8) in place: ppo.mojo:2356-2371, :2478-2511 + :637-653,
  * kernels.mojo:507-599 */
 int mrl_normalize_advantages(mrl_ctx *ctx, float *x, int n);
+/* RunningMeanStd.update / normalize of the reward stream, core/utils/normalization.mojo:188-292
+ * (used at deep_agents/ppo/ppo_continuous.mojo:2867-2871 on host copies).  state is a DEVICE
+ * array of 3 doubles (count, mean, var_sum), zero-initialised by the caller; all sums in Float64. */
+int mrl_rms_update(mrl_ctx *ctx, double *state, const float *x, int n);
+int mrl_rms_normalize(mrl_ctx *ctx, const double *state, float *x, int n);
+/* indices[0..n) = a pseudo-random permutation of 0..n-1 determined by seed; stands where the
+ * reference runs a host Fisher-Yates shuffle (deep_agents/ppo/ppo.mojo:2425-2434,
+ * core/utils/shuffle.mojo:21-82) and copies the indices to the device. */
+int mrl_permutation(mrl_ctx *ctx, int32_t *indices, int n, uint64_t seed);
+/* mean of kl[0..mb) against target_kl on the device: flag[0] is set to 1 when the mean exceeds
+ * target_kl (never cleared by the library), flag[1] receives the bits of the mean.  Replaces
+ * the per-minibatch D2H copy + host mean of ppo.mojo:2557-2573 / ppo_continuous.mojo:3062-3086. */
+int mrl_kl_check(mrl_ctx *ctx, const float *kl, int mb, float target_kl, int32_t *flag);
+/* params[i] = lo + u_i (hi - lo): the uniform fills behind Xavier / Kaiming
+ * (deep_rl/initializer/initializers.mojo:69-104) and StochasticActor.init_params_small
+ * (deep_rl/model/stochastic_actor.mojo:95-128); u from Philox(seed). */
+int mrl_init_uniform(mrl_ctx *ctx, float *params, int n, float lo, float hi, uint64_t seed);
 /* ppo_gather_minibatch_kernel ppo.mojo:135-191 / kernels.mojo:161-226: rows of the rollout
  * buffers picked by int32 indices */
 int mrl_gather_minibatch(mrl_ctx *ctx, const int32_t *indices, int mb, int obs_dim, int act_dim,
@@ -170,10 +187,10 @@ int mrl_adam_step(mrl_ctx *ctx, float *params, const float *grads, float *state,
 int mrl_clamp_log_std(mrl_ctx *ctx, float *params, int offset, int action_dim);
 
 /* ------------------------------------------------------------------ fused rollout step
- * One time step of train_gpu's collection loop for a discrete-action env
- * (deep_agents/ppo/ppo.mojo:2069-2285): actor + critic forward on obs, categorical
- * sampling, store of (obs, action, log_prob, value) into rollout row t, env step with
- * auto-reset, store of (reward, done), episode accounting.  The rollout buffers are the
+ * One time step of train_gpu's collection loop (deep_agents/ppo/ppo.mojo:2069-2285 for a
+ * discrete-action env, deep_agents/ppo/ppo_continuous.mojo:2619-2850 for a continuous one):
+ * actor + critic forward on obs, categorical or Gaussian sampling, store of (obs, action,
+ * log_prob, value) into rollout row t, env step with auto-reset, store of (reward, done), episode accounting.  The rollout buffers are the
  * reference's time-major ones ([T*N, ...], row = t*N + env); ep_return / ep_length are
  * the per-env accumulators of deep_rl/gpu/rl_kernels.mojo:103-227; finished episodes are
  * appended to done_returns / done_lengths (capacity done_cap) through the counter
@@ -188,6 +205,15 @@ int mrl_policy_step_discrete(mrl_ctx *ctx, const mrl_mlp_desc *actor, const mrl_
                              uint32_t seed, float *actions, float *r_obs, float *r_actions,
                              float *r_log_probs, float *r_values);
 
+/* Same for a continuous-action agent (deep_agents/ppo/ppo_continuous.mojo:2619-2686): the actor
+ * ends in a StochasticActor head, actions [n, A] are drawn as in kernels.mojo:12-98. */
+int mrl_policy_step_gaussian(mrl_ctx *ctx, const mrl_mlp_desc *actor, const mrl_mlp_desc *critic, int n,
+                             const float *obs, const float *actor_params, const float *critic_params,
+                             uint32_t seed, float *actions, float *r_obs, float *r_actions,
+                             float *r_log_probs, float *r_values);
+
+/* num_actions > 0: discrete agent (r_actions [T*N]); num_actions == 0: continuous agent whose
+ * actor ends in a StochasticActor head of the env's ACTION_DIM (r_actions [T*N, ACTION_DIM]). */
 typedef struct {
     int32_t env_id, n_envs, obs_dim, num_actions;
     float *states, *obs;                     /* [N, STATE_SIZE], [N, OBS] current observation */

@@ -13,9 +13,11 @@ from .context import DeviceContext  # noqa: E402
 from .envs import CartPoleEnv, PendulumV2, LunarLanderV2, BipedalWalkerV2, HalfCheetahPlanarV2  # noqa: E402
 from .model import Model, Linear, LinearReLU, LinearTanh, StochasticActor, seq  # noqa: E402
 from .optimizer import Adam  # noqa: E402
+from .training import Network, Xavier, Kaiming, init_params_small  # noqa: E402
 from . import ppo  # noqa: E402
 
 __all__ = ["DeviceContext", "CartPoleEnv", "PendulumV2", "LunarLanderV2", "BipedalWalkerV2",
            "HalfCheetahPlanarV2", "MrlError", "Model",
            "Linear", "LinearReLU", "LinearTanh", "StochasticActor", "seq", "Adam", "ppo",
+           "Network", "Xavier", "Kaiming", "init_params_small",
            "LINEAR", "LINEAR_RELU", "LINEAR_TANH", "STOCHASTIC_ACTOR"]

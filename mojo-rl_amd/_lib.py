@@ -76,7 +76,13 @@ SIGNATURES = {
     "mrl_clip_grad_norm": [P, P, I, F],
     "mrl_adam_step": [P, P, P, P, I, I, D, D, D, D],
     "mrl_clamp_log_std": [P, P, I, I],
+    "mrl_rms_update": [P, P, P, I],
+    "mrl_rms_normalize": [P, P, P, I],
+    "mrl_permutation": [P, P, I, U64],
+    "mrl_kl_check": [P, P, I, F, P],
+    "mrl_init_uniform": [P, P, I, F, F, U64],
     "mrl_policy_step_discrete": [P, DP, DP, I, P, P, P, U32, P, P, P, P, P],
+    "mrl_policy_step_gaussian": [P, DP, DP, I, P, P, P, U32, P, P, P, P, P],
     "mrl_rollout_step": [P, RP, I, U32, U64, U64],
 }
 _SPECIAL = {"mrl_version": (C.c_int, []), "mrl_last_error": (C.c_char_p, [])}

@@ -1,8 +1,11 @@
-// Fused collection-step policy kernel for discrete-action agents:
+// Fused collection-step policy kernel:
 //   actor  IN -> H -> H -> A   and   critic  IN -> H -> H -> 1   (ReLU or tanh hidden layers),
-//   categorical sampling, and the pre-step rollout stores, in ONE launch.
-// It replaces, per time step of deep_agents/ppo/ppo.mojo:2069-2146, six tiled-matmul launches,
-// _sample_actions_kernel (ppo.mojo:4064-4123) and _store_pre_step_kernel (ppo.mojo:662-690).
+//   action sampling, and the pre-step rollout stores, in ONE launch.
+// Discrete agents: logits head + categorical sampling.  It replaces, per time step of
+// deep_agents/ppo/ppo.mojo:2069-2146, six tiled-matmul launches, _sample_actions_kernel
+// (ppo.mojo:4064-4123) and _store_pre_step_kernel (ppo.mojo:662-690).
+// Continuous agents: StochasticActor head [mean | clamp(log_std)] + Gaussian sampling
+// (deep_agents/ppo/ppo_continuous.mojo:2619-2686, deep_agents/ppo/kernels.mojo:12-98).
 //
 // One workgroup = 32 environments (rows).  The 32 x H hidden activations never leave the CU:
 //   layer 0 (K = IN <= 32): one lane per hidden column, 32 row accumulators in registers, FMA;
@@ -100,8 +103,8 @@ MRL_DEV void head(const float *__restrict__ W2, int A, const float *h2, float *o
     }
 }
 
-template <int H, int ACT>
-__global__ __launch_bounds__(H) void policy_discrete_kernel(
+template <int H, int ACT, bool GAUSS>
+__global__ __launch_bounds__(H) void policy_kernel(
     const float *__restrict__ obs, int n, int IN, int A, const float *__restrict__ actor_p,
     const float *__restrict__ critic_p, uint32_t seed, float *__restrict__ actions,
     float *__restrict__ r_obs, float *__restrict__ r_actions, float *__restrict__ r_logp,
@@ -134,7 +137,7 @@ __global__ __launch_bounds__(H) void policy_discrete_kernel(
     head<H>(critic_p + IN * H + H + H * H + H, 1, h2, vals, 1);
     __syncthreads();
 
-    if (t < nrow) {   // categorical sampling, one lane per env
+    if (t < nrow && !GAUSS) {   // categorical sampling, one lane per env
         const int i = row0 + t;
         const float *l = logits + t * (PA_MAX + 1);
         uint32_t rng = seed ^ ((uint32_t)i * 2654435761u);
@@ -157,20 +160,46 @@ __global__ __launch_bounds__(H) void policy_discrete_kernel(
         r_logp[i] = logf(pr + 1e-8f);
         r_values[i] = vals[t];
     }
+    if (t < nrow && GAUSS) {    // Gaussian sampling, one lane per env, one Philox stream per (env, j)
+        const int i = row0 + t;
+        const float *mean_row = logits + t * (PA_MAX + 1);
+        const float *log_std_p = actor_p + IN * H + H + H * H + H + H * A + A;
+        const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
+        float total = 0.0f;
+        for (int j = 0; j < A; ++j) {
+            const float mean = mean_row[j];
+            float log_std = log_std_p[j];
+            if (log_std < -5.0f) log_std = -5.0f;
+            else if (log_std > 2.0f) log_std = 2.0f;
+            Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j), 0, 0);
+            const float u1 = rv.v[0] + 1e-8f;
+            const float mag = sqrtf(-2.0f * logf(u1));
+            const float noise = mag * cosf(rv.v[1] * (float)6.283185307179586);
+            const float std = expf(log_std);
+            const float action = mean + std * noise;
+            actions[(long)i * A + j] = action;
+            r_actions[(long)i * A + j] = action;
+            const float an = (action - mean) / (std + EPS);
+            total = total + -0.5f * (LOG_2PI + 2.0f * log_std + an * an);
+        }
+        r_logp[i] = total;
+        r_values[i] = vals[t];
+    }
 }
 
 // true when the pair (actor, critic) has the shape this kernel is specialised for
-bool policy_fusable(const mrl_mlp_desc &a, const mrl_mlp_desc &c, int *H, int *act) {
+bool policy_fusable(const mrl_mlp_desc &a, const mrl_mlp_desc &c, bool gauss, int *H, int *act) {
     if (a.n_layers != 3 || c.n_layers != 3) return false;
     const int k0 = a.layers[0].kind;
     if (k0 != MRL_LINEAR_RELU && k0 != MRL_LINEAR_TANH) return false;
     for (const mrl_mlp_desc *d : {&a, &c}) {
-        if (d->layers[0].kind != k0 || d->layers[1].kind != k0 || d->layers[2].kind != MRL_LINEAR)
-            return false;
+        if (d->layers[0].kind != k0 || d->layers[1].kind != k0) return false;
         if (d->layers[0].in_dim != a.layers[0].in_dim || d->layers[0].in_dim > PIN_MAX) return false;
         if (d->layers[0].out_dim != a.layers[0].out_dim || d->layers[1].out_dim != a.layers[0].out_dim)
             return false;
     }
+    if (a.layers[2].kind != (gauss ? MRL_STOCHASTIC_ACTOR : MRL_LINEAR) || c.layers[2].kind != MRL_LINEAR)
+        return false;
     const int h = a.layers[0].out_dim;
     if (h != 64 && h != 256) return false;
     if (a.layers[2].out_dim > PA_MAX || c.layers[2].out_dim != 1) return false;
@@ -179,20 +208,27 @@ bool policy_fusable(const mrl_mlp_desc &a, const mrl_mlp_desc &c, int *H, int *a
     return true;
 }
 
-int launch_policy_discrete(mrl_ctx *ctx, const mrl_mlp_desc &a, const mrl_mlp_desc &c, const float *obs,
-                           int n, const float *ap, const float *cp, uint32_t seed, float *actions,
-                           float *r_obs, float *r_actions, float *r_logp, float *r_values) {
+int launch_policy(mrl_ctx *ctx, const mrl_mlp_desc &a, const mrl_mlp_desc &c, bool gauss, const float *obs,
+                  int n, const float *ap, const float *cp, uint32_t seed, float *actions, float *r_obs,
+                  float *r_actions, float *r_logp, float *r_values) {
     int H = 0, act = 0;
-    if (!policy_fusable(a, c, &H, &act)) return MRL_E_UNSUPPORTED;
+    if (!policy_fusable(a, c, gauss, &H, &act)) return MRL_E_UNSUPPORTED;
     const int IN = a.layers[0].in_dim, A = a.layers[2].out_dim;
     dim3 grid((n + PR - 1) / PR);
-#define MRL_LAUNCH(HH, AA)                                                                          \
-    hipLaunchKernelGGL((policy_discrete_kernel<HH, AA>), grid, dim3(HH), 0, ctx->stream, obs, n, IN, \
-                       A, ap, cp, seed, actions, r_obs, r_actions, r_logp, r_values)
-    if (H == 256 && act == 1) MRL_LAUNCH(256, 1);
-    else if (H == 256 && act == 2) MRL_LAUNCH(256, 2);
-    else if (H == 64 && act == 1) MRL_LAUNCH(64, 1);
-    else MRL_LAUNCH(64, 2);
+#define MRL_LAUNCH(HH, AA, GG)                                                                         \
+    hipLaunchKernelGGL((policy_kernel<HH, AA, GG>), grid, dim3(HH), 0, ctx->stream, obs, n, IN, A, ap, \
+                       cp, seed, actions, r_obs, r_actions, r_logp, r_values)
+    if (gauss) {
+        if (H == 256 && act == 1) MRL_LAUNCH(256, 1, true);
+        else if (H == 256 && act == 2) MRL_LAUNCH(256, 2, true);
+        else if (H == 64 && act == 1) MRL_LAUNCH(64, 1, true);
+        else MRL_LAUNCH(64, 2, true);
+    } else {
+        if (H == 256 && act == 1) MRL_LAUNCH(256, 1, false);
+        else if (H == 256 && act == 2) MRL_LAUNCH(256, 2, false);
+        else if (H == 64 && act == 1) MRL_LAUNCH(64, 1, false);
+        else MRL_LAUNCH(64, 2, false);
+    }
 #undef MRL_LAUNCH
     MRL_CHECK_LAUNCH();
     return MRL_OK;

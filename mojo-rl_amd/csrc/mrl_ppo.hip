@@ -149,6 +149,160 @@ __global__ __launch_bounds__(TPB) void normalize_apply_kernel(float *__restrict_
     x[i] = (x[i] - mean) / (std + 1e-8f);
 }
 
+// ---------------------------------------------------------------- reward RunningMeanStd
+// core/utils/normalization.mojo:188-292 in Float64: batch mean and variance (two passes), merged
+// into (count, mean, var_sum) with Chan's formula; normalise with var = 1 while count < 2.
+MRL_DEV double wave_sum_d(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+MRL_DEV double block_sum_d(double v, double *smem) {
+    v = wave_sum_d(v);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) smem[w] = v;
+    __syncthreads();
+    double t = 0.0;
+    for (int k = 0; k < (int)(blockDim.x >> 6); ++k) t += smem[k];
+    __syncthreads();
+    return t;
+}
+
+// mean_ptr == nullptr: out[b] = sum x; else out[b] = sum (x - *mean_ptr)^2
+__global__ __launch_bounds__(TPB) void rms_partial_kernel(const float *__restrict__ x, int n,
+                                                          const double *__restrict__ mean_ptr,
+                                                          double *__restrict__ out) {
+    __shared__ double smem[4];
+    const double mean = mean_ptr ? *mean_ptr : 0.0;
+    double s = 0.0;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        double d = (double)x[i] - mean;
+        s += mean_ptr ? d * d : (double)x[i];
+    }
+    s = block_sum_d(s, smem);
+    if (threadIdx.x == 0) out[blockIdx.x] = s;
+}
+
+__global__ __launch_bounds__(TPB) void rms_batch_mean_kernel(const double *__restrict__ in, int nb, int n,
+                                                             double *__restrict__ out) {
+    __shared__ double smem[4];
+    double s = 0.0;
+    for (int i = threadIdx.x; i < nb; i += blockDim.x) s += in[i];
+    s = block_sum_d(s, smem);
+    if (threadIdx.x == 0) out[0] = s / (double)n;
+}
+
+// state = (count, mean, var_sum)
+__global__ __launch_bounds__(TPB) void rms_merge_kernel(const double *__restrict__ in, int nb, int n,
+                                                        const double *__restrict__ batch_mean,
+                                                        double *__restrict__ state) {
+    __shared__ double smem[4];
+    double s = 0.0;
+    for (int i = threadIdx.x; i < nb; i += blockDim.x) s += in[i];
+    s = block_sum_d(s, smem);
+    if (threadIdx.x != 0) return;
+    const double bm = *batch_mean, bv = s / (double)n;
+    const double count = state[0], mean = state[1], var_sum = state[2];
+    const double new_count = count + (double)n;
+    if (count == 0.0) {
+        state[1] = bm;
+        state[2] = bv * (double)n;
+    } else {
+        const double delta = bm - mean;
+        state[1] = mean + delta * (double)n / new_count;
+        state[2] = var_sum + bv * (double)n + delta * delta * count * (double)n / new_count;
+    }
+    state[0] = new_count;
+}
+
+__global__ __launch_bounds__(TPB) void rms_normalize_kernel(const double *__restrict__ state,
+                                                            float *__restrict__ x, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const double count = state[0], mean = state[1];
+    const double var = (count < 2.0) ? 1.0 : state[2] / count;
+    const double std = sqrt(var + 1e-8);
+    x[i] = (float)(((double)x[i] - mean) / (std + 1e-8));
+}
+
+// ---------------------------------------------------------------- permutation
+// A keyed bijection of [0, 2^k) (balanced Feistel network on k = 2h bits, round keys from
+// Philox) with cycle walking down to [0, n): idx[i] = P(i).  One pass, no sort, no scratch.
+// It stands where the reference shuffles on the host (Fisher-Yates driven by the global
+// random_float64 stream, deep_agents/ppo/ppo.mojo:2425-2434, core/utils/shuffle.mojo:21-82).
+constexpr int PERM_ROUNDS = 8;
+struct PermKeys { uint32_t k[PERM_ROUNDS]; };
+
+MRL_DEV uint32_t perm_mix(uint32_t x) {
+    x ^= x >> 16; x *= 0x85ebca6bu; x ^= x >> 13; x *= 0xc2b2ae35u; x ^= x >> 16;
+    return x;
+}
+
+__global__ __launch_bounds__(TPB) void permutation_kernel(int32_t *__restrict__ idx, int n, int half_bits,
+                                                          PermKeys keys) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t mask = (1u << half_bits) - 1u;
+    uint32_t x = (uint32_t)i;
+    do {
+        uint32_t l = x >> half_bits, r = x & mask;
+#pragma unroll
+        for (int k = 0; k < PERM_ROUNDS; ++k) {
+            const uint32_t f = perm_mix(r ^ keys.k[k]) & mask;
+            const uint32_t nl = r;
+            r = l ^ f;
+            l = nl;
+        }
+        x = (l << half_bits) | r;
+    } while (x >= (uint32_t)n);
+    idx[i] = (int32_t)x;
+}
+
+// host Philox4x32-10 block (round keys of the permutation)
+static void philox4x32_10_host(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+// ---------------------------------------------------------------- parameter initialisation
+// p[i] = lo + u_i * (hi - lo), u_i = lane (i % 4) of Philox(seed, offset = i / 4): the uniform
+// fills of deep_rl/initializer/initializers.mojo:69-104 (Xavier / Kaiming bounds are formed by
+// the caller) and StochasticActor.init_params_small (stochastic_actor.mojo:95-128).
+__global__ __launch_bounds__(TPB) void init_uniform_kernel(float *__restrict__ p, int n, float lo, float hi,
+                                                           uint64_t seed) {
+    int q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q * 4 >= n) return;
+    Uniform4 u = philox_uniform4(seed, (uint64_t)q, 0);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (q * 4 + k < n) p[q * 4 + k] = lo + u.v[k] * (hi - lo);
+}
+
+// ---------------------------------------------------------------- KL early stop
+// mean of the minibatch's per-sample KL estimates compared with target_kl on the device
+// (ppo.mojo:2557-2573, ppo_continuous.mojo:3062-3086 do this on the host after a copy):
+// flag[0] = 1 once mean KL > target (sticky), flag[1] = bit pattern of the last mean.
+__global__ __launch_bounds__(TPB) void kl_check_kernel(const float *__restrict__ kl, int mb, float target,
+                                                       int32_t *__restrict__ flag) {
+    __shared__ float smem[4];
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < mb; i += blockDim.x) s = s + kl[i];
+    s = block_sum(s, smem);
+    if (threadIdx.x == 0) {
+        const float mean = s / (float)mb;
+        flag[1] = __float_as_int(mean);
+        if (mean > target) flag[0] = 1;
+    }
+}
+
 // ---------------------------------------------------------------- gather
 __global__ __launch_bounds__(TPB) void gather_kernel(const int32_t *__restrict__ idx, int mb, int obs_dim,
                                                      int act_dim, const float *r_obs, const float *r_act,
@@ -433,6 +587,73 @@ int mrl_normalize_advantages(mrl_ctx *ctx, float *x, int n) {
     hipLaunchKernelGGL(partial_sum_kernel, dim3(nb), dim3(TPB), 0, ctx->stream, x, n, (const float *)stats, part);
     hipLaunchKernelGGL(finish_mean_kernel, dim3(1), dim3(TPB), 0, ctx->stream, part, nb, n, stats + 1);
     hipLaunchKernelGGL(normalize_apply_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream, x, n, stats);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_rms_update(mrl_ctx *ctx, double *state, const float *x, int n) {
+    MRL_CHECK_ARG(ctx, "mrl_rms_update: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0, "mrl_rms_update: negative size");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(state && x, "mrl_rms_update: NULL buffer");
+    const int nb = std::min(1024, grid_for(n, TPB));
+    double *part = reinterpret_cast<double *>(ctx->reduce_scratch);   // [0, nb) doubles
+    double *bm = part + 1024;
+    hipLaunchKernelGGL(rms_partial_kernel, dim3(nb), dim3(TPB), 0, ctx->stream, x, n, (const double *)nullptr, part);
+    hipLaunchKernelGGL(rms_batch_mean_kernel, dim3(1), dim3(TPB), 0, ctx->stream, part, nb, n, bm);
+    hipLaunchKernelGGL(rms_partial_kernel, dim3(nb), dim3(TPB), 0, ctx->stream, x, n, (const double *)bm, part);
+    hipLaunchKernelGGL(rms_merge_kernel, dim3(1), dim3(TPB), 0, ctx->stream, part, nb, n, bm, state);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_rms_normalize(mrl_ctx *ctx, const double *state, float *x, int n) {
+    MRL_CHECK_ARG(ctx, "mrl_rms_normalize: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0, "mrl_rms_normalize: negative size");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(state && x, "mrl_rms_normalize: NULL buffer");
+    hipLaunchKernelGGL(rms_normalize_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream, state, x, n);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_permutation(mrl_ctx *ctx, int32_t *indices, int n, uint64_t seed) {
+    MRL_CHECK_ARG(ctx, "mrl_permutation: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0 && n <= (1 << 30), "mrl_permutation: n = %d out of range", n);
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(indices, "mrl_permutation: NULL buffer");
+    int half_bits = 1;
+    while ((1ll << (2 * half_bits)) < (long long)n) ++half_bits;
+    PermKeys keys;
+    for (int k = 0; k < PERM_ROUNDS; k += 4) {
+        uint32_t ctr[4] = {(uint32_t)(k / 4), 0x7065726du, 0u, 0u};
+        uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+        uint32_t out[4];
+        philox4x32_10_host(ctr, key, out);
+        for (int j = 0; j < 4 && k + j < PERM_ROUNDS; ++j) keys.k[k + j] = out[j];
+    }
+    hipLaunchKernelGGL(permutation_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream, indices, n,
+                       half_bits, keys);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_kl_check(mrl_ctx *ctx, const float *kl, int mb, float target_kl, int32_t *flag) {
+    MRL_CHECK_ARG(ctx, "mrl_kl_check: ctx is NULL");
+    MRL_CHECK_ARG(mb > 0, "mrl_kl_check: minibatch must be positive");
+    MRL_CHECK_ARG(kl && flag, "mrl_kl_check: NULL buffer");
+    hipLaunchKernelGGL(kl_check_kernel, dim3(1), dim3(TPB), 0, ctx->stream, kl, mb, target_kl, flag);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_init_uniform(mrl_ctx *ctx, float *params, int n, float lo, float hi, uint64_t seed) {
+    MRL_CHECK_ARG(ctx, "mrl_init_uniform: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0, "mrl_init_uniform: negative size");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(params, "mrl_init_uniform: NULL buffer");
+    hipLaunchKernelGGL(init_uniform_kernel, dim3(grid_for((n + 3) / 4, TPB)), dim3(TPB), 0, ctx->stream,
+                       params, n, lo, hi, seed);
     MRL_CHECK_LAUNCH();
     return MRL_OK;
 }

@@ -7,9 +7,9 @@
 
 namespace mrl {
 
-int launch_policy_discrete(mrl_ctx *ctx, const mrl_mlp_desc &a, const mrl_mlp_desc &c, const float *obs,
-                           int n, const float *ap, const float *cp, uint32_t seed, float *actions,
-                           float *r_obs, float *r_actions, float *r_logp, float *r_values);
+int launch_policy(mrl_ctx *ctx, const mrl_mlp_desc &a, const mrl_mlp_desc &c, bool gauss, const float *obs,
+                  int n, const float *ap, const float *cp, uint32_t seed, float *actions, float *r_obs,
+                  float *r_actions, float *r_logp, float *r_values);
 
 // sampling (ppo.mojo:4064-4123) fused with _store_pre_step_kernel (ppo.mojo:662-690):
 // rollout row t gets obs, action, log-prob and value; `actions` feeds the env step.
@@ -38,6 +38,37 @@ __global__ __launch_bounds__(256) void sample_store_kernel(
     actions[i] = (float)sel;
     r_actions[i] = (float)sel;
     r_logp[i] = logf(p + 1e-8f);
+    r_values[i] = values[i];
+    for (int k = 0; k < obs_dim; ++k) r_obs[(long)i * obs_dim + k] = obs[(long)i * obs_dim + k];
+}
+
+// continuous counterpart: _sample_continuous_actions_kernel (kernels.mojo:12-98) fused with
+// the pre-step store (ppo_continuous.mojo:2672-2686)
+__global__ __launch_bounds__(256) void sample_store_gaussian_kernel(
+    const float *__restrict__ actor_out, const float *__restrict__ values, const float *__restrict__ obs,
+    int n, int A, int obs_dim, uint32_t seed, float *__restrict__ actions, float *__restrict__ r_obs,
+    float *__restrict__ r_actions, float *__restrict__ r_logp, float *__restrict__ r_values) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
+    float total = 0.0f;
+    for (int j = 0; j < A; ++j) {
+        float mean = actor_out[(long)i * 2 * A + j];
+        float log_std = actor_out[(long)i * 2 * A + A + j];
+        if (log_std < -5.0f) log_std = -5.0f;
+        else if (log_std > 2.0f) log_std = 2.0f;
+        Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j), 0, 0);
+        float u1 = rv.v[0] + 1e-8f;
+        float mag = sqrtf(-2.0f * logf(u1));
+        float noise = mag * cosf(rv.v[1] * (float)6.283185307179586);
+        float std = expf(log_std);
+        float action = mean + std * noise;
+        actions[(long)i * A + j] = action;
+        r_actions[(long)i * A + j] = action;
+        float an = (action - mean) / (std + EPS);
+        total = total + -0.5f * (LOG_2PI + 2.0f * log_std + an * an);
+    }
+    r_logp[i] = total;
     r_values[i] = values[i];
     for (int k = 0; k < obs_dim; ++k) r_obs[(long)i * obs_dim + k] = obs[(long)i * obs_dim + k];
 }
@@ -75,6 +106,9 @@ using namespace mrl;
 
 extern "C" {
 
+// floats per env after the policy temporaries: actions (<= 8), reward, done
+#define MRL_ROLLOUT_TAIL 10
+
 // layer-by-layer fallback needs logits/values temporaries
 static int ensure_rollout_ws(mrl_ctx *ctx, size_t need) {
     if (ctx->rollout_ws_floats < need) {
@@ -88,41 +122,67 @@ static int ensure_rollout_ws(mrl_ctx *ctx, size_t need) {
     return MRL_OK;
 }
 
-int mrl_policy_step_discrete(mrl_ctx *ctx, const mrl_mlp_desc *actor, const mrl_mlp_desc *critic, int n,
-                             const float *obs, const float *actor_params, const float *critic_params,
-                             uint32_t seed, float *actions, float *r_obs, float *r_actions,
-                             float *r_log_probs, float *r_values) {
-    MRL_CHECK_ARG(ctx && actor && critic, "mrl_policy_step_discrete: NULL argument");
-    MRL_CHECK_ARG(n >= 0, "mrl_policy_step_discrete: negative n");
+static int policy_step(mrl_ctx *ctx, const char *who, bool gauss, const mrl_mlp_desc *actor,
+                       const mrl_mlp_desc *critic, int n, const float *obs, const float *actor_params,
+                       const float *critic_params, uint32_t seed, float *actions, float *r_obs,
+                       float *r_actions, float *r_log_probs, float *r_values) {
+    MRL_CHECK_ARG(ctx && actor && critic, "%s: NULL argument", who);
+    MRL_CHECK_ARG(n >= 0, "%s: negative n", who);
     if (n == 0) return MRL_OK;
     MRL_CHECK_ARG(obs && actor_params && critic_params && actions && r_obs && r_actions && r_log_probs &&
-                      r_values, "mrl_policy_step_discrete: NULL buffer");
-    const int na = mrl_mlp_out_dim(actor), nv = mrl_mlp_out_dim(critic);
-    MRL_CHECK_ARG(na > 0 && nv == 1, "mrl_policy_step_discrete: actor must end in logits, critic in 1 value");
+                      r_values, "%s: NULL buffer", who);
+    MRL_CHECK_ARG(actor->n_layers >= 1 && actor->n_layers <= MRL_MAX_LAYERS && critic->n_layers >= 1 &&
+                      critic->n_layers <= MRL_MAX_LAYERS, "%s: bad layer count", who);
+    const bool head_is_actor = actor->layers[actor->n_layers - 1].kind == MRL_STOCHASTIC_ACTOR;
+    MRL_CHECK_ARG(head_is_actor == gauss,
+                  gauss ? "%s: actor must end in a StochasticActor head" : "%s: actor must end in logits", who);
+    const int na = mrl_mlp_out_dim(actor), nv = mrl_mlp_out_dim(critic);   // na = 2A for a Gaussian actor
+    MRL_CHECK_ARG(na > 0 && nv == 1, "%s: critic must end in 1 value", who);
     MRL_CHECK_ARG(actor->layers[0].in_dim == critic->layers[0].in_dim,
-                  "mrl_policy_step_discrete: actor and critic read different observation widths");
+                  "%s: actor and critic read different observation widths", who);
     const int od = actor->layers[0].in_dim;
     profile_mark(ctx, -1);
-    int rc = launch_policy_discrete(ctx, *actor, *critic, obs, n, actor_params, critic_params, seed,
-                                    actions, r_obs, r_actions, r_log_probs, r_values);
+    int rc = launch_policy(ctx, *actor, *critic, gauss, obs, n, actor_params, critic_params, seed, actions,
+                           r_obs, r_actions, r_log_probs, r_values);
     if (rc == MRL_OK) {
         profile_mark(ctx, MRL_PHASE_POLICY_FWD);
         return MRL_OK;
     }
     if (rc != MRL_E_UNSUPPORTED) return rc;
-    rc = ensure_rollout_ws(ctx, (size_t)n * (na + 5));
+    rc = ensure_rollout_ws(ctx, (size_t)n * (na + 1) + (size_t)n * (MRL_ROLLOUT_TAIL));
     if (rc) return rc;
-    float *logits = ctx->rollout_ws, *values = logits + (size_t)n * na;
-    rc = mrl_mlp_forward(ctx, actor, n, obs, actor_params, logits, nullptr);
+    float *head = ctx->rollout_ws, *values = head + (size_t)n * na;
+    rc = mrl_mlp_forward(ctx, actor, n, obs, actor_params, head, nullptr);
     if (rc) return rc;
     rc = mrl_mlp_forward(ctx, critic, n, obs, critic_params, values, nullptr);
     if (rc) return rc;
     profile_mark(ctx, MRL_PHASE_POLICY_FWD);
-    hipLaunchKernelGGL(sample_store_kernel, dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream, logits,
-                       values, obs, n, na, od, seed, actions, r_obs, r_actions, r_log_probs, r_values);
+    if (gauss)
+        hipLaunchKernelGGL(sample_store_gaussian_kernel, dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream,
+                           head, values, obs, n, na / 2, od, seed, actions, r_obs, r_actions, r_log_probs,
+                           r_values);
+    else
+        hipLaunchKernelGGL(sample_store_kernel, dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream, head,
+                           values, obs, n, na, od, seed, actions, r_obs, r_actions, r_log_probs, r_values);
     MRL_CHECK_LAUNCH();
     profile_mark(ctx, MRL_PHASE_SAMPLE);
     return MRL_OK;
+}
+
+int mrl_policy_step_discrete(mrl_ctx *ctx, const mrl_mlp_desc *actor, const mrl_mlp_desc *critic, int n,
+                             const float *obs, const float *actor_params, const float *critic_params,
+                             uint32_t seed, float *actions, float *r_obs, float *r_actions,
+                             float *r_log_probs, float *r_values) {
+    return policy_step(ctx, "mrl_policy_step_discrete", false, actor, critic, n, obs, actor_params,
+                       critic_params, seed, actions, r_obs, r_actions, r_log_probs, r_values);
+}
+
+int mrl_policy_step_gaussian(mrl_ctx *ctx, const mrl_mlp_desc *actor, const mrl_mlp_desc *critic, int n,
+                             const float *obs, const float *actor_params, const float *critic_params,
+                             uint32_t seed, float *actions, float *r_obs, float *r_actions,
+                             float *r_log_probs, float *r_values) {
+    return policy_step(ctx, "mrl_policy_step_gaussian", true, actor, critic, n, obs, actor_params,
+                       critic_params, seed, actions, r_obs, r_actions, r_log_probs, r_values);
 }
 
 int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_seed,
@@ -136,21 +196,24 @@ int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_
     int ss, od, na, ad;
     int rc = mrl_env_dims(r->env_id, &ss, &od, &na, &ad);
     if (rc) return rc;
-    MRL_CHECK_ARG(na > 0 && na == r->num_actions && od == r->obs_dim,
-                  "mrl_rollout_step: descriptor does not match a discrete-action env");
-    MRL_CHECK_ARG(mrl_mlp_out_dim(&r->actor) == na && r->actor.layers[0].in_dim == od,
-                  "mrl_rollout_step: actor must map obs_dim to num_actions logits");
+    const bool gauss = r->num_actions == 0;
+    MRL_CHECK_ARG(od == r->obs_dim && (gauss ? ad > 0 : (na > 0 && na == r->num_actions)),
+                  "mrl_rollout_step: descriptor does not match the env's observation / action space");
+    const int head = gauss ? 2 * ad : na;    // width of the actor's output
+    const int aw = gauss ? ad : 1;           // floats per stored action
+    MRL_CHECK_ARG(mrl_mlp_out_dim(&r->actor) == head && r->actor.layers[0].in_dim == od,
+                  "mrl_rollout_step: actor must map obs_dim to the env's action head");
     const int N = r->n_envs;
-    rc = ensure_rollout_ws(ctx, (size_t)N * (na + 5));
+    rc = ensure_rollout_ws(ctx, (size_t)N * (head + 1) + (size_t)N * MRL_ROLLOUT_TAIL);
     if (rc) return rc;
-    // [logits N*na | values N] are used by the layer-by-layer policy path; the tail holds the
-    // step's actions, rewards and dones
-    float *actions = ctx->rollout_ws + (size_t)N * (na + 1);
-    float *rewards = actions + N, *dones = rewards + N;
+    // [head N*head | values N] are used by the layer-by-layer policy path; the tail holds the
+    // step's actions (up to 8 per env), rewards and dones
+    float *actions = ctx->rollout_ws + (size_t)N * (head + 1);
+    float *rewards = actions + (size_t)N * 8, *dones = rewards + N;
     const size_t row = (size_t)t * N;
-    rc = mrl_policy_step_discrete(ctx, &r->actor, &r->critic, N, r->obs, r->actor_params,
-                                  r->critic_params, sample_seed, actions, r->r_obs + row * od,
-                                  r->r_actions + row, r->r_log_probs + row, r->r_values + row);
+    rc = policy_step(ctx, "mrl_rollout_step", gauss, &r->actor, &r->critic, N, r->obs, r->actor_params,
+                     r->critic_params, sample_seed, actions, r->r_obs + row * od, r->r_actions + row * aw,
+                     r->r_log_probs + row, r->r_values + row);
     if (rc) return rc;
     profile_mark(ctx, -1);
     rc = mrl_env_step_autoreset(ctx, r->env_id, N, r->states, actions, rewards, dones, r->obs, step_seed,

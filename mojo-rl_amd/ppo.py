@@ -80,21 +80,54 @@ def clamp_log_std_params(ctx, params, log_std_offset, action_dim):
     _lib.call("mrl_clamp_log_std", ctx.handle, _ptr(params), log_std_offset, action_dim)
 
 
-class RolloutBuffers:
-    """Device buffers of train_gpu's collection phase for a discrete-action env
-    (deep_agents/ppo/ppo.mojo:1616-1775): time-major rollout arrays, per-env episode
-    accumulators and the device-side list of finished episodes."""
+def permutation(ctx, indices, seed):
+    """Fills the int32 device buffer with a seeded pseudo-random permutation of 0..n-1; stands
+    where train_gpu shuffles on the host (ppo.mojo:2425-2434)."""
+    if indices.dtype != torch.int32:
+        raise _lib.MrlError("permutation indices must be int32")
+    _lib.call("mrl_permutation", ctx.handle, _ptr(indices), indices.numel(), int(seed) & (2**64 - 1))
 
-    def __init__(self, ctx, env, actor, critic, n_envs, rollout_len, done_cap=None):
+
+def kl_check(ctx, kl, target_kl, flag):
+    """Device-side early-stop test: flag[0] (int32) becomes 1 when mean(kl) > target_kl and stays
+    1; flag[1] holds the bits of the mean (ppo.mojo:2557-2573 without the host copy)."""
+    _lib.call("mrl_kl_check", ctx.handle, _ptr(kl), kl.numel(), float(target_kl), _ptr(flag))
+
+
+class RunningMeanStd:
+    """core/utils/normalization.mojo:188-292 with the state (count, mean, var_sum) in device
+    memory, Float64 throughout; used for reward normalisation (ppo_continuous.mojo:2867-2871)."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+        self.state = torch.zeros(3, dtype=torch.float64, device=ctx.device)
+
+    def update(self, x):
+        _lib.call("mrl_rms_update", self.ctx.handle, _ptr(self.state), _ptr(x), x.numel())
+
+    def normalize(self, x):
+        _lib.call("mrl_rms_normalize", self.ctx.handle, _ptr(self.state), _ptr(x), x.numel())
+
+
+class RolloutBuffers:
+    """Device buffers of train_gpu's collection phase (deep_agents/ppo/ppo.mojo:1616-1775,
+    ppo_continuous.mojo:2180-2470): time-major rollout arrays, per-env episode accumulators and
+    the device-side list of finished episodes.  A discrete agent (env.NUM_ACTIONS > 0 and
+    continuous=False) stores one float per action, a continuous one env.ACTION_DIM."""
+
+    def __init__(self, ctx, env, actor, critic, n_envs, rollout_len, done_cap=None, continuous=None):
         dev = ctx.device
         z = lambda *s: torch.zeros(*s, device=dev)
         self.ctx, self.env, self.actor, self.critic = ctx, env, actor, critic
         self.n_envs, self.rollout_len = n_envs, rollout_len
+        self.continuous = (env.NUM_ACTIONS == 0) if continuous is None else continuous
+        self.act_width = env.ACTION_DIM if self.continuous else 1
         self.states = z(n_envs * env.STATE_SIZE)
         self.obs = z(n_envs * env.OBS_DIM)
         T = rollout_len
         self.r_obs = z(T * n_envs * env.OBS_DIM)
-        self.r_actions, self.r_log_probs, self.r_values = z(T * n_envs), z(T * n_envs), z(T * n_envs)
+        self.r_actions = z(T * n_envs * self.act_width)
+        self.r_log_probs, self.r_values = z(T * n_envs), z(T * n_envs)
         self.r_rewards, self.r_dones = z(T * n_envs), z(T * n_envs)
         self.ep_return, self.ep_length = z(n_envs), z(n_envs)
         self.done_cap = done_cap or max(1024, 4 * n_envs)
@@ -106,7 +139,8 @@ class RolloutBuffers:
     def descriptor(self):
         r = _lib.Rollout()
         e = self.env
-        r.env_id, r.n_envs, r.obs_dim, r.num_actions = e.ENV_ID, self.n_envs, e.OBS_DIM, e.NUM_ACTIONS
+        r.env_id, r.n_envs, r.obs_dim = e.ENV_ID, self.n_envs, e.OBS_DIM
+        r.num_actions = 0 if self.continuous else e.NUM_ACTIONS
         r.states, r.obs = _ptr(self.states), _ptr(self.obs)
         r.actor_params, r.critic_params = _ptr(self.actor_params), _ptr(self.critic_params)
         r.actor, r.critic = self.actor.desc, self.critic.desc
@@ -119,79 +153,151 @@ class RolloutBuffers:
 
 
 def rollout_step(ctx, desc, t, sample_seed, step_seed=0, reset_seed=0):
-    """One pass of train_gpu's inner loop body (ppo.mojo:2069-2285), enqueue only."""
+    """One pass of train_gpu's inner loop body (ppo.mojo:2069-2285, ppo_continuous.mojo:2619-2850),
+    enqueue only."""
     _lib.call("mrl_rollout_step", ctx.handle, C.byref(desc), t, int(sample_seed) & 0xFFFFFFFF,
               int(step_seed) & (2**64 - 1), int(reset_seed) & (2**64 - 1))
 
 
-class DiscreteUpdate:
-    """Phases 2 and 3 of DeepPPOAgent.train_gpu (deep_agents/ppo/ppo.mojo:2296-2727) on device
-    buffers: bootstrap value, GAE, advantage normalisation, then epochs of shuffled minibatches,
-    each running actor forward / loss gradient / backward / clip / Adam and the same for the
-    critic.  Nothing is copied to the host inside an epoch; the mean KL of the last minibatch is
-    read once per epoch for the early-stop test."""
+class PPOUpdate:
+    """Phases 2 and 3 of train_gpu (deep_agents/ppo/ppo.mojo:2296-2727 for the discrete agent,
+    ppo_continuous.mojo:2852-3260 for the continuous one) on device buffers: bootstrap value,
+    optional reward normalisation, GAE, advantage normalisation, then epochs of shuffled
+    minibatches, each running actor forward / loss gradient / backward / clip / Adam
+    (/ log_std clamp) and the same for the critic.  Nothing is copied to the host inside an
+    epoch: the KL early-stop test runs on the device after every minibatch and its flag is read
+    once per epoch (kl_sync_every_minibatch=True reads it after every minibatch and stops before
+    that minibatch's update, as the reference does)."""
 
     def __init__(self, ctx, rb, minibatch, actor_opt, critic_opt, gamma=0.99, gae_lambda=0.95,
                  clip_epsilon=0.2, entropy_coef=0.01, value_loss_coef=0.5, max_grad_norm=0.5,
                  clip_value=True, normalize_advantages=True, norm_adv_per_minibatch=True,
-                 target_kl=0.015):
+                 target_kl=0.015, normalize_rewards=False, kl_sync_every_minibatch=False):
         self.ctx, self.rb, self.mb = ctx, rb, minibatch
         self.actor_opt, self.critic_opt = actor_opt, critic_opt
         self.gamma, self.gae_lambda = gamma, gae_lambda
         self.clip_epsilon, self.entropy_coef, self.value_loss_coef = clip_epsilon, entropy_coef, value_loss_coef
         self.max_grad_norm, self.clip_value = max_grad_norm, clip_value
         self.normalize_advantages, self.norm_adv_per_minibatch = normalize_advantages, norm_adv_per_minibatch
-        self.target_kl = target_kl
+        self.target_kl, self.kl_sync_every_minibatch = target_kl, kl_sync_every_minibatch
+        self.continuous = rb.continuous
+        self.reward_rms = RunningMeanStd(ctx) if normalize_rewards else None
         dev = ctx.device
         z = lambda n: torch.zeros(n, device=dev)
         total = rb.n_envs * rb.rollout_len
-        obs_dim, na = rb.env.OBS_DIM, rb.env.NUM_ACTIONS
+        obs_dim, aw = rb.env.OBS_DIM, rb.act_width
+        head = rb.actor.OUT_DIM
         self.total = total
         self.advantages, self.returns, self.bootstrap = z(total), z(total), z(rb.n_envs)
-        self.mb_obs, self.mb_actions = z(minibatch * obs_dim), z(minibatch)
+        self.mb_obs, self.mb_actions = z(minibatch * obs_dim), z(minibatch * aw)
         self.mb_adv, self.mb_ret, self.mb_logp, self.mb_val = z(minibatch), z(minibatch), z(minibatch), z(minibatch)
-        self.logits, self.values = z(minibatch * na), z(minibatch)
-        self.g_logits, self.g_values, self.kl = z(minibatch * na), z(minibatch), z(minibatch)
+        self.actor_out, self.values = z(minibatch * head), z(minibatch)
+        self.g_actor_out, self.g_values, self.kl = z(minibatch * head), z(minibatch), z(minibatch)
+        self.kl_flag = torch.zeros(2, dtype=torch.int32, device=dev)
         self.actor_cache = z(minibatch * rb.actor.CACHE_SIZE)
         self.critic_cache = z(minibatch * rb.critic.CACHE_SIZE)
         self.actor_grads, self.critic_grads = z(rb.actor.PARAM_SIZE), z(rb.critic.PARAM_SIZE)
         self.actor_state, self.critic_state = z(2 * rb.actor.PARAM_SIZE), z(2 * rb.critic.PARAM_SIZE)
+        self.indices = torch.zeros(total, dtype=torch.int32, device=dev)
+        if self.continuous:
+            a = rb.env.ACTION_DIM
+            self.log_std_offset = rb.actor.PARAM_SIZE - a
+
+    # compatibility names used by callers written against the discrete agent
+    @property
+    def logits(self):
+        return self.actor_out
+
+    @property
+    def g_logits(self):
+        return self.g_actor_out
 
     def compute_advantages(self):
         rb, ctx = self.rb, self.ctx
         rb.critic.forward_gpu_no_cache_ws(ctx, self.bootstrap, rb.obs, rb.critic_params)
+        if self.reward_rms is not None:
+            self.reward_rms.update(rb.r_rewards)
+            self.reward_rms.normalize(rb.r_rewards)
         compute_gae(ctx, rb.r_rewards, rb.r_values, rb.r_dones, self.bootstrap, self.gamma,
                     self.gae_lambda, self.advantages, self.returns)
         if self.normalize_advantages:
             normalize_advantages(ctx, self.advantages)
 
-    def minibatch_step(self, indices):
+    def actor_half(self, indices):
+        """gather -> (normalise) -> actor forward -> loss gradient + KL -> device KL test."""
         rb, ctx = self.rb, self.ctx
         gather_minibatch(ctx, indices,
                          (rb.r_obs, rb.r_actions, self.advantages, self.returns, rb.r_log_probs, rb.r_values),
                          (self.mb_obs, self.mb_actions, self.mb_adv, self.mb_ret, self.mb_logp, self.mb_val),
-                         rb.env.OBS_DIM, 1)
+                         rb.env.OBS_DIM, rb.act_width)
         if self.norm_adv_per_minibatch:
             normalize_advantages(ctx, self.mb_adv)
-        rb.actor.forward_gpu_ws(ctx, self.logits, self.mb_obs, rb.actor_params, self.actor_cache)
-        ppo_actor_grad_with_kl(ctx, self.g_logits, self.kl, self.logits, self.mb_logp, self.mb_adv,
-                               self.mb_actions, self.clip_epsilon, self.entropy_coef)
-        rb.actor.backward_gpu_ws(ctx, None, self.g_logits, rb.actor_params, self.actor_cache, self.actor_grads)
+        rb.actor.forward_gpu_ws(ctx, self.actor_out, self.mb_obs, rb.actor_params, self.actor_cache)
+        grad = ppo_continuous_actor_grad if self.continuous else ppo_actor_grad_with_kl
+        grad(ctx, self.g_actor_out, self.kl, self.actor_out, self.mb_logp, self.mb_adv, self.mb_actions,
+             self.clip_epsilon, self.entropy_coef)
+        if self.target_kl > 0.0:
+            kl_check(ctx, self.kl, self.target_kl, self.kl_flag)
+
+    def update_half(self):
+        rb, ctx = self.rb, self.ctx
+        rb.actor.backward_gpu_ws(ctx, None, self.g_actor_out, rb.actor_params, self.actor_cache, self.actor_grads)
         if self.max_grad_norm > 0.0:
             clip_grad_norm(ctx, self.actor_grads, self.max_grad_norm)
         self.actor_opt.step_gpu(ctx, rb.actor_params, self.actor_grads, self.actor_state)
+        if self.continuous:
+            clamp_log_std_params(ctx, rb.actor_params, self.log_std_offset, rb.env.ACTION_DIM)
         rb.critic.forward_gpu_ws(ctx, self.values, self.mb_obs, rb.critic_params, self.critic_cache)
         ppo_critic_grad(ctx, self.g_values, self.values, self.mb_ret, self.value_loss_coef,
-                        self.mb_val if self.clip_value else None, self.clip_epsilon)
+                        self.mb_val if self.clip_value else None, self.clip_epsilon,
+                        continuous=self.continuous)
         rb.critic.backward_gpu_ws(ctx, None, self.g_values, rb.critic_params, self.critic_cache, self.critic_grads)
         if self.max_grad_norm > 0.0:
             clip_grad_norm(ctx, self.critic_grads, self.max_grad_norm)
         self.critic_opt.step_gpu(ctx, rb.critic_params, self.critic_grads, self.critic_state)
 
-    def run_epoch(self, permutation):
-        """permutation: int32 device tensor over the T*N samples; only whole minibatches are used
-        (ppo.mojo:2438).  Returns the mean KL of the epoch's last minibatch."""
+    def minibatch_step(self, indices):
+        self.actor_half(indices)
+        self.update_half()
+
+    def kl_stopped(self):
+        """Reads the device flag (one synchronising copy of 8 bytes): (stopped, last mean KL)."""
+        f = self.kl_flag.cpu()
+        return bool(f[0].item()), float(f[1:2].view(torch.float32).item())
+
+    def run_epoch(self, permutation_or_seed):
+        """permutation_or_seed: an int32 device tensor over the T*N samples, or an int seed from
+        which the permutation is drawn on the device.  Only whole minibatches are used
+        (ppo.mojo:2438).  Returns (stopped, mean KL of the last minibatch tested)."""
+        if isinstance(permutation_or_seed, int):
+            permutation(self.ctx, self.indices, permutation_or_seed)
+            perm = self.indices
+        else:
+            perm = permutation_or_seed
         n_mb = self.total // self.mb
         for k in range(n_mb):
-            self.minibatch_step(permutation[k * self.mb:(k + 1) * self.mb])
-        return float(self.kl.mean().item()) if self.target_kl > 0.0 else 0.0
+            self.actor_half(perm[k * self.mb:(k + 1) * self.mb])
+            if self.target_kl > 0.0 and self.kl_sync_every_minibatch and self.kl_stopped()[0]:
+                break
+            self.update_half()
+        return self.kl_stopped() if self.target_kl > 0.0 else (False, 0.0)
+
+    def update(self, num_epochs, seed=0):
+        """compute_advantages + up to num_epochs epochs; stops after the epoch in which the KL
+        flag was raised.  Returns the number of epochs run."""
+        self.kl_flag.zero_()
+        self.compute_advantages()
+        for epoch in range(num_epochs):
+            stopped, _ = self.run_epoch(int(seed) * 1000003 + epoch)
+            if stopped:
+                return epoch + 1
+        return num_epochs
+
+
+class DiscreteUpdate(PPOUpdate):
+    """PPOUpdate for DeepPPOAgent (discrete actions, critic gradient 2*c_v*(V-R)/MB)."""
+
+
+class ContinuousUpdate(PPOUpdate):
+    """PPOUpdate for DeepPPOContinuousAgent (Gaussian actor with a StochasticActor head, critic
+    gradient (V-R)/MB, log_std clamp after every actor step, optional reward normalisation)."""

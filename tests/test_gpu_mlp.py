@@ -3,6 +3,8 @@ of the reference layers) and a torch fp32 reference.  Bar: outputs and gradients
 relative (floor 1e-5 absolute, scaled by the magnitude of the tensor)."""
 import sys
 
+import zlib
+
 import numpy as np
 import pytest
 import torch
@@ -45,7 +47,7 @@ CASES = [
 @pytest.mark.parametrize("name,spec,batch", CASES, ids=[c[0] for c in CASES])
 def test_forward_backward_parity(mrl, orc, orcmod, ctx, name, spec, batch):
     say("mlp case", name, batch)
-    rng = np.random.default_rng(abs(hash(name)) % 2**31)
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
     model = mk(mrl, spec)
     ls = orcmod.layers(spec)
     P, CS, OD = model.PARAM_SIZE, model.CACHE_SIZE, model.OUT_DIM
@@ -57,8 +59,6 @@ def test_forward_backward_parity(mrl, orc, orcmod, ctx, name, spec, batch):
 
     out_h = np.zeros((batch, OD), np.float32); cache_h = np.zeros(batch * CS, np.float32)
     orc.orc_mlp_forward(ls, len(spec), batch, x, params, out_h, cache_h.ctypes.data)
-    grads_h = np.zeros(P, np.float32); gin_h = np.zeros_like(x)
-    orc.orc_mlp_backward(ls, len(spec), batch, go, params, cache_h, grads_h, gin_h.ctypes.data)
 
     d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
     p_d, x_d, go_d = d(params), d(x.reshape(-1)), d(go.reshape(-1))
@@ -72,6 +72,11 @@ def test_forward_backward_parity(mrl, orc, orcmod, ctx, name, spec, batch):
     close(out_d.cpu().numpy().reshape(batch, OD), out_h, "forward")
     assert torch.equal(out_d, out_nc)
     close(cache_d.cpu().numpy(), cache_h, "cache")
+    # The oracle's backward runs on the cache the kernels wrote (just shown to agree with the
+    # oracle's own): a ReLU pre-activation within an ulp of zero may round to either side in the
+    # two forwards, and the gate it selects is a step function -- not a tolerance question.
+    grads_h = np.zeros(P, np.float32); gin_h = np.zeros_like(x)
+    orc.orc_mlp_backward(ls, len(spec), batch, go, params, cache_d.cpu().numpy(), grads_h, gin_h.ctypes.data)
     close(grads_d.cpu().numpy(), grads_h, "param grads")
     close(gin_d.cpu().numpy().reshape(x.shape), gin_h, "input grads")
     # backward without grad_input (what the PPO update asks for on the first layer)

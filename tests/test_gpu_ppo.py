@@ -278,3 +278,291 @@ def test_fused_policy_kernel_against_layerwise_path_and_oracle(mrl, orc, orcmod,
     same = r_actions == a_h
     assert same.mean() > 0.995, same.mean()
     np.testing.assert_allclose(r_logp[same], lp_h[same], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("hidden,kind,obs_dim,A,n", [(256, "tanh", 17, 6, 4096), (256, "relu", 24, 4, 333),
+                                                      (64, "tanh", 3, 1, 16384), (64, "relu", 5, 8, 31)])
+def test_fused_gaussian_policy_kernel_against_oracle(mrl, orc, orcmod, ctx, hidden, kind, obs_dim, A, n):
+    """Fused actor(StochasticActor head) + critic + Gaussian sampling + stores against the oracle's
+    forward and sampler.  The noise comes from the same Philox streams, so action = mean + std * z
+    differs from the oracle's only through the mean: MLP tolerance."""
+    say("fused gaussian policy", hidden, kind, n)
+    Lay = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
+    k = 1 if kind == "relu" else 2
+    actor = mrl.seq(Lay(obs_dim, hidden), Lay(hidden, hidden), mrl.StochasticActor(hidden, A))
+    critic = mrl.seq(Lay(obs_dim, hidden), Lay(hidden, hidden), mrl.Linear(hidden, 1))
+    rng = np.random.default_rng(hidden + n)
+    ap = rng.uniform(-0.15, 0.15, actor.PARAM_SIZE).astype(np.float32)
+    ap[-A:] = rng.uniform(-6.0, 2.5, A)          # log_std, partly outside the clamp range
+    cp = rng.uniform(-0.15, 0.15, critic.PARAM_SIZE).astype(np.float32)
+    obs = rng.normal(size=(n, obs_dim)).astype(np.float32)
+    la = orcmod.layers([(k, obs_dim, hidden), (k, hidden, hidden), (3, hidden, A)])
+    lc = orcmod.layers([(k, obs_dim, hidden), (k, hidden, hidden), (0, hidden, 1)])
+    out_h, values_h = np.zeros((n, 2 * A), np.float32), np.zeros((n, 1), np.float32)
+    orc.orc_mlp_forward(la, 3, n, obs, ap, out_h, None)
+    orc.orc_mlp_forward(lc, 3, n, obs, cp, values_h, None)
+    a_h, lp_h = np.zeros((n, A), np.float32), np.zeros(n, np.float32)
+    orc.orc_sample_gaussian(out_h, n, A, 4242, a_h, lp_h)
+    out = [torch.zeros(m, device="cuda") for m in (n * A, n * obs_dim, n * A, n, n)]
+    obs_d, ap_d, cp_d = d(obs.reshape(-1)), d(ap), d(cp)
+    mrl._lib.call("mrl_policy_step_gaussian", ctx.handle, ctypes.byref(actor.desc), ctypes.byref(critic.desc), n,
+                  obs_d.data_ptr(), ap_d.data_ptr(), cp_d.data_ptr(), 4242, *[o.data_ptr() for o in out])
+    ctx.synchronize()
+    actions, r_obs, r_actions, r_logp, r_values = (h(o) for o in out)
+    np.testing.assert_array_equal(r_obs.reshape(n, obs_dim), obs)
+    np.testing.assert_array_equal(actions, r_actions)
+    np.testing.assert_allclose(r_values, values_h[:, 0], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(actions.reshape(n, A), a_h, rtol=1e-4, atol=2e-5)
+    # log-prob: ((a - mean) / std)^2 amplifies the mean's rounding by 1/std (std down to e^-5)
+    np.testing.assert_allclose(r_logp, lp_h, rtol=1e-3, atol=2e-2)
+    wide = ap[-A:].min() > -2.0
+    if wide:
+        np.testing.assert_allclose(r_logp, lp_h, rtol=1e-4, atol=1e-3)
+
+
+def test_gaussian_policy_step_layerwise_path(mrl, orc, orcmod, ctx):
+    """A shape the fused kernel does not cover (hidden 128) takes the layer-by-layer path."""
+    n, obs_dim, hidden, A = 500, 11, 128, 3
+    actor = mrl.seq(mrl.LinearTanh(obs_dim, hidden), mrl.LinearTanh(hidden, hidden), mrl.StochasticActor(hidden, A))
+    critic = mrl.seq(mrl.LinearTanh(obs_dim, hidden), mrl.LinearTanh(hidden, hidden), mrl.Linear(hidden, 1))
+    rng = np.random.default_rng(5)
+    ap = rng.uniform(-0.15, 0.15, actor.PARAM_SIZE).astype(np.float32)
+    cp = rng.uniform(-0.15, 0.15, critic.PARAM_SIZE).astype(np.float32)
+    obs = rng.normal(size=(n, obs_dim)).astype(np.float32)
+    la = orcmod.layers([(2, obs_dim, hidden), (2, hidden, hidden), (3, hidden, A)])
+    lc = orcmod.layers([(2, obs_dim, hidden), (2, hidden, hidden), (0, hidden, 1)])
+    out_h, values_h = np.zeros((n, 2 * A), np.float32), np.zeros((n, 1), np.float32)
+    orc.orc_mlp_forward(la, 3, n, obs, ap, out_h, None)
+    orc.orc_mlp_forward(lc, 3, n, obs, cp, values_h, None)
+    a_h, lp_h = np.zeros((n, A), np.float32), np.zeros(n, np.float32)
+    orc.orc_sample_gaussian(out_h, n, A, 9, a_h, lp_h)
+    out = [torch.zeros(m, device="cuda") for m in (n * A, n * obs_dim, n * A, n, n)]
+    obs_d, ap_d, cp_d = d(obs.reshape(-1)), d(ap), d(cp)
+    mrl._lib.call("mrl_policy_step_gaussian", ctx.handle, ctypes.byref(actor.desc), ctypes.byref(critic.desc), n,
+                  obs_d.data_ptr(), ap_d.data_ptr(), cp_d.data_ptr(), 9, *[o.data_ptr() for o in out])
+    ctx.synchronize()
+    actions, r_obs, r_actions, r_logp, r_values = (h(o) for o in out)
+    np.testing.assert_array_equal(r_obs.reshape(n, obs_dim), obs)
+    np.testing.assert_allclose(actions.reshape(n, A), a_h, rtol=1e-4, atol=2e-5)
+    np.testing.assert_allclose(r_values, values_h[:, 0], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(r_logp, lp_h, rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("env_name,N", [("PendulumV2", 1000), ("HalfCheetahPlanarV2", 300)])
+def test_continuous_rollout_step_equals_its_parts(mrl, ctx, env_name, N):
+    """mrl_rollout_step for a continuous agent against forward + sample + step + selective reset."""
+    torch.manual_seed(1)
+    T = 4
+    E = getattr(mrl, env_name)
+    od, A, S = E.OBS_DIM, E.ACTION_DIM, E.STATE_SIZE
+    actor = mrl.seq(mrl.LinearTanh(od, 64), mrl.LinearTanh(64, 64), mrl.StochasticActor(64, A))
+    critic = mrl.seq(mrl.LinearTanh(od, 64), mrl.LinearTanh(64, 64), mrl.Linear(64, 1))
+    ap = (torch.rand(actor.PARAM_SIZE, device="cuda") - 0.5) * 0.3
+    cp = (torch.rand(critic.PARAM_SIZE, device="cuda") - 0.5) * 0.3
+    rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N, T)
+    assert rb.continuous and rb.act_width == A
+    rb.actor_params, rb.critic_params = ap, cp
+    E.reset_kernel_gpu(ctx, rb.states, 3)
+    rb.obs.copy_(rb.states.view(N, S)[:, :od].reshape(-1))
+    s2, o2 = rb.states.clone(), rb.obs.clone()
+    desc = rb.descriptor()
+    z = lambda n: torch.zeros(n, device="cuda")
+    head, values, acts, lps, rew, dn = z(N * 2 * A), z(N), z(N * A), z(N), z(N), z(N)
+    for t in range(T):
+        mrl.ppo.rollout_step(ctx, desc, t, 100 + t, 0, 500 + t)
+        actor.forward_gpu_no_cache_ws(ctx, head, o2, ap)
+        critic.forward_gpu_no_cache_ws(ctx, values, o2, cp)
+        mrl.ppo.sample_continuous_actions(ctx, head, acts, lps, 100 + t)
+        ctx.synchronize()
+        sl = slice(t * N, (t + 1) * N)
+        assert torch.equal(rb.r_obs[t * N * od:(t + 1) * N * od], o2)
+        torch.testing.assert_close(rb.r_actions[t * N * A:(t + 1) * N * A], acts, rtol=1e-4, atol=2e-5)
+        torch.testing.assert_close(rb.r_log_probs[sl], lps, rtol=1e-4, atol=1e-3)
+        torch.testing.assert_close(rb.r_values[sl], values, rtol=1e-4, atol=1e-5)
+        acts.copy_(rb.r_actions[t * N * A:(t + 1) * N * A])
+        E.step_kernel_gpu(ctx, s2, acts, rew, dn, o2, 0)
+        ctx.synchronize()
+        assert torch.equal(rb.r_rewards[sl], rew) and torch.equal(rb.r_dones[sl], dn)
+        E.selective_reset_kernel_gpu(ctx, s2, dn, 500 + t)
+        o2.copy_(s2.view(N, S)[:, :od].reshape(-1))
+        ctx.synchronize()
+        assert torch.equal(rb.states, s2) and torch.equal(rb.obs, o2)
+
+
+def test_running_mean_std(mrl, orc, orcmod, ctx):
+    rng = np.random.default_rng(3)
+    rms_h = orcmod.Rms(0.0, 0.0, 0.0)
+    rms = mrl.ppo.RunningMeanStd(ctx)
+    for n, scale, shift in ((1, 1.0, 0.0), (4096 * 50, 3.0, -2.0), (1000, 0.1, 7.0)):
+        x = (rng.normal(size=n) * scale + shift).astype(np.float32)
+        xd = d(x)
+        orc.orc_rms_update(ctypes.byref(rms_h), x, n)
+        rms.update(xd)
+        st = h(rms.state)
+        np.testing.assert_allclose(st, [rms_h.count, rms_h.mean, rms_h.var_sum], rtol=1e-12, atol=1e-12)
+        y = x.copy()
+        orc.orc_rms_normalize(ctypes.byref(rms_h), y, n)
+        rms.normalize(xd)
+        np.testing.assert_allclose(h(xd), y, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("n", [1, 2, 5, 1000, 4096, 65537, 4096 * 1000])
+def test_permutation_is_a_permutation(mrl, ctx, n):
+    idx = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    mrl.ppo.permutation(ctx, idx, 12345)
+    first = idx.clone()
+    assert torch.equal(torch.sort(idx.long()).values, torch.arange(n, device="cuda"))
+    mrl.ppo.permutation(ctx, idx, 12345)
+    assert torch.equal(idx, first)                      # deterministic in the seed
+    if n >= 1000:
+        mrl.ppo.permutation(ctx, idx, 12346)
+        assert (idx == first).float().mean() < 0.01     # another seed, another permutation
+        # no structure left from the identity: displacement |p(i) - i| of a random permutation
+        # has mean n/3, and each tenth of the range receives a tenth of the first tenth
+        # (tolerances: 4.5 standard deviations of the statistic under a uniform permutation)
+        disp = (first.double() - torch.arange(n, device="cuda").double()).abs().mean().item()
+        assert abs(disp / n - 1 / 3) < 4.5 * 0.236 / n ** 0.5 + 1e-3
+        head = first[: n // 10].long() * 10 // n
+        counts = torch.bincount(head, minlength=10).double()
+        assert (counts / counts.sum() - 0.1).abs().max() < 4.5 * (0.09 / (n // 10)) ** 0.5
+
+
+def test_kl_check_flag(mrl, ctx):
+    kl = torch.full((4096,), 0.01, device="cuda")
+    flag = torch.zeros(2, dtype=torch.int32, device="cuda")
+    mrl.ppo.kl_check(ctx, kl, 0.015, flag)
+    assert flag[0].item() == 0
+    assert abs(flag[1:2].view(torch.float32).item() - 0.01) < 1e-7
+    kl[:2048] = 0.03
+    mrl.ppo.kl_check(ctx, kl, 0.015, flag)
+    assert flag[0].item() == 1
+    kl.fill_(0.0)
+    mrl.ppo.kl_check(ctx, kl, 0.015, flag)
+    assert flag[0].item() == 1 and flag[1:2].view(torch.float32).item() == 0.0   # sticky
+
+
+def test_init_uniform_and_network(mrl, orc, ctx):
+    n = 1003
+    p = torch.zeros(n, device="cuda")
+    mrl._lib.call("mrl_init_uniform", ctx.handle, p.data_ptr(), n, -0.5, 1.5, 99)
+    got = h(p)
+    want = np.zeros(n + 1, np.float32)
+    u = np.zeros(4, np.float32)
+    for q in range((n + 3) // 4):
+        orc.orc_philox_uniform4(99, q, 0, u)
+        want[4 * q:4 * q + 4] = np.float32(-0.5) + u * np.float32(2.0)
+    np.testing.assert_array_equal(got, want[:n])
+    model = mrl.seq(mrl.LinearReLU(8, 256), mrl.LinearReLU(256, 256), mrl.Linear(256, 4))
+    net = mrl.Network(ctx, model, mrl.Adam(lr=3e-4), mrl.Xavier(seed=1))
+    w = h(net.params)
+    b = (2.0 / (8 + 4)) ** 0.5
+    assert w.shape == (69124,) and np.abs(w).max() <= b and np.abs(w).max() > 0.99 * b
+    assert abs(w.mean()) < 0.01 * b * 3 and abs(w.std() - b / 3 ** 0.5) < 0.01 * b
+    assert net.grads.abs().sum().item() == 0 and net.optimizer_state.numel() == 2 * 69124
+    amodel = mrl.seq(mrl.LinearTanh(17, 256), mrl.LinearTanh(256, 256), mrl.StochasticActor(256, 6))
+    anet = mrl.Network(ctx, amodel, mrl.Adam(lr=3e-4), mrl.Kaiming(seed=2))
+    off = 17 * 256 + 256 + 256 * 256 + 256
+    mrl.init_params_small(ctx, anet.params, off, 256, 6, seed=3)
+    a = h(anet.params)
+    assert np.abs(a[:off]).max() <= (2.0 / 17) ** 0.5
+    assert np.abs(a[off:off + 256 * 6]).max() <= 0.01 and np.all(a[off + 1536:off + 1542] == 0.0)
+    assert np.all(a[-6:] == np.float32(-0.5))
+
+
+def test_continuous_update_minibatch_against_oracle(mrl, orc, orcmod, ctx):
+    """One ContinuousUpdate minibatch (gather, per-minibatch normalisation, actor forward, Gaussian
+    loss gradient, backward, clip, Adam, log_std clamp, critic forward, gradient, backward, clip,
+    Adam) against the same sequence on the oracle."""
+    rng = np.random.default_rng(11)
+    N, T, MB = 64, 8, 256
+    E = mrl.HalfCheetahPlanarV2
+    od, A = E.OBS_DIM, E.ACTION_DIM
+    H = 64
+    actor = mrl.seq(mrl.LinearTanh(od, H), mrl.LinearTanh(H, H), mrl.StochasticActor(H, A))
+    critic = mrl.seq(mrl.LinearTanh(od, H), mrl.LinearTanh(H, H), mrl.Linear(H, 1))
+    la = orcmod.layers([(2, od, H), (2, H, H), (3, H, A)])
+    lc = orcmod.layers([(2, od, H), (2, H, H), (0, H, 1)])
+    ap = rng.uniform(-0.2, 0.2, actor.PARAM_SIZE).astype(np.float32)
+    ap[-A:] = -0.5
+    cp = rng.uniform(-0.2, 0.2, critic.PARAM_SIZE).astype(np.float32)
+    rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N, T)
+    rb.actor_params, rb.critic_params = d(ap), d(cp)
+    total = N * T
+    r_obs = rng.normal(size=(total, od)).astype(np.float32)
+    # behaviour policy = current policy: old log-probs from the oracle's own sampler
+    out0 = np.zeros((total, 2 * A), np.float32)
+    orc.orc_mlp_forward(la, 3, total, r_obs, ap, out0, None)
+    r_act, r_lp = np.zeros((total, A), np.float32), np.zeros(total, np.float32)
+    orc.orc_sample_gaussian(out0, total, A, 5, r_act, r_lp)
+    r_lp += rng.normal(size=total).astype(np.float32) * 0.05     # ratio != 1
+    r_val = rng.normal(size=total).astype(np.float32)
+    adv = rng.normal(size=total).astype(np.float32)
+    ret = (r_val + adv).astype(np.float32)
+    rb.r_obs.copy_(d(r_obs.reshape(-1))); rb.r_actions.copy_(d(r_act.reshape(-1)))
+    rb.r_log_probs.copy_(d(r_lp)); rb.r_values.copy_(d(r_val))
+    aopt, copt = mrl.Adam(lr=3e-4), mrl.Adam(lr=1e-3)
+    upd = mrl.ppo.ContinuousUpdate(ctx, rb, MB, aopt, copt, target_kl=0.0)
+    upd.advantages.copy_(d(adv)); upd.returns.copy_(d(ret))
+    idx = rng.permutation(total)[:MB].astype(np.int32)
+    upd.minibatch_step(d(idx))
+    ctx.synchronize()
+    # oracle
+    mo, ma, madv = r_obs[idx], r_act[idx], adv[idx].copy()
+    orc.orc_normalize_minibatch_host(madv, MB)
+    cache = np.zeros(MB * actor.CACHE_SIZE, np.float32)
+    out = np.zeros((MB, 2 * A), np.float32)
+    orc.orc_mlp_forward(la, 3, MB, mo, ap, out, cache.ctypes.data)
+    g_out, kl = np.zeros((MB, 2 * A), np.float32), np.zeros(MB, np.float32)
+    orc.orc_ppo_actor_grad_gaussian(out, r_lp[idx], madv, ma, MB, A, 0.2, 0.01, g_out, kl)
+    ga = np.zeros(actor.PARAM_SIZE, np.float32)
+    orc.orc_mlp_backward(la, 3, MB, g_out, ap, cache, ga, None)
+    orc.orc_clip_grad_norm(ga, ga.size, 0.5)
+    st = np.zeros(2 * ga.size, np.float32)
+    ap2 = ap.copy()
+    orc.orc_adam_step(ap2, ga, st, ga.size, 1, 3e-4, 0.9, 0.999, 1e-8)
+    orc.orc_clamp_log_std(ap2, ap2.size - A, A)
+    np.testing.assert_allclose(h(upd.kl), kl, rtol=1e-3, atol=1e-5)
+    np.testing.assert_allclose(h(upd.actor_grads), ga, rtol=1e-3, atol=1e-6)
+    np.testing.assert_allclose(h(rb.actor_params), ap2, rtol=1e-5, atol=2e-6)
+    ccache = np.zeros(MB * critic.CACHE_SIZE, np.float32)
+    v = np.zeros((MB, 1), np.float32)
+    orc.orc_mlp_forward(lc, 3, MB, mo, cp, v, ccache.ctypes.data)
+    gv = np.zeros(MB, np.float32)
+    orc.orc_ppo_critic_grad(v.reshape(-1), r_val[idx], ret[idx], MB, 1, 1, 0.5, 0.2, gv)
+    gc = np.zeros(critic.PARAM_SIZE, np.float32)
+    orc.orc_mlp_backward(lc, 3, MB, gv.reshape(MB, 1), cp, ccache, gc, None)
+    orc.orc_clip_grad_norm(gc, gc.size, 0.5)
+    st = np.zeros(2 * gc.size, np.float32)
+    cp2 = cp.copy()
+    orc.orc_adam_step(cp2, gc, st, gc.size, 1, 1e-3, 0.9, 0.999, 1e-8)
+    np.testing.assert_allclose(h(upd.critic_grads), gc, rtol=1e-3, atol=1e-6)
+    np.testing.assert_allclose(h(rb.critic_params), cp2, rtol=1e-5, atol=2e-6)
+
+
+def test_update_driver_runs_epochs_and_stops_on_kl(mrl, ctx):
+    """PPOUpdate.update end to end on a small LunarLander rollout: permutation drawn on the device,
+    the KL flag raised on the device stops the epochs, parameters stay finite."""
+    N, T, MB = 256, 16, 512
+    E = mrl.LunarLanderV2
+    actor = mrl.seq(mrl.LinearReLU(8, 64), mrl.LinearReLU(64, 64), mrl.Linear(64, 4))
+    critic = mrl.seq(mrl.LinearReLU(8, 64), mrl.LinearReLU(64, 64), mrl.Linear(64, 1))
+    anet = mrl.Network(ctx, actor, mrl.Adam(lr=3e-4), mrl.Xavier(seed=1))
+    cnet = mrl.Network(ctx, critic, mrl.Adam(lr=1e-3), mrl.Xavier(seed=2))
+    rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N, T)
+    rb.actor_params, rb.critic_params = anet.params, cnet.params
+    E.reset_kernel_gpu(ctx, rb.states, 5)
+    rb.obs.copy_(rb.states.view(N, 192)[:, :8].reshape(-1))
+    desc = rb.descriptor()
+    for t in range(T):
+        mrl.ppo.rollout_step(ctx, desc, t, 10 + t, 0, 900 + t)
+    upd = mrl.ppo.DiscreteUpdate(ctx, rb, MB, anet.optimizer, cnet.optimizer, target_kl=0.0)
+    before = anet.params.clone()
+    assert upd.update(2, seed=4) == 2
+    assert anet.optimizer.t == 2 * (N * T // MB)
+    assert torch.isfinite(anet.params).all() and not torch.equal(before, anet.params)
+    # a huge learning rate moves the policy far in one epoch: the device flag must stop the update
+    anet.optimizer.lr = 0.5
+    upd2 = mrl.ppo.DiscreteUpdate(ctx, rb, MB, anet.optimizer, cnet.optimizer, target_kl=1e-4)
+    ran = upd2.update(10, seed=5)
+    stopped, mean_kl = upd2.kl_stopped()
+    assert stopped and ran < 10
