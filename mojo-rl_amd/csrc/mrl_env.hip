@@ -13,6 +13,26 @@
 
 namespace mrl {
 
+// _store_post_step_kernel (deep_agents/ppo/ppo.mojo:692-708) + accumulate_rewards /
+// increment_steps / extract_completed_episodes (deep_rl/gpu/rl_kernels.mojo:103-200) for one env
+MRL_DEV void account(const Accounting &acc, int i, float r, float d) {
+    if (acc.r_rewards == nullptr) return;
+    acc.r_rewards[i] = r;
+    acc.r_dones[i] = d;
+    float er = acc.ep_return[i] + r;
+    float el = acc.ep_length[i] + 1.0f;
+    if (d > 0.5f) {
+        int slot = atomicAdd(acc.done_count, 1);
+        if (slot < acc.done_cap) {
+            acc.done_returns[slot] = er;
+            acc.done_lengths[slot] = el;
+        }
+        er = 0.0f;
+        el = 0.0f;
+    }
+    acc.ep_return[i] = er;
+    acc.ep_length[i] = el;
+}
 
 // ---------------------------------------------------------------- CartPole / Pendulum
 
@@ -21,7 +41,8 @@ namespace mrl {
 __global__ __launch_bounds__(256) void cartpole_step_kernel(float *states, int32_t *steps,
                                                             const float *actions, float *rewards,
                                                             float *dones, float *obs, int batch,
-                                                            int autoreset, uint32_t reset_seed) {
+                                                            int autoreset, uint32_t reset_seed,
+                                                            Accounting acc) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= batch) return;
     float4 v = reinterpret_cast<const float4 *>(states)[i];
@@ -36,6 +57,7 @@ __global__ __launch_bounds__(256) void cartpole_step_kernel(float *states, int32
     steps[i] = st;
     rewards[i] = r;
     dones[i] = d;
+    account(acc, i, r, d);
 }
 
 // mode 0: reset every env; mode 1: reset envs with dones > 0.5 and clear the flag
@@ -58,7 +80,7 @@ __global__ __launch_bounds__(256) void cartpole_reset_kernel(float *states, int3
 __global__ __launch_bounds__(256) void pendulum_step_kernel(float *states, const float *actions,
                                                             float *rewards, float *dones,
                                                             float *obs, int batch, int autoreset,
-                                                            uint64_t reset_seed) {
+                                                            uint64_t reset_seed, Accounting acc) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= batch) return;
     float4 *row = reinterpret_cast<float4 *>(states) + 2 * (size_t)i;
@@ -74,6 +96,7 @@ __global__ __launch_bounds__(256) void pendulum_step_kernel(float *states, const
     obs[3 * (size_t)i + 2] = s[2];
     rewards[i] = r;
     dones[i] = d;
+    account(acc, i, r, d);
 }
 
 __global__ __launch_bounds__(256) void pendulum_reset_kernel(float *states, float *dones, int batch,
@@ -204,7 +227,7 @@ template <class E, bool AUTORESET>
 __global__ __launch_bounds__(BLOCK) void phys_step_kernel(float *states, const float *actions,
                                                           float *rewards, float *dones, float *obs,
                                                           const float *shapes_g, int batch,
-                                                          uint64_t reset_seed) {
+                                                          uint64_t reset_seed, Accounting acc) {
     using S = Stage<E>;
     __shared__ float rows[E::EPB * S::STRIDE];
     __shared__ float cts[E::EPB * S::CSTRIDE];
@@ -229,6 +252,7 @@ __global__ __launch_bounds__(BLOCK) void phys_step_kernel(float *states, const f
                     actions + (size_t)env * E::ACT_W, r, d);
             rewards[env] = r;
             dones[env] = d;
+            account(acc, env, r, d);
             finished = d > 0.5f;
         }
         if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, tid);
@@ -274,14 +298,14 @@ static int launch_phys_reset(mrl_ctx *ctx, int batch, float *states, const float
 template <class E>
 static int launch_phys_step(mrl_ctx *ctx, int batch, float *states, const float *actions, float *rewards,
                             float *dones, float *obs, const float *shapes, bool autoreset,
-                            uint64_t reset_seed) {
+                            uint64_t reset_seed, const Accounting &acc) {
     dim3 grid(grid_for(batch, E::EPB));
     if (autoreset)
         hipLaunchKernelGGL((phys_step_kernel<E, true>), grid, dim3(BLOCK), 0, ctx->stream, states, actions,
-                           rewards, dones, obs, shapes, batch, reset_seed);
+                           rewards, dones, obs, shapes, batch, reset_seed, acc);
     else
         hipLaunchKernelGGL((phys_step_kernel<E, false>), grid, dim3(BLOCK), 0, ctx->stream, states, actions,
-                           rewards, dones, obs, shapes, batch, reset_seed);
+                           rewards, dones, obs, shapes, batch, reset_seed, acc);
     return MRL_OK;
 }
 
@@ -371,7 +395,7 @@ int mrl_env_selective_reset(mrl_ctx *ctx, int env_id, int batch, float *states, 
 
 static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, const float *actions,
                          float *rewards, float *dones, float *obs, uint64_t seed, bool autoreset,
-                         uint64_t reset_seed) {
+                         uint64_t reset_seed, const Accounting &acc) {
     (void)seed;  // none of the built envs consumes the step seed (their streams are keyed by env/step)
     MRL_CHECK_ARG(ctx, "mrl_env_step: NULL ctx");
     MRL_CHECK_ARG(batch >= 0, "mrl_env_step: negative batch");
@@ -384,25 +408,25 @@ static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, con
             if (rc) return rc;
             hipLaunchKernelGGL(cartpole_step_kernel, dim3(grid_for(batch, 256)), dim3(256), 0,
                                ctx->stream, states, steps, actions, rewards, dones, obs, batch,
-                               autoreset ? 1 : 0, (uint32_t)reset_seed);
+                               autoreset ? 1 : 0, (uint32_t)reset_seed, acc);
             break;
         }
         case MRL_ENV_PENDULUM:
             hipLaunchKernelGGL(pendulum_step_kernel, dim3(grid_for(batch, 256)), dim3(256), 0,
                                ctx->stream, states, actions, rewards, dones, obs, batch,
-                               autoreset ? 1 : 0, reset_seed);
+                               autoreset ? 1 : 0, reset_seed, acc);
             break;
         case MRL_ENV_LUNARLANDER:
             launch_phys_step<LunarLander>(ctx, batch, states, actions, rewards, dones, obs, ctx->ll_shapes,
-                                          autoreset, reset_seed);
+                                          autoreset, reset_seed, acc);
             break;
         case MRL_ENV_BIPEDAL:
             launch_phys_step<BipedalWalker>(ctx, batch, states, actions, rewards, dones, obs, ctx->bw_shapes,
-                                            autoreset, reset_seed);
+                                            autoreset, reset_seed, acc);
             break;
         case MRL_ENV_HALFCHEETAH:
             launch_phys_step<HalfCheetah>(ctx, batch, states, actions, rewards, dones, obs, ctx->hc_shapes,
-                                          autoreset, reset_seed);
+                                          autoreset, reset_seed, acc);
             break;
         default:
             return set_error(MRL_E_UNSUPPORTED, "mrl_env_step: env_id %d is not built", env_id);
@@ -413,14 +437,22 @@ static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, con
 
 int mrl_env_step(mrl_ctx *ctx, int env_id, int batch, float *states, const float *actions,
                  float *rewards, float *dones, float *obs, uint64_t seed) {
-    return env_step_impl(ctx, env_id, batch, states, actions, rewards, dones, obs, seed, false, 0);
+    return env_step_impl(ctx, env_id, batch, states, actions, rewards, dones, obs, seed, false, 0,
+                         Accounting{});
 }
 
 int mrl_env_step_autoreset(mrl_ctx *ctx, int env_id, int batch, float *states, const float *actions,
                            float *rewards, float *dones, float *obs, uint64_t step_seed,
                            uint64_t reset_seed) {
     return env_step_impl(ctx, env_id, batch, states, actions, rewards, dones, obs, step_seed, true,
-                         reset_seed);
+                         reset_seed, Accounting{});
 }
 
 }  // extern "C"
+
+int mrl::env_step_accounting(mrl_ctx *ctx, int env_id, int batch, float *states, const float *actions,
+                             float *rewards, float *dones, float *obs, uint64_t step_seed,
+                             uint64_t reset_seed, const Accounting &acc) {
+    return env_step_impl(ctx, env_id, batch, states, actions, rewards, dones, obs, step_seed, true,
+                         reset_seed, acc);
+}

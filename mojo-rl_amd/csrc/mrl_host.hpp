@@ -40,6 +40,22 @@ namespace mrl {
 
 int set_error(int code, const char *fmt, ...);
 
+// Post-step bookkeeping of a collection step, done by the env-step kernel itself when the rollout
+// step asks for it (all pointers null otherwise): rollout rows of reward / done, per-env episode
+// return and length, and the device-side list of finished episodes.
+struct Accounting {
+    float *r_rewards, *r_dones;        // [N] row t of the time-major buffers
+    float *ep_return, *ep_length;      // [N]
+    float *done_returns, *done_lengths;
+    int32_t *done_count;
+    int32_t done_cap;
+};
+
+// mrl_env_step_autoreset with the bookkeeping folded into the same launch
+int env_step_accounting(mrl_ctx *ctx, int env_id, int batch, float *states, const float *actions,
+                        float *rewards, float *dones, float *obs, uint64_t step_seed, uint64_t reset_seed,
+                        const Accounting &acc);
+
 inline int grid_for(long n, int block) { return (int)((n + block - 1) / block); }
 
 // records a phase boundary: the time since the previous mark is charged to `tag` (tag < 0: start)

@@ -7,13 +7,15 @@
 // Continuous agents: StochasticActor head [mean | clamp(log_std)] + Gaussian sampling
 // (deep_agents/ppo/ppo_continuous.mojo:2619-2686, deep_agents/ppo/kernels.mojo:12-98).
 //
-// One workgroup = 32 environments (rows).  The 32 x H hidden activations never leave the CU:
-//   layer 0 (K = IN <= 32): one lane per hidden column, 32 row accumulators in registers, FMA;
-//   layer 1 (H x H):        fp32 MFMA 32x32x2, each wavefront owns 64 output columns (two
-//                           accumulator tiles), A operand from LDS (k-major), B operand (the
-//                           weights) streamed from L2 -- all blocks read the same 256 KB;
+// One workgroup = 32 environments (rows) and 2H threads: threads [0, H) run the actor, threads
+// [H, 2H) the critic, side by side (two wavefronts per SIMD hide each other's LDS and L2
+// latencies).  The 32 x H hidden activations never leave the CU:
+//   layers 0 and 1:         fp32 MFMA 32x32x2, each wavefront owns 64 output columns (two
+//                           accumulator tiles), A operand from LDS, B operand (the weights)
+//                           streamed from L2 a block of k-steps ahead of the MFMAs that use it
+//                           -- all workgroups read the same 256 KB;
 //   layer 2 (N = A or 1):   H/32 lanes per row, shuffle reduction.
-// With 8192 envs this is 256 workgroups: one per CU of the MI355X.
+// With 8192 envs this is 256 workgroups of 8 wavefronts: one per CU of the MI355X.
 #include "mrl_host.hpp"
 #include "mrl_device.hpp"
 
@@ -37,36 +39,63 @@ MRL_DEV float activate(float x) {
 // hidden stack of one net for the block's 32 rows; leaves act(layer1) in h2[32][H+1]
 template <int H, int ACT>
 MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2) {
-    const int t = threadIdx.x, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
+    const int t = threadIdx.x % H, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
     const float *W0 = p, *b0 = p + IN * H;
     const float *W1 = b0 + H, *b1 = W1 + H * H;
-    {   // layer 0: lane t owns hidden column t
-        float acc[PR];
-        const float b = b0[t];
-#pragma unroll
-        for (int r = 0; r < PR; ++r) acc[r] = b;
-        for (int k = 0; k < IN; ++k) {
-            const float wv = W0[k * H + t];
-#pragma unroll
-            for (int r = 0; r < PR; ++r) acc[r] = fmaf(xs[r * XS_LD + k], wv, acc[r]);
-        }
-#pragma unroll
-        for (int r = 0; r < PR; ++r) hT[t * HT_LD + r] = activate<ACT>(acc[r]);
-    }
-    __syncthreads();
-    {   // layer 1: wavefront w owns columns [64w, 64w + 64)
+    const int col0 = 64 * w + l31, col1 = col0 + 32;
+    {   // layer 0 (K = IN <= 32, padded to even with zeros): wavefront w owns columns [64w, 64w + 64)
         floatx16 c0 = {0}, c1 = {0};
-        const float *Wc = W1 + 64 * w + l31;
-#pragma unroll 8
-        for (int kk = 0; kk < H / 2; ++kk) {
+        for (int kk = 0; kk < (IN + 1) / 2; ++kk) {
             const int k = 2 * kk + half;
-            const float a = hT[k * HT_LD + l31];
-            const float bv0 = Wc[k * H];
-            const float bv1 = Wc[k * H + 32];
+            const bool in = k < IN;
+            const float a = in ? xs[l31 * XS_LD + k] : 0.0f;
+            const float bv0 = in ? W0[k * H + col0] : 0.0f;
+            const float bv1 = in ? W0[k * H + col1] : 0.0f;
             c0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bv0, c0, 0, 0, 0);
             c1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bv1, c1, 0, 0, 0);
         }
-        const int col0 = 64 * w + l31, col1 = col0 + 32;
+        const float bb0 = b0[col0], bb1 = b0[col1];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int row = 8 * (v >> 2) + 4 * half + (v & 3);
+            hT[col0 * HT_LD + row] = activate<ACT>(c0[v] + bb0);
+            hT[col1 * HT_LD + row] = activate<ACT>(c1[v] + bb1);
+        }
+    }
+    __syncthreads();
+    {   // layer 1 (H x H): weights streamed from L2 one block of KB k-steps ahead of the MFMAs
+        constexpr int KB = 8;
+        floatx16 c0 = {0}, c1 = {0};
+        const float *Wc = W1 + col0;
+        float a[KB], bv0[KB], bv1[KB], na[KB], nb0[KB], nb1[KB];
+#pragma unroll
+        for (int j = 0; j < KB; ++j) {
+            const int k = 2 * j + half;
+            a[j] = hT[k * HT_LD + l31];
+            bv0[j] = Wc[k * H];
+            bv1[j] = Wc[k * H + 32];
+        }
+        for (int blk = 0; blk < H / (2 * KB); ++blk) {
+            const bool more = blk + 1 < H / (2 * KB);
+            if (more) {
+#pragma unroll
+                for (int j = 0; j < KB; ++j) {
+                    const int k = 2 * ((blk + 1) * KB + j) + half;
+                    na[j] = hT[k * HT_LD + l31];
+                    nb0[j] = Wc[k * H];
+                    nb1[j] = Wc[k * H + 32];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < KB; ++j) {
+                c0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], bv0[j], c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], bv1[j], c1, 0, 0, 0);
+            }
+            if (more) {
+#pragma unroll
+                for (int j = 0; j < KB; ++j) { a[j] = na[j]; bv0[j] = nb0[j]; bv1[j] = nb1[j]; }
+            }
+        }
         const float bb0 = b1[col0], bb1 = b1[col1];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -82,7 +111,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
 template <int H>
 MRL_DEV void head(const float *__restrict__ W2, int A, const float *h2, float *out, int out_ld) {
     constexpr int TPR = H / PR;
-    const int t = threadIdx.x, r = t / TPR, part = t % TPR;
+    const int t = threadIdx.x % H, r = t / TPR, part = t % TPR;
     const float *b2 = W2 + H * A;
     float acc[PA_MAX];
 #pragma unroll
@@ -104,22 +133,23 @@ MRL_DEV void head(const float *__restrict__ W2, int A, const float *h2, float *o
 }
 
 template <int H, int ACT, bool GAUSS>
-__global__ __launch_bounds__(H) void policy_kernel(
+__global__ __launch_bounds__(2 * H) void policy_kernel(
     const float *__restrict__ obs, int n, int IN, int A, const float *__restrict__ actor_p,
     const float *__restrict__ critic_p, uint32_t seed, float *__restrict__ actions,
     float *__restrict__ r_obs, float *__restrict__ r_actions, float *__restrict__ r_logp,
     float *__restrict__ r_values) {
     __shared__ float xs[PR * XS_LD];
-    __shared__ float hT[H * HT_LD];
-    __shared__ float h2[PR * (H + 1)];
+    __shared__ float hT[2][H * HT_LD];
+    __shared__ float h2[2][PR * (H + 1)];
     __shared__ float logits[PR * (PA_MAX + 1)];
     __shared__ float vals[PR];
     const int t = threadIdx.x;
+    const int net = t / H;                   // 0 = actor, 1 = critic
     const int row0 = blockIdx.x * PR;
     const int nrow = min(PR, n - row0);
 
     // observation tile in (rows beyond the batch read as zero), and straight out to rollout[t]
-    for (int i = t; i < PR * IN; i += H) {
+    for (int i = t; i < PR * IN; i += 2 * H) {
         const int r = i / IN, k = i - r * IN;
         float v = 0.0f;
         if (r < nrow) {
@@ -130,11 +160,10 @@ __global__ __launch_bounds__(H) void policy_kernel(
     }
     __syncthreads();
 
-    hidden_stack<H, ACT>(actor_p, IN, xs, hT, h2);
-    head<H>(actor_p + IN * H + H + H * H + H, A, h2, logits, PA_MAX + 1);
-    __syncthreads();
-    hidden_stack<H, ACT>(critic_p, IN, xs, hT, h2);
-    head<H>(critic_p + IN * H + H + H * H + H, 1, h2, vals, 1);
+    const float *p = net ? critic_p : actor_p;
+    hidden_stack<H, ACT>(p, IN, xs, hT[net], h2[net]);
+    if (net == 0) head<H>(p + IN * H + H + H * H + H, A, h2[0], logits, PA_MAX + 1);
+    else head<H>(p + IN * H + H + H * H + H, 1, h2[1], vals, 1);
     __syncthreads();
 
     if (t < nrow && !GAUSS) {   // categorical sampling, one lane per env
@@ -216,7 +245,7 @@ int launch_policy(mrl_ctx *ctx, const mrl_mlp_desc &a, const mrl_mlp_desc &c, bo
     const int IN = a.layers[0].in_dim, A = a.layers[2].out_dim;
     dim3 grid((n + PR - 1) / PR);
 #define MRL_LAUNCH(HH, AA, GG)                                                                         \
-    hipLaunchKernelGGL((policy_kernel<HH, AA, GG>), grid, dim3(HH), 0, ctx->stream, obs, n, IN, A, ap, \
+    hipLaunchKernelGGL((policy_kernel<HH, AA, GG>), grid, dim3(2 * HH), 0, ctx->stream, obs, n, IN, A, ap, \
                        cp, seed, actions, r_obs, r_actions, r_logp, r_values)
     if (gauss) {
         if (H == 256 && act == 1) MRL_LAUNCH(256, 1, true);

@@ -1,6 +1,6 @@
 // One time step of the PPO collection loop (deep_agents/ppo/ppo.mojo:2069-2285) without any
-// host round trip: policy + value forward, categorical sampling, rollout stores, env step with
-// auto-reset, episode accounting.  Finished episodes are appended to a device-side list through
+// host round trip, in two launches: [policy + value forward, sampling, pre-step stores] and
+// [env step with auto-reset, post-step stores, episode accounting].  Finished episodes are appended to a device-side list through
 // a counter instead of being copied to the host after every step.
 #include "mrl_host.hpp"
 #include "mrl_device.hpp"
@@ -71,33 +71,6 @@ __global__ __launch_bounds__(256) void sample_store_gaussian_kernel(
     r_logp[i] = total;
     r_values[i] = values[i];
     for (int k = 0; k < obs_dim; ++k) r_obs[(long)i * obs_dim + k] = obs[(long)i * obs_dim + k];
-}
-
-// _store_post_step_kernel (ppo.mojo:692-708) + accumulate_rewards / increment_steps /
-// extract_completed_episodes (deep_rl/gpu/rl_kernels.mojo:103-200) in one pass
-__global__ __launch_bounds__(256) void post_store_kernel(
-    const float *__restrict__ rewards, const float *__restrict__ dones, int n,
-    float *__restrict__ r_rewards, float *__restrict__ r_dones, float *__restrict__ ep_return,
-    float *__restrict__ ep_length, float *__restrict__ done_returns, float *__restrict__ done_lengths,
-    int32_t *__restrict__ done_count, int done_cap) {
-    int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    float r = rewards[i], d = dones[i];
-    r_rewards[i] = r;
-    r_dones[i] = d;
-    float er = ep_return[i] + r;
-    float el = ep_length[i] + 1.0f;
-    if (d > 0.5f) {
-        int slot = atomicAdd(done_count, 1);
-        if (slot < done_cap) {
-            done_returns[slot] = er;
-            done_lengths[slot] = el;
-        }
-        er = 0.0f;
-        el = 0.0f;
-    }
-    ep_return[i] = er;
-    ep_length[i] = el;
 }
 
 }  // namespace mrl
@@ -216,15 +189,14 @@ int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_
                      r->r_log_probs + row, r->r_values + row);
     if (rc) return rc;
     profile_mark(ctx, -1);
-    rc = mrl_env_step_autoreset(ctx, r->env_id, N, r->states, actions, rewards, dones, r->obs, step_seed,
-                                reset_seed);
+    // the env-step kernel also stores (reward, done) into rollout row t and does the episode
+    // accounting for its envs
+    const Accounting acc{r->r_rewards + row, r->r_dones + row, r->ep_return, r->ep_length,
+                         r->done_returns, r->done_lengths, r->done_count, r->done_cap};
+    rc = env_step_accounting(ctx, r->env_id, N, r->states, actions, rewards, dones, r->obs, step_seed,
+                             reset_seed, acc);
     if (rc) return rc;
     profile_mark(ctx, MRL_PHASE_ENV);
-    hipLaunchKernelGGL(post_store_kernel, dim3(grid_for(N, 256)), dim3(256), 0, ctx->stream, rewards,
-                       dones, N, r->r_rewards + row, r->r_dones + row, r->ep_return, r->ep_length,
-                       r->done_returns, r->done_lengths, r->done_count, r->done_cap);
-    MRL_CHECK_LAUNCH();
-    profile_mark(ctx, MRL_PHASE_POST);
     return MRL_OK;
 }
 
