@@ -16,6 +16,13 @@
 namespace mrl {
 namespace ll {
 
+// joint j hangs leg j + 1 on the lander body (reset_row below, lunar_lander_v2.mojo:560-634)
+struct Topology {
+    static constexpr bool STATIC = true;
+    static constexpr MRL_DEV int a(int) { return 0; }
+    static constexpr MRL_DEV int b(int j) { return j + 1; }
+};
+
 using L = LunarLanderLayout;
 constexpr int STATE = L::STATE_SIZE;  // 192
 constexpr int OBS = 8;
@@ -298,7 +305,7 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
     const float gx = (float)0.0, gy = (float)-10.0, dt = (float)DT;
     const float friction = (float)0.1, restitution = (float)0.0;
     const float baumgarte = (float)0.2, slop = (float)0.005;
-    const int n = reg_physics_substep<L, false>(row, shapes, contacts, gx, gy, dt, friction, restitution,
+    const int n = reg_physics_substep<L, Topology, false, true>(row, shapes, contacts, gx, gy, dt, friction, restitution,
                                                 baumgarte, slop, 6, 2);
 
     step_count += 1;

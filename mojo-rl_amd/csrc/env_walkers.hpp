@@ -9,7 +9,7 @@
 // :745-846; constants envs/half_cheetah/constants.mojo.
 // Reset seed for both: Int(f32(seed)) * 2654435761 + (env + 1) * 12345 (:1444 / :1108).
 #pragma once
-#include "physics2d.hpp"
+#include "physics2d_reg.hpp"
 
 namespace mrl {
 
@@ -46,30 +46,17 @@ MRL_DEV uint64_t walker_seed(uint64_t seed, int env) {
     return (uint64_t)seed_i * 2654435761ull + (uint64_t)(env + 1) * 12345ull;
 }
 
-template <class L, bool FLAT>
-MRL_DEV int physics_substep(float *row, const float *shapes, float *contacts, float gx, float gy,
-                            float dt, float friction, float restitution, float baumgarte, float slop,
-                            int vel_iters, int pos_iters) {
-    integrate_velocities<L>(row, gx, gy, dt);
-    int n = FLAT ? flat_detect<L>(row, shapes, 0.0f, contacts) : edge_detect<L>(row, shapes, contacts);
-    JointAnchors<L> an;
-    joint_anchors_all<L>(row, an);
-    for (int it = 0; it < vel_iters; ++it) {
-        contact_solve_velocity<L>(row, contacts, n, friction, restitution);
-        joint_solve_velocity<L>(row, an, dt);
-    }
-    integrate_positions<L>(row, dt);
-    for (int it = 0; it < pos_iters; ++it) {
-        contact_solve_position<L>(row, contacts, n, baumgarte, slop);
-        joint_solve_position<L>(row, baumgarte, slop);
-    }
-    for (int k = 0; k < L::NUM_BODIES * 3; ++k) row[L::FORCES_OFF + k] = 0.0f;
-    return n;
-}
 
 // ================================================================ BipedalWalker
 namespace bw {
 using L = BipedalWalkerLayout;
+
+// hull(0) - upper leg(1) - lower leg(2), hull(0) - upper leg(3) - lower leg(4): reset_row below
+struct Topology {
+    static constexpr bool STATIC = true;
+    static constexpr MRL_DEV int a(int j) { return (j & 1) ? j : 0; }
+    static constexpr MRL_DEV int b(int j) { return j + 1; }
+};
 constexpr int STATE = L::STATE_SIZE, OBS = 24, ACT = 4, NSHAPE_FLOATS = 5 * SHAPE_SIZE;
 constexpr double SCALE = 30.0, FPS = 50.0;
 constexpr double LEG_DOWN = -8.0 / SCALE, LEG_H = 34.0 / SCALE;
@@ -115,12 +102,17 @@ MRL_DEV void observe(float *row) {
     }
     const float hull_x = B[IDX_X], hull_y = B[IDX_Y], hull_angle_rad = B[IDX_ANGLE];
     const float lidar_range = (float)LIDAR_RANGE;
+    // every ray stays within lidar_range of the hull in x: select those edges once for the ten rays
+    EdgeMask<L> near;
+    const bool plain = !(hull_x == hull_x);
+    if (!plain) edges_near<L>(row, hull_x - lidar_range, hull_x + lidar_range, 0.02f, near);
     for (int i = 0; i < 10; ++i) {
         float local_angle = (float)i * 1.5f / (float)9;
         float world_angle = hull_angle_rad - local_angle - (float)(3.14159265358979323846 / 2.0);
         float sn, cs;
         sincos32(world_angle, sn, cs);
-        o[14 + i] = lidar_ray<L>(row, hull_x, hull_y, cs * lidar_range, sn * lidar_range);
+        o[14 + i] = plain ? lidar_ray<L>(row, hull_x, hull_y, cs * lidar_range, sn * lidar_range)
+                          : lidar_ray_near<L>(row, near, hull_x, hull_y, cs * lidar_range, sn * lidar_range);
     }
 #pragma unroll
     for (int k = 0; k < OBS; ++k) row[k] = o[k];
@@ -190,7 +182,7 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
         J[J_MOTOR_SPEED] = sign * (float)((j & 1) ? 6.0 : 4.0);
         J[J_MAX_TORQUE] = (float)MOTORS_TORQUE * fabsf(a);
     }
-    int n = physics_substep<L, false>(row, shapes, contacts, (float)0.0, (float)-10.0, (float)(1.0 / FPS),
+    int n = reg_physics_substep<L, Topology, false, false>(row, shapes, contacts, (float)0.0, (float)-10.0, (float)(1.0 / FPS),
                                       (float)2.5, (float)0.0, (float)0.2, (float)0.005, 6, 2);
     bool left = false, right = false, hull = false;
     for (int c = 0; c < n; ++c) {
@@ -237,6 +229,13 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
 // ================================================================ HalfCheetah
 namespace hc {
 using L = HalfCheetahLayout;
+
+// torso(0) - thigh - shin - foot for the back (1,2,3) and front (4,5,6) legs: reset_row below
+struct Topology {
+    static constexpr bool STATIC = true;
+    static constexpr MRL_DEV int a(int j) { return (j == 0 || j == 3) ? 0 : j; }
+    static constexpr MRL_DEV int b(int j) { return j + 1; }
+};
 constexpr int STATE = L::STATE_SIZE, OBS = 17, ACT = 6, NSHAPE_FLOATS = 7 * SHAPE_SIZE;
 enum { META_STEP = 0, META_PREV_X = 1, META_PREV_SHAPING = 2, META_DONE = 3, META_TOTAL = 4 };
 __device__ constexpr double LEN[7] = {1.0, 0.145, 0.15, 0.094, 0.133, 0.106, 0.07};
@@ -316,7 +315,7 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
     const double x_before = B[IDX_X];
     int n = 0;
     for (int s = 0; s < 5; ++s)
-        n = physics_substep<L, true>(row, shapes, contacts, (float)0.0, (float)-9.81, (float)0.01, (float)0.9,
+        n = reg_physics_substep<L, Topology, true, false>(row, shapes, contacts, (float)0.0, (float)-9.81, (float)0.01, (float)0.9,
                                      (float)0.0, (float)0.2, (float)0.005, 4, 2);
     const double x_after = B[IDX_X], torso_z = B[IDX_Y];
     const double forward_velocity = (x_after - x_before) / (0.01 * (double)5);

@@ -41,6 +41,7 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     c->rollout_ws_floats = 0;
     c->profiling = false;
     c->prof_used = 0;
+    c->prof_chained = false;
     MRL_CHECK_HIP(hipMalloc(&c->ll_shapes, sizeof(mrl::ll::Shapes)));
     mrl::ll::Shapes sh = mrl::ll::make_shapes();
     MRL_CHECK_HIP(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));
@@ -88,6 +89,7 @@ int mrl_profile_begin(mrl_ctx *ctx, int max_marks) {
     }
     ctx->prof_tags.assign(ctx->prof_events.size(), -1);
     ctx->prof_used = 0;
+    ctx->prof_chained = false;
     ctx->profiling = true;
     return MRL_OK;
 }

@@ -168,7 +168,7 @@ constexpr int BLOCK = 256;  // all four wavefronts of the workgroup move the row
 template <class E>
 struct Stage {
     static constexpr int STRIDE = E::STATE | 1;                            // odd => conflict-free lane access
-    static constexpr int CSTRIDE = (E::L::MAX_CONTACTS * CONTACT_SIZE) | 1;
+    static constexpr int CSTRIDE = (E::L::MAX_CONTACTS * CONTACT_SCRATCH) | 1;
 
     static MRL_DEV void in(float *lds, const float *g, int nenv, int lane) {
         if (E::STATE % 4 == 0) {   // rows are whole float4s, never straddled by a 16-byte load

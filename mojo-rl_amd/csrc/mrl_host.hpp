@@ -34,6 +34,7 @@ struct mrl_ctx {
     std::vector<hipEvent_t> prof_events;
     std::vector<int> prof_tags;
     size_t prof_used;
+    bool prof_chained;   // the last event recorded closes a phase and can open the next one
 };
 
 namespace mrl {
@@ -58,11 +59,16 @@ int env_step_accounting(mrl_ctx *ctx, int env_id, int batch, float *states, cons
 
 inline int grid_for(long n, int block) { return (int)((n + block - 1) / block); }
 
-// records a phase boundary: the time since the previous mark is charged to `tag` (tag < 0: start)
+// Records a phase boundary: the time since the previous mark is charged to `tag`; tag < 0 opens
+// a phase without charging anything.  An opening mark that directly follows a closing one reuses
+// its event (two events per collection step instead of four), so work that the caller enqueues
+// between two rollout steps is charged to the first phase of the second step.
 inline void profile_mark(mrl_ctx *ctx, int tag) {
     if (!ctx->profiling || ctx->prof_used >= ctx->prof_events.size()) return;
+    if (tag < 0 && ctx->prof_chained) return;
     if (hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream) != hipSuccess) return;
     ctx->prof_tags[ctx->prof_used++] = tag;
+    ctx->prof_chained = tag >= 0;
 }
 
 }  // namespace mrl

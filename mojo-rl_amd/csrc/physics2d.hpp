@@ -120,6 +120,38 @@ MRL_DEV bool edge_x_pass(float e_x0, float e_x1, float world_x) {
     return !(world_x < x_min || world_x > x_max);
 }
 
+// Bit e of a mask is set when terrain edge e can matter for an x interval.
+template <class L>
+struct EdgeMask {
+    static constexpr int WORDS = (L::MAX_EDGES + 31) / 32;
+    unsigned w[WORDS];
+};
+
+// Edges whose x-range pre-check (edge_x_pass) can succeed for some x in [xlo, xhi]: a superset of
+// the edges any such vertex passes, decided with the same fp32 bounds the pre-check uses.
+// widen = 0 gives exactly that; lidar passes its own safety margin on top.
+template <class L>
+MRL_DEV void edges_near(const float *row, float xlo, float xhi, float widen, EdgeMask<L> &m) {
+    int n_edges = (int)row[L::EDGE_COUNT_OFF];
+    if (n_edges > L::MAX_EDGES) n_edges = L::MAX_EDGES;
+    const float *edges = row + L::EDGES_OFF;
+#pragma unroll
+    for (int q = 0; q < EdgeMask<L>::WORDS; ++q) {
+        unsigned bits = 0;
+        const int e0 = q * 32;
+        for (int k = 0; k < 32; ++k) {
+            const int e = e0 + k;
+            if (e >= n_edges) break;
+            const float e_x0 = edges[e * 6], e_x1 = edges[e * 6 + 2];
+            const float margin = 0.1f;
+            float x_min = e_x0 - margin, x_max = e_x1 + margin;
+            if (e_x0 > e_x1) { x_min = e_x1 - margin; x_max = e_x0 + margin; }
+            if (!(xhi < x_min - widen || xlo > x_max + widen)) bits |= 1u << k;
+        }
+        m.w[q] = bits;
+    }
+}
+
 // vertex / circle against the row's terrain polyline; contacts in (body, vertex, edge) order.
 //
 // The x-range pre-check rejects almost every (vertex, edge) pair, but which pairs survive differs
@@ -143,13 +175,39 @@ MRL_DEV int edge_detect(const float *row, const float *shapes, float *contacts) 
             ex1[e] = edges[e * 6 + 2];
         }
     }
+    // long polylines: one pass over the edges picks those near the env's polygon vertices at all
+    // (x interval of every vertex of every body); the per-vertex loops then visit only these
+    float sins[L::NUM_BODIES], coss[L::NUM_BODIES];
+#pragma unroll
+    for (int b = 0; b < L::NUM_BODIES; ++b) sincos32(row[L::BODIES_OFF + b * BODY_SIZE + IDX_ANGLE], sins[b], coss[b]);
+    EdgeMask<L> near;
+    if (!SMALL) {
+        float xlo = 3.0e38f, xhi = -3.0e38f;
+        bool odd = false;   // a NaN coordinate passes the pre-check of every edge
+#pragma unroll
+        for (int b = 0; b < L::NUM_BODIES; ++b) {
+            const float *B = row + L::BODIES_OFF + b * BODY_SIZE;
+            const float *S = shapes + (int)B[IDX_SHAPE] * SHAPE_SIZE;
+            if ((int)S[0] != SHAPE_POLYGON) continue;
+            int n_verts = (int)S[1];
+            if (n_verts > MAX_POLY_VERTS) n_verts = MAX_POLY_VERTS;
+            for (int v = 0; v < n_verts; ++v) {
+                const float world_x = B[IDX_X] + S[2 + v * 2] * coss[b] - S[3 + v * 2] * sins[b];
+                odd = odd || !(world_x == world_x);
+                xlo = world_x < xlo ? world_x : xlo;
+                xhi = world_x > xhi ? world_x : xhi;
+            }
+        }
+        if (odd) { xlo = -3.0e38f; xhi = 3.0e38f; }
+        edges_near<L>(row, xlo, xhi, 0.0f, near);
+    }
+#pragma unroll
     for (int b = 0; b < L::NUM_BODIES; ++b) {
         const float *B = row + L::BODIES_OFF + b * BODY_SIZE;
         float body_x = B[IDX_X], body_y = B[IDX_Y];
         const float *S = shapes + (int)B[IDX_SHAPE] * SHAPE_SIZE;
         int shape_type = (int)S[0];
-        float sin_a, cos_a;
-        sincos32(B[IDX_ANGLE], sin_a, cos_a);
+        const float sin_a = sins[b], cos_a = coss[b];
         if (shape_type == SHAPE_POLYGON) {
             int n_verts = (int)S[1];
             if (n_verts > MAX_POLY_VERTS) n_verts = MAX_POLY_VERTS;
@@ -169,18 +227,15 @@ MRL_DEV int edge_detect(const float *row, const float *shapes, float *contacts) 
                                          L::MAX_CONTACTS);
                     }
                 } else {
-                    for (int e0 = 0; e0 < n_edges; e0 += 32) {
-                        const int m = min(32, n_edges - e0);
-                        unsigned mask = 0;
-                        for (int k = 0; k < m; ++k) {
-                            const float *E = edges + (e0 + k) * 6;
-                            if (edge_x_pass(E[0], E[2], world_x)) mask |= 1u << k;
-                        }
+#pragma unroll
+                    for (int q = 0; q < EdgeMask<L>::WORDS; ++q) {
+                        unsigned mask = near.w[q];
                         while (mask) {
-                            const int e = e0 + __ffs((int)mask) - 1;
+                            const int e = q * 32 + __ffs((int)mask) - 1;
                             mask &= mask - 1;
-                            vertex_edge_test(edges + e * 6, b, world_x, world_y, contacts, count,
-                                             L::MAX_CONTACTS);
+                            const float *E = edges + e * 6;
+                            if (edge_x_pass(E[0], E[2], world_x))
+                                vertex_edge_test(E, b, world_x, world_y, contacts, count, L::MAX_CONTACTS);
                         }
                     }
                 }
@@ -526,20 +581,49 @@ MRL_DEV void joint_solve_position(float *row, float baumgarte, float slop) {
     }
 }
 
+// ray / edge test of physics2d/lidar/lidar.mojo:25-141 for one edge
+MRL_DEV void lidar_edge(const float *E, float ox, float oy, float rdx, float rdy, float &min_t) {
+    float ex = E[2] - E[0], ey = E[3] - E[1];
+    float denom = rdx * ey - rdy * ex;
+    if (denom > -1e-10f && denom < 1e-10f) return;
+    float dx = ox - E[0], dy = oy - E[1];
+    float t = (ex * dy - ey * dx) / denom;
+    float u = (rdx * dy - rdy * dx) / denom;
+    if (t >= 0.0f && t <= 1.0f && u >= 0.0f && u <= 1.0f && t < min_t) min_t = t;
+}
+
 template <class L>
 MRL_DEV float lidar_ray(const float *row, float ox, float oy, float rdx, float rdy) {
     int n_edges = (int)row[L::EDGE_COUNT_OFF];
     if (n_edges > L::MAX_EDGES) n_edges = L::MAX_EDGES;
     float min_t = 1.0f;
-    for (int e = 0; e < n_edges; ++e) {
-        const float *E = row + L::EDGES_OFF + e * 6;
-        float ex = E[2] - E[0], ey = E[3] - E[1];
-        float denom = rdx * ey - rdy * ex;
-        if (denom > -1e-10f && denom < 1e-10f) continue;
-        float dx = ox - E[0], dy = oy - E[1];
-        float t = (ex * dy - ey * dx) / denom;
-        float u = (rdx * dy - rdy * dx) / denom;
-        if (t >= 0.0f && t <= 1.0f && u >= 0.0f && u <= 1.0f && t < min_t) min_t = t;
+    for (int e = 0; e < n_edges; ++e) lidar_edge(row + L::EDGES_OFF + e * 6, ox, oy, rdx, rdy, min_t);
+    return min_t;
+}
+
+// Same result from a pre-selected edge set.  A hit needs a point common to the ray segment and the
+// edge, so an edge whose x extent stays clear of the ray's x extent cannot hit; `near` must hold
+// every edge within 0.01 of the ray's x extent (the tests t, u in [0, 1] are evaluated in fp32:
+// the slack is orders of magnitude above their rounding error, and where the denominator is tiny
+// a far-away edge yields |t| or |u| in the millions, never a value in [0, 1]).
+template <class L>
+MRL_DEV float lidar_ray_near(const float *row, const EdgeMask<L> &near, float ox, float oy, float rdx,
+                             float rdy) {
+    float min_t = 1.0f;
+    const float ex_ = ox + rdx;
+    const float rlo = (ox < ex_ ? ox : ex_) - 0.01f, rhi = (ox > ex_ ? ox : ex_) + 0.01f;
+#pragma unroll
+    for (int q = 0; q < EdgeMask<L>::WORDS; ++q) {
+        unsigned mask = near.w[q];
+        while (mask) {
+            const int e = q * 32 + __ffs((int)mask) - 1;
+            mask &= mask - 1;
+            const float *E = row + L::EDGES_OFF + e * 6;
+            const float x0 = E[0], x1 = E[2];
+            const float elo = x0 < x1 ? x0 : x1, ehi = x0 < x1 ? x1 : x0;
+            if (ehi < rlo || elo > rhi) continue;
+            lidar_edge(E, ox, oy, rdx, rdy, min_t);
+        }
     }
     return min_t;
 }
