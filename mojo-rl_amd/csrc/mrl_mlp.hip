@@ -291,6 +291,14 @@ static void launch_fwd(hipStream_t s, const float *X, int ldx, const float *W, c
                        M, K, N);
 }
 
+// fused three-layer path (mrl_mlp3.hip); MRL_E_UNSUPPORTED when the shape is not covered
+bool mlp3_fusable(const mrl_mlp_desc &d, int *H, int *act, bool *gauss);
+int mlp3_forward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *in, const float *params,
+                 float *out, float *cache);
+int mlp3_backward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *grad_out, const float *params,
+                  const float *cache, float *grads, float *ws);
+size_t mlp3_backward_ws(const mrl_mlp_desc &d, int batch);
+
 }  // namespace mrl
 
 using namespace mrl;
@@ -327,6 +335,8 @@ int mrl_mlp_forward(mrl_ctx *ctx, const mrl_mlp_desc *d, int batch, const float 
     MRL_CHECK_ARG(batch >= 0, "mrl_mlp_forward: negative batch");
     if (batch == 0) return MRL_OK;
     MRL_CHECK_ARG(in && params && out, "mrl_mlp_forward: NULL buffer");
+    rc = mlp3_forward(ctx, *d, batch, in, params, out, cache);
+    if (rc != MRL_E_UNSUPPORTED) return rc;
     // two ping-pong activation buffers of the widest hidden size
     int widest = 0;
     for (int i = 0; i + 1 < d->n_layers; ++i) widest = std::max(widest, layer_out_dim(d->layers[i]));
@@ -369,6 +379,17 @@ int mrl_mlp_backward(mrl_ctx *ctx, const mrl_mlp_desc *d, int batch, const float
     if (rc) return rc;
     MRL_CHECK_ARG(batch > 0, "mrl_mlp_backward: batch must be positive");
     MRL_CHECK_ARG(grad_out && params && cache && grads, "mrl_mlp_backward: NULL buffer");
+    {
+        int fh, fa;
+        bool fg;
+        if (grad_in == nullptr && mlp3_fusable(*d, &fh, &fa, &fg)) {
+            float *fws = nullptr;
+            rc = ensure_ws(ctx, mlp3_backward_ws(*d, batch), &fws);
+            if (rc) return rc;
+            rc = mlp3_backward(ctx, *d, batch, grad_out, params, cache, grads, fws);
+            if (rc != MRL_E_UNSUPPORTED) return rc;
+        }
+    }
 
     size_t poff[MRL_MAX_LAYERS], coff[MRL_MAX_LAYERS];
     size_t p = 0, c = 0;

@@ -79,11 +79,12 @@ def test_forward_backward_parity(mrl, orc, orcmod, ctx, name, spec, batch):
     orc.orc_mlp_backward(ls, len(spec), batch, go, params, cache_d.cpu().numpy(), grads_h, gin_h.ctypes.data)
     close(grads_d.cpu().numpy(), grads_h, "param grads")
     close(gin_d.cpu().numpy().reshape(x.shape), gin_h, "input grads")
-    # backward without grad_input (what the PPO update asks for on the first layer)
-    grads2 = torch.zeros(P, device="cuda")
+    # backward without grad_input (what the PPO update asks for): three-layer nets of the agents'
+    # shapes take the fused kernels here, which sum in another order than the per-layer ones
+    grads2 = torch.full((P,), 9.0, device="cuda")
     model.backward_gpu_ws(ctx, None, go_d, p_d, cache_d, grads2)
     ctx.synchronize()
-    assert torch.equal(grads2, grads_d)
+    close(grads2.cpu().numpy(), grads_h, "param grads (no input gradient)")
 
 
 def test_forward_matches_torch_fp32_at_update_size(mrl, ctx):
