@@ -149,7 +149,8 @@ int mrl_rms_normalize(mrl_ctx *ctx, const double *state, float *x, int n);
  * core/utils/shuffle.mojo:21-82) and copies the indices to the device. */
 int mrl_permutation(mrl_ctx *ctx, int32_t *indices, int n, uint64_t seed);
 /* mean of kl[0..mb) against target_kl on the device: flag[0] is set to 1 when the mean exceeds
- * target_kl (never cleared by the library), flag[1] receives the bits of the mean.  Replaces
+ * target_kl (never cleared by the library), flag[1] receives the bits of the mean (flag holds 4
+ * int32; [2] and [3] belong to mrl_ppo_update_minibatch).  Replaces
  * the per-minibatch D2H copy + host mean of ppo.mojo:2557-2573 / ppo_continuous.mojo:3062-3086. */
 int mrl_kl_check(mrl_ctx *ctx, const float *kl, int mb, float target_kl, int32_t *flag);
 /* params[i] = lo + u_i (hi - lo): the uniform fills behind Xavier / Kaiming
@@ -228,6 +229,44 @@ typedef struct {
 
 int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_seed,
                      uint64_t step_seed, uint64_t reset_seed);
+
+/* ------------------------------------------------------------------ minibatch update
+ * The body of train_gpu's minibatch loop (deep_agents/ppo/ppo.mojo:2438-2727 for DeepPPOAgent,
+ * deep_agents/ppo/ppo_continuous.mojo:3000-3260 for DeepPPOContinuousAgent) as one enqueue-only
+ * call: gather the rows `indices` of the rollout, normalise the minibatch's advantages, actor
+ * forward / loss gradient (+ per-sample KL) / backward / global-norm clip / Adam (/ log_std
+ * clamp), and the same for the critic.  On return (in stream order) the parameter and optimiser
+ * buffers are updated in place and actor_grads / critic_grads hold the clipped gradients.
+ * continuous = 0: logits head, critic gradient 2 c_v (V - R) / MB; continuous = 1: StochasticActor
+ * head, critic gradient (V - R) / MB.  actor_t / critic_t are the optimisers' step counts after
+ * this step (Adam.t += 1 stays on the host, deep_rl/optimizer/adam.mojo:170).
+ * KL early stop (target_kl > 0): the mean KL is tested on the device; kl_flag is 4 int32 --
+ * [0] raised (and left raised) when a minibatch's mean KL exceeds target_kl, [1] bits of the
+ * last mean, [2] number of updates applied since the caller cleared it; once [0] is up the call
+ * still computes gradients but leaves parameters and optimiser state untouched, which is where
+ * the reference's `break` (ppo.mojo:2566-2573) leaves them. */
+typedef struct {
+    int32_t minibatch, obs_dim, act_width, continuous;
+    mrl_mlp_desc actor, critic;
+    float *actor_params, *critic_params;
+    float *actor_grads, *critic_grads;
+    float *actor_state, *critic_state;       /* Adam (m, v) interleaved, [P, 2] */
+    const float *r_obs, *r_actions, *r_log_probs, *r_values, *advantages, *returns; /* [T*N, ...] */
+    float *mb_obs, *mb_actions, *mb_adv, *mb_ret, *mb_logp, *mb_val;                /* [MB, ...] */
+    float *actor_out, *values, *g_actor_out, *g_values, *kl;
+    float *actor_cache, *critic_cache;       /* [MB * CACHE_SIZE] */
+    int32_t *kl_flag;                        /* [4], may be NULL when target_kl <= 0 */
+    float clip_epsilon, entropy_coef, value_loss_coef, max_grad_norm, target_kl;
+    int32_t clip_value, norm_adv_per_minibatch;
+    double actor_lr, critic_lr, beta1, beta2, eps;
+} mrl_update;
+
+int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int actor_t,
+                             int critic_t);
+/* n_minibatches consecutive minibatches of `indices` (a permutation of the rollout); minibatch k
+ * runs with step counts actor_t0 + k + 1 / critic_t0 + k + 1 */
+int mrl_ppo_update_epoch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int n_minibatches,
+                         int actor_t0, int critic_t0);
 
 #ifdef __cplusplus
 }

@@ -41,12 +41,27 @@ class Rollout(C.Structure):
     ]
 
 
+class Update(C.Structure):
+    _fields_ = (
+        [(n, C.c_int32) for n in ("minibatch", "obs_dim", "act_width", "continuous")]
+        + [("actor", MlpDesc), ("critic", MlpDesc)]
+        + [(n, C.c_void_p) for n in (
+            "actor_params", "critic_params", "actor_grads", "critic_grads", "actor_state", "critic_state",
+            "r_obs", "r_actions", "r_log_probs", "r_values", "advantages", "returns",
+            "mb_obs", "mb_actions", "mb_adv", "mb_ret", "mb_logp", "mb_val",
+            "actor_out", "values", "g_actor_out", "g_values", "kl", "actor_cache", "critic_cache", "kl_flag")]
+        + [(n, C.c_float) for n in ("clip_epsilon", "entropy_coef", "value_loss_coef", "max_grad_norm", "target_kl")]
+        + [(n, C.c_int32) for n in ("clip_value", "norm_adv_per_minibatch")]
+        + [(n, C.c_double) for n in ("actor_lr", "critic_lr", "beta1", "beta2", "eps")]
+    )
+
+
 class MrlError(RuntimeError):
     pass
 
 
 P, I, U32, U64, F, D = C.c_void_p, C.c_int, C.c_uint32, C.c_uint64, C.c_float, C.c_double
-DP, RP = C.POINTER(MlpDesc), C.POINTER(Rollout)
+DP, RP, UP = C.POINTER(MlpDesc), C.POINTER(Rollout), C.POINTER(Update)
 
 # name -> argtypes; every function returns int (0 = ok) unless listed in _SPECIAL
 SIGNATURES = {
@@ -84,6 +99,8 @@ SIGNATURES = {
     "mrl_policy_step_discrete": [P, DP, DP, I, P, P, P, U32, P, P, P, P, P],
     "mrl_policy_step_gaussian": [P, DP, DP, I, P, P, P, U32, P, P, P, P, P],
     "mrl_rollout_step": [P, RP, I, U32, U64, U64],
+    "mrl_ppo_update_minibatch": [P, UP, P, I, I],
+    "mrl_ppo_update_epoch": [P, UP, P, I, I, I],
 }
 _SPECIAL = {"mrl_version": (C.c_int, []), "mrl_last_error": (C.c_char_p, [])}
 # size queries return a count, not a status

@@ -17,6 +17,7 @@
 // 64 lanes of an MFMA operand read are consecutive words.
 #include "mrl_host.hpp"
 #include "mrl_device.hpp"
+#include "mlp3.hpp"
 
 namespace mrl {
 
@@ -291,13 +292,7 @@ static void launch_fwd(hipStream_t s, const float *X, int ldx, const float *W, c
                        M, K, N);
 }
 
-// fused three-layer path (mrl_mlp3.hip); MRL_E_UNSUPPORTED when the shape is not covered
-bool mlp3_fusable(const mrl_mlp_desc &d, int *H, int *act, bool *gauss);
-int mlp3_forward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *in, const float *params,
-                 float *out, float *cache);
-int mlp3_backward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *grad_out, const float *params,
-                  const float *cache, float *grads, float *ws);
-size_t mlp3_backward_ws(const mrl_mlp_desc &d, int batch);
+int mlp_ensure_ws(mrl_ctx *ctx, size_t floats, float **out) { return ensure_ws(ctx, floats, out); }
 
 }  // namespace mrl
 
@@ -384,7 +379,8 @@ int mrl_mlp_backward(mrl_ctx *ctx, const mrl_mlp_desc *d, int batch, const float
         bool fg;
         if (grad_in == nullptr && mlp3_fusable(*d, &fh, &fa, &fg)) {
             float *fws = nullptr;
-            rc = ensure_ws(ctx, mlp3_backward_ws(*d, batch), &fws);
+            const mrl_mlp_desc *ds[1] = {d};
+            rc = ensure_ws(ctx, mlp3_backward_ws(ds, 1, batch), &fws);
             if (rc) return rc;
             rc = mlp3_backward(ctx, *d, batch, grad_out, params, cache, grads, fws);
             if (rc != MRL_E_UNSUPPORTED) return rc;

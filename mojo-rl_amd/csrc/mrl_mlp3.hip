@@ -13,17 +13,25 @@
 #include "mrl_host.hpp"
 #include "mrl_device.hpp"
 #include "mlp_tile.hpp"
+#include "mlp3.hpp"
 
 namespace mrl {
 
-template <int H, int ACT, bool GAUSS>
-__global__ __launch_bounds__(H) void mlp3_fwd_kernel(const float *__restrict__ x, int B, int IN, int A,
-                                                     const float *__restrict__ params,
-                                                     float *__restrict__ out, float *__restrict__ cache) {
+// grid = (row tiles, nets): blockIdx.y picks the net, so that an actor and a critic that read the
+// same inputs go through the chip side by side
+template <int H, int ACT>
+__global__ __launch_bounds__(H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets nets) {
     __shared__ float xs[PR * XS_LD];
     __shared__ float hT[H * HT_LD];
     __shared__ float h2[PR * (H + 1)];
     __shared__ float ys[PR * (PA_MAX + 1)];
+    const Mlp3Net &nn = nets.n[blockIdx.y];
+    const float *__restrict__ x = nn.x;
+    const float *__restrict__ params = nn.params;
+    float *__restrict__ out = nn.out;
+    float *__restrict__ cache = nn.cache;
+    const int A = nn.A;
+    const bool GAUSS = nn.gauss != 0;
     const int t = threadIdx.x;
     const long row0 = (long)blockIdx.x * PR;
     const int nrow = (int)min((long)PR, B - row0);
@@ -70,13 +78,18 @@ MRL_DEV float act_deriv(float cached) {
 }
 
 // grad_out [B, ld] (ld = A, or 2A for the Gaussian head: mean gradients first); g1, g0 [B, H];
-// ls_part [tiles, A]: per-tile sums of the log_std gradient columns
-template <int H, int ACT, bool GAUSS>
-__global__ __launch_bounds__(H) void mlp3_bwd_dx_kernel(const float *__restrict__ grad_out, int B, int IN,
-                                                        int A, const float *__restrict__ params,
-                                                        const float *__restrict__ cache,
-                                                        float *__restrict__ g1, float *__restrict__ g0,
-                                                        float *__restrict__ ls_part) {
+// ls_part [tiles, A]: per-tile sums of the log_std gradient columns.  grid = (row tiles, nets).
+template <int H, int ACT>
+__global__ __launch_bounds__(H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3Nets nets) {
+    const Mlp3Net &nn = nets.n[blockIdx.y];
+    const float *__restrict__ grad_out = nn.grad_out;
+    const float *__restrict__ params = nn.params;
+    const float *__restrict__ cache = nn.cache;
+    float *__restrict__ g1 = nn.g1;
+    float *__restrict__ g0 = nn.g0;
+    float *__restrict__ ls_part = nn.ls_part;
+    const int A = nn.A;
+    const bool GAUSS = nn.gauss != 0;
     constexpr int KCH = 32;                       // k-chunk of W1 staged per round
     __shared__ float g2s[PR * (2 * PA_MAX + 1)];
     __shared__ float gT[H * HT_LD];               // g1 of the tile, k-major
@@ -163,15 +176,15 @@ struct DwProblem {
     int poff;         // offset of the layer in the flat parameter vector
     int tiles_n, tiles;   // tiles_n = ceil(N / 64); tiles = tiles_n * ceil((K + 1) / 64)
 };
-struct Dw3 { DwProblem p[3]; };
+struct DwSet { DwProblem p[6]; int n; };
 
-// grid.x = sum of the layers' tiles, grid.y = batch splits; partial[z][P]
-__global__ __launch_bounds__(256) void dw3_kernel(Dw3 d, int M, int rows_per_split, int P,
+// grid.x = sum of the problems' tiles, grid.y = batch splits; partial[z][P]
+__global__ __launch_bounds__(256) void dw3_kernel(DwSet d, int M, int rows_per_split, int P,
                                                   float *__restrict__ partial) {
     __shared__ float As[DKC * DLD];
     __shared__ float Bs[DKC * DLD];
     int tile = blockIdx.x, li = 0;
-    while (li < 2 && tile >= d.p[li].tiles) { tile -= d.p[li].tiles; ++li; }
+    while (li < d.n - 1 && tile >= d.p[li].tiles) { tile -= d.p[li].tiles; ++li; }
     const DwProblem &pr = d.p[li];
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wr = w >> 1, wc = w & 1;
     const int half = lane >> 5, l31 = lane & 31;
@@ -220,20 +233,29 @@ __global__ __launch_bounds__(256) void dw3_kernel(Dw3 d, int M, int rows_per_spl
 }
 
 // grads[i] = sum_z partial[z][i] for the [W | b] blocks; the log_std tail (Gaussian head) sums the
-// per-tile column sums of the backward-dx kernel
-__global__ __launch_bounds__(256) void sum3_kernel(const float *__restrict__ partial, int splits, int P,
-                                                   int n_wb, const float *__restrict__ ls_part, int tiles,
-                                                   int A, float *__restrict__ grads) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= P) return;
+// per-tile column sums of the backward-dx kernel.  The nets' vectors lie back to back in `partial`.
+struct SumNets {
+    float *grads[2];
+    const float *ls_part[2];
+    int P[2], n_wb[2], A[2];
+    int n;
+};
+
+__global__ __launch_bounds__(256) void sum3_kernel(const float *__restrict__ partial, int splits, int Ptot,
+                                                   int tiles, SumNets sn) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= Ptot) return;
+    const int gi = i;
+    int net = 0;
+    if (sn.n > 1 && i >= sn.P[0]) { net = 1; i -= sn.P[0]; }
     float s = 0.0f;
-    if (i < n_wb) {
-        for (int z = 0; z < splits; ++z) s += partial[(size_t)z * P + i];
+    if (i < sn.n_wb[net]) {
+        for (int z = 0; z < splits; ++z) s += partial[(size_t)z * Ptot + gi];
     } else {
-        const int j = i - n_wb;
-        for (int q = 0; q < tiles; ++q) s += ls_part[(size_t)q * A + j];
+        const int j = i - sn.n_wb[net];
+        for (int q = 0; q < tiles; ++q) s += sn.ls_part[net][(size_t)q * sn.A[net] + j];
     }
-    grads[i] = s;
+    sn.grads[net][i] = s;
 }
 
 // ---------------------------------------------------------------- host side
@@ -253,78 +275,142 @@ bool mlp3_fusable(const mrl_mlp_desc &d, int *H, int *act, bool *gauss) {
     return true;
 }
 
-int mlp3_forward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *in, const float *params,
-                 float *out, float *cache) {
+static int net_P(const mrl_mlp_desc &d) {
+    const int IN = d.layers[0].in_dim, H = d.layers[0].out_dim, A = d.layers[2].out_dim;
+    return (IN + 1) * H + (H + 1) * H + (H + 1) * A + (d.layers[2].kind == MRL_STOCHASTIC_ACTOR ? A : 0);
+}
+
+// true when the two nets can share launches: both fusable, same input width, width and activation
+bool mlp3_pair_fusable(const mrl_mlp_desc &a, const mrl_mlp_desc &b) {
+    int ha, hb, aa, ab;
+    bool ga, gb;
+    return mlp3_fusable(a, &ha, &aa, &ga) && mlp3_fusable(b, &hb, &ab, &gb) && ha == hb && aa == ab &&
+           a.layers[0].in_dim == b.layers[0].in_dim;
+}
+
+template <int H, int ACT>
+static void launch_fwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, int n_nets) {
+    dim3 grid((batch + PR - 1) / PR, n_nets);
+    hipLaunchKernelGGL((mlp3_fwd_kernel<H, ACT>), grid, dim3(H), 0, ctx->stream, batch, IN, nets);
+}
+template <int H, int ACT>
+static void launch_bwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, int n_nets) {
+    dim3 grid((batch + PR - 1) / PR, n_nets);
+    hipLaunchKernelGGL((mlp3_bwd_dx_kernel<H, ACT>), grid, dim3(H), 0, ctx->stream, batch, IN, nets);
+}
+
+// forward of one or two nets (descs[i], io.n[i]) in one launch
+int mlp3_forward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io) {
     int H = 0, act = 0;
     bool gauss = false;
-    if (!mlp3_fusable(d, &H, &act, &gauss)) return MRL_E_UNSUPPORTED;
-    const int IN = d.layers[0].in_dim, A = d.layers[2].out_dim;
-    dim3 grid((batch + PR - 1) / PR);
-#define MRL_F(HH, AA, GG)                                                                          \
-    hipLaunchKernelGGL((mlp3_fwd_kernel<HH, AA, GG>), grid, dim3(HH), 0, ctx->stream, in, batch, IN, A, \
-                       params, out, cache)
-#define MRL_F2(HH, AA) do { if (gauss) MRL_F(HH, AA, true); else MRL_F(HH, AA, false); } while (0)
-    if (H == 256 && act == 1) MRL_F2(256, 1);
-    else if (H == 256) MRL_F2(256, 2);
-    else if (act == 1) MRL_F2(64, 1);
-    else MRL_F2(64, 2);
-#undef MRL_F2
-#undef MRL_F
+    for (int i = 0; i < n_nets; ++i) {
+        if (!mlp3_fusable(*descs[i], &H, &act, &gauss)) return MRL_E_UNSUPPORTED;
+        io.n[i].A = descs[i]->layers[2].out_dim;
+        io.n[i].gauss = gauss ? 1 : 0;
+    }
+    if (n_nets == 2 && !mlp3_pair_fusable(*descs[0], *descs[1])) return MRL_E_UNSUPPORTED;
+    const int IN = descs[0]->layers[0].in_dim;
+    if (H == 256 && act == 1) launch_fwd_t<256, 1>(ctx, batch, IN, io, n_nets);
+    else if (H == 256) launch_fwd_t<256, 2>(ctx, batch, IN, io, n_nets);
+    else if (act == 1) launch_fwd_t<64, 1>(ctx, batch, IN, io, n_nets);
+    else launch_fwd_t<64, 2>(ctx, batch, IN, io, n_nets);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mlp3_forward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *in, const float *params,
+                 float *out, float *cache) {
+    Mlp3Nets io{};
+    io.n[0].x = in; io.n[0].params = params; io.n[0].out = out; io.n[0].cache = cache;
+    const mrl_mlp_desc *ds[1] = {&d};
+    return mlp3_forward_n(ctx, ds, 1, batch, io);
+}
+
+// floats of workspace mlp3_backward_n needs for these nets
+size_t mlp3_backward_ws(const mrl_mlp_desc *const *descs, int n_nets, int batch) {
+    size_t total = 0, P = 0;
+    for (int i = 0; i < n_nets; ++i) {
+        const int H = descs[i]->layers[0].out_dim;
+        total += (size_t)2 * batch * H + (size_t)((batch + PR - 1) / PR) * PA_MAX;
+        P += net_P(*descs[i]);
+    }
+    return total + (size_t)32 * P;
+}
+
+// backward (parameter gradients only) of one or two nets: io.n[i].grad_out / params / cache in,
+// grads[i] out; ws as sized by mlp3_backward_ws
+int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io,
+                    float *const *grads, float *ws) {
+    int H = 0, act = 0;
+    bool gauss = false;
+    for (int i = 0; i < n_nets; ++i) {
+        if (!mlp3_fusable(*descs[i], &H, &act, &gauss)) return MRL_E_UNSUPPORTED;
+        io.n[i].A = descs[i]->layers[2].out_dim;
+        io.n[i].gauss = gauss ? 1 : 0;
+        // the W1 rows are staged with 16-byte loads
+        const int IN = descs[i]->layers[0].in_dim;
+        if (reinterpret_cast<uintptr_t>(io.n[i].params + IN * H + H) % 16 != 0) return MRL_E_UNSUPPORTED;
+    }
+    if (n_nets == 2 && !mlp3_pair_fusable(*descs[0], *descs[1])) return MRL_E_UNSUPPORTED;
+    const int IN = descs[0]->layers[0].in_dim;
+    const int tiles = (batch + PR - 1) / PR;
+    int splits = std::max(1, std::min(32, batch / 128));
+    int rows_per = ((batch + splits - 1) / splits + DKC - 1) / DKC * DKC;
+    splits = (batch + rows_per - 1) / rows_per;
+    // workspace: per net g1 [B, H] | g0 [B, H] | ls_part [tiles, PA_MAX]; then partial [splits, Ptot]
+    float *w = ws;
+    for (int i = 0; i < n_nets; ++i) {
+        io.n[i].g1 = w; w += (size_t)batch * H;
+        io.n[i].g0 = w; w += (size_t)batch * H;
+        io.n[i].ls_part = w; w += (size_t)tiles * PA_MAX;
+    }
+    float *partial = w;
+    if (H == 256 && act == 1) launch_bwd_t<256, 1>(ctx, batch, IN, io, n_nets);
+    else if (H == 256) launch_bwd_t<256, 2>(ctx, batch, IN, io, n_nets);
+    else if (act == 1) launch_bwd_t<64, 1>(ctx, batch, IN, io, n_nets);
+    else launch_bwd_t<64, 2>(ctx, batch, IN, io, n_nets);
+    MRL_CHECK_LAUNCH();
+    DwSet dw;
+    dw.n = 3 * n_nets;
+    SumNets sn{};
+    sn.n = n_nets;
+    auto fill = [](DwProblem &p, const float *X, int xs, const float *G, int gs, int K, int N, int poff) {
+        p.X = X; p.G = G; p.xs = xs; p.gs = gs; p.K = K; p.N = N; p.poff = poff;
+        p.tiles_n = (N + DBN - 1) / DBN;
+        p.tiles = p.tiles_n * ((K + 1 + DBM - 1) / DBM);
+    };
+    int base = 0, total_tiles = 0;
+    for (int i = 0; i < n_nets; ++i) {
+        const Mlp3Net &nn = io.n[i];
+        const int A = nn.A;
+        const float *c0 = nn.cache, *c1 = c0 + (size_t)batch * (IN + H), *c2 = c1 + (size_t)batch * 2 * H;
+        fill(dw.p[3 * i + 0], c0, IN + H, nn.g0, H, IN, H, base);
+        fill(dw.p[3 * i + 1], c1, 2 * H, nn.g1, H, H, H, base + (IN + 1) * H);
+        fill(dw.p[3 * i + 2], c2, H, nn.grad_out, nn.gauss ? 2 * A : A, H, A, base + (IN + 1) * H + (H + 1) * H);
+        for (int q = 0; q < 3; ++q) total_tiles += dw.p[3 * i + q].tiles;
+        sn.grads[i] = grads[i];
+        sn.ls_part[i] = nn.ls_part;
+        sn.P[i] = net_P(*descs[i]);
+        sn.n_wb[i] = (IN + 1) * H + (H + 1) * H + (H + 1) * A;
+        sn.A[i] = A;
+        base += sn.P[i];
+    }
+    const int Ptot = base;
+    hipLaunchKernelGGL(dw3_kernel, dim3(total_tiles, splits), dim3(256), 0, ctx->stream, dw, batch, rows_per,
+                       Ptot, partial);
+    hipLaunchKernelGGL(sum3_kernel, dim3(grid_for(Ptot, 256)), dim3(256), 0, ctx->stream, partial, splits,
+                       Ptot, tiles, sn);
     MRL_CHECK_LAUNCH();
     return MRL_OK;
 }
 
 int mlp3_backward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *grad_out, const float *params,
                   const float *cache, float *grads, float *ws) {
-    int H = 0, act = 0;
-    bool gauss = false;
-    if (!mlp3_fusable(d, &H, &act, &gauss)) return MRL_E_UNSUPPORTED;
-    const int IN = d.layers[0].in_dim, A = d.layers[2].out_dim;
-    // the W1 rows are staged with 16-byte loads
-    if (reinterpret_cast<uintptr_t>(params + IN * H + H) % 16 != 0) return MRL_E_UNSUPPORTED;
-    const int tiles = (batch + PR - 1) / PR;
-    const int n_wb = (IN + 1) * H + (H + 1) * H + (H + 1) * A;
-    const int P = n_wb + (gauss ? A : 0);
-    int splits = std::max(1, std::min(32, batch / 128));
-    int rows_per = ((batch + splits - 1) / splits + DKC - 1) / DKC * DKC;
-    splits = (batch + rows_per - 1) / rows_per;
-    // workspace: g1 [B, H] | g0 [B, H] | ls_part [tiles, A] | partial [splits, P]
-    float *g1 = ws, *g0 = g1 + (size_t)batch * H, *ls_part = g0 + (size_t)batch * H;
-    float *partial = ls_part + (size_t)tiles * PA_MAX;
-#define MRL_B(HH, AA, GG)                                                                               \
-    hipLaunchKernelGGL((mlp3_bwd_dx_kernel<HH, AA, GG>), dim3(tiles), dim3(HH), 0, ctx->stream, grad_out,    \
-                       batch, IN, A, params, cache, g1, g0, ls_part)
-#define MRL_B2(HH, AA) do { if (gauss) MRL_B(HH, AA, true); else MRL_B(HH, AA, false); } while (0)
-    if (H == 256 && act == 1) MRL_B2(256, 1);
-    else if (H == 256) MRL_B2(256, 2);
-    else if (act == 1) MRL_B2(64, 1);
-    else MRL_B2(64, 2);
-#undef MRL_B2
-#undef MRL_B
-    MRL_CHECK_LAUNCH();
-    const float *c0 = cache, *c1 = cache + (size_t)batch * (IN + H), *c2 = c1 + (size_t)batch * 2 * H;
-    Dw3 dw;
-    auto fill = [](DwProblem &p, const float *X, int xs, const float *G, int gs, int K, int N, int poff) {
-        p.X = X; p.G = G; p.xs = xs; p.gs = gs; p.K = K; p.N = N; p.poff = poff;
-        p.tiles_n = (N + DBN - 1) / DBN;
-        p.tiles = p.tiles_n * ((K + 1 + DBM - 1) / DBM);
-    };
-    fill(dw.p[0], c0, IN + H, g0, H, IN, H, 0);
-    fill(dw.p[1], c1, 2 * H, g1, H, H, H, (IN + 1) * H);
-    fill(dw.p[2], c2, H, grad_out, gauss ? 2 * A : A, H, A, (IN + 1) * H + (H + 1) * H);
-    dim3 gdw(dw.p[0].tiles + dw.p[1].tiles + dw.p[2].tiles, splits);
-    hipLaunchKernelGGL(dw3_kernel, gdw, dim3(256), 0, ctx->stream, dw, batch, rows_per, P, partial);
-    hipLaunchKernelGGL(sum3_kernel, dim3(grid_for(P, 256)), dim3(256), 0, ctx->stream, partial, splits, P,
-                       n_wb, ls_part, tiles, A, grads);
-    MRL_CHECK_LAUNCH();
-    return MRL_OK;
-}
-
-// floats of workspace mlp3_backward needs
-size_t mlp3_backward_ws(const mrl_mlp_desc &d, int batch) {
-    const int H = d.layers[0].out_dim, IN = d.layers[0].in_dim, A = d.layers[2].out_dim;
-    const size_t P = (size_t)(IN + 1) * H + (size_t)(H + 1) * H + (size_t)(H + 1) * A + A;
-    return (size_t)2 * batch * H + (size_t)((batch + PR - 1) / PR) * PA_MAX + (size_t)32 * P;
+    Mlp3Nets io{};
+    io.n[0].grad_out = grad_out; io.n[0].params = params; io.n[0].cache = const_cast<float *>(cache);
+    const mrl_mlp_desc *ds[1] = {&d};
+    float *gs[1] = {grads};
+    return mlp3_backward_n(ctx, ds, 1, batch, io, gs, ws);
 }
 
 }  // namespace mrl

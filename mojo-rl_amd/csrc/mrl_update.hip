@@ -1,0 +1,255 @@
+// One PPO minibatch update -- the body of the minibatch loop of train_gpu
+// (deep_agents/ppo/ppo.mojo:2438-2727, deep_agents/ppo/ppo_continuous.mojo:3000-3260) -- as one
+// call that only enqueues: gather, per-minibatch advantage normalisation, actor and critic
+// forward, loss gradients, KL test, backward, global-norm clip, Adam (and the log_std clamp).
+// The actor and the critic do not depend on each other inside a minibatch, so when both have one
+// of the fused shapes every stage runs them side by side in ONE launch: 11 launches per
+// minibatch instead of about 40, and twice the workgroups per launch.
+//
+// KL early stop: the reference copies the per-sample KL to the host after the actor's loss
+// gradient and breaks out of the minibatch and epoch loops when its mean exceeds target_kl.
+// Here the mean is tested on the device (kl_flag[0] is raised and stays raised) and the kernel
+// that applies the update does nothing once the flag is up: the parameters end exactly where
+// the reference's break leaves them, without a host round trip.  kl_flag[2] counts the updates
+// that were applied, for the host's optimiser step counters.
+#include "mrl_host.hpp"
+#include "mrl_device.hpp"
+#include "mlp3.hpp"
+
+namespace mrl {
+
+constexpr int UTPB = 256;
+
+MRL_DEV float u_wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+template <int NW>
+MRL_DEV float u_block_sum(float v, float *smem) {
+    v = u_wave_sum(v);
+    if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NW; ++k) t += smem[k];
+    __syncthreads();
+    return t;
+}
+
+// (x - mean) / (sqrt(var + 1e-8) + 1e-8) over one minibatch in a single workgroup
+// (deep_agents/ppo/kernels.mojo:507-599 is a single-block kernel as well)
+__global__ __launch_bounds__(1024) void normalize_small_kernel(float *__restrict__ x, int n) {
+    __shared__ float smem[16];
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 1024) s += x[i];
+    const float mean = u_block_sum<16>(s, smem) / (float)n;
+    float q = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        const float d = x[i] - mean;
+        q += d * d;
+    }
+    const float variance = u_block_sum<16>(q, smem) / (float)n;
+    const float std = sqrtf(variance + 1e-8f);
+    for (int i = threadIdx.x; i < n; i += 1024) x[i] = (x[i] - mean) / (std + 1e-8f);
+}
+
+struct AdamNet {
+    float *p, *g;
+    float2 *state;
+    int n;
+    float lr, bc1, bc2;
+    int clamp_off, clamp_n;   // log_std slice to clamp to [-5, 2] after the step (clamp_n = 0: none)
+};
+struct AdamNets { AdamNet n[2]; };
+
+// partial[net][block] = sum of g^2 over the block's grid-stride slice; grid = (nb, nets)
+__global__ __launch_bounds__(UTPB) void sq_partial2_kernel(AdamNets nets, float *__restrict__ partial) {
+    __shared__ float smem[4];
+    const AdamNet &a = nets.n[blockIdx.y];
+    float s = 0.0f;
+    for (long i = (long)blockIdx.x * UTPB + threadIdx.x; i < a.n; i += (long)gridDim.x * UTPB) s += a.g[i] * a.g[i];
+    s = u_block_sum<4>(s, smem);
+    if (threadIdx.x == 0) partial[blockIdx.y * gridDim.x + blockIdx.x] = s;
+}
+
+// global-norm clip (ppo.mojo:382-534; actor and critic separately) + Adam (adam.mojo:52-105)
+// + log_std clamp (kernels.mojo:842-873); grid = (blocks, nets).  Does nothing once stop[0] != 0.
+__global__ __launch_bounds__(UTPB) void clip_adam2_kernel(AdamNets nets, const float *__restrict__ partial,
+                                                          int nb, float max_norm, float beta1, float beta2,
+                                                          float omb1, float omb2, float eps,
+                                                          int32_t *__restrict__ stop) {
+    __shared__ float smem[4];
+    __shared__ float scale_s;
+    if (stop != nullptr && stop[0] != 0) return;
+    const AdamNet &a = nets.n[blockIdx.y];
+    float scale = 1.0f;
+    if (max_norm > 0.0f) {
+        float s = 0.0f;
+        for (int i = threadIdx.x; i < nb; i += UTPB) s += partial[blockIdx.y * nb + i];
+        s = u_block_sum<4>(s, smem);
+        if (threadIdx.x == 0) {
+            const float norm = sqrtf(s);
+            scale_s = norm > max_norm ? max_norm / (norm + 1e-8f) : 1.0f;
+        }
+        __syncthreads();
+        scale = scale_s;
+    }
+    if (stop != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) stop[2] = stop[2] + 1;
+    const int i = blockIdx.x * UTPB + threadIdx.x;
+    if (i >= a.n) return;
+    const float gi = a.g[i] * scale;
+    a.g[i] = gi;
+    const float2 mv = a.state[i];
+    const float m_new = beta1 * mv.x + omb1 * gi;
+    const float v_new = beta2 * mv.y + omb2 * gi * gi;
+    a.state[i] = make_float2(m_new, v_new);
+    const float m_hat = m_new / a.bc1, v_hat = v_new / a.bc2;
+    float p = a.p[i] - a.lr * m_hat / (sqrtf(v_hat) + eps);
+    if (i >= a.clamp_off && i < a.clamp_off + a.clamp_n) {
+        if (p < -5.0f) p = -5.0f;
+        else if (p > 2.0f) p = 2.0f;
+    }
+    a.p[i] = p;
+}
+
+}  // namespace mrl
+
+using namespace mrl;
+
+extern "C" {
+
+static int update_check(const mrl_update *u, const char *who) {
+    MRL_CHECK_ARG(u != nullptr, "%s: descriptor is NULL", who);
+    MRL_CHECK_ARG(u->minibatch > 0 && u->obs_dim > 0 && u->act_width > 0, "%s: bad sizes", who);
+    MRL_CHECK_ARG(u->actor_params && u->critic_params && u->actor_grads && u->critic_grads && u->actor_state &&
+                      u->critic_state, "%s: NULL parameter / gradient / optimiser buffer", who);
+    MRL_CHECK_ARG(u->r_obs && u->r_actions && u->r_log_probs && u->r_values && u->advantages && u->returns,
+                  "%s: NULL rollout buffer", who);
+    MRL_CHECK_ARG(u->mb_obs && u->mb_actions && u->mb_adv && u->mb_ret && u->mb_logp && u->mb_val &&
+                      u->actor_out && u->values && u->g_actor_out && u->g_values && u->kl && u->actor_cache &&
+                      u->critic_cache, "%s: NULL minibatch buffer", who);
+    MRL_CHECK_ARG(u->target_kl <= 0.0f || u->kl_flag != nullptr, "%s: target_kl needs kl_flag", who);
+    const int head = mrl_mlp_out_dim(&u->actor);
+    MRL_CHECK_ARG(head > 0 && mrl_mlp_out_dim(&u->critic) == 1, "%s: bad actor / critic description", who);
+    const bool gauss = u->actor.layers[u->actor.n_layers - 1].kind == MRL_STOCHASTIC_ACTOR;
+    MRL_CHECK_ARG(gauss == (u->continuous != 0), "%s: a continuous agent needs a StochasticActor head (and only it)",
+                  who);
+    MRL_CHECK_ARG(!gauss || head == 2 * u->act_width, "%s: act_width does not match the actor head", who);
+    MRL_CHECK_ARG(gauss || u->act_width == 1, "%s: a discrete agent stores one float per action", who);
+    MRL_CHECK_ARG(u->actor.layers[0].in_dim == u->obs_dim && u->critic.layers[0].in_dim == u->obs_dim,
+                  "%s: nets do not read obs_dim inputs", who);
+    return MRL_OK;
+}
+
+int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int actor_t,
+                             int critic_t) {
+    MRL_CHECK_ARG(ctx != nullptr, "mrl_ppo_update_minibatch: ctx is NULL");
+    int rc = update_check(u, "mrl_ppo_update_minibatch");
+    if (rc) return rc;
+    MRL_CHECK_ARG(indices != nullptr && actor_t >= 1 && critic_t >= 1,
+                  "mrl_ppo_update_minibatch: need indices and step counts >= 1");
+    const int mb = u->minibatch, head = mrl_mlp_out_dim(&u->actor);
+    const int Pa = mrl_mlp_param_size(&u->actor), Pc = mrl_mlp_param_size(&u->critic);
+    const bool cont = u->continuous != 0;
+
+    rc = mrl_gather_minibatch(ctx, indices, mb, u->obs_dim, u->act_width, u->r_obs, u->r_actions, u->advantages,
+                              u->returns, u->r_log_probs, u->r_values, u->mb_obs, u->mb_actions, u->mb_adv,
+                              u->mb_ret, u->mb_logp, u->mb_val);
+    if (rc) return rc;
+    if (u->norm_adv_per_minibatch) {
+        if (mb <= 65536) {
+            hipLaunchKernelGGL(normalize_small_kernel, dim3(1), dim3(1024), 0, ctx->stream, u->mb_adv, mb);
+            MRL_CHECK_LAUNCH();
+        } else {
+            rc = mrl_normalize_advantages(ctx, u->mb_adv, mb);
+            if (rc) return rc;
+        }
+    }
+
+    const mrl_mlp_desc *descs[2] = {&u->actor, &u->critic};
+    const bool paired = mlp3_pair_fusable(u->actor, u->critic) &&
+                        reinterpret_cast<uintptr_t>(u->actor_params) % 16 == 0 &&
+                        reinterpret_cast<uintptr_t>(u->critic_params) % 16 == 0;
+    Mlp3Nets io{};
+    io.n[0].x = u->mb_obs; io.n[0].params = u->actor_params; io.n[0].out = u->actor_out; io.n[0].cache = u->actor_cache;
+    io.n[1].x = u->mb_obs; io.n[1].params = u->critic_params; io.n[1].out = u->values; io.n[1].cache = u->critic_cache;
+    if (paired) {
+        rc = mlp3_forward_n(ctx, descs, 2, mb, io);
+        if (rc) return rc;
+    } else {
+        rc = mrl_mlp_forward(ctx, &u->actor, mb, u->mb_obs, u->actor_params, u->actor_out, u->actor_cache);
+        if (rc) return rc;
+        rc = mrl_mlp_forward(ctx, &u->critic, mb, u->mb_obs, u->critic_params, u->values, u->critic_cache);
+        if (rc) return rc;
+    }
+
+    if (cont)
+        rc = mrl_ppo_actor_grad_gaussian(ctx, u->actor_out, u->mb_logp, u->mb_adv, u->mb_actions, mb, u->act_width,
+                                         u->clip_epsilon, u->entropy_coef, u->g_actor_out, u->kl);
+    else
+        rc = mrl_ppo_actor_grad_discrete(ctx, u->actor_out, u->mb_logp, u->mb_adv, u->mb_actions, mb, head,
+                                         u->clip_epsilon, u->entropy_coef, u->g_actor_out, u->kl);
+    if (rc) return rc;
+    if (u->target_kl > 0.0f) {
+        rc = mrl_kl_check(ctx, u->kl, mb, u->target_kl, u->kl_flag);
+        if (rc) return rc;
+    }
+    rc = mrl_ppo_critic_grad(ctx, u->values, u->clip_value ? u->mb_val : nullptr, u->mb_ret, mb, cont ? 1 : 0,
+                             u->clip_value ? 1 : 0, u->value_loss_coef, u->clip_epsilon, u->g_values);
+    if (rc) return rc;
+
+    io.n[0].grad_out = u->g_actor_out;
+    io.n[1].grad_out = u->g_values;
+    float *grads[2] = {u->actor_grads, u->critic_grads};
+    if (paired) {
+        float *ws = nullptr;
+        rc = mlp_ensure_ws(ctx, mlp3_backward_ws(descs, 2, mb), &ws);
+        if (rc) return rc;
+        rc = mlp3_backward_n(ctx, descs, 2, mb, io, grads, ws);
+        if (rc) return rc;
+    } else {
+        rc = mrl_mlp_backward(ctx, &u->actor, mb, u->g_actor_out, u->actor_params, u->actor_cache, u->actor_grads,
+                              nullptr);
+        if (rc) return rc;
+        rc = mrl_mlp_backward(ctx, &u->critic, mb, u->g_values, u->critic_params, u->critic_cache, u->critic_grads,
+                              nullptr);
+        if (rc) return rc;
+    }
+
+    AdamNets an{};
+    auto fill = [&](AdamNet &a, float *p, float *g, float *st, int n, double lr, int t) {
+        a.p = p; a.g = g; a.state = reinterpret_cast<float2 *>(st); a.n = n; a.lr = (float)lr;
+        // bias corrections in fp64 then rounded, as the host code of the reference does
+        a.bc1 = (float)(1.0 - pow(u->beta1, (double)t));
+        a.bc2 = (float)(1.0 - pow(u->beta2, (double)t));
+        a.clamp_off = 0; a.clamp_n = 0;
+    };
+    fill(an.n[0], u->actor_params, u->actor_grads, u->actor_state, Pa, u->actor_lr, actor_t);
+    fill(an.n[1], u->critic_params, u->critic_grads, u->critic_state, Pc, u->critic_lr, critic_t);
+    if (cont) { an.n[0].clamp_off = Pa - u->act_width; an.n[0].clamp_n = u->act_width; }
+    const int nmax = std::max(Pa, Pc);
+    const int nb = std::min(256, grid_for(nmax, UTPB));
+    float *part = ctx->reduce_scratch + 1024;   // [2][nb], nb <= 256
+    if (u->max_grad_norm > 0.0f)
+        hipLaunchKernelGGL(sq_partial2_kernel, dim3(nb, 2), dim3(UTPB), 0, ctx->stream, an, part);
+    hipLaunchKernelGGL(clip_adam2_kernel, dim3(grid_for(nmax, UTPB), 2), dim3(UTPB), 0, ctx->stream, an, part, nb,
+                       u->max_grad_norm, (float)u->beta1, (float)u->beta2, (float)(1.0 - u->beta1),
+                       (float)(1.0 - u->beta2), (float)u->eps, u->target_kl > 0.0f ? u->kl_flag : nullptr);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_ppo_update_epoch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int n_minibatches,
+                         int actor_t0, int critic_t0) {
+    MRL_CHECK_ARG(ctx != nullptr && u != nullptr, "mrl_ppo_update_epoch: NULL argument");
+    MRL_CHECK_ARG(n_minibatches >= 0 && actor_t0 >= 0 && critic_t0 >= 0, "mrl_ppo_update_epoch: negative count");
+    for (int k = 0; k < n_minibatches; ++k) {
+        int rc = mrl_ppo_update_minibatch(ctx, u, indices + (size_t)k * u->minibatch, actor_t0 + k + 1,
+                                          critic_t0 + k + 1);
+        if (rc) return rc;
+    }
+    return MRL_OK;
+}
+
+}  // extern "C"

@@ -163,23 +163,23 @@ class PPOUpdate:
     """Phases 2 and 3 of train_gpu (deep_agents/ppo/ppo.mojo:2296-2727 for the discrete agent,
     ppo_continuous.mojo:2852-3260 for the continuous one) on device buffers: bootstrap value,
     optional reward normalisation, GAE, advantage normalisation, then epochs of shuffled
-    minibatches, each running actor forward / loss gradient / backward / clip / Adam
-    (/ log_std clamp) and the same for the critic.  Nothing is copied to the host inside an
-    epoch: the KL early-stop test runs on the device after every minibatch and its flag is read
-    once per epoch (kl_sync_every_minibatch=True reads it after every minibatch and stops before
-    that minibatch's update, as the reference does)."""
+    minibatches, each one library call (mrl_ppo_update_minibatch / _epoch) that runs actor and
+    critic forward / loss gradient / backward / clip / Adam (/ log_std clamp).  Nothing is copied
+    to the host inside an epoch: the KL early-stop test runs on the device after every actor
+    loss gradient, an update is not applied once it has fired (the reference's `break`), and
+    the flag is read once per epoch."""
 
     def __init__(self, ctx, rb, minibatch, actor_opt, critic_opt, gamma=0.99, gae_lambda=0.95,
                  clip_epsilon=0.2, entropy_coef=0.01, value_loss_coef=0.5, max_grad_norm=0.5,
                  clip_value=True, normalize_advantages=True, norm_adv_per_minibatch=True,
-                 target_kl=0.015, normalize_rewards=False, kl_sync_every_minibatch=False):
+                 target_kl=0.015, normalize_rewards=False):
         self.ctx, self.rb, self.mb = ctx, rb, minibatch
         self.actor_opt, self.critic_opt = actor_opt, critic_opt
         self.gamma, self.gae_lambda = gamma, gae_lambda
         self.clip_epsilon, self.entropy_coef, self.value_loss_coef = clip_epsilon, entropy_coef, value_loss_coef
         self.max_grad_norm, self.clip_value = max_grad_norm, clip_value
         self.normalize_advantages, self.norm_adv_per_minibatch = normalize_advantages, norm_adv_per_minibatch
-        self.target_kl, self.kl_sync_every_minibatch = target_kl, kl_sync_every_minibatch
+        self.target_kl = target_kl
         self.continuous = rb.continuous
         self.reward_rms = RunningMeanStd(ctx) if normalize_rewards else None
         dev = ctx.device
@@ -193,17 +193,15 @@ class PPOUpdate:
         self.mb_adv, self.mb_ret, self.mb_logp, self.mb_val = z(minibatch), z(minibatch), z(minibatch), z(minibatch)
         self.actor_out, self.values = z(minibatch * head), z(minibatch)
         self.g_actor_out, self.g_values, self.kl = z(minibatch * head), z(minibatch), z(minibatch)
-        self.kl_flag = torch.zeros(2, dtype=torch.int32, device=dev)
+        self.kl_flag = torch.zeros(4, dtype=torch.int32, device=dev)
         self.actor_cache = z(minibatch * rb.actor.CACHE_SIZE)
         self.critic_cache = z(minibatch * rb.critic.CACHE_SIZE)
         self.actor_grads, self.critic_grads = z(rb.actor.PARAM_SIZE), z(rb.critic.PARAM_SIZE)
         self.actor_state, self.critic_state = z(2 * rb.actor.PARAM_SIZE), z(2 * rb.critic.PARAM_SIZE)
         self.indices = torch.zeros(total, dtype=torch.int32, device=dev)
-        if self.continuous:
-            a = rb.env.ACTION_DIM
-            self.log_std_offset = rb.actor.PARAM_SIZE - a
+        self._t_base = (actor_opt.t, critic_opt.t)
 
-    # compatibility names used by callers written against the discrete agent
+    # names used by callers written against the discrete agent
     @property
     def logits(self):
         return self.actor_out
@@ -211,6 +209,33 @@ class PPOUpdate:
     @property
     def g_logits(self):
         return self.g_actor_out
+
+    def descriptor(self):
+        """The mrl_update view of this object (buffers, hyper-parameters, current learning rates)."""
+        rb, u = self.rb, _lib.Update()
+        u.minibatch, u.obs_dim, u.act_width = self.mb, rb.env.OBS_DIM, rb.act_width
+        u.continuous = 1 if self.continuous else 0
+        u.actor, u.critic = rb.actor.desc, rb.critic.desc
+        for name, t in (("actor_params", rb.actor_params), ("critic_params", rb.critic_params),
+                        ("actor_grads", self.actor_grads), ("critic_grads", self.critic_grads),
+                        ("actor_state", self.actor_state), ("critic_state", self.critic_state),
+                        ("r_obs", rb.r_obs), ("r_actions", rb.r_actions), ("r_log_probs", rb.r_log_probs),
+                        ("r_values", rb.r_values), ("advantages", self.advantages), ("returns", self.returns),
+                        ("mb_obs", self.mb_obs), ("mb_actions", self.mb_actions), ("mb_adv", self.mb_adv),
+                        ("mb_ret", self.mb_ret), ("mb_logp", self.mb_logp), ("mb_val", self.mb_val),
+                        ("actor_out", self.actor_out), ("values", self.values),
+                        ("g_actor_out", self.g_actor_out), ("g_values", self.g_values), ("kl", self.kl),
+                        ("actor_cache", self.actor_cache), ("critic_cache", self.critic_cache),
+                        ("kl_flag", self.kl_flag)):
+            setattr(u, name, _ptr(t))
+        u.clip_epsilon, u.entropy_coef, u.value_loss_coef = self.clip_epsilon, self.entropy_coef, self.value_loss_coef
+        u.max_grad_norm, u.target_kl = self.max_grad_norm, self.target_kl
+        u.clip_value, u.norm_adv_per_minibatch = int(self.clip_value), int(self.norm_adv_per_minibatch)
+        a, c = self.actor_opt, self.critic_opt
+        if (a.beta1, a.beta2, a.eps) != (c.beta1, c.beta2, c.eps):
+            raise _lib.MrlError("actor and critic optimisers must share beta1, beta2 and eps")
+        u.actor_lr, u.critic_lr, u.beta1, u.beta2, u.eps = a.lr, c.lr, a.beta1, a.beta2, a.eps
+        return u
 
     def compute_advantages(self):
         rb, ctx = self.rb, self.ctx
@@ -223,47 +248,30 @@ class PPOUpdate:
         if self.normalize_advantages:
             normalize_advantages(ctx, self.advantages)
 
-    def actor_half(self, indices):
-        """gather -> (normalise) -> actor forward -> loss gradient + KL -> device KL test."""
-        rb, ctx = self.rb, self.ctx
-        gather_minibatch(ctx, indices,
-                         (rb.r_obs, rb.r_actions, self.advantages, self.returns, rb.r_log_probs, rb.r_values),
-                         (self.mb_obs, self.mb_actions, self.mb_adv, self.mb_ret, self.mb_logp, self.mb_val),
-                         rb.env.OBS_DIM, rb.act_width)
-        if self.norm_adv_per_minibatch:
-            normalize_advantages(ctx, self.mb_adv)
-        rb.actor.forward_gpu_ws(ctx, self.actor_out, self.mb_obs, rb.actor_params, self.actor_cache)
-        grad = ppo_continuous_actor_grad if self.continuous else ppo_actor_grad_with_kl
-        grad(ctx, self.g_actor_out, self.kl, self.actor_out, self.mb_logp, self.mb_adv, self.mb_actions,
-             self.clip_epsilon, self.entropy_coef)
-        if self.target_kl > 0.0:
-            kl_check(ctx, self.kl, self.target_kl, self.kl_flag)
-
-    def update_half(self):
-        rb, ctx = self.rb, self.ctx
-        rb.actor.backward_gpu_ws(ctx, None, self.g_actor_out, rb.actor_params, self.actor_cache, self.actor_grads)
-        if self.max_grad_norm > 0.0:
-            clip_grad_norm(ctx, self.actor_grads, self.max_grad_norm)
-        self.actor_opt.step_gpu(ctx, rb.actor_params, self.actor_grads, self.actor_state)
-        if self.continuous:
-            clamp_log_std_params(ctx, rb.actor_params, self.log_std_offset, rb.env.ACTION_DIM)
-        rb.critic.forward_gpu_ws(ctx, self.values, self.mb_obs, rb.critic_params, self.critic_cache)
-        ppo_critic_grad(ctx, self.g_values, self.values, self.mb_ret, self.value_loss_coef,
-                        self.mb_val if self.clip_value else None, self.clip_epsilon,
-                        continuous=self.continuous)
-        rb.critic.backward_gpu_ws(ctx, None, self.g_values, rb.critic_params, self.critic_cache, self.critic_grads)
-        if self.max_grad_norm > 0.0:
-            clip_grad_norm(ctx, self.critic_grads, self.max_grad_norm)
-        self.critic_opt.step_gpu(ctx, rb.critic_params, self.critic_grads, self.critic_state)
+    def reset_kl(self):
+        """Clears the device flag and the applied-update counter (start of an update phase)."""
+        self.kl_flag.zero_()
+        self._t_base = (self.actor_opt.t, self.critic_opt.t)
 
     def minibatch_step(self, indices):
-        self.actor_half(indices)
-        self.update_half()
+        if indices.dtype != torch.int32 or indices.numel() != self.mb:
+            raise _lib.MrlError("minibatch_step needs %d int32 indices" % self.mb)
+        u = self.descriptor()
+        _lib.call("mrl_ppo_update_minibatch", self.ctx.handle, C.byref(u), _ptr(indices),
+                  self.actor_opt.t + 1, self.critic_opt.t + 1)
+        self.actor_opt.t += 1
+        self.critic_opt.t += 1
 
     def kl_stopped(self):
-        """Reads the device flag (one synchronising copy of 8 bytes): (stopped, last mean KL)."""
+        """Reads the device flag (one synchronising copy of 16 bytes): (stopped, last mean KL).
+        When the stop has fired the optimisers' step counters are set to the updates applied."""
         f = self.kl_flag.cpu()
-        return bool(f[0].item()), float(f[1:2].view(torch.float32).item())
+        stopped = bool(f[0].item())
+        if stopped:
+            applied = int(f[2].item())
+            self.actor_opt.t = self._t_base[0] + applied
+            self.critic_opt.t = self._t_base[1] + applied
+        return stopped, float(f[1:2].view(torch.float32).item())
 
     def run_epoch(self, permutation_or_seed):
         """permutation_or_seed: an int32 device tensor over the T*N samples, or an int seed from
@@ -274,18 +282,20 @@ class PPOUpdate:
             perm = self.indices
         else:
             perm = permutation_or_seed
-        n_mb = self.total // self.mb
-        for k in range(n_mb):
-            self.actor_half(perm[k * self.mb:(k + 1) * self.mb])
-            if self.target_kl > 0.0 and self.kl_sync_every_minibatch and self.kl_stopped()[0]:
-                break
-            self.update_half()
+            if perm.dtype != torch.int32:
+                raise _lib.MrlError("permutation must be int32")
+        n_mb = min(self.total, perm.numel()) // self.mb
+        u = self.descriptor()
+        _lib.call("mrl_ppo_update_epoch", self.ctx.handle, C.byref(u), _ptr(perm), n_mb,
+                  self.actor_opt.t, self.critic_opt.t)
+        self.actor_opt.t += n_mb
+        self.critic_opt.t += n_mb
         return self.kl_stopped() if self.target_kl > 0.0 else (False, 0.0)
 
     def update(self, num_epochs, seed=0):
         """compute_advantages + up to num_epochs epochs; stops after the epoch in which the KL
         flag was raised.  Returns the number of epochs run."""
-        self.kl_flag.zero_()
+        self.reset_kl()
         self.compute_advantages()
         for epoch in range(num_epochs):
             stopped, _ = self.run_epoch(int(seed) * 1000003 + epoch)

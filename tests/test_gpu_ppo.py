@@ -469,7 +469,8 @@ def test_init_uniform_and_network(mrl, orc, ctx):
     assert np.all(a[-6:] == np.float32(-0.5))
 
 
-def test_continuous_update_minibatch_against_oracle(mrl, orc, orcmod, ctx):
+@pytest.mark.parametrize("H", [64, 128])     # 64: actor and critic share fused launches; 128: layer-by-layer path
+def test_continuous_update_minibatch_against_oracle(mrl, orc, orcmod, ctx, H):
     """One ContinuousUpdate minibatch (gather, per-minibatch normalisation, actor forward, Gaussian
     loss gradient, backward, clip, Adam, log_std clamp, critic forward, gradient, backward, clip,
     Adam) against the same sequence on the oracle."""
@@ -477,7 +478,6 @@ def test_continuous_update_minibatch_against_oracle(mrl, orc, orcmod, ctx):
     N, T, MB = 64, 8, 256
     E = mrl.HalfCheetahPlanarV2
     od, A = E.OBS_DIM, E.ACTION_DIM
-    H = 64
     actor = mrl.seq(mrl.LinearTanh(od, H), mrl.LinearTanh(H, H), mrl.StochasticActor(H, A))
     critic = mrl.seq(mrl.LinearTanh(od, H), mrl.LinearTanh(H, H), mrl.Linear(H, 1))
     la = orcmod.layers([(2, od, H), (2, H, H), (3, H, A)])
@@ -523,7 +523,9 @@ def test_continuous_update_minibatch_against_oracle(mrl, orc, orcmod, ctx):
     orc.orc_clamp_log_std(ap2, ap2.size - A, A)
     np.testing.assert_allclose(h(upd.kl), kl, rtol=1e-3, atol=1e-5)
     np.testing.assert_allclose(h(upd.actor_grads), ga, rtol=1e-3, atol=1e-6)
-    np.testing.assert_allclose(h(rb.actor_params), ap2, rtol=1e-5, atol=2e-6)
+    # the first Adam step is lr * g / (|g| + eps): for a gradient entry near eps = 1e-8 the step
+    # follows the entry's absolute rounding error, so parameters are compared to a few % of lr
+    np.testing.assert_allclose(h(rb.actor_params), ap2, rtol=1e-5, atol=0.03 * 3e-4)
     ccache = np.zeros(MB * critic.CACHE_SIZE, np.float32)
     v = np.zeros((MB, 1), np.float32)
     orc.orc_mlp_forward(lc, 3, MB, mo, cp, v, ccache.ctypes.data)
@@ -536,7 +538,7 @@ def test_continuous_update_minibatch_against_oracle(mrl, orc, orcmod, ctx):
     cp2 = cp.copy()
     orc.orc_adam_step(cp2, gc, st, gc.size, 1, 1e-3, 0.9, 0.999, 1e-8)
     np.testing.assert_allclose(h(upd.critic_grads), gc, rtol=1e-3, atol=1e-6)
-    np.testing.assert_allclose(h(rb.critic_params), cp2, rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(h(rb.critic_params), cp2, rtol=1e-5, atol=0.03 * 1e-3)
 
 
 def test_update_driver_runs_epochs_and_stops_on_kl(mrl, ctx):
@@ -565,4 +567,12 @@ def test_update_driver_runs_epochs_and_stops_on_kl(mrl, ctx):
     upd2 = mrl.ppo.DiscreteUpdate(ctx, rb, MB, anet.optimizer, cnet.optimizer, target_kl=1e-4)
     ran = upd2.update(10, seed=5)
     stopped, mean_kl = upd2.kl_stopped()
-    assert stopped and ran < 10
+    assert stopped and ran < 10 and mean_kl > 1e-4
+    applied = int(upd2.kl_flag[2].item())
+    assert applied < ran * (N * T // MB)
+    assert anet.optimizer.t == 2 * (N * T // MB) + applied == cnet.optimizer.t
+    # nothing moves once the stop has fired
+    frozen = anet.params.clone()
+    upd2.minibatch_step(upd2.indices[:MB])
+    ctx.synchronize()
+    assert torch.equal(frozen, anet.params)
