@@ -34,52 +34,77 @@ struct TileCache {
     int nrow;    // rows of the tile inside the batch
 };
 
-// hidden stack of one net for the block's 32 rows; leaves act(layer1) in h2[32][H+1]
-template <int H, int ACT>
+// Hidden stack of one net for the block's 32 rows; leaves act(layer1) in h2[32][H+1].
+// TPW = accumulator tiles (32 columns each) per wavefront: the net is worked on by 2H / TPW
+// threads (threadIdx.x modulo that count picks the role), so TPW = 1 spreads the same MFMA chain
+// over twice the wavefronts.  Everything a later phase needs from global memory and that does not
+// depend on earlier phases (biases, the layer-0 weights) is requested up front, so that a block
+// pays the L2 latency once rather than once per phase.
+template <int H, int ACT, int TPW = 2>
 MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
                           const TileCache tc) {
-    const int t = threadIdx.x % H, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
+    constexpr int T = 2 * H / TPW;
+    constexpr int K0 = PIN_MAX / 2;   // k-steps of layer 0 at the widest input
+    const int t = threadIdx.x % T, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
     const float *W0 = p, *b0 = p + IN * H;
     const float *W1 = b0 + H, *b1 = W1 + H * H;
-    const int col0 = 64 * w + l31, col1 = col0 + 32;
-    {   // layer 0 (K = IN <= 32, padded to even with zeros): wavefront w owns columns [64w, 64w + 64)
-        floatx16 c0 = {0}, c1 = {0};
-        for (int kk = 0; kk < (IN + 1) / 2; ++kk) {
+    int col[TPW];
+    float bias0[TPW], bias1[TPW];
+#pragma unroll
+    for (int q = 0; q < TPW; ++q) {
+        col[q] = 32 * (TPW * w + q) + l31;
+        bias0[q] = b0[col[q]];
+        bias1[q] = b1[col[q]];
+    }
+    {   // layer 0 (K = IN <= 32, padded to even with zeros): all operands first, then the MFMAs
+        float a0[K0], w0[TPW][K0];
+#pragma unroll
+        for (int kk = 0; kk < K0; ++kk) {
             const int k = 2 * kk + half;
             const bool in = k < IN;
-            const float a = in ? xs[l31 * XS_LD + k] : 0.0f;
-            const float bv0 = in ? W0[k * H + col0] : 0.0f;
-            const float bv1 = in ? W0[k * H + col1] : 0.0f;
-            c0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bv0, c0, 0, 0, 0);
-            c1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bv1, c1, 0, 0, 0);
-        }
-        const float bb0 = b0[col0], bb1 = b0[col1];
+            a0[kk] = in ? xs[l31 * XS_LD + k] : 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int row = 8 * (v >> 2) + 4 * half + (v & 3);
-            const float p0 = c0[v] + bb0, p1 = c1[v] + bb1;
-            const float y0 = activate<ACT>(p0), y1 = activate<ACT>(p1);
-            hT[col0 * HT_LD + row] = y0;
-            hT[col1 * HT_LD + row] = y1;
-            if (tc.c0 != nullptr && row < tc.nrow) {
-                float *q0 = tc.c0 + (tc.row0 + row) * (IN + H) + IN, *q1 = tc.c1 + (tc.row0 + row) * (2 * H);
-                q0[col0] = ACT == 1 ? p0 : y0; q0[col1] = ACT == 1 ? p1 : y1;
-                q1[col0] = y0; q1[col1] = y1;
+            for (int q = 0; q < TPW; ++q) w0[q][kk] = in ? W0[k * H + col[q]] : 0.0f;
+        }
+        floatx16 c[TPW];
+#pragma unroll
+        for (int q = 0; q < TPW; ++q) c[q] = floatx16{0};
+#pragma unroll
+        for (int kk = 0; kk < K0; ++kk) {
+            if (2 * kk < IN) {
+#pragma unroll
+                for (int q = 0; q < TPW; ++q)
+                    c[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[kk], w0[q][kk], c[q], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < TPW; ++q) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = 8 * (v >> 2) + 4 * half + (v & 3);
+                const float pre = c[q][v] + bias0[q];
+                const float y = activate<ACT>(pre);
+                hT[col[q] * HT_LD + row] = y;
+                if (tc.c0 != nullptr && row < tc.nrow) {
+                    tc.c0[(tc.row0 + row) * (IN + H) + IN + col[q]] = ACT == 1 ? pre : y;
+                    tc.c1[(tc.row0 + row) * (2 * H) + col[q]] = y;
+                }
             }
         }
     }
     __syncthreads();
     {   // layer 1 (H x H): weights streamed from L2 one block of KB k-steps ahead of the MFMAs
-        constexpr int KB = 8;
-        floatx16 c0 = {0}, c1 = {0};
-        const float *Wc = W1 + col0;
-        float a[KB], bv0[KB], bv1[KB], na[KB], nb0[KB], nb1[KB];
+        constexpr int KB = TPW == 2 ? 8 : 32;
+        floatx16 c[TPW];
+#pragma unroll
+        for (int q = 0; q < TPW; ++q) c[q] = floatx16{0};
+        float a[KB], bv[TPW][KB], na[KB], nb[TPW][KB];
 #pragma unroll
         for (int j = 0; j < KB; ++j) {
             const int k = 2 * j + half;
             a[j] = hT[k * HT_LD + l31];
-            bv0[j] = Wc[k * H];
-            bv1[j] = Wc[k * H + 32];
+#pragma unroll
+            for (int q = 0; q < TPW; ++q) bv[q][j] = W1[k * H + col[q]];
         }
         for (int blk = 0; blk < H / (2 * KB); ++blk) {
             const bool more = blk + 1 < H / (2 * KB);
@@ -88,53 +113,71 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
                 for (int j = 0; j < KB; ++j) {
                     const int k = 2 * ((blk + 1) * KB + j) + half;
                     na[j] = hT[k * HT_LD + l31];
-                    nb0[j] = Wc[k * H];
-                    nb1[j] = Wc[k * H + 32];
+#pragma unroll
+                    for (int q = 0; q < TPW; ++q) nb[q][j] = W1[k * H + col[q]];
                 }
             }
 #pragma unroll
             for (int j = 0; j < KB; ++j) {
-                c0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], bv0[j], c0, 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], bv1[j], c1, 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < TPW; ++q)
+                    c[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], bv[q][j], c[q], 0, 0, 0);
             }
             if (more) {
 #pragma unroll
-                for (int j = 0; j < KB; ++j) { a[j] = na[j]; bv0[j] = nb0[j]; bv1[j] = nb1[j]; }
+                for (int j = 0; j < KB; ++j) {
+                    a[j] = na[j];
+#pragma unroll
+                    for (int q = 0; q < TPW; ++q) bv[q][j] = nb[q][j];
+                }
             }
         }
-        const float bb0 = b1[col0], bb1 = b1[col1];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int row = 8 * (v >> 2) + 4 * half + (v & 3);
-            const float p0 = c0[v] + bb0, p1 = c1[v] + bb1;
-            const float y0 = activate<ACT>(p0), y1 = activate<ACT>(p1);
-            h2[row * (H + 1) + col0] = y0;
-            h2[row * (H + 1) + col1] = y1;
-            if (tc.c0 != nullptr && row < tc.nrow) {
-                float *q1 = tc.c1 + (tc.row0 + row) * (2 * H) + H, *q2 = tc.c2 + (tc.row0 + row) * H;
-                q1[col0] = ACT == 1 ? p0 : y0; q1[col1] = ACT == 1 ? p1 : y1;
-                q2[col0] = y0; q2[col1] = y1;
+        for (int q = 0; q < TPW; ++q) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = 8 * (v >> 2) + 4 * half + (v & 3);
+                const float pre = c[q][v] + bias1[q];
+                const float y = activate<ACT>(pre);
+                h2[row * (H + 1) + col[q]] = y;
+                if (tc.c0 != nullptr && row < tc.nrow) {
+                    tc.c1[(tc.row0 + row) * (2 * H) + H + col[q]] = ACT == 1 ? pre : y;
+                    tc.c2[(tc.row0 + row) * H + col[q]] = y;
+                }
             }
         }
     }
     __syncthreads();
 }
 
-// out[r][a] = h2[r] . W2[:, a] + b2[a] for the block's rows; TPR = H/32 lanes cooperate per row
+// floats of LDS that hold one net's head parameters [W2 (H x A) | b2 (A) | log_std (A)]
+constexpr int HEAD_LDS(int H) { return (H + 2) * PA_MAX; }
+
+// copies the head parameters of a net into LDS (call by `nthreads` threads with 0 <= t < nthreads,
+// early in the kernel: the head then never waits on global memory)
+MRL_DEV void stage_head(const float *__restrict__ W2, int H, int A, bool with_log_std, float *w2s, int t,
+                        int nthreads) {
+    const int n = (H + 1) * A + (with_log_std ? A : 0);
+    for (int i = t; i < n; i += nthreads) w2s[i] = W2[i];
+}
+
+// out[r][a] = h2[r] . W2[:, a] + b2[a] for the block's rows; TPR = H/32 lanes cooperate per row.
+// w2s: the head parameters in LDS (stage_head); called by the first H threads of the net.
 template <int H>
-MRL_DEV void head(const float *__restrict__ W2, int A, const float *h2, float *out, int out_ld) {
+MRL_DEV void head(const float *w2s, int A, const float *h2, float *out, int out_ld) {
     constexpr int TPR = H / PR;
     const int t = threadIdx.x % H, r = t / TPR, part = t % TPR;
-    const float *b2 = W2 + H * A;
+    const float *b2 = w2s + H * A;
     float acc[PA_MAX];
 #pragma unroll
     for (int a = 0; a < PA_MAX; ++a) acc[a] = 0.0f;
+#pragma unroll 8
     for (int i = 0; i < PR; ++i) {
         const int n = i * TPR + part;
         const float hv = h2[r * (H + 1) + n];
 #pragma unroll
         for (int a = 0; a < PA_MAX; ++a)
-            if (a < A) acc[a] = fmaf(hv, W2[n * A + a], acc[a]);
+            if (a < A) acc[a] = fmaf(hv, w2s[n * A + a], acc[a]);
     }
 #pragma unroll
     for (int a = 0; a < PA_MAX; ++a) {

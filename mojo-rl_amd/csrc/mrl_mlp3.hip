@@ -20,11 +20,13 @@ namespace mrl {
 // grid = (row tiles, nets): blockIdx.y picks the net, so that an actor and a critic that read the
 // same inputs go through the chip side by side
 template <int H, int ACT>
-__global__ __launch_bounds__(H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets nets) {
+__global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets nets) {
+    constexpr int T = 2 * H;   // one 32-column accumulator tile per wavefront
     __shared__ float xs[PR * XS_LD];
     __shared__ float hT[H * HT_LD];
     __shared__ float h2[PR * (H + 1)];
     __shared__ float ys[PR * (PA_MAX + 1)];
+    __shared__ float w2s[HEAD_LDS(H)];
     const Mlp3Net &nn = nets.n[blockIdx.y];
     const float *__restrict__ x = nn.x;
     const float *__restrict__ params = nn.params;
@@ -41,7 +43,7 @@ __global__ __launch_bounds__(H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets net
         tc.c1 = cache + (size_t)B * (IN + H);
         tc.c2 = tc.c1 + (size_t)B * 2 * H;
     }
-    for (int i = t; i < PR * IN; i += H) {
+    for (int i = t; i < PR * IN; i += T) {
         const int r = i / IN, k = i - r * IN;
         float v = 0.0f;
         if (r < nrow) {
@@ -51,18 +53,18 @@ __global__ __launch_bounds__(H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets net
         xs[r * XS_LD + k] = v;
     }
     __syncthreads();
-    hidden_stack<H, ACT>(params, IN, xs, hT, h2, tc);
-    const float *W2 = params + IN * H + H + H * H + H;
-    head<H>(W2, A, h2, ys, PA_MAX + 1);
+    stage_head(params + IN * H + H + H * H + H, H, A, GAUSS, w2s, t, T);
+    hidden_stack<H, ACT, 1>(params, IN, xs, hT, h2, tc);
+    if (t < H) head<H>(w2s, A, h2, ys, PA_MAX + 1);
     __syncthreads();
     const int ld = GAUSS ? 2 * A : A;
-    for (int i = t; i < nrow * ld; i += H) {
+    for (int i = t; i < nrow * ld; i += T) {
         const int r = i / ld, a = i - r * ld;
         float v;
         if (a < A) {
             v = ys[r * (PA_MAX + 1) + a];
         } else {   // state-independent log_std, clamped (deep_rl/model/stochastic_actor.mojo:260-275)
-            v = W2[H * A + A + (a - A)];
+            v = w2s[H * A + A + (a - A)];
             if (v < -5.0f) v = -5.0f;
             else if (v > 2.0f) v = 2.0f;
         }
@@ -80,7 +82,8 @@ MRL_DEV float act_deriv(float cached) {
 // grad_out [B, ld] (ld = A, or 2A for the Gaussian head: mean gradients first); g1, g0 [B, H];
 // ls_part [tiles, A]: per-tile sums of the log_std gradient columns.  grid = (row tiles, nets).
 template <int H, int ACT>
-__global__ __launch_bounds__(H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3Nets nets) {
+__global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3Nets nets) {
+    constexpr int T = 2 * H;   // one 32-column accumulator tile per wavefront
     const Mlp3Net &nn = nets.n[blockIdx.y];
     const float *__restrict__ grad_out = nn.grad_out;
     const float *__restrict__ params = nn.params;
@@ -88,6 +91,7 @@ __global__ __launch_bounds__(H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3Nets 
     float *__restrict__ g1 = nn.g1;
     float *__restrict__ g0 = nn.g0;
     float *__restrict__ ls_part = nn.ls_part;
+    float *__restrict__ db_part = nn.db_part + (size_t)blockIdx.x * (2 * H + PA_MAX);   // this tile's slice
     const int A = nn.A;
     const bool GAUSS = nn.gauss != 0;
     constexpr int KCH = 32;                       // k-chunk of W1 staged per round
@@ -101,20 +105,22 @@ __global__ __launch_bounds__(H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3Nets 
     const float *c0 = cache, *c1 = cache + (size_t)B * (IN + H);
     const float *W1 = params + IN * H + H;
     const float *W2 = W1 + H * H + H;
-    for (int i = t; i < PR * ld; i += H) {
+    for (int i = t; i < PR * ld; i += T) {
         const int r = i / ld, a = i - r * ld;
         g2s[r * (2 * PA_MAX + 1) + a] = r < nrow ? grad_out[row0 * ld + i] : 0.0f;
     }
     __syncthreads();
-    if (GAUSS && t < A) {
+    if (t < ld) {   // column sums of the tile: bias gradient of the head, log_std gradient
         float s = 0.0f;
-        for (int r = 0; r < PR; ++r) s += g2s[r * (2 * PA_MAX + 1) + A + t];
-        ls_part[(long)blockIdx.x * A + t] = s;
+        for (int r = 0; r < PR; ++r) s += g2s[r * (2 * PA_MAX + 1) + t];
+        if (t < A) db_part[2 * H + t] = s;
+        else ls_part[(long)blockIdx.x * A + (t - A)] = s;
     }
-    {   // g1[r][n] = (sum_a g2[r][a] W2[n][a]) * act'(layer 1); thread t owns column n = t
+    if (t < H) {   // g1[r][n] = (sum_a g2[r][a] W2[n][a]) * act'(layer 1); thread t owns column n = t
         float wrow[PA_MAX];
 #pragma unroll
         for (int a = 0; a < PA_MAX; ++a) wrow[a] = a < A ? W2[t * A + a] : 0.0f;
+        float colsum = 0.0f;
         for (int r = 0; r < PR; ++r) {
             float s = 0.0f;
 #pragma unroll
@@ -126,44 +132,54 @@ __global__ __launch_bounds__(H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3Nets 
                 g1[(row0 + r) * H + t] = g;
             }
             gT[t * HT_LD + r] = g;
+            colsum += g;
         }
+        db_part[H + t] = colsum;   // bias gradient of layer 1, this tile's rows
     }
-    // dh1 = g1 W1^T: wavefront w owns input columns [64w, 64w + 64)
-    floatx16 acc0 = {0}, acc1 = {0};
-    const int col0 = 64 * w + l31, col1 = col0 + 32;
+    // dh1 = g1 W1^T: wavefront w owns input columns [32w, 32w + 32).  The next chunk of W1 is
+    // fetched into registers while the matrix cores work on the current one.
+    floatx16 acc = {0};
+    const int col = 32 * w + l31;
+    const int wrow = t % H, wseg = (t / H) * (KCH / 2);   // thread copies W1[wrow][o0 + wseg .. + 16)
+    float4 nxt[KCH / 8];
+    auto fetch = [&](int o0) {
+        const float4 *src = reinterpret_cast<const float4 *>(W1 + (size_t)wrow * H + o0 + wseg);
+#pragma unroll
+        for (int q = 0; q < KCH / 8; ++q) nxt[q] = src[q];
+    };
+    fetch(0);
     for (int o0 = 0; o0 < H; o0 += KCH) {
         __syncthreads();   // gT complete (first round) / previous chunk consumed
-        {   // thread t copies W1[t][o0 .. o0 + 32) -> wT[k][t]
-            const float4 *src = reinterpret_cast<const float4 *>(W1 + (size_t)t * H + o0);
 #pragma unroll
-            for (int q = 0; q < KCH / 4; ++q) {
-                const float4 v = src[q];
-                wT[(4 * q + 0) * (H + 1) + t] = v.x;
-                wT[(4 * q + 1) * (H + 1) + t] = v.y;
-                wT[(4 * q + 2) * (H + 1) + t] = v.z;
-                wT[(4 * q + 3) * (H + 1) + t] = v.w;
-            }
+        for (int q = 0; q < KCH / 8; ++q) {
+            wT[(wseg + 4 * q + 0) * (H + 1) + wrow] = nxt[q].x;
+            wT[(wseg + 4 * q + 1) * (H + 1) + wrow] = nxt[q].y;
+            wT[(wseg + 4 * q + 2) * (H + 1) + wrow] = nxt[q].z;
+            wT[(wseg + 4 * q + 3) * (H + 1) + wrow] = nxt[q].w;
         }
         __syncthreads();
+        if (o0 + KCH < H) fetch(o0 + KCH);
+        __builtin_amdgcn_sched_barrier(0);   // keep the loads ahead of the MFMAs that hide them
 #pragma unroll
         for (int kk = 0; kk < KCH / 2; ++kk) {
             const int k = 2 * kk + half;
             const float a = gT[(o0 + k) * HT_LD + l31];
-            const float b0 = wT[k * (H + 1) + col0];
-            const float b1 = wT[k * (H + 1) + col1];
-            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b0, acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b1, acc1, 0, 0, 0);
+            const float b = wT[k * (H + 1) + col];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
         }
     }
+    float cs = 0.0f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         const int row = 8 * (v >> 2) + 4 * half + (v & 3);
         if (row >= nrow) continue;
-        const float *q = c0 + (row0 + row) * (IN + H) + IN;
-        float *o = g0 + (row0 + row) * H;
-        o[col0] = acc0[v] * act_deriv<ACT>(q[col0]);
-        o[col1] = acc1[v] * act_deriv<ACT>(q[col1]);
+        const float val = acc[v] * act_deriv<ACT>(c0[(row0 + row) * (IN + H) + IN + col]);
+        g0[(row0 + row) * H + col] = val;
+        cs += val;
     }
+    // the two halves of the wavefront hold the other 16 rows of the same column
+    cs += __shfl_xor(cs, 32, 64);
+    if (half == 0) db_part[col] = cs;   // bias gradient of layer 0, this tile's rows
 }
 
 // ---------------------------------------------------------------- [dW | db] of the three layers
@@ -172,13 +188,15 @@ constexpr int DBM = 64, DBN = 64, DKC = 32, DLD = 65;
 struct DwProblem {
     const float *X;   // layer input per batch row (row stride xs)
     const float *G;   // gradient at the layer's pre-activation (row stride gs)
-    int xs, gs, K, N; // K inputs, N outputs: the block written is [(K + 1), N] (last row = bias)
-    int poff;         // offset of the layer in the flat parameter vector
-    int tiles_n, tiles;   // tiles_n = ceil(N / 64); tiles = tiles_n * ceil((K + 1) / 64)
+    int xs, gs, K, N; // K inputs, N outputs: the block written is dW [K, N]
+    int poff;         // offset of the layer's W in the flat parameter vector
+    int tiles_n, tiles;   // tiles_n = ceil(N / 64); tiles = tiles_n * ceil(K / 64)
 };
 struct DwSet { DwProblem p[6]; int n; };
 
-// grid.x = sum of the problems' tiles, grid.y = batch splits; partial[z][P]
+// dW = X^T G of every problem, split over the batch: grid.x = sum of the problems' tiles,
+// grid.y = batch splits; partial[z][P].  The next 32-row chunk is fetched into registers while
+// the matrix cores work on the current one.
 __global__ __launch_bounds__(256) void dw3_kernel(DwSet d, int M, int rows_per_split, int P,
                                                   float *__restrict__ partial) {
     __shared__ float As[DKC * DLD];
@@ -194,25 +212,27 @@ __global__ __launch_bounds__(256) void dw3_kernel(DwSet d, int M, int rows_per_s
     if (b_end > M) b_end = M;
     floatx16 acc = {0};
     const int bb = t >> 3, seg = (t & 7) * 8;
-    for (long b0 = b_begin; b0 < b_end; b0 += DKC) {
+    float xa[8], gb[8];
+    auto fetch = [&](long b0) {
         const long b = b0 + bb;
         const bool inb = b < b_end;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const int ii = i0 + seg + i;
-            float v = 0.0f;
-            if (inb) {
-                if (ii < pr.K) v = pr.X[b * pr.xs + ii];
-                else if (ii == pr.K) v = 1.0f;
-            }
-            As[bb * DLD + seg + i] = v;
+            const int ii = i0 + seg + i, j = j0 + seg + i;
+            xa[i] = (inb && ii < pr.K) ? pr.X[b * pr.xs + ii] : 0.0f;
+            gb[i] = (inb && j < pr.N) ? pr.G[b * pr.gs + j] : 0.0f;
         }
+    };
+    fetch(b_begin);
+    for (long b0 = b_begin; b0 < b_end; b0 += DKC) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const int j = j0 + seg + i;
-            Bs[bb * DLD + seg + i] = (inb && j < pr.N) ? pr.G[b * pr.gs + j] : 0.0f;
+            As[bb * DLD + seg + i] = xa[i];
+            Bs[bb * DLD + seg + i] = gb[i];
         }
         __syncthreads();
+        if (b0 + DKC < b_end) fetch(b0 + DKC);
+        __builtin_amdgcn_sched_barrier(0);   // keep the loads ahead of the MFMAs that hide them
 #pragma unroll
         for (int kk = 0; kk < DKC; kk += 2) {
             const float a = As[(kk + half) * DLD + 32 * wr + l31];
@@ -227,18 +247,19 @@ __global__ __launch_bounds__(256) void dw3_kernel(DwSet d, int M, int rows_per_s
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int row = i0 + 32 * wr + 8 * (v >> 2) + 4 * half + (v & 3);
-            if (row <= pr.K) out[(size_t)row * pr.N + col] = acc[v];
+            if (row < pr.K) out[(size_t)row * pr.N + col] = acc[v];
         }
     }
 }
 
-// grads[i] = sum_z partial[z][i] for the [W | b] blocks; the log_std tail (Gaussian head) sums the
-// per-tile column sums of the backward-dx kernel.  The nets' vectors lie back to back in `partial`.
+// Flat gradient vector of each net from the pieces: weight blocks = sum over the batch splits of
+// `partial`, bias rows and the log_std tail (Gaussian head) = sum over the row tiles of the column
+// sums the backward-dx kernel left.  The nets' vectors lie back to back in `partial`.
 struct SumNets {
     float *grads[2];
-    const float *ls_part[2];
-    int P[2], n_wb[2], A[2];
-    int n;
+    const float *ls_part[2], *db_part[2];
+    int P[2], A[2], gauss[2];
+    int n, IN, H;
 };
 
 __global__ __launch_bounds__(256) void sum3_kernel(const float *__restrict__ partial, int splits, int Ptot,
@@ -248,13 +269,36 @@ __global__ __launch_bounds__(256) void sum3_kernel(const float *__restrict__ par
     const int gi = i;
     int net = 0;
     if (sn.n > 1 && i >= sn.P[0]) { net = 1; i -= sn.P[0]; }
-    float s = 0.0f;
-    if (i < sn.n_wb[net]) {
-        for (int z = 0; z < splits; ++z) s += partial[(size_t)z * Ptot + gi];
-    } else {
-        const int j = i - sn.n_wb[net];
-        for (int q = 0; q < tiles; ++q) s += sn.ls_part[net][(size_t)q * sn.A[net] + j];
+    const int IN = sn.IN, H = sn.H, A = sn.A[net];
+    const int o1 = (IN + 1) * H, o2 = o1 + (H + 1) * H, o3 = o2 + (H + 1) * A;
+    // which bias row (or the log_std tail) does i fall in?  -1: a weight
+    int bias_layer = -1, j = 0;
+    if (i >= IN * H && i < o1) { bias_layer = 0; j = i - IN * H; }
+    else if (i >= o1 + H * H && i < o2) { bias_layer = 1; j = i - (o1 + H * H); }
+    else if (i >= o2 + H * A && i < o3) { bias_layer = 2; j = i - (o2 + H * A); }
+    else if (i >= o3) { bias_layer = 3; j = i - o3; }
+    // n terms, `stride` floats apart, added in order; loads are issued 16 at a time so that the
+    // chain is 16 times shorter than one dependent load per term
+    const float *p;
+    size_t stride;
+    int n;
+    if (bias_layer < 0) { p = partial + gi; stride = (size_t)Ptot; n = splits; }
+    else if (bias_layer == 3) { p = sn.ls_part[net] + j; stride = (size_t)A; n = tiles; }
+    else {
+        p = sn.db_part[net] + (bias_layer == 0 ? 0 : (bias_layer == 1 ? H : 2 * H)) + j;
+        stride = (size_t)(2 * H + PA_MAX);
+        n = tiles;
     }
+    float s = 0.0f;
+    int q = 0;
+    for (; q + 16 <= n; q += 16) {
+        float v[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) v[k] = p[(size_t)(q + k) * stride];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) s += v[k];
+    }
+    for (; q < n; ++q) s += p[(size_t)q * stride];
     sn.grads[net][i] = s;
 }
 
@@ -291,12 +335,12 @@ bool mlp3_pair_fusable(const mrl_mlp_desc &a, const mrl_mlp_desc &b) {
 template <int H, int ACT>
 static void launch_fwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, int n_nets) {
     dim3 grid((batch + PR - 1) / PR, n_nets);
-    hipLaunchKernelGGL((mlp3_fwd_kernel<H, ACT>), grid, dim3(H), 0, ctx->stream, batch, IN, nets);
+    hipLaunchKernelGGL((mlp3_fwd_kernel<H, ACT>), grid, dim3(2 * H), 0, ctx->stream, batch, IN, nets);
 }
 template <int H, int ACT>
 static void launch_bwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, int n_nets) {
     dim3 grid((batch + PR - 1) / PR, n_nets);
-    hipLaunchKernelGGL((mlp3_bwd_dx_kernel<H, ACT>), grid, dim3(H), 0, ctx->stream, batch, IN, nets);
+    hipLaunchKernelGGL((mlp3_bwd_dx_kernel<H, ACT>), grid, dim3(2 * H), 0, ctx->stream, batch, IN, nets);
 }
 
 // forward of one or two nets (descs[i], io.n[i]) in one launch
@@ -331,7 +375,7 @@ size_t mlp3_backward_ws(const mrl_mlp_desc *const *descs, int n_nets, int batch)
     size_t total = 0, P = 0;
     for (int i = 0; i < n_nets; ++i) {
         const int H = descs[i]->layers[0].out_dim;
-        total += (size_t)2 * batch * H + (size_t)((batch + PR - 1) / PR) * PA_MAX;
+        total += (size_t)2 * batch * H + (size_t)((batch + PR - 1) / PR) * (2 * PA_MAX + 2 * H);
         P += net_P(*descs[i]);
     }
     return total + (size_t)32 * P;
@@ -354,15 +398,17 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
     if (n_nets == 2 && !mlp3_pair_fusable(*descs[0], *descs[1])) return MRL_E_UNSUPPORTED;
     const int IN = descs[0]->layers[0].in_dim;
     const int tiles = (batch + PR - 1) / PR;
-    int splits = std::max(1, std::min(32, batch / 128));
+    int splits = std::max(1, std::min(32, batch / 256));
     int rows_per = ((batch + splits - 1) / splits + DKC - 1) / DKC * DKC;
     splits = (batch + rows_per - 1) / rows_per;
-    // workspace: per net g1 [B, H] | g0 [B, H] | ls_part [tiles, PA_MAX]; then partial [splits, Ptot]
+    // workspace: per net g1 [B, H] | g0 [B, H] | ls_part [tiles, PA_MAX] | db_part [tiles, 2H + PA_MAX];
+    // then partial [splits, Ptot]
     float *w = ws;
     for (int i = 0; i < n_nets; ++i) {
         io.n[i].g1 = w; w += (size_t)batch * H;
         io.n[i].g0 = w; w += (size_t)batch * H;
         io.n[i].ls_part = w; w += (size_t)tiles * PA_MAX;
+        io.n[i].db_part = w; w += (size_t)tiles * (2 * H + PA_MAX);
     }
     float *partial = w;
     if (H == 256 && act == 1) launch_bwd_t<256, 1>(ctx, batch, IN, io, n_nets);
@@ -374,10 +420,12 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
     dw.n = 3 * n_nets;
     SumNets sn{};
     sn.n = n_nets;
+    sn.IN = IN;
+    sn.H = H;
     auto fill = [](DwProblem &p, const float *X, int xs, const float *G, int gs, int K, int N, int poff) {
         p.X = X; p.G = G; p.xs = xs; p.gs = gs; p.K = K; p.N = N; p.poff = poff;
         p.tiles_n = (N + DBN - 1) / DBN;
-        p.tiles = p.tiles_n * ((K + 1 + DBM - 1) / DBM);
+        p.tiles = p.tiles_n * ((K + DBM - 1) / DBM);
     };
     int base = 0, total_tiles = 0;
     for (int i = 0; i < n_nets; ++i) {
@@ -390,9 +438,10 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
         for (int q = 0; q < 3; ++q) total_tiles += dw.p[3 * i + q].tiles;
         sn.grads[i] = grads[i];
         sn.ls_part[i] = nn.ls_part;
+        sn.db_part[i] = nn.db_part;
         sn.P[i] = net_P(*descs[i]);
-        sn.n_wb[i] = (IN + 1) * H + (H + 1) * H + (H + 1) * A;
         sn.A[i] = A;
+        sn.gauss[i] = nn.gauss;
         base += sn.P[i];
     }
     const int Ptot = base;

@@ -33,6 +33,7 @@ __global__ __launch_bounds__(2 * H) void policy_kernel(
     __shared__ float h2[2][PR * (H + 1)];
     __shared__ float logits[PR * (PA_MAX + 1)];
     __shared__ float vals[PR];
+    __shared__ float w2s[2][HEAD_LDS(H)];
     const int t = threadIdx.x;
     const int net = t / H;                   // 0 = actor, 1 = critic
     const int row0 = blockIdx.x * PR;
@@ -51,9 +52,10 @@ __global__ __launch_bounds__(2 * H) void policy_kernel(
     __syncthreads();
 
     const float *p = net ? critic_p : actor_p;
+    stage_head(p + IN * H + H + H * H + H, H, net ? 1 : A, GAUSS && net == 0, w2s[net], t % H, H);
     hidden_stack<H, ACT>(p, IN, xs, hT[net], h2[net], TileCache{});
-    if (net == 0) head<H>(p + IN * H + H + H * H + H, A, h2[0], logits, PA_MAX + 1);
-    else head<H>(p + IN * H + H + H * H + H, 1, h2[1], vals, 1);
+    if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1);
+    else head<H>(w2s[1], 1, h2[1], vals, 1);
     __syncthreads();
 
     if (t < nrow && !GAUSS) {   // categorical sampling, one lane per env
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(2 * H) void policy_kernel(
     if (t < nrow && GAUSS) {    // Gaussian sampling, one lane per env, one Philox stream per (env, j)
         const int i = row0 + t;
         const float *mean_row = logits + t * (PA_MAX + 1);
-        const float *log_std_p = actor_p + IN * H + H + H * H + H + H * A + A;
+        const float *log_std_p = w2s[0] + H * A + A;
         const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
         float total = 0.0f;
         for (int j = 0; j < A; ++j) {
