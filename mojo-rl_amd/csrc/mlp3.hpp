@@ -24,8 +24,10 @@ int mlp3_forward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, i
 size_t mlp3_backward_ws(const mrl_mlp_desc *const *descs, int n_nets, int batch);
 int mlp3_backward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *grad_out, const float *params,
                   const float *cache, float *grads, float *ws);
+// sq_part (nullable): receives per-block sums of squares of the gradients, [net * 1024 + block];
+// *sq_blocks = number of blocks written (0 when none were)
 int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io,
-                    float *const *grads, float *ws);
+                    float *const *grads, float *ws, float *sq_part, int *sq_blocks);
 // grows the context's MLP workspace to at least `floats`
 int mlp_ensure_ws(mrl_ctx *ctx, size_t floats, float **out);
 

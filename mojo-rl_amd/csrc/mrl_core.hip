@@ -55,6 +55,9 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
         MRL_CHECK_HIP(hipMemcpy(c->hc_shapes, &hs, sizeof(hs), hipMemcpyHostToDevice));
     }
     MRL_CHECK_HIP(hipMalloc(&c->reduce_scratch, sizeof(float) * c->reduce_scratch_floats));
+    c->upd_scratch = nullptr;
+    MRL_CHECK_HIP(hipMalloc(&c->upd_scratch, sizeof(float) * 4096));
+    MRL_CHECK_HIP(hipMemset(c->upd_scratch, 0, sizeof(float) * 4096));
     *out = c;
     return MRL_OK;
 }
@@ -67,6 +70,7 @@ int mrl_ctx_destroy(mrl_ctx *ctx) {
     if (ctx->bw_shapes) hipFree(ctx->bw_shapes);
     if (ctx->hc_shapes) hipFree(ctx->hc_shapes);
     if (ctx->reduce_scratch) hipFree(ctx->reduce_scratch);
+    if (ctx->upd_scratch) hipFree(ctx->upd_scratch);
     if (ctx->mlp_ws) hipFree(ctx->mlp_ws);
     if (ctx->rollout_ws) hipFree(ctx->rollout_ws);
     for (hipEvent_t e : ctx->prof_events) hipEventDestroy(e);

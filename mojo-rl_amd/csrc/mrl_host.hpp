@@ -29,6 +29,9 @@ struct mrl_ctx {
     // rewards, dones for n_envs), grown on demand
     float *rollout_ws;
     size_t rollout_ws_floats;
+    // scratch of the minibatch update: per-block KL partials [0, 1024), their arrival counter
+    // (int, at float index 1024; zero between launches), sum-of-squares partials [2048, 4096)
+    float *upd_scratch;
     // phase timing: events recorded on `stream` at phase boundaries while armed
     bool profiling;
     std::vector<hipEvent_t> prof_events;

@@ -105,6 +105,24 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
     const float *c0 = cache, *c1 = cache + (size_t)B * (IN + H);
     const float *W1 = params + IN * H + H;
     const float *W2 = W1 + H * H + H;
+    // what the later phases need from global memory is requested now, so that the block waits
+    // for L2 once: the cached activations behind act' of both hidden layers, the head weights
+    float d1[PR];          // thread t < H: layer-1 cache entries of column t, rows of the tile
+    float w2row[PA_MAX];   // thread t < H: W2[t][:]
+    float d0[16];          // layer-0 cache entries at this lane's accumulator positions
+    {
+        const int n1 = t % H;
+#pragma unroll
+        for (int r = 0; r < PR; ++r) d1[r] = r < nrow ? c1[(row0 + r) * (2 * H) + H + n1] : 0.0f;
+#pragma unroll
+        for (int a = 0; a < PA_MAX; ++a) w2row[a] = a < A ? W2[n1 * A + a] : 0.0f;
+        const int colq = 32 * w + l31;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int row = 8 * (v >> 2) + 4 * half + (v & 3);
+            d0[v] = row < nrow ? c0[(row0 + row) * (IN + H) + IN + colq] : 0.0f;
+        }
+    }
     for (int i = t; i < PR * ld; i += T) {
         const int r = i / ld, a = i - r * ld;
         g2s[r * (2 * PA_MAX + 1) + a] = r < nrow ? grad_out[row0 * ld + i] : 0.0f;
@@ -117,18 +135,16 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
         else ls_part[(long)blockIdx.x * A + (t - A)] = s;
     }
     if (t < H) {   // g1[r][n] = (sum_a g2[r][a] W2[n][a]) * act'(layer 1); thread t owns column n = t
-        float wrow[PA_MAX];
-#pragma unroll
-        for (int a = 0; a < PA_MAX; ++a) wrow[a] = a < A ? W2[t * A + a] : 0.0f;
         float colsum = 0.0f;
+#pragma unroll
         for (int r = 0; r < PR; ++r) {
             float s = 0.0f;
 #pragma unroll
             for (int a = 0; a < PA_MAX; ++a)
-                if (a < A) s = fmaf(g2s[r * (2 * PA_MAX + 1) + a], wrow[a], s);
+                if (a < A) s = fmaf(g2s[r * (2 * PA_MAX + 1) + a], w2row[a], s);
             float g = 0.0f;
             if (r < nrow) {
-                g = s * act_deriv<ACT>(c1[(row0 + r) * (2 * H) + H + t]);
+                g = s * act_deriv<ACT>(d1[r]);
                 g1[(row0 + r) * H + t] = g;
             }
             gT[t * HT_LD + r] = g;
@@ -173,7 +189,7 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
     for (int v = 0; v < 16; ++v) {
         const int row = 8 * (v >> 2) + 4 * half + (v & 3);
         if (row >= nrow) continue;
-        const float val = acc[v] * act_deriv<ACT>(c0[(row0 + row) * (IN + H) + IN + col]);
+        const float val = acc[v] * act_deriv<ACT>(d0[v]);
         g0[(row0 + row) * H + col] = val;
         cs += val;
     }
@@ -263,43 +279,60 @@ struct SumNets {
 };
 
 __global__ __launch_bounds__(256) void sum3_kernel(const float *__restrict__ partial, int splits, int Ptot,
-                                                   int tiles, SumNets sn) {
-    int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= Ptot) return;
-    const int gi = i;
+                                                   int tiles, SumNets sn, float *__restrict__ sq_part) {
+    __shared__ float red[2][4];
+    const int gi = blockIdx.x * blockDim.x + threadIdx.x;
     int net = 0;
-    if (sn.n > 1 && i >= sn.P[0]) { net = 1; i -= sn.P[0]; }
-    const int IN = sn.IN, H = sn.H, A = sn.A[net];
-    const int o1 = (IN + 1) * H, o2 = o1 + (H + 1) * H, o3 = o2 + (H + 1) * A;
-    // which bias row (or the log_std tail) does i fall in?  -1: a weight
-    int bias_layer = -1, j = 0;
-    if (i >= IN * H && i < o1) { bias_layer = 0; j = i - IN * H; }
-    else if (i >= o1 + H * H && i < o2) { bias_layer = 1; j = i - (o1 + H * H); }
-    else if (i >= o2 + H * A && i < o3) { bias_layer = 2; j = i - (o2 + H * A); }
-    else if (i >= o3) { bias_layer = 3; j = i - o3; }
-    // n terms, `stride` floats apart, added in order; loads are issued 16 at a time so that the
-    // chain is 16 times shorter than one dependent load per term
-    const float *p;
-    size_t stride;
-    int n;
-    if (bias_layer < 0) { p = partial + gi; stride = (size_t)Ptot; n = splits; }
-    else if (bias_layer == 3) { p = sn.ls_part[net] + j; stride = (size_t)A; n = tiles; }
-    else {
-        p = sn.db_part[net] + (bias_layer == 0 ? 0 : (bias_layer == 1 ? H : 2 * H)) + j;
-        stride = (size_t)(2 * H + PA_MAX);
-        n = tiles;
-    }
     float s = 0.0f;
-    int q = 0;
-    for (; q + 16 <= n; q += 16) {
-        float v[16];
+    if (gi < Ptot) {
+        int i = gi;
+        if (sn.n > 1 && i >= sn.P[0]) { net = 1; i -= sn.P[0]; }
+        const int IN = sn.IN, H = sn.H, A = sn.A[net];
+        const int o1 = (IN + 1) * H, o2 = o1 + (H + 1) * H, o3 = o2 + (H + 1) * A;
+        // which bias row (or the log_std tail) does i fall in?  -1: a weight
+        int bias_layer = -1, j = 0;
+        if (i >= IN * H && i < o1) { bias_layer = 0; j = i - IN * H; }
+        else if (i >= o1 + H * H && i < o2) { bias_layer = 1; j = i - (o1 + H * H); }
+        else if (i >= o2 + H * A && i < o3) { bias_layer = 2; j = i - (o2 + H * A); }
+        else if (i >= o3) { bias_layer = 3; j = i - o3; }
+        // n terms, `stride` floats apart, added in order; loads are issued 16 at a time so that the
+        // chain is 16 times shorter than one dependent load per term
+        const float *p;
+        size_t stride;
+        int n;
+        if (bias_layer < 0) { p = partial + gi; stride = (size_t)Ptot; n = splits; }
+        else if (bias_layer == 3) { p = sn.ls_part[net] + j; stride = (size_t)A; n = tiles; }
+        else {
+            p = sn.db_part[net] + (bias_layer == 0 ? 0 : (bias_layer == 1 ? H : 2 * H)) + j;
+            stride = (size_t)(2 * H + PA_MAX);
+            n = tiles;
+        }
+        int q = 0;
+        for (; q + 16 <= n; q += 16) {
+            float v[16];
 #pragma unroll
-        for (int k = 0; k < 16; ++k) v[k] = p[(size_t)(q + k) * stride];
+            for (int k = 0; k < 16; ++k) v[k] = p[(size_t)(q + k) * stride];
 #pragma unroll
-        for (int k = 0; k < 16; ++k) s += v[k];
+            for (int k = 0; k < 16; ++k) s += v[k];
+        }
+        for (; q < n; ++q) s += p[(size_t)q * stride];
+        sn.grads[net][i] = s;
     }
-    for (; q < n; ++q) s += p[(size_t)q * stride];
-    sn.grads[net][i] = s;
+    if (sq_part == nullptr) return;
+    // per-block sums of squares, one per net (a block may straddle the two vectors): the partials
+    // of the global-norm clip, sq_part[net * 1024 + block]
+    float v0 = net == 0 ? s * s : 0.0f, v1 = net == 1 ? s * s : 0.0f;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        v0 += __shfl_xor(v0, off, 64);
+        v1 += __shfl_xor(v1, off, 64);
+    }
+    if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = v0; red[1][threadIdx.x >> 6] = v1; }
+    __syncthreads();
+    if (threadIdx.x < 2) {
+        const float *r = red[threadIdx.x];
+        sq_part[threadIdx.x * 1024 + blockIdx.x] = r[0] + r[1] + r[2] + r[3];
+    }
 }
 
 // ---------------------------------------------------------------- host side
@@ -384,7 +417,7 @@ size_t mlp3_backward_ws(const mrl_mlp_desc *const *descs, int n_nets, int batch)
 // backward (parameter gradients only) of one or two nets: io.n[i].grad_out / params / cache in,
 // grads[i] out; ws as sized by mlp3_backward_ws
 int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io,
-                    float *const *grads, float *ws) {
+                    float *const *grads, float *ws, float *sq_part, int *sq_blocks) {
     int H = 0, act = 0;
     bool gauss = false;
     for (int i = 0; i < n_nets; ++i) {
@@ -447,8 +480,11 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
     const int Ptot = base;
     hipLaunchKernelGGL(dw3_kernel, dim3(total_tiles, splits), dim3(256), 0, ctx->stream, dw, batch, rows_per,
                        Ptot, partial);
-    hipLaunchKernelGGL(sum3_kernel, dim3(grid_for(Ptot, 256)), dim3(256), 0, ctx->stream, partial, splits,
-                       Ptot, tiles, sn);
+    const int sum_blocks = grid_for(Ptot, 256);
+    if (sum_blocks > 1024) sq_part = nullptr;   // more partials than the caller's buffer holds
+    if (sq_blocks) *sq_blocks = sq_part ? sum_blocks : 0;
+    hipLaunchKernelGGL(sum3_kernel, dim3(sum_blocks), dim3(256), 0, ctx->stream, partial, splits, Ptot, tiles,
+                       sn, sq_part);
     MRL_CHECK_LAUNCH();
     return MRL_OK;
 }
@@ -459,7 +495,7 @@ int mlp3_backward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *g
     io.n[0].grad_out = grad_out; io.n[0].params = params; io.n[0].cache = const_cast<float *>(cache);
     const mrl_mlp_desc *ds[1] = {&d};
     float *gs[1] = {grads};
-    return mlp3_backward_n(ctx, ds, 1, batch, io, gs, ws);
+    return mlp3_backward_n(ctx, ds, 1, batch, io, gs, ws, nullptr, nullptr);
 }
 
 }  // namespace mrl

@@ -3,8 +3,9 @@
 // call that only enqueues: gather, per-minibatch advantage normalisation, actor and critic
 // forward, loss gradients, KL test, backward, global-norm clip, Adam (and the log_std clamp).
 // The actor and the critic do not depend on each other inside a minibatch, so when both have one
-// of the fused shapes every stage runs them side by side in ONE launch: 11 launches per
-// minibatch instead of about 40, and twice the workgroups per launch.
+// of the fused shapes every stage runs them side by side in ONE launch: 7 launches per
+// minibatch (gather + normalise, forward, loss gradients + KL test, backward dx, dW, sum,
+// clip + Adam) instead of about 40, and twice the workgroups per launch.
 //
 // KL early stop: the reference copies the per-sample KL to the host after the actor's loss
 // gradient and breaks out of the minibatch and epoch loops when its mean exceeds target_kl.
@@ -15,6 +16,7 @@
 #include "mrl_host.hpp"
 #include "mrl_device.hpp"
 #include "mlp3.hpp"
+#include "ppo_grads.hpp"
 
 namespace mrl {
 
@@ -37,21 +39,133 @@ MRL_DEV float u_block_sum(float v, float *smem) {
     return t;
 }
 
-// (x - mean) / (sqrt(var + 1e-8) + 1e-8) over one minibatch in a single workgroup
-// (deep_agents/ppo/kernels.mojo:507-599 is a single-block kernel as well)
-__global__ __launch_bounds__(1024) void normalize_small_kernel(float *__restrict__ x, int n) {
-    __shared__ float smem[16];
-    float s = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 1024) s += x[i];
-    const float mean = u_block_sum<16>(s, smem) / (float)n;
-    float q = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 1024) {
-        const float d = x[i] - mean;
-        q += d * d;
+// ppo_gather_minibatch_kernel (ppo.mojo:135-191) with the per-minibatch advantage normalisation
+// (ppo.mojo:2478-2511) done by one extra workgroup: that one gathers the advantages itself and
+// writes them normalised, the others copy the remaining fields.
+struct GatherArgs {
+    const int32_t *idx;
+    const float *r_obs, *r_act, *r_adv, *r_ret, *r_logp, *r_val;
+    float *mb_obs, *mb_act, *mb_adv, *mb_ret, *mb_logp, *mb_val;
+    int mb, obs_dim, act_dim, normalize;
+};
+
+__global__ __launch_bounds__(UTPB) void gather_norm_kernel(GatherArgs g) {
+    __shared__ float smem[4];
+    if (blockIdx.x == gridDim.x - 1) {
+        constexpr int PER = 32;   // minibatches up to 8192 samples stay in registers
+        if (g.mb <= PER * UTPB) {
+            int src[PER];
+            float v[PER];
+#pragma unroll
+            for (int k = 0; k < PER; ++k) {
+                const int i = threadIdx.x + k * UTPB;
+                src[k] = i < g.mb ? g.idx[i] : -1;
+            }
+#pragma unroll
+            for (int k = 0; k < PER; ++k) v[k] = src[k] >= 0 ? g.r_adv[src[k]] : 0.0f;
+            if (g.normalize) {
+                float s = 0.0f;
+#pragma unroll
+                for (int k = 0; k < PER; ++k) s += v[k];
+                const float mean = u_block_sum<4>(s, smem) / (float)g.mb;
+                float q = 0.0f;
+#pragma unroll
+                for (int k = 0; k < PER; ++k) {
+                    const float d = v[k] - mean;
+                    q += src[k] >= 0 ? d * d : 0.0f;
+                }
+                const float variance = u_block_sum<4>(q, smem) / (float)g.mb;
+                const float std = sqrtf(variance + 1e-8f);
+#pragma unroll
+                for (int k = 0; k < PER; ++k) v[k] = (v[k] - mean) / (std + 1e-8f);
+            }
+#pragma unroll
+            for (int k = 0; k < PER; ++k)
+                if (src[k] >= 0) g.mb_adv[threadIdx.x + k * UTPB] = v[k];
+            return;
+        }
+        float s = 0.0f;
+        for (int i = threadIdx.x; i < g.mb; i += UTPB) s += g.r_adv[g.idx[i]];
+        if (!g.normalize) {
+            for (int i = threadIdx.x; i < g.mb; i += UTPB) g.mb_adv[i] = g.r_adv[g.idx[i]];
+            return;
+        }
+        const float mean = u_block_sum<4>(s, smem) / (float)g.mb;
+        float q = 0.0f;
+        for (int i = threadIdx.x; i < g.mb; i += UTPB) {
+            const float d = g.r_adv[g.idx[i]] - mean;
+            q += d * d;
+        }
+        const float variance = u_block_sum<4>(q, smem) / (float)g.mb;
+        const float std = sqrtf(variance + 1e-8f);
+        for (int i = threadIdx.x; i < g.mb; i += UTPB) g.mb_adv[i] = (g.r_adv[g.idx[i]] - mean) / (std + 1e-8f);
+        return;
     }
-    const float variance = u_block_sum<16>(q, smem) / (float)n;
-    const float std = sqrtf(variance + 1e-8f);
-    for (int i = threadIdx.x; i < n; i += 1024) x[i] = (x[i] - mean) / (std + 1e-8f);
+    const long i = (long)blockIdx.x * UTPB + threadIdx.x;
+    const int w = g.obs_dim;
+    if (i >= (long)g.mb * w) return;
+    const int b = (int)(i / w), c = (int)(i - (long)b * w);
+    const long src = g.idx[b];
+    g.mb_obs[i] = g.r_obs[src * g.obs_dim + c];
+    if (c < g.act_dim) g.mb_act[(long)b * g.act_dim + c] = g.r_act[src * g.act_dim + c];
+    if (c == 0) {
+        g.mb_ret[b] = g.r_ret[src];
+        g.mb_logp[b] = g.r_logp[src];
+        g.mb_val[b] = g.r_val[src];
+    }
+}
+
+// Actor and critic loss gradients in one launch (grid.y = 0: actor, 1: critic) and the KL test:
+// every actor workgroup leaves the sum of its samples' KL estimates, the last one to arrive adds
+// them up in workgroup order, compares the mean with target_kl and re-arms the counter.
+struct LossArgs {
+    const float *actor_out, *mb_logp, *mb_adv, *mb_act, *values, *mb_val, *mb_ret;
+    float *g_actor_out, *g_values, *kl;
+    float *kl_part;      // [grid.x]
+    int *arrived;        // zero between launches
+    int32_t *kl_flag;    // nullable: no test
+    int mb, A, continuous, clip_value;
+    float clip_eps, ent_coef, value_coef, target_kl;
+};
+
+__global__ __launch_bounds__(UTPB) void loss_grads_kernel(LossArgs a) {
+    __shared__ float smem[4];
+    __shared__ int last;
+    const int b = blockIdx.x * UTPB + threadIdx.x;
+    if (blockIdx.y == 1) {
+        if (b < a.mb)
+            a.g_values[b] = critic_grad_one(b, a.values, a.mb_val, a.mb_ret, a.mb, a.continuous, a.clip_value,
+                                            a.value_coef, a.clip_eps);
+        return;
+    }
+    float kl = 0.0f;
+    if (b < a.mb) {
+        kl = a.continuous ? actor_grad_gaussian_one(b, a.actor_out, a.mb_logp, a.mb_adv, a.mb_act, a.mb, a.A,
+                                                    a.clip_eps, a.ent_coef, a.g_actor_out)
+                          : actor_grad_discrete_one(b, a.actor_out, a.mb_logp, a.mb_adv, a.mb_act, a.mb, a.A,
+                                                    a.clip_eps, a.ent_coef, a.g_actor_out);
+        a.kl[b] = kl;
+    }
+    if (a.kl_flag == nullptr) return;
+    const float s = u_block_sum<4>(kl, smem);
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&a.kl_part[blockIdx.x], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence();
+        last = atomicAdd(a.arrived, 1) == (int)gridDim.x - 1;
+    }
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    float t = 0.0f;
+    for (int i = threadIdx.x; i < (int)gridDim.x; i += UTPB)
+        t += __hip_atomic_load(&a.kl_part[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    t = u_block_sum<4>(t, smem);
+    if (threadIdx.x == 0) {
+        const float mean = t / (float)a.mb;
+        a.kl_flag[1] = __float_as_int(mean);
+        if (mean > a.target_kl) a.kl_flag[0] = 1;
+        *a.arrived = 0;
+    }
 }
 
 struct AdamNet {
@@ -76,7 +190,8 @@ __global__ __launch_bounds__(UTPB) void sq_partial2_kernel(AdamNets nets, float 
 // global-norm clip (ppo.mojo:382-534; actor and critic separately) + Adam (adam.mojo:52-105)
 // + log_std clamp (kernels.mojo:842-873); grid = (blocks, nets).  Does nothing once stop[0] != 0.
 __global__ __launch_bounds__(UTPB) void clip_adam2_kernel(AdamNets nets, const float *__restrict__ partial,
-                                                          int nb, float max_norm, float beta1, float beta2,
+                                                          int nb, int part_stride, float max_norm, float beta1,
+                                                          float beta2,
                                                           float omb1, float omb2, float eps,
                                                           int32_t *__restrict__ stop) {
     __shared__ float smem[4];
@@ -86,7 +201,7 @@ __global__ __launch_bounds__(UTPB) void clip_adam2_kernel(AdamNets nets, const f
     float scale = 1.0f;
     if (max_norm > 0.0f) {
         float s = 0.0f;
-        for (int i = threadIdx.x; i < nb; i += UTPB) s += partial[blockIdx.y * nb + i];
+        for (int i = threadIdx.x; i < nb; i += UTPB) s += partial[blockIdx.y * part_stride + i];
         s = u_block_sum<4>(s, smem);
         if (threadIdx.x == 0) {
             const float norm = sqrtf(s);
@@ -153,18 +268,14 @@ int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *i
     const int Pa = mrl_mlp_param_size(&u->actor), Pc = mrl_mlp_param_size(&u->critic);
     const bool cont = u->continuous != 0;
 
-    rc = mrl_gather_minibatch(ctx, indices, mb, u->obs_dim, u->act_width, u->r_obs, u->r_actions, u->advantages,
-                              u->returns, u->r_log_probs, u->r_values, u->mb_obs, u->mb_actions, u->mb_adv,
-                              u->mb_ret, u->mb_logp, u->mb_val);
-    if (rc) return rc;
-    if (u->norm_adv_per_minibatch) {
-        if (mb <= 65536) {
-            hipLaunchKernelGGL(normalize_small_kernel, dim3(1), dim3(1024), 0, ctx->stream, u->mb_adv, mb);
-            MRL_CHECK_LAUNCH();
-        } else {
-            rc = mrl_normalize_advantages(ctx, u->mb_adv, mb);
-            if (rc) return rc;
-        }
+    {
+        GatherArgs g{indices, u->r_obs, u->r_actions, u->advantages, u->returns, u->r_log_probs, u->r_values,
+                     u->mb_obs, u->mb_actions, u->mb_adv, u->mb_ret, u->mb_logp, u->mb_val,
+                     mb, u->obs_dim, u->act_width, u->norm_adv_per_minibatch};
+        MRL_CHECK_ARG(u->act_width <= u->obs_dim, "mrl_ppo_update_minibatch: action wider than observation");
+        hipLaunchKernelGGL(gather_norm_kernel, dim3(grid_for((long)mb * u->obs_dim, UTPB) + 1), dim3(UTPB), 0,
+                           ctx->stream, g);
+        MRL_CHECK_LAUNCH();
     }
 
     const mrl_mlp_desc *descs[2] = {&u->actor, &u->critic};
@@ -184,29 +295,32 @@ int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *i
         if (rc) return rc;
     }
 
-    if (cont)
-        rc = mrl_ppo_actor_grad_gaussian(ctx, u->actor_out, u->mb_logp, u->mb_adv, u->mb_actions, mb, u->act_width,
-                                         u->clip_epsilon, u->entropy_coef, u->g_actor_out, u->kl);
-    else
-        rc = mrl_ppo_actor_grad_discrete(ctx, u->actor_out, u->mb_logp, u->mb_adv, u->mb_actions, mb, head,
-                                         u->clip_epsilon, u->entropy_coef, u->g_actor_out, u->kl);
-    if (rc) return rc;
-    if (u->target_kl > 0.0f) {
-        rc = mrl_kl_check(ctx, u->kl, mb, u->target_kl, u->kl_flag);
-        if (rc) return rc;
+    {
+        const int nblk = grid_for(mb, UTPB);
+        const bool test = u->target_kl > 0.0f && nblk <= 1024;
+        LossArgs a{u->actor_out, u->mb_logp, u->mb_adv, u->mb_actions, u->values, u->mb_val, u->mb_ret,
+                   u->g_actor_out, u->g_values, u->kl, ctx->upd_scratch,
+                   reinterpret_cast<int *>(ctx->upd_scratch + 1024), test ? u->kl_flag : nullptr,
+                   mb, cont ? u->act_width : head, cont ? 1 : 0, u->clip_value ? 1 : 0,
+                   u->clip_epsilon, u->entropy_coef, u->value_loss_coef, u->target_kl};
+        hipLaunchKernelGGL(loss_grads_kernel, dim3(nblk, 2), dim3(UTPB), 0, ctx->stream, a);
+        MRL_CHECK_LAUNCH();
+        if (u->target_kl > 0.0f && !test) {
+            rc = mrl_kl_check(ctx, u->kl, mb, u->target_kl, u->kl_flag);
+            if (rc) return rc;
+        }
     }
-    rc = mrl_ppo_critic_grad(ctx, u->values, u->clip_value ? u->mb_val : nullptr, u->mb_ret, mb, cont ? 1 : 0,
-                             u->clip_value ? 1 : 0, u->value_loss_coef, u->clip_epsilon, u->g_values);
-    if (rc) return rc;
 
     io.n[0].grad_out = u->g_actor_out;
     io.n[1].grad_out = u->g_values;
     float *grads[2] = {u->actor_grads, u->critic_grads};
+    int sq_blocks = 0;   // > 0: the backward pass already left the sum-of-squares partials
     if (paired) {
         float *ws = nullptr;
         rc = mlp_ensure_ws(ctx, mlp3_backward_ws(descs, 2, mb), &ws);
         if (rc) return rc;
-        rc = mlp3_backward_n(ctx, descs, 2, mb, io, grads, ws);
+        rc = mlp3_backward_n(ctx, descs, 2, mb, io, grads, ws,
+                             u->max_grad_norm > 0.0f ? ctx->upd_scratch + 2048 : nullptr, &sq_blocks);
         if (rc) return rc;
     } else {
         rc = mrl_mlp_backward(ctx, &u->actor, mb, u->g_actor_out, u->actor_params, u->actor_cache, u->actor_grads,
@@ -229,12 +343,17 @@ int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *i
     fill(an.n[1], u->critic_params, u->critic_grads, u->critic_state, Pc, u->critic_lr, critic_t);
     if (cont) { an.n[0].clamp_off = Pa - u->act_width; an.n[0].clamp_n = u->act_width; }
     const int nmax = std::max(Pa, Pc);
-    const int nb = std::min(256, grid_for(nmax, UTPB));
-    float *part = ctx->reduce_scratch + 1024;   // [2][nb], nb <= 256
-    if (u->max_grad_norm > 0.0f)
-        hipLaunchKernelGGL(sq_partial2_kernel, dim3(nb, 2), dim3(UTPB), 0, ctx->stream, an, part);
+    int nb = sq_blocks, stride = 1024;
+    const float *part = ctx->upd_scratch + 2048;
+    if (u->max_grad_norm > 0.0f && sq_blocks == 0) {
+        nb = std::min(256, grid_for(nmax, UTPB));
+        stride = nb;
+        float *p2 = ctx->reduce_scratch + 1024;   // [2][nb], nb <= 256
+        hipLaunchKernelGGL(sq_partial2_kernel, dim3(nb, 2), dim3(UTPB), 0, ctx->stream, an, p2);
+        part = p2;
+    }
     hipLaunchKernelGGL(clip_adam2_kernel, dim3(grid_for(nmax, UTPB), 2), dim3(UTPB), 0, ctx->stream, an, part, nb,
-                       u->max_grad_norm, (float)u->beta1, (float)u->beta2, (float)(1.0 - u->beta1),
+                       stride, u->max_grad_norm, (float)u->beta1, (float)u->beta2, (float)(1.0 - u->beta1),
                        (float)(1.0 - u->beta2), (float)u->eps, u->target_kl > 0.0f ? u->kl_flag : nullptr);
     MRL_CHECK_LAUNCH();
     return MRL_OK;

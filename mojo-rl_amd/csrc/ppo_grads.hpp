@@ -1,0 +1,143 @@
+// Per-sample loss gradients of the PPO agents, shared by the stand-alone kernels (mrl_ppo.hip) and
+// the merged kernel of the minibatch update (mrl_update.hip).
+#pragma once
+#include "mrl_device.hpp"
+
+namespace mrl {
+
+// deep_agents/ppo/ppo.mojo:285-378; returns the sample's KL estimate (old - new log-prob)
+MRL_DEV float actor_grad_discrete_one(int b, const float *__restrict__ logits, const float *__restrict__ old_logp,
+                                      const float *__restrict__ adv, const float *__restrict__ actions, int mb,
+                                      int A, float clip_eps, float ent_coef, float *__restrict__ grad_logits) {
+    const float *l = logits + (long)b * A;
+    int action = (int)actions[b];
+    float advantage = adv[b];
+    float max_logit = l[0];
+    for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
+    float sum_exp = 0.0f;
+    for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
+    float p_action = 0.0f;
+    for (int a = 0; a < A; ++a) {
+        float p = expf(l[a] - max_logit) / sum_exp;
+        if (a == action) p_action = p;
+    }
+    float new_logp = logf(p_action + 1e-8f);
+    float old = old_logp[b];
+    float ratio = expf(new_logp - old);
+    bool clipped = (ratio < 1.0f - clip_eps) || (ratio > 1.0f + clip_eps);
+    for (int a = 0; a < A; ++a) {
+        float g = 0.0f;
+        if (!clipped) {
+            float p = expf(l[a] - max_logit) / sum_exp;
+            float d_log_prob = (a == action) ? 1.0f - p : -p;
+            float log_prob_ent = logf(p + 1e-8f);
+            float d_entropy = -p * (1.0f + log_prob_ent);
+            g = (-advantage * ratio * d_log_prob - ent_coef * d_entropy) / (float)mb;
+        }
+        grad_logits[(long)b * A + a] = g;
+    }
+    return old - new_logp;
+}
+
+// deep_agents/ppo/kernels.mojo:230-412; returns the sample's KL estimate ((ratio - 1) - diff, clamped)
+MRL_DEV float actor_grad_gaussian_one(int b, const float *__restrict__ actor_out, const float *__restrict__ old_logp,
+                                      const float *__restrict__ adv, const float *__restrict__ actions, int mb,
+                                      int A, float clip_eps, float ent_coef, float *__restrict__ grad_out) {
+    const float eps = 1e-6f, log_2pi = (float)1.8378770664093453;
+    const float *o = actor_out + (long)b * 2 * A;
+    const float *act = actions + (long)b * A;
+    float advantage = adv[b], old_log_prob = old_logp[b];
+    float new_log_prob = 0.0f;
+    for (int j = 0; j < A; ++j) {
+        float log_std = o[A + j];
+        if (log_std < -5.0f) log_std = -5.0f;
+        else if (log_std > 2.0f) log_std = 2.0f;
+        float std = expf(log_std);
+        float an = (act[j] - o[j]) / (std + eps);
+        float lg = -0.5f * (log_2pi + 2.0f * log_std + an * an);
+        new_log_prob = new_log_prob + lg;
+    }
+    float diff = new_log_prob - old_log_prob;
+    if (diff > 20.0f) diff = 20.0f;
+    else if (diff < -20.0f) diff = -20.0f;
+    float ratio = expf(diff);
+    float kl = (ratio - 1.0f) - diff;
+    if (kl < 0.0f) kl = 0.0f;
+    else if (kl > 100.0f) kl = 100.0f;
+    float clipped_ratio = ratio;
+    if (clipped_ratio < 1.0f - clip_eps) clipped_ratio = 1.0f - clip_eps;
+    else if (clipped_ratio > 1.0f + clip_eps) clipped_ratio = 1.0f + clip_eps;
+    bool is_clipped = clipped_ratio * advantage < ratio * advantage;
+    float *g = grad_out + (long)b * 2 * A;
+    for (int j = 0; j < A; ++j) {
+        float gm = 0.0f, gs = 0.0f;
+        if (!is_clipped) {
+            float log_std = o[A + j];
+            if (log_std < -5.0f) log_std = -5.0f;
+            else if (log_std > 2.0f) log_std = 2.0f;
+            float std = expf(log_std);
+            float an = (act[j] - o[j]) / (std + eps);
+            float d_mean = an / (std + eps);
+            float d_log_std = an * an - 1.0f;
+            gm = (-advantage * ratio * d_mean) / (float)mb;
+            gs = (-advantage * ratio * d_log_std - ent_coef * 1.0f) / (float)mb;
+            if (gm > 10.0f) gm = 10.0f;
+            else if (gm < -10.0f) gm = -10.0f;
+            if (gs > 10.0f) gs = 10.0f;
+            else if (gs < -10.0f) gs = -10.0f;
+        }
+        g[j] = gm;
+        g[A + j] = gs;
+    }
+    return kl;
+}
+
+// ppo.mojo:538-633 (convention 0) and kernels.mojo:416-486 (convention 1)
+MRL_DEV float critic_grad_one(int b, const float *__restrict__ values, const float *__restrict__ old_values,
+                              const float *__restrict__ returns, int mb, int convention, int clipped,
+                              float value_coef, float clip_eps) {
+    float v = values[b], ret = returns[b];
+    float out;
+    if (convention == 0) {
+        if (!clipped) {
+            out = 2.0f * value_coef * (v - ret) / (float)mb;
+        } else {
+            float v_old = old_values[b];
+            float v_diff = v - v_old;
+            float v_clipped;
+            if (v_diff > clip_eps) v_clipped = v_old + clip_eps;
+            else if (v_diff < -clip_eps) v_clipped = v_old - clip_eps;
+            else v_clipped = v;
+            float loss_unclipped = (v - ret) * (v - ret);
+            float loss_clipped = (v_clipped - ret) * (v_clipped - ret);
+            float g;
+            if (loss_unclipped > loss_clipped) g = 2.0f * (v - ret);
+            else if (v_diff > clip_eps || v_diff < -clip_eps) g = 0.0f;
+            else g = 2.0f * (v - ret);
+            out = value_coef * g / (float)mb;
+        }
+    } else {
+        if (!clipped) {
+            out = (v - ret) / (float)mb;
+        } else {
+            float old_value = old_values[b];
+            float d = v - old_value;
+            float mn = d < clip_eps ? d : clip_eps;
+            float mx = mn > -clip_eps ? mn : -clip_eps;
+            float value_clipped = old_value + mx;
+            float loss_unclipped = (v - ret) * (v - ret);
+            float loss_clipped = (value_clipped - ret) * (value_clipped - ret);
+            if (loss_clipped > loss_unclipped) {
+                float clip_sign = 1.0f;
+                if (v - old_value > clip_eps) clip_sign = 0.0f;
+                else if (v - old_value < -clip_eps) clip_sign = 0.0f;
+                out = clip_sign * (value_clipped - ret) / (float)mb;
+            } else {
+                out = (v - ret) / (float)mb;
+            }
+        }
+    }
+    return out;
+}
+
+}  // namespace mrl
