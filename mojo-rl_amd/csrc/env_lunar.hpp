@@ -287,26 +287,44 @@ MRL_DEV void apply_engines(float *row, int env, int step_count, double m_power, 
     B[IDX_OMEGA] = (float)(omega + domega);
 }
 
-// one env step on an LDS-resident row; `contacts` = this lane's 8*9 scratch
-MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env, int action,
-                      float &reward, float &done) {
-    if (row[L::META_OFF + META_DONE] > 0.5f) {
+// An env step in two halves, so that contact detection -- which reads positions only -- can run
+// on other wavefronts while this one applies the engines (which write velocities only):
+//   step_begin   already-finished short-circuit, engine impulses;
+//   step_finish  physics with the `n` contacts given in `contacts` (n < 0: detect here),
+//                observation, reward, termination.
+struct StepCarry {
+    int step_count;
+    double m_power, s_power;
+    bool skip;   // the row was already finished: reward 0, done 1, nothing moves
+};
+
+MRL_DEV StepCarry step_begin(float *row, int env, int action) {
+    StepCarry c;
+    c.skip = row[L::META_OFF + META_DONE] > 0.5f;
+    c.step_count = (int)row[L::META_OFF + META_STEP];
+    c.m_power = 0.0; c.s_power = 0.0;
+    double direction = 0.0;
+    if (action == 2) c.m_power = 1.0;
+    else if (action == 1) { c.s_power = 1.0; direction = -1.0; }
+    else if (action == 3) { c.s_power = 1.0; direction = 1.0; }
+    if (!c.skip) apply_engines(row, env, c.step_count, c.m_power, c.s_power, direction);
+    return c;
+}
+
+MRL_DEV void step_finish(float *row, float *contacts, int n_given, const float *shapes, const StepCarry &c,
+                         float &reward, float &done) {
+    if (c.skip) {
         reward = 0.0f;
         done = 1.0f;
         return;
     }
-    int step_count = (int)row[L::META_OFF + META_STEP];
-    double m_power = 0.0, s_power = 0.0, direction = 0.0;
-    if (action == 2) m_power = 1.0;
-    else if (action == 1) { s_power = 1.0; direction = -1.0; }
-    else if (action == 3) { s_power = 1.0; direction = 1.0; }
-    apply_engines(row, env, step_count, m_power, s_power, direction);
-
+    const double m_power = c.m_power, s_power = c.s_power;
+    int step_count = c.step_count;
     const float gx = (float)0.0, gy = (float)-10.0, dt = (float)DT;
     const float friction = (float)0.1, restitution = (float)0.0;
     const float baumgarte = (float)0.2, slop = (float)0.005;
-    const int n = reg_physics_substep<L, Topology, false, true>(row, shapes, contacts, gx, gy, dt, friction, restitution,
-                                                baumgarte, slop, 6, 2);
+    const int n = reg_physics_substep<L, Topology, false, true>(row, shapes, contacts, gx, gy, dt, friction,
+                                                                restitution, baumgarte, slop, 6, 2, n_given);
 
     step_count += 1;
     float obs[8];
@@ -322,8 +340,8 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
     bool both_legs = obs[6] > 0.5f && obs[7] > 0.5f;
     double speed = ::sqrt(vx * vx + vy * vy);
     bool lander_contact = false;
-    for (int c = 0; c < n; ++c)
-        if ((int)contacts[c * CONTACT_SIZE + C_BODY_A] == 0) lander_contact = true;
+    for (int k = 0; k < n; ++k)
+        if ((int)contacts[k * CONTACT_SIZE + C_BODY_A] == 0) lander_contact = true;
     if (lander_contact) { terminated = true; r = -100.0f; }
     if (speed < 0.01 && ::fabs(omega) < 0.01 && both_legs) { terminated = true; r = r + 100.0f; }
     if (step_count >= 1000) terminated = true;
@@ -335,6 +353,13 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
     row[L::META_OFF + META_DONE] = terminated ? 1.0f : 0.0f;
     reward = r;
     done = terminated ? 1.0f : 0.0f;
+}
+
+// one env step on an LDS-resident row by one lane; `contacts` = this lane's contact scratch
+MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env, int action,
+                      float &reward, float &done) {
+    const StepCarry c = step_begin(row, env, action);
+    step_finish(row, contacts, -1, shapes, c, reward, done);
 }
 
 }  // namespace ll

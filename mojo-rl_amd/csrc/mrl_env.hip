@@ -134,6 +134,14 @@ struct LunarLander {
     static MRL_DEV void reset_wave(float *row, uint64_t seed, int env, int lane) {
         ll::reset_row_wave(row, ll::combined_seed(seed, env), lane);
     }
+    // contact detection of body k runs on wavefront k + 1 while wavefront 0 applies the engines
+    static constexpr int DETECT_WAVES = L::NUM_BODIES;
+    using Carry = ll::StepCarry;
+    static MRL_DEV Carry step_begin(float *row, int env, const float *a) { return ll::step_begin(row, env, (int)a[0]); }
+    static MRL_DEV void step_finish(float *row, float *cts, int n, const float *shapes, const Carry &c, float &r,
+                                    float &d) {
+        ll::step_finish(row, cts, n, shapes, c, r, d);
+    }
 };
 
 struct BipedalWalker {
@@ -147,6 +155,10 @@ struct BipedalWalker {
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { bw::reset_row(row, walker_seed(seed, env)); }
     static constexpr bool WAVE_RESET = false;
     static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
+    static constexpr int DETECT_WAVES = 0;
+    struct Carry {};
+    static MRL_DEV Carry step_begin(float *, int, const float *) { return Carry{}; }
+    static MRL_DEV void step_finish(float *, float *, int, const float *, const Carry &, float &, float &) {}
 };
 
 struct HalfCheetah {
@@ -160,6 +172,10 @@ struct HalfCheetah {
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { hc::reset_row(row, walker_seed(seed, env)); }
     static constexpr bool WAVE_RESET = false;
     static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
+    static constexpr int DETECT_WAVES = 0;
+    struct Carry {};
+    static MRL_DEV Carry step_begin(float *, int, const float *) { return Carry{}; }
+    static MRL_DEV void step_finish(float *, float *, int, const float *, const Carry &, float &, float &) {}
 };
 
 constexpr int WAVE = 64;    // the compute phase runs on one wavefront, one lane per env
@@ -243,19 +259,61 @@ __global__ __launch_bounds__(BLOCK) void phys_step_kernel(float *states, const f
     if (tid < E::EPB) was_reset[tid] = 0;
     __syncthreads();
 
-    if (tid < WAVE) {
-        bool finished = false;
-        if (tid < nenv) {
-            const int env = env0 + tid;
-            float r, d;
-            E::step(rows + tid * S::STRIDE, cts + tid * S::CSTRIDE, shapes, env,
-                    actions + (size_t)env * E::ACT_W, r, d);
-            rewards[env] = r;
-            dones[env] = d;
-            account(acc, env, r, d);
-            finished = d > 0.5f;
+    if constexpr (E::DETECT_WAVES > 0) {
+        // wavefront 0: first half of the step (reads and writes velocities only); wavefronts
+        // 1 .. DETECT_WAVES: contacts of one body each (read positions only), into their own lists
+        constexpr int DW = E::DETECT_WAVES > 0 ? E::DETECT_WAVES : 1;
+        constexpr int LSTRIDE = (E::L::MAX_CONTACTS * CONTACT_SIZE) | 1;
+        __shared__ float dlist[DW * E::EPB * LSTRIDE];
+        __shared__ int dcount[DW * E::EPB];
+        static_assert(E::DETECT_WAVES < BLOCK / WAVE, "one wavefront per body besides wavefront 0");
+        const int wave = tid / WAVE, lane = tid % WAVE;
+        typename E::Carry carry{};
+        if (wave == 0) {
+            if (lane < nenv)
+                carry = E::step_begin(rows + lane * S::STRIDE, env0 + lane, actions + (size_t)(env0 + lane) * E::ACT_W);
+        } else if (wave <= E::DETECT_WAVES && lane < nenv) {
+            dcount[(wave - 1) * E::EPB + lane] = edge_detect_body<typename E::L>(
+                rows + lane * S::STRIDE, shapes, wave - 1, dlist + ((wave - 1) * E::EPB + lane) * LSTRIDE);
         }
-        if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, tid);
+        __syncthreads();
+        if (wave == 0) {
+            bool finished = false;
+            if (lane < nenv) {
+                // concatenate the bodies' lists in body order, cut at MAX_CONTACTS
+                float *mine = cts + lane * S::CSTRIDE;
+                int n = 0;
+                for (int k = 0; k < E::DETECT_WAVES; ++k) {
+                    const float *src = dlist + (k * E::EPB + lane) * LSTRIDE;
+                    const int m = dcount[k * E::EPB + lane];
+                    for (int c = 0; c < m && n < E::L::MAX_CONTACTS; ++c, ++n)
+                        for (int f = 0; f < CONTACT_SIZE; ++f) mine[n * CONTACT_SIZE + f] = src[c * CONTACT_SIZE + f];
+                }
+                const int env = env0 + lane;
+                float r, d;
+                E::step_finish(rows + lane * S::STRIDE, mine, n, shapes, carry, r, d);
+                rewards[env] = r;
+                dones[env] = d;
+                account(acc, env, r, d);
+                finished = d > 0.5f;
+            }
+            if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, lane);
+        }
+    } else {
+        if (tid < WAVE) {
+            bool finished = false;
+            if (tid < nenv) {
+                const int env = env0 + tid;
+                float r, d;
+                E::step(rows + tid * S::STRIDE, cts + tid * S::CSTRIDE, shapes, env,
+                        actions + (size_t)env * E::ACT_W, r, d);
+                rewards[env] = r;
+                dones[env] = d;
+                account(acc, env, r, d);
+                finished = d > 0.5f;
+            }
+            if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, tid);
+        }
     }
     __syncthreads();
 

@@ -270,6 +270,73 @@ MRL_DEV int edge_detect(const float *row, const float *shapes, float *contacts) 
     return count;
 }
 
+// edge_detect restricted to body b (short polylines only): the contacts body b contributes, in
+// the same (vertex, edge) order, counted from zero.  Concatenating the lists of bodies 0, 1, ...
+// and cutting at MAX_CONTACTS reproduces edge_detect, which lets different wavefronts detect
+// different bodies of the same env at the same time.
+template <class L>
+MRL_DEV int edge_detect_body(const float *row, const float *shapes, int b, float *contacts) {
+    static_assert(L::MAX_EDGES <= 16, "per-body detection keeps the edge x ranges in registers");
+    int count = 0;
+    const int n_edges = (int)row[L::EDGE_COUNT_OFF];
+    const float *edges = row + L::EDGES_OFF;
+    float ex0[L::MAX_EDGES], ex1[L::MAX_EDGES];
+#pragma unroll
+    for (int e = 0; e < L::MAX_EDGES; ++e) {
+        ex0[e] = edges[e * 6];
+        ex1[e] = edges[e * 6 + 2];
+    }
+    const float *B = row + L::BODIES_OFF + b * BODY_SIZE;
+    const float body_x = B[IDX_X], body_y = B[IDX_Y];
+    const float *S = shapes + (int)B[IDX_SHAPE] * SHAPE_SIZE;
+    const int shape_type = (int)S[0];
+    float sin_a, cos_a;
+    sincos32(B[IDX_ANGLE], sin_a, cos_a);
+    if (shape_type == SHAPE_POLYGON) {
+        int n_verts = (int)S[1];
+        if (n_verts > MAX_POLY_VERTS) n_verts = MAX_POLY_VERTS;
+        for (int v = 0; v < n_verts; ++v) {
+            const float local_x = S[2 + v * 2], local_y = S[3 + v * 2];
+            const float world_x = body_x + local_x * cos_a - local_y * sin_a;
+            const float world_y = body_y + local_x * sin_a + local_y * cos_a;
+            unsigned mask = 0;
+#pragma unroll
+            for (int e = 0; e < L::MAX_EDGES; ++e)
+                if (e < n_edges && edge_x_pass(ex0[e], ex1[e], world_x)) mask |= 1u << e;
+            while (mask) {
+                const int e = __ffs((int)mask) - 1;
+                mask &= mask - 1;
+                vertex_edge_test(edges + e * 6, b, world_x, world_y, contacts, count, L::MAX_CONTACTS);
+            }
+        }
+    } else if (shape_type == SHAPE_CIRCLE) {
+        const float radius = S[1], cox = S[2], coy = S[3];
+        const float cwx = body_x + cox * cos_a - coy * sin_a;
+        const float cwy = body_y + cox * sin_a + coy * cos_a;
+        for (int e = 0; e < n_edges; ++e) {
+            const float *E = edges + e * 6;
+            float e_x0 = E[0], e_y0 = E[1], e_x1 = E[2], e_y1 = E[3], e_nx = E[4], e_ny = E[5];
+            float edge_dx = e_x1 - e_x0, edge_dy = e_y1 - e_y0;
+            float edge_len_sq = edge_dx * edge_dx + edge_dy * edge_dy;
+            if (edge_len_sq < 1e-6f) continue;
+            float t = ((cwx - e_x0) * edge_dx + (cwy - e_y0) * edge_dy) / edge_len_sq;
+            if (t < 0.0f) t = 0.0f;
+            if (t > 1.0f) t = 1.0f;
+            float closest_x = e_x0 + t * edge_dx, closest_y = e_y0 + t * edge_dy;
+            float dist_x = cwx - closest_x, dist_y = cwy - closest_y;
+            float dist = sqrtf(dist_x * dist_x + dist_y * dist_y);
+            float penetration = radius - dist;
+            if (penetration > 0.0f && count < L::MAX_CONTACTS) {
+                float cnx = e_nx, cny = e_ny;
+                if (dist > 1e-6f) { cnx = dist_x / dist; cny = dist_y / dist; }
+                put_contact(contacts + count * CONTACT_SIZE, b, closest_x, closest_y, cnx, cny, penetration);
+                count += 1;
+            }
+        }
+    }
+    return count;
+}
+
 template <class L>
 MRL_DEV int flat_detect(const float *row, const float *shapes, float ground_y, float *contacts) {
     int count = 0;

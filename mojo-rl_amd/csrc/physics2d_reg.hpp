@@ -477,12 +477,13 @@ MRL_DEV bool topology_matches(const float *row) {
 template <class L, class T, bool FLAT, bool REG_CONTACTS>
 MRL_DEV int reg_physics_substep_impl(float *row, const float *shapes, float *contacts, float gx, float gy,
                                      float dt, float friction, float restitution, float baumgarte,
-                                     float slop, int vel_iters, int pos_iters) {
+                                     float slop, int vel_iters, int pos_iters, int n_given) {
     RegBodies<L> B;
     B.load(row);
     reg_integrate_velocities<L>(B, row, gx, gy, dt);
     // the detectors read positions and angles only, which the velocity update has not touched
-    const int n = FLAT ? flat_detect<L>(row, shapes, 0.0f, contacts) : edge_detect<L>(row, shapes, contacts);
+    const int n = n_given >= 0 ? n_given
+                  : (FLAT ? flat_detect<L>(row, shapes, 0.0f, contacts) : edge_detect<L>(row, shapes, contacts));
     typename std::conditional<REG_CONTACTS, RegContacts<L>, LdsContacts<L>>::type C;
     C.load(B, contacts, n);
     RegJoints<L, T> J;
@@ -507,17 +508,19 @@ MRL_DEV int reg_physics_substep_impl(float *row, const float *shapes, float *con
 // MAX_CONTACTS * CONTACT_SCRATCH floats (detection order and the MAX_CONTACTS cut-off unchanged;
 // afterwards the body indices of the contacts are still readable at
 // contacts[c * CONTACT_SIZE + C_BODY_A / C_BODY_B], the contact-point slots are not), then
-// everything iterative runs on registers.
+// everything iterative runs on registers.  n_given >= 0: `contacts` already holds that many
+// contacts detected from the row's current positions (detection is skipped).
 template <class L, class T, bool FLAT, bool REG_CONTACTS>
 MRL_DEV int reg_physics_substep(float *row, const float *shapes, float *contacts, float gx, float gy,
                                 float dt, float friction, float restitution, float baumgarte, float slop,
-                                int vel_iters, int pos_iters) {
+                                int vel_iters, int pos_iters, int n_given = -1) {
     if (T::STATIC && __all(topology_matches<L, T>(row) ? 1 : 0))
         return reg_physics_substep_impl<L, T, FLAT, REG_CONTACTS>(row, shapes, contacts, gx, gy, dt, friction,
                                                                   restitution, baumgarte, slop, vel_iters,
-                                                                  pos_iters);
+                                                                  pos_iters, n_given);
     return reg_physics_substep_impl<L, DynamicTopology, FLAT, REG_CONTACTS>(
-        row, shapes, contacts, gx, gy, dt, friction, restitution, baumgarte, slop, vel_iters, pos_iters);
+        row, shapes, contacts, gx, gy, dt, friction, restitution, baumgarte, slop, vel_iters, pos_iters,
+        n_given);
 }
 
 }  // namespace mrl
