@@ -11,7 +11,7 @@ struct Mlp3Net {
     float *out;              // forward: [B, A] or [B, 2A]
     float *cache;            // forward: written when non-null; backward: read
     const float *grad_out;   // backward
-    float *g1, *g0, *ls_part, *db_part;  // backward workspace (set by the host function)
+    float *g1, *g0, *ls_part, *db_part, *thin_part;  // backward workspace (set by the host function)
     int A, gauss;            // set by the host function from the description
 };
 struct Mlp3Nets { Mlp3Net n[2]; };

@@ -93,27 +93,34 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
     float *__restrict__ ls_part = nn.ls_part;
     float *__restrict__ db_part = nn.db_part + (size_t)blockIdx.x * (2 * H + PA_MAX);   // this tile's slice
     const int A = nn.A;
+    // this tile's share of the two thin weight gradients: [dW0 (IN x H) | dW2 (H x A)]
+    float *__restrict__ thin_part = nn.thin_part + (size_t)blockIdx.x * ((size_t)IN * H + (size_t)H * A);
     const bool GAUSS = nn.gauss != 0;
     constexpr int KCH = 32;                       // k-chunk of W1 staged per round
     __shared__ float g2s[PR * (2 * PA_MAX + 1)];
+    __shared__ float xs[PR * XS_LD];              // the tile's inputs, for dW0
     __shared__ float gT[H * HT_LD];               // g1 of the tile, k-major
     __shared__ float wT[KCH * (H + 1)];           // W1[i][o0 + k] stored as [k][i]
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
     const long row0 = (long)blockIdx.x * PR;
     const int nrow = (int)min((long)PR, B - row0);
     const int ld = GAUSS ? 2 * A : A;
-    const float *c0 = cache, *c1 = cache + (size_t)B * (IN + H);
+    const float *c0 = cache, *c1 = cache + (size_t)B * (IN + H), *c2 = c1 + (size_t)B * 2 * H;
     const float *W1 = params + IN * H + H;
     const float *W2 = W1 + H * H + H;
     // what the later phases need from global memory is requested now, so that the block waits
     // for L2 once: the cached activations behind act' of both hidden layers, the head weights
     float d1[PR];          // thread t < H: layer-1 cache entries of column t, rows of the tile
+    float d2[PR];          // thread t < H: h2 of column t, rows of the tile
     float w2row[PA_MAX];   // thread t < H: W2[t][:]
     float d0[16];          // layer-0 cache entries at this lane's accumulator positions
     {
         const int n1 = t % H;
 #pragma unroll
-        for (int r = 0; r < PR; ++r) d1[r] = r < nrow ? c1[(row0 + r) * (2 * H) + H + n1] : 0.0f;
+        for (int r = 0; r < PR; ++r) {
+            d1[r] = r < nrow ? c1[(row0 + r) * (2 * H) + H + n1] : 0.0f;
+            d2[r] = r < nrow ? c2[(row0 + r) * H + n1] : 0.0f;
+        }
 #pragma unroll
         for (int a = 0; a < PA_MAX; ++a) w2row[a] = a < A ? W2[n1 * A + a] : 0.0f;
         const int colq = 32 * w + l31;
@@ -126,6 +133,10 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
     for (int i = t; i < PR * ld; i += T) {
         const int r = i / ld, a = i - r * ld;
         g2s[r * (2 * PA_MAX + 1) + a] = r < nrow ? grad_out[row0 * ld + i] : 0.0f;
+    }
+    for (int i = t; i < PR * IN; i += T) {
+        const int r = i / IN, k = i - r * IN;
+        xs[r * XS_LD + k] = r < nrow ? c0[(row0 + r) * (IN + H) + k] : 0.0f;
     }
     __syncthreads();
     if (t < ld) {   // column sums of the tile: bias gradient of the head, log_std gradient
@@ -151,6 +162,17 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
             colsum += g;
         }
         db_part[H + t] = colsum;   // bias gradient of layer 1, this tile's rows
+        // dW2[t][a] of the tile = sum_r h2[r][t] g2[r][a]
+        float *o2 = thin_part + (size_t)IN * H + (size_t)t * A;
+#pragma unroll
+        for (int a = 0; a < PA_MAX; ++a) {
+            if (a < A) {
+                float s = 0.0f;
+#pragma unroll
+                for (int r = 0; r < PR; ++r) s = fmaf(d2[r], g2s[r * (2 * PA_MAX + 1) + a], s);
+                o2[a] = s;
+            }
+        }
     }
     // dh1 = g1 W1^T: wavefront w owns input columns [32w, 32w + 32).  The next chunk of W1 is
     // fetched into registers while the matrix cores work on the current one.
@@ -185,17 +207,28 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
         }
     }
     float cs = 0.0f;
+    float gv[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         const int row = 8 * (v >> 2) + 4 * half + (v & 3);
+        gv[v] = 0.0f;
         if (row >= nrow) continue;
         const float val = acc[v] * act_deriv<ACT>(d0[v]);
         g0[(row0 + row) * H + col] = val;
+        gv[v] = val;
         cs += val;
     }
     // the two halves of the wavefront hold the other 16 rows of the same column
     cs += __shfl_xor(cs, 32, 64);
     if (half == 0) db_part[col] = cs;   // bias gradient of layer 0, this tile's rows
+    // dW0[i][col] of the tile = sum_r x[r][i] g0[r][col]
+    for (int i = 0; i < IN; ++i) {
+        float s = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s = fmaf(xs[(8 * (v >> 2) + 4 * half + (v & 3)) * XS_LD + i], gv[v], s);
+        s += __shfl_xor(s, 32, 64);
+        if (half == 0) thin_part[(size_t)i * H + col] = s;
+    }
 }
 
 // ---------------------------------------------------------------- [dW | db] of the three layers
@@ -207,6 +240,7 @@ struct DwProblem {
     int xs, gs, K, N; // K inputs, N outputs: the block written is dW [K, N]
     int poff;         // offset of the layer's W in the flat parameter vector
     int tiles_n, tiles;   // tiles_n = ceil(N / 64); tiles = tiles_n * ceil(K / 64)
+    int vec;              // rows of X and G can be read with 16-byte loads, K and N are multiples of 64
 };
 struct DwSet { DwProblem p[6]; int n; };
 
@@ -229,9 +263,23 @@ __global__ __launch_bounds__(256) void dw3_kernel(DwSet d, int M, int rows_per_s
     floatx16 acc = {0};
     const int bb = t >> 3, seg = (t & 7) * 8;
     float xa[8], gb[8];
+    // each thread moves 8 consecutive floats of X and of G per chunk: two 16-byte loads each when
+    // the problem allows (whole tiles inside K and N, 16-byte aligned rows), scalar loads otherwise
+    const bool vec = pr.vec != 0;
     auto fetch = [&](long b0) {
         const long b = b0 + bb;
         const bool inb = b < b_end;
+        if (vec) {
+            float4 x0 = {0, 0, 0, 0}, x1 = x0, g0 = x0, g1 = x0;
+            if (inb) {
+                const float4 *px = reinterpret_cast<const float4 *>(pr.X + b * pr.xs + i0 + seg);
+                const float4 *pg = reinterpret_cast<const float4 *>(pr.G + b * pr.gs + j0 + seg);
+                x0 = px[0]; x1 = px[1]; g0 = pg[0]; g1 = pg[1];
+            }
+            xa[0] = x0.x; xa[1] = x0.y; xa[2] = x0.z; xa[3] = x0.w; xa[4] = x1.x; xa[5] = x1.y; xa[6] = x1.z; xa[7] = x1.w;
+            gb[0] = g0.x; gb[1] = g0.y; gb[2] = g0.z; gb[3] = g0.w; gb[4] = g1.x; gb[5] = g1.y; gb[6] = g1.z; gb[7] = g1.w;
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int ii = i0 + seg + i, j = j0 + seg + i;
@@ -273,7 +321,7 @@ __global__ __launch_bounds__(256) void dw3_kernel(DwSet d, int M, int rows_per_s
 // sums the backward-dx kernel left.  The nets' vectors lie back to back in `partial`.
 struct SumNets {
     float *grads[2];
-    const float *ls_part[2], *db_part[2];
+    const float *ls_part[2], *db_part[2], *thin_part[2];
     int P[2], A[2], gauss[2];
     int n, IN, H;
 };
@@ -300,7 +348,12 @@ __global__ __launch_bounds__(256) void sum3_kernel(const float *__restrict__ par
         const float *p;
         size_t stride;
         int n;
-        if (bias_layer < 0) { p = partial + gi; stride = (size_t)Ptot; n = splits; }
+        if (bias_layer < 0 && i >= o1 && i < o1 + H * H) { p = partial + gi; stride = (size_t)Ptot; n = splits; }
+        else if (bias_layer < 0) {   // a weight of layer 0 or of the head: per-tile pieces of the dx kernel
+            p = sn.thin_part[net] + (i < o1 ? i : (size_t)IN * H + (i - o2));
+            stride = (size_t)IN * H + (size_t)H * A;
+            n = tiles;
+        }
         else if (bias_layer == 3) { p = sn.ls_part[net] + j; stride = (size_t)A; n = tiles; }
         else {
             p = sn.db_part[net] + (bias_layer == 0 ? 0 : (bias_layer == 1 ? H : 2 * H)) + j;
@@ -408,7 +461,9 @@ size_t mlp3_backward_ws(const mrl_mlp_desc *const *descs, int n_nets, int batch)
     size_t total = 0, P = 0;
     for (int i = 0; i < n_nets; ++i) {
         const int H = descs[i]->layers[0].out_dim;
-        total += (size_t)2 * batch * H + (size_t)((batch + PR - 1) / PR) * (2 * PA_MAX + 2 * H);
+        const int IN = descs[i]->layers[0].in_dim, A = descs[i]->layers[2].out_dim;
+        total += (size_t)2 * batch * H +
+                 (size_t)((batch + PR - 1) / PR) * (2 * PA_MAX + 2 * H + (size_t)IN * H + (size_t)H * A);
         P += net_P(*descs[i]);
     }
     return total + (size_t)32 * P;
@@ -434,14 +489,15 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
     int splits = std::max(1, std::min(32, batch / 256));
     int rows_per = ((batch + splits - 1) / splits + DKC - 1) / DKC * DKC;
     splits = (batch + rows_per - 1) / rows_per;
-    // workspace: per net g1 [B, H] | g0 [B, H] | ls_part [tiles, PA_MAX] | db_part [tiles, 2H + PA_MAX];
-    // then partial [splits, Ptot]
+    // workspace: per net g1 [B, H] | g0 [B, H] | ls_part [tiles, PA_MAX] | db_part [tiles, 2H + PA_MAX] |
+    // thin_part [tiles, IN H + H A]; then partial [splits, Ptot]
     float *w = ws;
     for (int i = 0; i < n_nets; ++i) {
         io.n[i].g1 = w; w += (size_t)batch * H;
         io.n[i].g0 = w; w += (size_t)batch * H;
         io.n[i].ls_part = w; w += (size_t)tiles * PA_MAX;
         io.n[i].db_part = w; w += (size_t)tiles * (2 * H + PA_MAX);
+        io.n[i].thin_part = w; w += (size_t)tiles * ((size_t)IN * H + (size_t)H * descs[i]->layers[2].out_dim);
     }
     float *partial = w;
     if (H == 256 && act == 1) launch_bwd_t<256, 1>(ctx, batch, IN, io, n_nets);
@@ -450,28 +506,27 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
     else launch_bwd_t<64, 2>(ctx, batch, IN, io, n_nets);
     MRL_CHECK_LAUNCH();
     DwSet dw;
-    dw.n = 3 * n_nets;
+    dw.n = n_nets;   // the H x H layer of each net; the thin layers come out of the dx kernel
     SumNets sn{};
     sn.n = n_nets;
     sn.IN = IN;
     sn.H = H;
-    auto fill = [](DwProblem &p, const float *X, int xs, const float *G, int gs, int K, int N, int poff) {
-        p.X = X; p.G = G; p.xs = xs; p.gs = gs; p.K = K; p.N = N; p.poff = poff;
-        p.tiles_n = (N + DBN - 1) / DBN;
-        p.tiles = p.tiles_n * ((K + DBM - 1) / DBM);
-    };
     int base = 0, total_tiles = 0;
     for (int i = 0; i < n_nets; ++i) {
         const Mlp3Net &nn = io.n[i];
         const int A = nn.A;
-        const float *c0 = nn.cache, *c1 = c0 + (size_t)batch * (IN + H), *c2 = c1 + (size_t)batch * 2 * H;
-        fill(dw.p[3 * i + 0], c0, IN + H, nn.g0, H, IN, H, base);
-        fill(dw.p[3 * i + 1], c1, 2 * H, nn.g1, H, H, H, base + (IN + 1) * H);
-        fill(dw.p[3 * i + 2], c2, H, nn.grad_out, nn.gauss ? 2 * A : A, H, A, base + (IN + 1) * H + (H + 1) * H);
-        for (int q = 0; q < 3; ++q) total_tiles += dw.p[3 * i + q].tiles;
+        const float *c1 = nn.cache + (size_t)batch * (IN + H);
+        DwProblem &p = dw.p[i];
+        p.X = c1; p.xs = 2 * H; p.G = nn.g1; p.gs = H; p.K = H; p.N = H; p.poff = base + (IN + 1) * H;
+        p.tiles_n = (H + DBN - 1) / DBN;
+        p.tiles = p.tiles_n * ((H + DBM - 1) / DBM);
+        p.vec = (H % 64 == 0 && reinterpret_cast<uintptr_t>(c1) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(nn.g1) % 16 == 0) ? 1 : 0;
+        total_tiles += p.tiles;
         sn.grads[i] = grads[i];
         sn.ls_part[i] = nn.ls_part;
         sn.db_part[i] = nn.db_part;
+        sn.thin_part[i] = nn.thin_part;
         sn.P[i] = net_P(*descs[i]);
         sn.A[i] = A;
         sn.gauss[i] = nn.gauss;
