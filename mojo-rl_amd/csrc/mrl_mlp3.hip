@@ -96,7 +96,7 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
     // this tile's share of the two thin weight gradients: [dW0 (IN x H) | dW2 (H x A)]
     float *__restrict__ thin_part = nn.thin_part + (size_t)blockIdx.x * ((size_t)IN * H + (size_t)H * A);
     const bool GAUSS = nn.gauss != 0;
-    constexpr int KCH = 32;                       // k-chunk of W1 staged per round
+    constexpr int KCH = 64;                       // k-chunk of W1 staged per round
     __shared__ float g2s[PR * (2 * PA_MAX + 1)];
     __shared__ float xs[PR * XS_LD];              // the tile's inputs, for dW0
     __shared__ float gT[H * HT_LD];               // g1 of the tile, k-major
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
     // fetched into registers while the matrix cores work on the current one.
     floatx16 acc = {0};
     const int col = 32 * w + l31;
-    const int wrow = t % H, wseg = (t / H) * (KCH / 2);   // thread copies W1[wrow][o0 + wseg .. + 16)
+    const int wrow = t % H, wseg = (t / H) * (KCH / 2);   // thread copies W1[wrow][o0 + wseg .. + KCH / 2)
     float4 nxt[KCH / 8];
     auto fetch = [&](int o0) {
         const float4 *src = reinterpret_cast<const float4 *>(W1 + (size_t)wrow * H + o0 + wseg);
