@@ -1,12 +1,14 @@
 #!/usr/bin/env python3
-"""Headline benchmark: LunarLander 8192-env rollout (policy + value forward, sampling, env step
-with auto-reset, rollout stores) and the PPO update, on one MI355X.
+"""Headline benchmark: batched rollout (policy + value forward, sampling, env step with auto-reset,
+rollout stores) and the PPO update, on one MI355X.
 
-One "step" = one collection step over all 8192 envs.  `value` = env-steps/s including the policy
-forward, inputs resident in HBM.  The PPO update throughput (samples/s) is reported beside it in
-the same JSON line, with the roofline figures of the dominant kernel (device time measured live
-with HIP events on the launch stream) and the CPU baseline (the oracle's C restatement of the
-reference's CPU path, timed on this box's host cores on a bounded sample).
+Default workload: LunarLander, 8192 envs, nets 8-256-256-4 / 8-256-256-1 (the north-star
+configuration).  One "step" = one collection step over all envs.  `value` = env-steps/s including
+the policy forward, inputs resident in HBM.  The PPO update throughput (samples/s) is reported
+beside it in the same JSON line, with the roofline figures of the dominant kernel (device time
+measured live with HIP events on the launch stream) and the CPU baseline (the oracle's C
+restatement of the reference's CPU path, timed on this box's host cores on a bounded sample).
+`--workload` selects one of the other benchmark configurations (parity-test cases otherwise).
 """
 import argparse
 import importlib
@@ -19,20 +21,46 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-N_ENVS, HIDDEN, OBS, NA = 8192, 256, 8, 4
-ENV_STEP_BYTES = 672                  # algorithmic HBM bytes per LunarLander env-step (live fields)
-FWD_FLOPS = 2 * ((OBS * HIDDEN + HIDDEN * HIDDEN + HIDDEN * NA) + (OBS * HIDDEN + HIDDEN * HIDDEN + HIDDEN * 1))
 HBM_PEAK_GBS, MFMA_FP32_PEAK_TFLOPS = 8000.0, 157.3
+
+# name -> env class, envs, hidden width, hidden activation, algorithmic bytes per env-step (live
+# fields of the reference row layout, each read once and written once), description
+WORKLOADS = {
+    "cartpole": ("CartPoleEnv", 4096, 64, "relu", 60, "CartPole-v1 discrete, 4096 envs, nets 4-64-64-2 / 4-64-64-1"),
+    "pendulum": ("PendulumV2", 16384, 64, "tanh", 72, "Pendulum continuous, 16384 envs, Gaussian 3-64-64-1 + value"),
+    "lunarlander": ("LunarLanderV2", 8192, 256, "relu", 672,
+                    "LunarLander-v2 discrete, 8192 envs, policy 8-256-256-4 + value 8-256-256-1 "
+                    "(BASELINE.json configs[2])"),
+    "bipedal": ("BipedalWalkerV2", 4096, 256, "tanh", 3964,
+                "BipedalWalker continuous, 4096 envs, Gaussian 24-256-256-4 + value"),
+    "halfcheetah": ("HalfCheetahPlanarV2", 4096, 256, "tanh", 1112,
+                    "HalfCheetah planar continuous, 4096 envs, Gaussian 17-256-256-6 + value"),
+}
+ORACLE = {"cartpole": None, "pendulum": None, "lunarlander": "ll", "bipedal": "bw", "halfcheetah": "hc"}
+
+
+def build_nets(mrl, E, hidden, act):
+    lay = mrl.LinearReLU if act == "relu" else mrl.LinearTanh
+    continuous = E.NUM_ACTIONS == 0
+    head = mrl.StochasticActor(hidden, E.ACTION_DIM) if continuous else mrl.Linear(hidden, E.NUM_ACTIONS)
+    actor = mrl.seq(lay(E.OBS_DIM, hidden), lay(hidden, hidden), head)
+    critic = mrl.seq(lay(E.OBS_DIM, hidden), lay(hidden, hidden), mrl.Linear(hidden, 1))
+    return actor, critic, continuous
+
+
+def fwd_flops(E, hidden):
+    a = E.ACTION_DIM if E.NUM_ACTIONS == 0 else E.NUM_ACTIONS
+    return 2 * ((E.OBS_DIM * hidden + hidden * hidden + hidden * a) + (E.OBS_DIM * hidden + hidden * hidden + hidden))
 
 
 def cpu_baseline(np, n_envs=2048, steps=60):
-    """Oracle (C restatement of the reference CPU path): env step + policy/value forward + sampling,
-    single thread, on a bounded sample of the same workload."""
+    """Oracle (C restatement of the reference CPU path): LunarLander env step + policy/value forward
+    + sampling, single thread, on a bounded sample of the default workload."""
     from oracle import orc
     o = orc.load()
-    spec_a = [(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, NA)]
-    spec_c = [(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, 1)]
-    la, lc = orc.layers(spec_a), orc.layers(spec_c)
+    OBS, HIDDEN, NA = 8, 256, 4
+    la = orc.layers([(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, NA)])
+    lc = orc.layers([(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, 1)])
     rng = np.random.default_rng(0)
     pa = rng.uniform(-0.1, 0.1, o.orc_mlp_param_size(la, 3)).astype(np.float32)
     pc = rng.uniform(-0.1, 0.1, o.orc_mlp_param_size(lc, 3)).astype(np.float32)
@@ -52,7 +80,7 @@ def cpu_baseline(np, n_envs=2048, steps=60):
         obs[:] = s[:, :8]
     dt = time.perf_counter() - t0
     return {"value": n_envs * steps / dt, "unit": "env-steps/s", "cores": 1, "kind": "port",
-            "sample": "%d envs x %d collection steps (env step + actor/critic forward + sampling), "
+            "sample": "LunarLander, %d envs x %d collection steps (env step + actor/critic forward + sampling), "
                       "single thread, %.1f s" % (n_envs, steps, dt)}
 
 
@@ -78,6 +106,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="lunarlander")
     ap.add_argument("--update-minibatches", type=int, default=200,
                     help="minibatches of 4096 timed for the PPO-update figure")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -93,14 +122,21 @@ def main():
     import torch
     mrl = importlib.import_module("mojo-rl_amd")
     ctx = mrl.DeviceContext("cuda:0")
-    E = mrl.LunarLanderV2
-    actor = mrl.seq(mrl.LinearReLU(OBS, HIDDEN), mrl.LinearReLU(HIDDEN, HIDDEN), mrl.Linear(HIDDEN, NA))
-    critic = mrl.seq(mrl.LinearReLU(OBS, HIDDEN), mrl.LinearReLU(HIDDEN, HIDDEN), mrl.Linear(HIDDEN, 1))
+    env_name, N_ENVS, HIDDEN, ACT, ENV_STEP_BYTES, describe = WORKLOADS[args.workload]
+    E = getattr(mrl, env_name)
+    OBS = E.OBS_DIM
+    actor, critic, continuous = build_nets(mrl, E, HIDDEN, ACT)
+    FWD_FLOPS = fwd_flops(E, HIDDEN)
     T = max(args.steps, 1)
     rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N_ENVS, T, done_cap=4 * N_ENVS + 64 * T)
-    # reference init: Xavier over the flat vector with the network's in/out dims (initializers.mojo:69-76)
-    anet = mrl.Network(ctx, actor, mrl.Adam(lr=3e-4), mrl.Xavier(seed=0x5EED + 2))
-    cnet = mrl.Network(ctx, critic, mrl.Adam(lr=1e-3), mrl.Xavier(seed=0x5EED + 3))
+    # reference initialisers: Xavier for the discrete agent, Kaiming + small Gaussian head for the
+    # continuous one (deep_agents/ppo/ppo.mojo:807-817, ppo_continuous.mojo:171-342)
+    init = mrl.Kaiming if continuous else mrl.Xavier
+    anet = mrl.Network(ctx, actor, mrl.Adam(lr=3e-4), init(seed=0x5EED + 2))
+    cnet = mrl.Network(ctx, critic, mrl.Adam(lr=1e-3), init(seed=0x5EED + 3))
+    if continuous:
+        mrl.init_params_small(ctx, anet.params, OBS * HIDDEN + HIDDEN + HIDDEN * HIDDEN + HIDDEN, HIDDEN,
+                              E.ACTION_DIM, seed=0x5EED + 4)
     rb.actor_params, rb.critic_params = anet.params, cnet.params
     E.reset_kernel_gpu(ctx, rb.states, 0x5EED + 2)
     rb.obs.copy_(rb.states.view(N_ENVS, E.STATE_SIZE)[:, :OBS].reshape(-1))
@@ -113,7 +149,7 @@ def main():
     ctx.synchronize()
 
     # ---- timed region: exactly `steps` collection steps
-    ctx.profile_begin(8 * T + 16)
+    ctx.profile_begin(4 * T + 16)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for t in range(T):
@@ -128,33 +164,36 @@ def main():
     fwd_us, env_us = ph_us["policy_fwd"], ph_us["env_step"]
     fwd_tflops = FWD_FLOPS * N_ENVS / (fwd_us * 1e-6) / 1e12
     env_gbs = ENV_STEP_BYTES * N_ENVS / (env_us * 1e-6) / 1e9
-    traffic = measured_traffic()
+    traffic = measured_traffic() if args.workload == "lunarlander" else {}
     if fwd_us >= env_us:
-        name = "mrl::policy_kernel<256, 1, false>"
+        name = "mrl::policy_kernel<%d, %d, %s>" % (HIDDEN, 1 if ACT == "relu" else 2, "true" if continuous else "false")
         roofline = {"kernel": name + " (actor + critic forward, sampling, stores)", "bound": "mfma",
                     "achieved": fwd_tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": fwd_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": traffic.get(name),
                     "avg_launch_us": fwd_us}
     else:
-        name = "mrl::phys_step_kernel<mrl::LunarLander, true>"
-        roofline = {"kernel": name + " (env step + auto-reset)", "bound": "hbm", "achieved": env_gbs,
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": env_gbs / HBM_PEAK_GBS,
+        name = {"lunarlander": "mrl::phys_step_kernel<mrl::LunarLander, true>",
+                "bipedal": "mrl::phys_step_kernel<mrl::BipedalWalker, true>",
+                "halfcheetah": "mrl::phys_step_kernel<mrl::HalfCheetah, true>",
+                "cartpole": "mrl::cartpole_step_kernel", "pendulum": "mrl::pendulum_step_kernel"}[args.workload]
+        roofline = {"kernel": name + " (env step + auto-reset + post-step stores)", "bound": "hbm",
+                    "achieved": env_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": env_gbs / HBM_PEAK_GBS,
                     "traffic": traffic.get(name), "avg_launch_us": env_us}
 
     # ---- PPO update on the collected batch (minibatch 4096, reference defaults)
-    MB = 4096
-    upd = mrl.ppo.DiscreteUpdate(ctx, rb, MB, anet.optimizer, cnet.optimizer, target_kl=0.0)
+    MB = min(4096, N_ENVS * T)
+    cls = mrl.ppo.ContinuousUpdate if continuous else mrl.ppo.DiscreteUpdate
+    upd = cls(ctx, rb, MB, anet.optimizer, cnet.optimizer, target_kl=0.0, normalize_rewards=continuous)
     upd.compute_advantages()
     total = N_ENVS * T
     n_mb = max(1, min(args.update_minibatches, total // MB))
     perm = upd.indices
     mrl.ppo.permutation(ctx, perm, 0x5EED)
-    for k in range(3):
+    for k in range(min(3, n_mb)):
         upd.minibatch_step(perm[k * MB:(k + 1) * MB])
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    for k in range(n_mb):
-        upd.minibatch_step(perm[k * MB:(k + 1) * MB])
+    upd.run_epoch(perm[:n_mb * MB])
     torch.cuda.synchronize()
     dtu = time.perf_counter() - t1
     update_sps = n_mb * MB / dtu
@@ -168,8 +207,7 @@ def main():
         "value": env_steps_per_s, "unit": "env-steps/s", "n_gpus": 1, "steps": T, "warmup": args.warmup,
         "ms_per_step": 1e3 * dt / T, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "LunarLander-v2 discrete, 8192 envs, policy 8-256-256-4 + value 8-256-256-1 "
-                               "(BASELINE.json configs[2]); update: minibatch 4096, clip 0.2, Adam",
+        "config": {"workload": describe + "; update: minibatch %d, clip 0.2, Adam" % MB,
                    "n_envs": N_ENVS, "rollout_steps": T, "minibatch": MB},
         "ppo_update_samples_per_s": update_sps,
         "ppo_update": {"minibatches_timed": n_mb, "ms_per_minibatch": 1e3 * dtu / n_mb,
@@ -178,7 +216,8 @@ def main():
         "phase_us_per_step": ph_us,
         "kernels": {"policy_fwd_TFLOPs": fwd_tflops, "env_step_GBs": env_gbs,
                     "env_step_frac_hbm": env_gbs / HBM_PEAK_GBS,
-                    "policy_fwd_frac_mfma": fwd_tflops / MFMA_FP32_PEAK_TFLOPS},
+                    "policy_fwd_frac_mfma": fwd_tflops / MFMA_FP32_PEAK_TFLOPS,
+                    "update_TFLOPs": 3.0 * FWD_FLOPS * update_sps / 1e12},
         "roofline": roofline,
     }
     if args.copy_calibration:
