@@ -30,7 +30,7 @@ WORKLOADS = {
     "pendulum": ("PendulumV2", 16384, 64, "tanh", 72, "Pendulum continuous, 16384 envs, Gaussian 3-64-64-1 + value"),
     "lunarlander": ("LunarLanderV2", 8192, 256, "relu", 672,
                     "LunarLander-v2 discrete, 8192 envs, policy 8-256-256-4 + value 8-256-256-1 "
-                    "(BASELINE.json configs[2])"),
+                    "(the north-star configuration)"),
     "bipedal": ("BipedalWalkerV2", 4096, 256, "tanh", 3964,
                 "BipedalWalker continuous, 4096 envs, Gaussian 24-256-256-4 + value"),
     "halfcheetah": ("HalfCheetahPlanarV2", 4096, 256, "tanh", 1112,

@@ -40,7 +40,7 @@ struct TileCache {
 // over twice the wavefronts.  Everything a later phase needs from global memory and that does not
 // depend on earlier phases (biases, the layer-0 weights) is requested up front, so that a block
 // pays the L2 latency once rather than once per phase.
-template <int H, int ACT, int TPW = 2>
+template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32)>
 MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
                           const TileCache tc) {
     constexpr int T = 2 * H / TPW;
@@ -94,7 +94,6 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
     }
     __syncthreads();
     {   // layer 1 (H x H): weights streamed from L2 one block of KB k-steps ahead of the MFMAs
-        constexpr int KB = TPW == 2 ? 8 : 32;
         floatx16 c[TPW];
 #pragma unroll
         for (int q = 0; q < TPW; ++q) c[q] = floatx16{0};

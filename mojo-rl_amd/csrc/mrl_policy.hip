@@ -22,8 +22,8 @@
 
 namespace mrl {
 
-template <int H, int ACT, bool GAUSS>
-__global__ __launch_bounds__(2 * H) void policy_kernel(
+template <int H, int ACT, bool GAUSS, int TPW>
+__global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
     const float *__restrict__ obs, int n, int IN, int A, const float *__restrict__ actor_p,
     const float *__restrict__ critic_p, uint32_t seed, float *__restrict__ actions,
     float *__restrict__ r_obs, float *__restrict__ r_actions, float *__restrict__ r_logp,
@@ -34,13 +34,14 @@ __global__ __launch_bounds__(2 * H) void policy_kernel(
     __shared__ float logits[PR * (PA_MAX + 1)];
     __shared__ float vals[PR];
     __shared__ float w2s[2][HEAD_LDS(H)];
+    constexpr int TN = 2 * H / TPW;          // threads per net
     const int t = threadIdx.x;
-    const int net = t / H;                   // 0 = actor, 1 = critic
+    const int net = t / TN;                  // 0 = actor, 1 = critic
     const int row0 = blockIdx.x * PR;
     const int nrow = min(PR, n - row0);
 
     // observation tile in (rows beyond the batch read as zero), and straight out to rollout[t]
-    for (int i = t; i < PR * IN; i += 2 * H) {
+    for (int i = t; i < PR * IN; i += 2 * TN) {
         const int r = i / IN, k = i - r * IN;
         float v = 0.0f;
         if (r < nrow) {
@@ -52,10 +53,12 @@ __global__ __launch_bounds__(2 * H) void policy_kernel(
     __syncthreads();
 
     const float *p = net ? critic_p : actor_p;
-    stage_head(p + IN * H + H + H * H + H, H, net ? 1 : A, GAUSS && net == 0, w2s[net], t % H, H);
-    hidden_stack<H, ACT>(p, IN, xs, hT[net], h2[net], TileCache{});
-    if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1);
-    else head<H>(w2s[1], 1, h2[1], vals, 1);
+    stage_head(p + IN * H + H + H * H + H, H, net ? 1 : A, GAUSS && net == 0, w2s[net], t % TN, TN);
+    hidden_stack<H, ACT, TPW, 8>(p, IN, xs, hT[net], h2[net], TileCache{});
+    if (t % TN < H) {
+        if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1);
+        else head<H>(w2s[1], 1, h2[1], vals, 1);
+    }
     __syncthreads();
 
     if (t < nrow && !GAUSS) {   // categorical sampling, one lane per env
@@ -109,6 +112,8 @@ __global__ __launch_bounds__(2 * H) void policy_kernel(
 }
 
 // true when the pair (actor, critic) has the shape this kernel is specialised for
+constexpr int PTPW = 2;   // accumulator tiles per wavefront in the policy kernel (1 measured no faster)
+
 bool policy_fusable(const mrl_mlp_desc &a, const mrl_mlp_desc &c, bool gauss, int *H, int *act) {
     if (a.n_layers != 3 || c.n_layers != 3) return false;
     const int k0 = a.layers[0].kind;
@@ -137,7 +142,7 @@ int launch_policy(mrl_ctx *ctx, const mrl_mlp_desc &a, const mrl_mlp_desc &c, bo
     const int IN = a.layers[0].in_dim, A = a.layers[2].out_dim;
     dim3 grid((n + PR - 1) / PR);
 #define MRL_LAUNCH(HH, AA, GG)                                                                         \
-    hipLaunchKernelGGL((policy_kernel<HH, AA, GG>), grid, dim3(2 * HH), 0, ctx->stream, obs, n, IN, A, ap, \
+    hipLaunchKernelGGL((policy_kernel<HH, AA, GG, PTPW>), grid, dim3(4 * HH / PTPW), 0, ctx->stream, obs, n, IN, A, ap, \
                        cp, seed, actions, r_obs, r_actions, r_logp, r_values)
     if (gauss) {
         if (H == 256 && act == 1) MRL_LAUNCH(256, 1, true);
