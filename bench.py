@@ -36,7 +36,6 @@ WORKLOADS = {
     "halfcheetah": ("HalfCheetahPlanarV2", 4096, 256, "tanh", 1112,
                     "HalfCheetah planar continuous, 4096 envs, Gaussian 17-256-256-6 + value"),
 }
-ORACLE = {"cartpole": None, "pendulum": None, "lunarlander": "ll", "bipedal": "bw", "halfcheetah": "hc"}
 
 
 def build_nets(mrl, E, hidden, act):

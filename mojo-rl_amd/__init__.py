@@ -15,9 +15,11 @@ from .model import Model, Linear, LinearReLU, LinearTanh, StochasticActor, seq  
 from .optimizer import Adam  # noqa: E402
 from .training import Network, Xavier, Kaiming, init_params_small  # noqa: E402
 from . import ppo  # noqa: E402
+from .agents import DeepPPOAgent, DeepPPOContinuousAgent, TrainingMetrics  # noqa: E402
 
 __all__ = ["DeviceContext", "CartPoleEnv", "PendulumV2", "LunarLanderV2", "BipedalWalkerV2",
            "HalfCheetahPlanarV2", "MrlError", "Model",
            "Linear", "LinearReLU", "LinearTanh", "StochasticActor", "seq", "Adam", "ppo",
            "Network", "Xavier", "Kaiming", "init_params_small",
+           "DeepPPOAgent", "DeepPPOContinuousAgent", "TrainingMetrics",
            "LINEAR", "LINEAR_RELU", "LINEAR_TANH", "STOCHASTIC_ACTOR"]

@@ -1,0 +1,164 @@
+"""DeepPPOAgent / DeepPPOContinuousAgent: the host side of the reference's GPU training loop
+(deep_agents/ppo/ppo.mojo:742-960, 1558-2840; deep_agents/ppo/ppo_continuous.mojo:171-390,
+2180-3300) over this library's fused calls.
+
+`train_gpu` keeps the reference's structure -- collect `rollout_len` steps on `n_envs` device
+envs, bootstrap + GAE, `num_epochs` epochs of shuffled minibatches, learning-rate and entropy
+annealing, KL early stop -- and its seed schedule for sampling and resets.  What differs is where
+the work runs: a collection step is one library call (two launches), an epoch is one library
+call, and the host reads back only the list of finished episodes and the KL flag, once per
+rollout / epoch.  Network sizes, hyper-parameter names and defaults are the reference's.
+"""
+import torch
+
+from . import ppo
+from .model import Linear, LinearReLU, LinearTanh, StochasticActor, seq
+from .optimizer import Adam
+from .training import Network, Xavier, Kaiming, init_params_small
+
+
+class TrainingMetrics:
+    """Episode returns / lengths in completion order (core/metrics TrainingMetrics of the reference,
+    reduced to what the PPO agents record)."""
+
+    def __init__(self, algorithm_name, environment_name):
+        self.algorithm_name, self.environment_name = algorithm_name, environment_name
+        self.episode_rewards, self.episode_steps = [], []
+        self.rollouts, self.total_steps = 0, 0
+
+    def log_episodes(self, rewards, steps):
+        self.episode_rewards.extend(rewards)
+        self.episode_steps.extend(steps)
+
+    def mean_reward(self, last=100):
+        r = self.episode_rewards[-last:]
+        return sum(r) / len(r) if r else 0.0
+
+
+class _PPOAgentBase:
+    continuous = False
+
+    def _build(self, ctx, env):
+        raise NotImplementedError
+
+    def train_gpu(self, ctx, env, num_episodes, verbose=False, print_every=10, max_rollouts=None,
+                  seed=0):
+        """Train on device envs of class `env` until `num_episodes` episodes have finished (or
+        `max_rollouts` rollouts have run).  Returns TrainingMetrics."""
+        if env.OBS_DIM != self.obs_dim:
+            raise ValueError("env OBS_DIM %d != agent obs_dim %d" % (env.OBS_DIM, self.obs_dim))
+        self._build(ctx, env)
+        metrics = TrainingMetrics("Deep PPO (GPU)" + (" continuous" if self.continuous else ""), env.__name__)
+        rb, upd = self.rb, self.upd
+        N, T = self.n_envs, self.rollout_len
+        env.reset_kernel_gpu(ctx, rb.states, seed)
+        rb.obs.copy_(rb.states.view(N, env.STATE_SIZE)[:, :env.OBS_DIM].reshape(-1))
+        rb.ep_return.zero_(); rb.ep_length.zero_()
+        desc = rb.descriptor()
+        total_steps, completed = 0, 0
+        target_steps = self.target_total_steps or num_episodes * 200
+        a_lr0, c_lr0, ent0 = self.actor_lr, self.critic_lr, self.entropy_coef
+        while completed < num_episodes:
+            if max_rollouts is not None and metrics.rollouts >= max_rollouts:
+                break
+            rb.done_count.zero_()
+            for t in range(T):
+                ppo.rollout_step(ctx, desc, t,
+                                 (total_steps * 2654435761 + t * 7919) & 0xFFFFFFFF,
+                                 (total_steps * 1103515245 + t * 12345) & (2**64 - 1),
+                                 (total_steps * 1013904223 + t * 2654435761) & (2**64 - 1))
+                total_steps += N
+            # annealing (ppo.mojo:2385-2406)
+            progress = min(1.0, total_steps / float(target_steps))
+            if self.anneal_lr:
+                self.actor.optimizer.lr = a_lr0 * (1.0 - progress)
+                self.critic.optimizer.lr = c_lr0 * (1.0 - progress)
+            upd.entropy_coef = ent0 * (1.0 - progress) if self.anneal_entropy else ent0
+            upd.update(self.num_epochs, seed=seed * 7919 + metrics.rollouts)
+            # the only read-back of the rollout: the finished episodes
+            cnt = min(int(rb.done_count.item()), rb.done_cap)
+            if cnt:
+                metrics.log_episodes(rb.done_returns[:cnt].tolist(), rb.done_lengths[:cnt].tolist())
+            completed += cnt
+            metrics.rollouts += 1
+            metrics.total_steps = total_steps
+            if verbose and metrics.rollouts % print_every == 0:
+                print("rollout %d  steps %d  episodes %d  mean return (last 100) %.2f" % (
+                    metrics.rollouts, total_steps, completed, metrics.mean_reward()), flush=True)
+        return metrics
+
+
+class DeepPPOAgent(_PPOAgentBase):
+    """deep_agents/ppo/ppo.mojo:742-960: actor obs -> hidden (ReLU) -> hidden (ReLU) -> logits,
+    critic obs -> hidden (ReLU) -> hidden (ReLU) -> 1, Xavier initialisation, Adam."""
+
+    def __init__(self, obs_dim, num_actions, hidden_dim=64, rollout_len=128, n_envs=1024,
+                 gpu_minibatch_size=256, gamma=0.99, gae_lambda=0.95, clip_epsilon=0.2, actor_lr=0.0003,
+                 critic_lr=0.001, entropy_coef=0.01, value_loss_coef=0.5, num_epochs=4,
+                 normalize_advantages=True, target_kl=0.015, max_grad_norm=0.5, anneal_lr=True,
+                 anneal_entropy=False, target_total_steps=0, clip_value=True, norm_adv_per_minibatch=True,
+                 init_seed=0):
+        self.obs_dim, self.num_actions, self.hidden_dim = obs_dim, num_actions, hidden_dim
+        self.rollout_len, self.n_envs, self.gpu_minibatch_size = rollout_len, n_envs, gpu_minibatch_size
+        self.gamma, self.gae_lambda, self.clip_epsilon = gamma, gae_lambda, clip_epsilon
+        self.actor_lr, self.critic_lr, self.entropy_coef = actor_lr, critic_lr, entropy_coef
+        self.value_loss_coef, self.num_epochs = value_loss_coef, num_epochs
+        self.normalize_advantages, self.target_kl, self.max_grad_norm = normalize_advantages, target_kl, max_grad_norm
+        self.anneal_lr, self.anneal_entropy, self.target_total_steps = anneal_lr, anneal_entropy, target_total_steps
+        self.clip_value, self.norm_adv_per_minibatch, self.init_seed = clip_value, norm_adv_per_minibatch, init_seed
+        self.actor = self.critic = self.rb = self.upd = None
+
+    def _nets(self):
+        H = self.hidden_dim
+        return (seq(LinearReLU(self.obs_dim, H), LinearReLU(H, H), Linear(H, self.num_actions)),
+                seq(LinearReLU(self.obs_dim, H), LinearReLU(H, H), Linear(H, 1)))
+
+    def _build(self, ctx, env):
+        if self.actor is None:
+            am, cm = self._nets()
+            self.actor = Network(ctx, am, Adam(lr=self.actor_lr), Xavier(seed=2 * self.init_seed + 1))
+            self.critic = Network(ctx, cm, Adam(lr=self.critic_lr), Xavier(seed=2 * self.init_seed + 2))
+        self.rb = ppo.RolloutBuffers(ctx, env, self.actor.model, self.critic.model, self.n_envs, self.rollout_len,
+                                     done_cap=max(1024, 2 * self.n_envs * self.rollout_len // 8),
+                                     continuous=self.continuous)
+        self.rb.actor_params, self.rb.critic_params = self.actor.params, self.critic.params
+        cls = ppo.ContinuousUpdate if self.continuous else ppo.DiscreteUpdate
+        self.upd = cls(ctx, self.rb, self.gpu_minibatch_size, self.actor.optimizer, self.critic.optimizer,
+                       gamma=self.gamma, gae_lambda=self.gae_lambda, clip_epsilon=self.clip_epsilon,
+                       entropy_coef=self.entropy_coef, value_loss_coef=self.value_loss_coef,
+                       max_grad_norm=self.max_grad_norm, clip_value=self.clip_value,
+                       normalize_advantages=self.normalize_advantages,
+                       norm_adv_per_minibatch=self.norm_adv_per_minibatch, target_kl=self.target_kl,
+                       normalize_rewards=getattr(self, "normalize_rewards", False))
+        # the optimiser state lives with the update object; share the networks' buffers
+        self.upd.actor_state, self.upd.critic_state = self.actor.optimizer_state, self.critic.optimizer_state
+        self.upd.actor_grads, self.upd.critic_grads = self.actor.grads, self.critic.grads
+
+
+class DeepPPOContinuousAgent(DeepPPOAgent):
+    """deep_agents/ppo/ppo_continuous.mojo:171-390: tanh hidden layers, StochasticActor head
+    (state-independent log_std, small initial weights), Kaiming initialisation, critic gradient
+    (V - R) / MB, optional reward normalisation."""
+    continuous = True
+
+    def __init__(self, obs_dim, action_dim, hidden_dim=64, rollout_len=128, n_envs=1024,
+                 gpu_minibatch_size=256, normalize_rewards=True, entropy_coef=0.0, **kw):
+        super().__init__(obs_dim, action_dim, hidden_dim, rollout_len, n_envs, gpu_minibatch_size,
+                         entropy_coef=entropy_coef, **kw)
+        self.action_dim, self.normalize_rewards = action_dim, normalize_rewards
+
+    def _nets(self):
+        H = self.hidden_dim
+        return (seq(LinearTanh(self.obs_dim, H), LinearTanh(H, H), StochasticActor(H, self.action_dim)),
+                seq(LinearTanh(self.obs_dim, H), LinearTanh(H, H), Linear(H, 1)))
+
+    def _build(self, ctx, env):
+        fresh = self.actor is None
+        if fresh:
+            am, cm = self._nets()
+            self.actor = Network(ctx, am, Adam(lr=self.actor_lr), Kaiming(seed=2 * self.init_seed + 1))
+            self.critic = Network(ctx, cm, Adam(lr=self.critic_lr), Kaiming(seed=2 * self.init_seed + 2))
+            H = self.hidden_dim
+            init_params_small(ctx, self.actor.params, self.obs_dim * H + H + H * H + H, H, self.action_dim,
+                              seed=2 * self.init_seed + 3)
+        super()._build(ctx, env)
