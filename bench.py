@@ -100,6 +100,9 @@ def measured_traffic():
     return out
 
 
+EVENT_STRIDE = 8
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -148,7 +151,9 @@ def main():
     ctx.synchronize()
 
     # ---- timed region: exactly `steps` collection steps
-    ctx.profile_begin(4 * T + 16)
+    # HIP events around the two kernels of every 8th step: an event between two launches costs
+    # device time (about 3 us each here), so timing every step would slow the region it measures
+    ctx.profile_begin(4 * T + 16, sample_every=EVENT_STRIDE)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for t in range(T):
@@ -213,6 +218,7 @@ def main():
                        "gae_plus_normalise_ms": gae_ms},
         "episodes_finished": episodes,
         "phase_us_per_step": ph_us,
+        "phase_events": {"sampled_every_n_steps": EVENT_STRIDE, "launches_timed": phases["env_step"][1]},
         "kernels": {"policy_fwd_TFLOPs": fwd_tflops, "env_step_GBs": env_gbs,
                     "env_step_frac_hbm": env_gbs / HBM_PEAK_GBS,
                     "policy_fwd_frac_mfma": fwd_tflops / MFMA_FP32_PEAK_TFLOPS,

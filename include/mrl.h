@@ -84,6 +84,10 @@ enum {
     MRL_PHASE_COUNT = 4
 };
 int mrl_profile_begin(mrl_ctx *ctx, int max_marks);
+/* Time only every `every`-th call of mrl_rollout_step (1, the default: all of them).  An event
+ * between two kernels costs device time of its own; sampling keeps a long timed run close to an
+ * untimed one while the per-phase averages still come from launches inside it. */
+int mrl_profile_sample_every(mrl_ctx *ctx, int every);
 int mrl_profile_end(mrl_ctx *ctx, int n_phases, double *total_ms, int *counts);
 
 /* ------------------------------------------------------------------ environments

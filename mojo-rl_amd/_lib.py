@@ -69,6 +69,7 @@ SIGNATURES = {
     "mrl_ctx_destroy": [P],
     "mrl_ctx_synchronize": [P],
     "mrl_profile_begin": [P, I],
+    "mrl_profile_sample_every": [P, I],
     "mrl_profile_end": [P, I, C.POINTER(D), C.POINTER(I)],
     "mrl_env_dims": [I, C.POINTER(I), C.POINTER(I), C.POINTER(I), C.POINTER(I)],
     "mrl_env_reset": [P, I, I, P, U64],

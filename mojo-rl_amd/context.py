@@ -43,8 +43,10 @@ class DeviceContext:
 
     PHASES = ("policy_fwd", "sample_store", "env_step", "post_store")
 
-    def profile_begin(self, max_marks=8192):
-        """Arm per-phase device timing (HIP events on this context's stream)."""
+    def profile_begin(self, max_marks=8192, sample_every=1):
+        """Arm per-phase device timing (HIP events on this context's stream); with sample_every = k
+        only every k-th rollout step carries events."""
+        _lib.call("mrl_profile_sample_every", self.handle, sample_every)
         _lib.call("mrl_profile_begin", self.handle, max_marks)
 
     def profile_end(self):

@@ -56,6 +56,12 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
         bias0[q] = b0[col[q]];
         bias1[q] = b1[col[q]];
     }
+    float bv[TPW][KB];   // first block of layer-1 weights: on its way while layer 0 runs
+#pragma unroll
+    for (int j = 0; j < KB; ++j) {
+#pragma unroll
+        for (int q = 0; q < TPW; ++q) bv[q][j] = W1[(2 * j + half) * H + col[q]];
+    }
     {   // layer 0 (K = IN <= 32, padded to even with zeros): all operands first, then the MFMAs
         float a0[K0], w0[TPW][K0];
 #pragma unroll
@@ -97,14 +103,9 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
         floatx16 c[TPW];
 #pragma unroll
         for (int q = 0; q < TPW; ++q) c[q] = floatx16{0};
-        float a[KB], bv[TPW][KB], na[KB], nb[TPW][KB];
+        float a[KB], na[KB], nb[TPW][KB];
 #pragma unroll
-        for (int j = 0; j < KB; ++j) {
-            const int k = 2 * j + half;
-            a[j] = hT[k * HT_LD + l31];
-#pragma unroll
-            for (int q = 0; q < TPW; ++q) bv[q][j] = W1[k * H + col[q]];
-        }
+        for (int j = 0; j < KB; ++j) a[j] = hT[(2 * j + half) * HT_LD + l31];
         for (int blk = 0; blk < H / (2 * KB); ++blk) {
             const bool more = blk + 1 < H / (2 * KB);
             if (more) {
@@ -149,35 +150,56 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
     __syncthreads();
 }
 
-// floats of LDS that hold one net's head parameters [W2 (H x A) | b2 (A) | log_std (A)]
+// floats of LDS that hold one net's head parameters, every row padded to PA_MAX columns with
+// zeros: [W2 (H x PA_MAX) | b2 (PA_MAX) | log_std (PA_MAX)]; the array must be 16-byte aligned
 constexpr int HEAD_LDS(int H) { return (H + 2) * PA_MAX; }
+constexpr int HEAD_B2(int H) { return H * PA_MAX; }
+constexpr int HEAD_LOG_STD(int H) { return (H + 1) * PA_MAX; }
 
 // copies the head parameters of a net into LDS (call by `nthreads` threads with 0 <= t < nthreads,
-// early in the kernel: the head then never waits on global memory)
+// early in the kernel: the head then never waits on global memory).  The padding lets head() read
+// whole rows with two 16-byte loads and no test on A.
 MRL_DEV void stage_head(const float *__restrict__ W2, int H, int A, bool with_log_std, float *w2s, int t,
                         int nthreads) {
-    const int n = (H + 1) * A + (with_log_std ? A : 0);
-    for (int i = t; i < n; i += nthreads) w2s[i] = W2[i];
+    const int rows = H + 1 + (with_log_std ? 1 : 0);   // the parameters are [H + 1 (+ 1)][A], row-major
+    const int total = rows * PA_MAX;
+    for (int i0 = t; i0 < total; i0 += 4 * nthreads) {   // four independent loads in flight per thread
+        float v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int i = i0 + k * nthreads, n = i / PA_MAX, a = i % PA_MAX;
+            v[k] = (i < total && a < A) ? W2[n * A + a] : 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (i0 + k * nthreads < total) w2s[i0 + k * nthreads] = v[k];
+    }
 }
 
-// out[r][a] = h2[r] . W2[:, a] + b2[a] for the block's rows; TPR = H/32 lanes cooperate per row.
-// w2s: the head parameters in LDS (stage_head); called by the first H threads of the net.
+// out[r][a] = h2[r] . W2[:, a] + b2[a] for the block's rows; TPR = H/32 lanes cooperate per row,
+// each over 32 consecutive columns that it walks from a different starting point (the lanes of a
+// wavefront then read distinct LDS banks).  w2s: the head parameters in LDS (stage_head); called
+// by the first H threads of the net.
 template <int H>
 MRL_DEV void head(const float *w2s, int A, const float *h2, float *out, int out_ld) {
     constexpr int TPR = H / PR;
     const int t = threadIdx.x % H, r = t / TPR, part = t % TPR;
-    const float *b2 = w2s + H * A;
     float acc[PA_MAX];
 #pragma unroll
     for (int a = 0; a < PA_MAX; ++a) acc[a] = 0.0f;
 #pragma unroll 8
     for (int i = 0; i < PR; ++i) {
-        const int n = i * TPR + part;
+        const int n = part * PR + ((i + 4 * part) & (PR - 1));
         const float hv = h2[r * (H + 1) + n];
-#pragma unroll
-        for (int a = 0; a < PA_MAX; ++a)
-            if (a < A) acc[a] = fmaf(hv, w2s[n * A + a], acc[a]);
+        const float4 wa = *reinterpret_cast<const float4 *>(w2s + n * PA_MAX);
+        const float4 wb = *reinterpret_cast<const float4 *>(w2s + n * PA_MAX + 4);
+        acc[0] = fmaf(hv, wa.x, acc[0]); acc[1] = fmaf(hv, wa.y, acc[1]);
+        acc[2] = fmaf(hv, wa.z, acc[2]); acc[3] = fmaf(hv, wa.w, acc[3]);
+        acc[4] = fmaf(hv, wb.x, acc[4]); acc[5] = fmaf(hv, wb.y, acc[5]);
+        acc[6] = fmaf(hv, wb.z, acc[6]); acc[7] = fmaf(hv, wb.w, acc[7]);
     }
+    static_assert(PA_MAX == 8, "two float4 per padded row");
+    const float *b2 = w2s + HEAD_B2(H);
 #pragma unroll
     for (int a = 0; a < PA_MAX; ++a) {
         float v = acc[a];

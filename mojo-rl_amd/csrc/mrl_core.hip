@@ -42,6 +42,9 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     c->profiling = false;
     c->prof_used = 0;
     c->prof_chained = false;
+    c->prof_every = 1;
+    c->prof_step = 0;
+    c->prof_active = true;
     MRL_CHECK_HIP(hipMalloc(&c->ll_shapes, sizeof(mrl::ll::Shapes)));
     mrl::ll::Shapes sh = mrl::ll::make_shapes();
     MRL_CHECK_HIP(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));
@@ -94,7 +97,15 @@ int mrl_profile_begin(mrl_ctx *ctx, int max_marks) {
     ctx->prof_tags.assign(ctx->prof_events.size(), -1);
     ctx->prof_used = 0;
     ctx->prof_chained = false;
+    ctx->prof_step = 0;
+    ctx->prof_active = true;
     ctx->profiling = true;
+    return MRL_OK;
+}
+
+int mrl_profile_sample_every(mrl_ctx *ctx, int every) {
+    MRL_CHECK_ARG(ctx != nullptr && every >= 1, "mrl_profile_sample_every: bad arguments");
+    ctx->prof_every = every;
     return MRL_OK;
 }
 

@@ -1,11 +1,12 @@
 // Environment kernels and their C entry points.
 //
-// Physics envs (LunarLander): one wavefront-sized workgroup handles 64 consecutive env rows.
-// The rows are contiguous in the reference's [B, STATE_SIZE] buffer, so the block copies them
-// HBM -> LDS with coalesced 16-byte loads, each lane then steps its own env entirely out of
-// LDS (row stride odd => the 64 lanes touch 64 distinct banks for any field), and the fields
-// that a step can change are copied back with coalesced stores.  HBM sees each row once in
-// and the changed part once out; nothing is re-read.
+// Physics envs: a workgroup handles EPB consecutive env rows.  The rows are contiguous in the
+// reference's [B, STATE_SIZE] buffer, so all wavefronts of the block copy them HBM -> LDS with
+// coalesced 16-byte loads, one lane of wavefront 0 per env then steps it entirely out of LDS
+// (row stride odd => the lanes touch distinct banks for any field) while the other wavefronts
+// detect its contacts where the env splits that off, and the fields that a step can change are
+// copied back with coalesced stores.  HBM sees each row once in and the changed part once out;
+// nothing is re-read.
 #include "mrl_host.hpp"
 #include "env_classic.hpp"
 #include "env_lunar.hpp"
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(256) void pendulum_reset_kernel(float *states, floa
 
 struct LunarLander {
     using L = ll::L;
-    static constexpr int STATE = ll::STATE, OBS = ll::OBS, ACT_W = 1, EPB = 64;
+    static constexpr int STATE = ll::STATE, OBS = ll::OBS, ACT_W = 1, EPB = 32, THREADS = 512;
     static constexpr int DYN_END = L::JOINTS_OFF, NSHAPE = 3 * SHAPE_SIZE;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
@@ -134,8 +135,14 @@ struct LunarLander {
     static MRL_DEV void reset_wave(float *row, uint64_t seed, int env, int lane) {
         ll::reset_row_wave(row, ll::combined_seed(seed, env), lane);
     }
-    // contact detection of body k runs on wavefront k + 1 while wavefront 0 applies the engines
-    static constexpr int DETECT_WAVES = L::NUM_BODIES;
+    // contact detection runs beside the engines of wavefront 0: every half of wavefronts 1 .. 7
+    // takes one (body, vertex) pair of the block's 32 envs -- hull 6 vertices, legs 4 each
+    static constexpr int DETECT_TASKS = 14;
+    static MRL_DEV void detect_task(int k, int &body, int &vertex, int &max_verts) {
+        if (k < 6) { body = 0; vertex = k; max_verts = 6; }
+        else if (k < 10) { body = 1; vertex = k - 6; max_verts = 4; }
+        else { body = 2; vertex = k - 10; max_verts = 4; }
+    }
     using Carry = ll::StepCarry;
     static MRL_DEV Carry step_begin(float *row, int env, const float *a) { return ll::step_begin(row, env, (int)a[0]); }
     static MRL_DEV void step_finish(float *row, float *cts, int n, const float *shapes, const Carry &c, float &r,
@@ -146,7 +153,7 @@ struct LunarLander {
 
 struct BipedalWalker {
     using L = bw::L;
-    static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 32;
+    static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 32, THREADS = 256;
     static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = bw::NSHAPE_FLOATS;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
@@ -155,7 +162,8 @@ struct BipedalWalker {
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { bw::reset_row(row, walker_seed(seed, env)); }
     static constexpr bool WAVE_RESET = false;
     static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
-    static constexpr int DETECT_WAVES = 0;
+    static constexpr int DETECT_TASKS = 0;
+    static MRL_DEV void detect_task(int, int &, int &, int &) {}
     struct Carry {};
     static MRL_DEV Carry step_begin(float *, int, const float *) { return Carry{}; }
     static MRL_DEV void step_finish(float *, float *, int, const float *, const Carry &, float &, float &) {}
@@ -163,7 +171,7 @@ struct BipedalWalker {
 
 struct HalfCheetah {
     using L = hc::L;
-    static constexpr int STATE = hc::STATE, OBS = hc::OBS, ACT_W = hc::ACT, EPB = 64;
+    static constexpr int STATE = hc::STATE, OBS = hc::OBS, ACT_W = hc::ACT, EPB = 64, THREADS = 256;
     static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = hc::NSHAPE_FLOATS;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
@@ -172,75 +180,123 @@ struct HalfCheetah {
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { hc::reset_row(row, walker_seed(seed, env)); }
     static constexpr bool WAVE_RESET = false;
     static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
-    static constexpr int DETECT_WAVES = 0;
+    static constexpr int DETECT_TASKS = 0;
+    static MRL_DEV void detect_task(int, int &, int &, int &) {}
     struct Carry {};
     static MRL_DEV Carry step_begin(float *, int, const float *) { return Carry{}; }
     static MRL_DEV void step_finish(float *, float *, int, const float *, const Carry &, float &, float &) {}
 };
 
 constexpr int WAVE = 64;    // the compute phase runs on one wavefront, one lane per env
-constexpr int BLOCK = 256;  // all four wavefronts of the workgroup move the rows between HBM and LDS
 
 template <class E>
 struct Stage {
     static constexpr int STRIDE = E::STATE | 1;                            // odd => conflict-free lane access
     static constexpr int CSTRIDE = (E::L::MAX_CONTACTS * CONTACT_SCRATCH) | 1;
 
+    // Copies run in batches of UNROLL independent elements per thread (all loads of a batch are
+    // issued before the first store), so a thread waits for memory once per batch and not once
+    // per element.
+    static constexpr int UNROLL = 8;
+
     static MRL_DEV void in(float *lds, const float *g, int nenv, int lane) {
         if (E::STATE % 4 == 0) {   // rows are whole float4s, never straddled by a 16-byte load
             const float4 *src = reinterpret_cast<const float4 *>(g);
             const int total4 = nenv * (E::STATE / 4);
-            for (int i = lane; i < total4; i += BLOCK) {
-                float4 v = src[i];
-                int f = i * 4;
-                int r = f / E::STATE, c = f - r * E::STATE;
-                float *d = lds + r * STRIDE + c;
-                d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+            for (int i0 = lane; i0 < total4; i0 += UNROLL * E::THREADS) {
+                float4 v[UNROLL];
+#pragma unroll
+                for (int k = 0; k < UNROLL; ++k)
+                    if (i0 + k * E::THREADS < total4) v[k] = src[i0 + k * E::THREADS];
+#pragma unroll
+                for (int k = 0; k < UNROLL; ++k) {
+                    if (i0 + k * E::THREADS >= total4) continue;
+                    const int f = (i0 + k * E::THREADS) * 4;
+                    const int r = f / E::STATE, c = f - r * E::STATE;
+                    float *d = lds + r * STRIDE + c;
+                    d[0] = v[k].x; d[1] = v[k].y; d[2] = v[k].z; d[3] = v[k].w;
+                }
             }
         } else {
             const int total = nenv * E::STATE;
-            for (int i = lane; i < total; i += BLOCK) {
-                int r = i / E::STATE, c = i - r * E::STATE;
-                lds[r * STRIDE + c] = g[i];
+            for (int i0 = lane; i0 < total; i0 += UNROLL * E::THREADS) {
+                float v[UNROLL];
+#pragma unroll
+                for (int k = 0; k < UNROLL; ++k)
+                    if (i0 + k * E::THREADS < total) v[k] = g[i0 + k * E::THREADS];
+#pragma unroll
+                for (int k = 0; k < UNROLL; ++k) {
+                    const int i = i0 + k * E::THREADS;
+                    if (i >= total) continue;
+                    const int r = i / E::STATE, c = i - r * E::STATE;
+                    lds[r * STRIDE + c] = v[k];
+                }
             }
         }
     }
 
+    // columns [c0, c1) of every row whose bit is set in `rows` (row r = bit r)
     static MRL_DEV void out(const float *lds, float *g, int nenv, int lane, int c0, int c1,
-                            const int *row_flag) {
+                            unsigned long long rows = ~0ull) {
         const int w = c1 - c0;
         const int total = nenv * w;
-        for (int i = lane; i < total; i += BLOCK) {
-            int r = i / w, c = c0 + (i - r * w);
-            if (row_flag == nullptr || row_flag[r]) g[(size_t)r * E::STATE + c] = lds[r * STRIDE + c];
+        for (int i0 = lane; i0 < total; i0 += UNROLL * E::THREADS) {
+            float v[UNROLL];
+            int at[UNROLL];
+#pragma unroll
+            for (int k = 0; k < UNROLL; ++k) {
+                const int i = i0 + k * E::THREADS;
+                at[k] = -1;
+                if (i >= total) continue;
+                const int r = i / w, c = c0 + (i - r * w);
+                if (!((rows >> r) & 1ull)) continue;
+                v[k] = lds[r * STRIDE + c];
+                at[k] = r * E::STATE + c;
+            }
+#pragma unroll
+            for (int k = 0; k < UNROLL; ++k)
+                if (at[k] >= 0) g[at[k]] = v[k];
+        }
+    }
+
+    // the same for a set of rows that is usually small: a few rows are copied one after the other
+    static MRL_DEV void out_rows(const float *lds, float *g, int nenv, unsigned long long mask, int lane,
+                                 int c0, int c1) {
+        if (__popcll(mask) > 8) {
+            out(lds, g, nenv, lane, c0, c1, mask);
+            return;
+        }
+        while (mask) {
+            const int r = __ffsll((long long)mask) - 1;
+            mask &= mask - 1;
+            for (int c = c0 + lane; c < c1; c += E::THREADS) g[(size_t)r * E::STATE + c] = lds[r * STRIDE + c];
         }
     }
 };
 
-// Resets the rows whose bit is set in `mask` (lanes of wavefront 0).  A handful of rows -- the
+// Resets the rows whose bit is set in `mask` (lanes of wavefront 0) and records the mask.  A handful of rows -- the
 // usual case inside a step -- are rebuilt one after the other by all 64 lanes together; many rows
 // (a full reset) are rebuilt by their own lanes in parallel.
 template <class E>
-MRL_DEV void reset_rows(float *rows, int *was_reset, unsigned long long mask, uint64_t seed, int env0,
-                        int lane) {
+MRL_DEV void reset_rows(float *rows, unsigned long long *was_reset, unsigned long long mask, uint64_t seed,
+                        int env0, int lane) {
     using S = Stage<E>;
+    if (lane == 0) *was_reset = mask;
     if (E::WAVE_RESET && __popcll(mask) <= 8) {
         while (mask) {
             const int src = __ffsll((long long)mask) - 1;
             mask &= mask - 1;
             E::reset_wave(rows + src * S::STRIDE, seed, env0 + src, lane);
-            if (lane == 0) was_reset[src] = 1;
         }
     } else if ((mask >> lane) & 1ull) {
         E::reset(rows + lane * S::STRIDE, seed, env0 + lane);
-        was_reset[lane] = 1;
     }
 }
 
 // AUTORESET = false: step_kernel_gpu of the trait.  AUTORESET = true: step, then rows that
 // finished are re-initialised in place (selective reset) before the observation is copied out.
 template <class E, bool AUTORESET>
-__global__ __launch_bounds__(BLOCK) void phys_step_kernel(float *states, const float *actions,
+__global__ __launch_bounds__(E::THREADS) void phys_step_kernel(float *states, const float *actions,
                                                           float *rewards, float *dones, float *obs,
                                                           const float *shapes_g, int batch,
                                                           uint64_t reset_seed, Accounting acc) {
@@ -248,56 +304,65 @@ __global__ __launch_bounds__(BLOCK) void phys_step_kernel(float *states, const f
     __shared__ float rows[E::EPB * S::STRIDE];
     __shared__ float cts[E::EPB * S::CSTRIDE];
     __shared__ float shapes[E::NSHAPE];
-    __shared__ int was_reset[E::EPB];
+    __shared__ unsigned long long was_reset;   // rows re-initialised by this launch, one bit each
     const int tid = threadIdx.x;
     const int env0 = blockIdx.x * E::EPB;
     const int nenv = min(E::EPB, batch - env0);
     float *gbase = states + (size_t)env0 * E::STATE;
 
     S::in(rows, gbase, nenv, tid);
-    for (int i = tid; i < E::NSHAPE; i += BLOCK) shapes[i] = shapes_g[i];
-    if (tid < E::EPB) was_reset[tid] = 0;
+    for (int i = tid; i < E::NSHAPE; i += E::THREADS) shapes[i] = shapes_g[i];
+    if (tid == 0) was_reset = 0;
     __syncthreads();
 
-    if constexpr (E::DETECT_WAVES > 0) {
-        // wavefront 0: first half of the step (reads and writes velocities only); wavefronts
-        // 1 .. DETECT_WAVES: contacts of one body each (read positions only), into their own lists
-        constexpr int DW = E::DETECT_WAVES > 0 ? E::DETECT_WAVES : 1;
-        constexpr int LSTRIDE = (E::L::MAX_CONTACTS * CONTACT_SIZE) | 1;
-        __shared__ float dlist[DW * E::EPB * LSTRIDE];
-        __shared__ int dcount[DW * E::EPB];
-        static_assert(E::DETECT_WAVES < BLOCK / WAVE, "one wavefront per body besides wavefront 0");
+    if constexpr (E::DETECT_TASKS > 0) {
+        // wavefront 0: first half of the step (reads and writes velocities only); the halves of the
+        // other wavefronts: contacts of one (body, vertex) pair each (read positions only), into
+        // lists of their own.  A list holds DCAP records; a vertex that fills it, or a body whose
+        // shape the task table does not cover, sends that env back to detection inside step_finish.
+        constexpr int NT = E::DETECT_TASKS, HALF = WAVE / 2, DCAP = 4;
+        constexpr int LSTRIDE = (DCAP * CONTACT_SIZE) | 1;
+        __shared__ float dlist[NT * E::EPB * LSTRIDE];
+        __shared__ int dcount[NT * E::EPB];
+        static_assert(E::EPB <= HALF && (NT + 1) / 2 < E::THREADS / WAVE, "two tasks per wavefront besides wavefront 0");
         const int wave = tid / WAVE, lane = tid % WAVE;
         typename E::Carry carry{};
         if (wave == 0) {
             if (lane < nenv)
                 carry = E::step_begin(rows + lane * S::STRIDE, env0 + lane, actions + (size_t)(env0 + lane) * E::ACT_W);
-        } else if (wave <= E::DETECT_WAVES && lane < nenv) {
-            dcount[(wave - 1) * E::EPB + lane] = edge_detect_body<typename E::L>(
-                rows + lane * S::STRIDE, shapes, wave - 1, dlist + ((wave - 1) * E::EPB + lane) * LSTRIDE);
+        } else {
+            const int task = (wave - 1) * 2 + lane / HALF, e = lane % HALF;
+            if (task < NT && e < nenv) {
+                int body, vertex, max_verts;
+                E::detect_task(task, body, vertex, max_verts);
+                dcount[task * E::EPB + e] = edge_detect_vertex<typename E::L>(
+                    rows + e * S::STRIDE, shapes, body, vertex, max_verts, dlist + (task * E::EPB + e) * LSTRIDE, DCAP);
+            }
         }
         __syncthreads();
         if (wave == 0) {
             bool finished = false;
             if (lane < nenv) {
-                // concatenate the bodies' lists in body order, cut at MAX_CONTACTS
+                // concatenate the lists in (body, vertex) order, cut at MAX_CONTACTS
                 float *mine = cts + lane * S::CSTRIDE;
                 int n = 0;
-                for (int k = 0; k < E::DETECT_WAVES; ++k) {
+                bool redo = false;
+                for (int k = 0; k < NT; ++k) {
                     const float *src = dlist + (k * E::EPB + lane) * LSTRIDE;
                     const int m = dcount[k * E::EPB + lane];
+                    redo |= m < 0;
                     for (int c = 0; c < m && n < E::L::MAX_CONTACTS; ++c, ++n)
                         for (int f = 0; f < CONTACT_SIZE; ++f) mine[n * CONTACT_SIZE + f] = src[c * CONTACT_SIZE + f];
                 }
                 const int env = env0 + lane;
                 float r, d;
-                E::step_finish(rows + lane * S::STRIDE, mine, n, shapes, carry, r, d);
+                E::step_finish(rows + lane * S::STRIDE, mine, redo ? -1 : n, shapes, carry, r, d);
                 rewards[env] = r;
                 dones[env] = d;
                 account(acc, env, r, d);
                 finished = d > 0.5f;
             }
-            if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, lane);
+            if (AUTORESET) reset_rows<E>(rows, &was_reset, __ballot(finished), reset_seed, env0, lane);
         }
     } else {
         if (tid < WAVE) {
@@ -312,43 +377,43 @@ __global__ __launch_bounds__(BLOCK) void phys_step_kernel(float *states, const f
                 account(acc, env, r, d);
                 finished = d > 0.5f;
             }
-            if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, tid);
+            if (AUTORESET) reset_rows<E>(rows, &was_reset, __ballot(finished), reset_seed, env0, tid);
         }
     }
     __syncthreads();
 
-    for (int i = tid; i < nenv * E::OBS; i += BLOCK) {   // observation out: [nenv, OBS] contiguous
+    for (int i = tid; i < nenv * E::OBS; i += E::THREADS) {   // observation out: [nenv, OBS] contiguous
         int r = i / E::OBS, c = i - r * E::OBS;
         obs[(size_t)env0 * E::OBS + i] = rows[r * S::STRIDE + c];
     }
-    S::out(rows, gbase, nenv, tid, 0, E::DYN_END, nullptr);
-    S::out(rows, gbase, nenv, tid, E::L::META_OFF, E::STATE, nullptr);
-    if (AUTORESET) S::out(rows, gbase, nenv, tid, E::DYN_END, E::L::META_OFF, was_reset);
+    S::out(rows, gbase, nenv, tid, 0, E::DYN_END);
+    S::out(rows, gbase, nenv, tid, E::L::META_OFF, E::STATE);
+    if (AUTORESET) S::out_rows(rows, gbase, nenv, was_reset, tid, E::DYN_END, E::L::META_OFF);
 }
 
 template <class E>
-__global__ __launch_bounds__(BLOCK) void phys_reset_kernel(float *states, const float *dones, int batch,
+__global__ __launch_bounds__(E::THREADS) void phys_reset_kernel(float *states, const float *dones, int batch,
                                                            uint64_t seed, int selective) {
     using S = Stage<E>;
     __shared__ float rows[E::EPB * S::STRIDE];
-    __shared__ int was_reset[E::EPB];
+    __shared__ unsigned long long was_reset;   // rows re-initialised by this launch, one bit each
     const int tid = threadIdx.x;
     const int env0 = blockIdx.x * E::EPB;
     const int nenv = min(E::EPB, batch - env0);
-    if (tid < E::EPB) was_reset[tid] = 0;
+    if (tid == 0) was_reset = 0;
     __syncthreads();
     if (tid < WAVE) {
         const bool want = tid < nenv && (!selective || dones[env0 + tid] > 0.5f);
-        reset_rows<E>(rows, was_reset, __ballot(want), seed, env0, tid);
+        reset_rows<E>(rows, &was_reset, __ballot(want), seed, env0, tid);
     }
     __syncthreads();
-    S::out(rows, states + (size_t)env0 * E::STATE, nenv, tid, 0, E::STATE, was_reset);
+    S::out_rows(rows, states + (size_t)env0 * E::STATE, nenv, was_reset, tid, 0, E::STATE);
 }
 
 template <class E>
 static int launch_phys_reset(mrl_ctx *ctx, int batch, float *states, const float *dones, uint64_t seed,
                              int selective) {
-    hipLaunchKernelGGL(phys_reset_kernel<E>, dim3(grid_for(batch, E::EPB)), dim3(BLOCK), 0, ctx->stream,
+    hipLaunchKernelGGL(phys_reset_kernel<E>, dim3(grid_for(batch, E::EPB)), dim3(E::THREADS), 0, ctx->stream,
                        states, dones, batch, seed, selective);
     return MRL_OK;
 }
@@ -359,10 +424,10 @@ static int launch_phys_step(mrl_ctx *ctx, int batch, float *states, const float 
                             uint64_t reset_seed, const Accounting &acc) {
     dim3 grid(grid_for(batch, E::EPB));
     if (autoreset)
-        hipLaunchKernelGGL((phys_step_kernel<E, true>), grid, dim3(BLOCK), 0, ctx->stream, states, actions,
+        hipLaunchKernelGGL((phys_step_kernel<E, true>), grid, dim3(E::THREADS), 0, ctx->stream, states, actions,
                            rewards, dones, obs, shapes, batch, reset_seed, acc);
     else
-        hipLaunchKernelGGL((phys_step_kernel<E, false>), grid, dim3(BLOCK), 0, ctx->stream, states, actions,
+        hipLaunchKernelGGL((phys_step_kernel<E, false>), grid, dim3(E::THREADS), 0, ctx->stream, states, actions,
                            rewards, dones, obs, shapes, batch, reset_seed, acc);
     return MRL_OK;
 }

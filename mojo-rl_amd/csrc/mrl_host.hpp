@@ -38,6 +38,9 @@ struct mrl_ctx {
     std::vector<int> prof_tags;
     size_t prof_used;
     bool prof_chained;   // the last event recorded closes a phase and can open the next one
+    int prof_every;      // rollout steps between two that are timed (1 = every step)
+    long prof_step;      // rollout steps seen since profiling was armed
+    bool prof_active;    // marks of the current rollout step are recorded
 };
 
 namespace mrl {
@@ -68,11 +71,21 @@ inline int grid_for(long n, int block) { return (int)((n + block - 1) / block); 
 // between two rollout steps is charged to the first phase of the second step.
 inline void profile_mark(mrl_ctx *ctx, int tag) {
     if (!ctx->profiling || ctx->prof_used >= ctx->prof_events.size()) return;
+    if (!ctx->prof_active) {
+        ctx->prof_chained = false;
+        return;
+    }
     if (tag < 0 && ctx->prof_chained) return;
     if (hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream) != hipSuccess) return;
     ctx->prof_tags[ctx->prof_used++] = tag;
     ctx->prof_chained = tag >= 0;
 }
+
+// Decides whether the rollout step that starts now is one of the timed ones.
+inline void profile_step_begin(mrl_ctx *ctx) {
+    ctx->prof_active = !ctx->profiling || ctx->prof_every <= 1 || (ctx->prof_step++ % ctx->prof_every) == 0;
+}
+inline void profile_step_end(mrl_ctx *ctx) { ctx->prof_active = true; }
 
 }  // namespace mrl
 

@@ -26,7 +26,7 @@ __global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets
     __shared__ float hT[H * HT_LD];
     __shared__ float h2[PR * (H + 1)];
     __shared__ float ys[PR * (PA_MAX + 1)];
-    __shared__ float w2s[HEAD_LDS(H)];
+    __shared__ __align__(16) float w2s[HEAD_LDS(H)];
     const Mlp3Net &nn = nets.n[blockIdx.y];
     const float *__restrict__ x = nn.x;
     const float *__restrict__ params = nn.params;
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets
         if (a < A) {
             v = ys[r * (PA_MAX + 1) + a];
         } else {   // state-independent log_std, clamped (deep_rl/model/stochastic_actor.mojo:260-275)
-            v = w2s[H * A + A + (a - A)];
+            v = w2s[HEAD_LOG_STD(H) + (a - A)];
             if (v < -5.0f) v = -5.0f;
             else if (v > 2.0f) v = 2.0f;
         }
@@ -108,27 +108,48 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
     const float *c0 = cache, *c1 = cache + (size_t)B * (IN + H), *c2 = c1 + (size_t)B * 2 * H;
     const float *W1 = params + IN * H + H;
     const float *W2 = W1 + H * H + H;
-    // what the later phases need from global memory is requested now, so that the block waits
-    // for L2 once: the cached activations behind act' of both hidden layers, the head weights
-    float d1[PR];          // thread t < H: layer-1 cache entries of column t, rows of the tile
-    float d2[PR];          // thread t < H: h2 of column t, rows of the tile
+    // what the later phases need from global memory is requested now, in few wide loads (a
+    // wavefront can keep 64 vector-memory instructions in flight), so that the block waits for
+    // memory once: the cached activations behind act' of both hidden layers as row tiles, the head
+    // weights, the first chunk of W1
+    static_assert(PR * H == 4 * 4 * T && 2 * PR * H <= KCH * (H + 1), "tile staging layout");
+    float4 t1[4], t2[4];   // 32 x H tiles of the layer-1 cache entries and of h2, 16 bytes per thread and load
     float w2row[PA_MAX];   // thread t < H: W2[t][:]
     float d0[16];          // layer-0 cache entries at this lane's accumulator positions
-    {
-        const int n1 = t % H;
+    const int wrow = t % H, wseg = (t / H) * (KCH / 2);   // thread copies W1[wrow][o0 + wseg .. + KCH / 2)
+    float4 nxt[KCH / 8];
+    auto fetch = [&](int o0) {
+        const float4 *src = reinterpret_cast<const float4 *>(W1 + (size_t)wrow * H + o0 + wseg);
 #pragma unroll
-        for (int r = 0; r < PR; ++r) {
-            d1[r] = r < nrow ? c1[(row0 + r) * (2 * H) + H + n1] : 0.0f;
-            d2[r] = r < nrow ? c2[(row0 + r) * H + n1] : 0.0f;
+        for (int q = 0; q < KCH / 8; ++q) nxt[q] = src[q];
+    };
+    {
+        const bool vec = ((reinterpret_cast<uintptr_t>(c1) | reinterpret_cast<uintptr_t>(c2)) & 15) == 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int e = 4 * (t + q * T), r = e / H, ci = e % H;
+            const float *s1 = c1 + (row0 + r) * (2 * H) + H + ci;
+            const float *s2 = c2 + (row0 + r) * H + ci;
+            t1[q] = t2[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (r < nrow) {
+                if (vec) {
+                    t1[q] = *reinterpret_cast<const float4 *>(s1);
+                    t2[q] = *reinterpret_cast<const float4 *>(s2);
+                } else {
+                    t1[q] = make_float4(s1[0], s1[1], s1[2], s1[3]);
+                    t2[q] = make_float4(s2[0], s2[1], s2[2], s2[3]);
+                }
+            }
         }
 #pragma unroll
-        for (int a = 0; a < PA_MAX; ++a) w2row[a] = a < A ? W2[n1 * A + a] : 0.0f;
+        for (int a = 0; a < PA_MAX; ++a) w2row[a] = a < A ? W2[wrow * A + a] : 0.0f;
         const int colq = 32 * w + l31;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int row = 8 * (v >> 2) + 4 * half + (v & 3);
             d0[v] = row < nrow ? c0[(row0 + row) * (IN + H) + IN + colq] : 0.0f;
         }
+        fetch(0);
     }
     for (int i = t; i < PR * ld; i += T) {
         const int r = i / ld, a = i - r * ld;
@@ -138,13 +159,15 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
         const int r = i / IN, k = i - r * IN;
         xs[r * XS_LD + k] = r < nrow ? c0[(row0 + r) * (IN + H) + k] : 0.0f;
     }
-    __syncthreads();
-    if (t < ld) {   // column sums of the tile: bias gradient of the head, log_std gradient
-        float s = 0.0f;
-        for (int r = 0; r < PR; ++r) s += g2s[r * (2 * PA_MAX + 1) + t];
-        if (t < A) db_part[2 * H + t] = s;
-        else ls_part[(long)blockIdx.x * A + (t - A)] = s;
+    // the two tiles rest in the W1 staging buffer until the chunk loop claims it
+    float *tile1 = wT, *tile2 = wT + PR * H;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int e = 4 * (t + q * T);
+        *reinterpret_cast<float4 *>(tile1 + e) = t1[q];
+        *reinterpret_cast<float4 *>(tile2 + e) = t2[q];
     }
+    __syncthreads();
     if (t < H) {   // g1[r][n] = (sum_a g2[r][a] W2[n][a]) * act'(layer 1); thread t owns column n = t
         float colsum = 0.0f;
 #pragma unroll
@@ -155,37 +178,40 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
                 if (a < A) s = fmaf(g2s[r * (2 * PA_MAX + 1) + a], w2row[a], s);
             float g = 0.0f;
             if (r < nrow) {
-                g = s * act_deriv<ACT>(d1[r]);
+                g = s * act_deriv<ACT>(tile1[r * H + t]);
                 g1[(row0 + r) * H + t] = g;
             }
             gT[t * HT_LD + r] = g;
             colsum += g;
         }
         db_part[H + t] = colsum;   // bias gradient of layer 1, this tile's rows
-        // dW2[t][a] of the tile = sum_r h2[r][t] g2[r][a]
-        float *o2 = thin_part + (size_t)IN * H + (size_t)t * A;
+    } else {       // meanwhile the other half of the block: dW2[n][a] of the tile = sum_r h2[r][n] g2[r][a]
+        const int n = t - H;
+        float s[PA_MAX];
 #pragma unroll
-        for (int a = 0; a < PA_MAX; ++a) {
-            if (a < A) {
-                float s = 0.0f;
+        for (int a = 0; a < PA_MAX; ++a) s[a] = 0.0f;
 #pragma unroll
-                for (int r = 0; r < PR; ++r) s = fmaf(d2[r], g2s[r * (2 * PA_MAX + 1) + a], s);
-                o2[a] = s;
-            }
+        for (int r = 0; r < PR; ++r) {
+            const float h = tile2[r * H + n];
+#pragma unroll
+            for (int a = 0; a < PA_MAX; ++a)
+                if (a < A) s[a] = fmaf(h, g2s[r * (2 * PA_MAX + 1) + a], s[a]);
+        }
+        float *o2 = thin_part + (size_t)IN * H + (size_t)n * A;
+#pragma unroll
+        for (int a = 0; a < PA_MAX; ++a)
+            if (a < A) o2[a] = s[a];
+        if (n < ld) {   // column sums of the tile: bias gradient of the head, log_std gradient
+            float cs2 = 0.0f;
+            for (int r = 0; r < PR; ++r) cs2 += g2s[r * (2 * PA_MAX + 1) + n];
+            if (n < A) db_part[2 * H + n] = cs2;
+            else ls_part[(long)blockIdx.x * A + (n - A)] = cs2;
         }
     }
     // dh1 = g1 W1^T: wavefront w owns input columns [32w, 32w + 32).  The next chunk of W1 is
     // fetched into registers while the matrix cores work on the current one.
     floatx16 acc = {0};
     const int col = 32 * w + l31;
-    const int wrow = t % H, wseg = (t / H) * (KCH / 2);   // thread copies W1[wrow][o0 + wseg .. + KCH / 2)
-    float4 nxt[KCH / 8];
-    auto fetch = [&](int o0) {
-        const float4 *src = reinterpret_cast<const float4 *>(W1 + (size_t)wrow * H + o0 + wseg);
-#pragma unroll
-        for (int q = 0; q < KCH / 8; ++q) nxt[q] = src[q];
-    };
-    fetch(0);
     for (int o0 = 0; o0 < H; o0 += KCH) {
         __syncthreads();   // gT complete (first round) / previous chunk consumed
 #pragma unroll

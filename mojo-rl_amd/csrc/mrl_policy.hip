@@ -33,7 +33,7 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
     __shared__ float h2[2][PR * (H + 1)];
     __shared__ float logits[PR * (PA_MAX + 1)];
     __shared__ float vals[PR];
-    __shared__ float w2s[2][HEAD_LDS(H)];
+    __shared__ __align__(16) float w2s[2][HEAD_LDS(H)];
     constexpr int TN = 2 * H / TPW;          // threads per net
     const int t = threadIdx.x;
     const int net = t / TN;                  // 0 = actor, 1 = critic
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
     if (t < nrow && GAUSS) {    // Gaussian sampling, one lane per env, one Philox stream per (env, j)
         const int i = row0 + t;
         const float *mean_row = logits + t * (PA_MAX + 1);
-        const float *log_std_p = w2s[0] + H * A + A;
+        const float *log_std_p = w2s[0] + HEAD_LOG_STD(H);
         const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
         float total = 0.0f;
         for (int j = 0; j < A; ++j) {

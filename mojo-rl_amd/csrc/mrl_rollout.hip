@@ -184,10 +184,14 @@ int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_
     float *actions = ctx->rollout_ws + (size_t)N * (head + 1);
     float *rewards = actions + (size_t)N * 8, *dones = rewards + N;
     const size_t row = (size_t)t * N;
+    profile_step_begin(ctx);
     rc = policy_step(ctx, "mrl_rollout_step", gauss, &r->actor, &r->critic, N, r->obs, r->actor_params,
                      r->critic_params, sample_seed, actions, r->r_obs + row * od, r->r_actions + row * aw,
                      r->r_log_probs + row, r->r_values + row);
-    if (rc) return rc;
+    if (rc) {
+        profile_step_end(ctx);
+        return rc;
+    }
     profile_mark(ctx, -1);
     // the env-step kernel also stores (reward, done) into rollout row t and does the episode
     // accounting for its envs
@@ -195,9 +199,9 @@ int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_
                          r->done_returns, r->done_lengths, r->done_count, r->done_cap};
     rc = env_step_accounting(ctx, r->env_id, N, r->states, actions, rewards, dones, r->obs, step_seed,
                              reset_seed, acc);
-    if (rc) return rc;
-    profile_mark(ctx, MRL_PHASE_ENV);
-    return MRL_OK;
+    if (rc == MRL_OK) profile_mark(ctx, MRL_PHASE_ENV);
+    profile_step_end(ctx);
+    return rc;
 }
 
 }  // extern "C"

@@ -270,71 +270,40 @@ MRL_DEV int edge_detect(const float *row, const float *shapes, float *contacts) 
     return count;
 }
 
-// edge_detect restricted to body b (short polylines only): the contacts body b contributes, in
-// the same (vertex, edge) order, counted from zero.  Concatenating the lists of bodies 0, 1, ...
-// and cutting at MAX_CONTACTS reproduces edge_detect, which lets different wavefronts detect
-// different bodies of the same env at the same time.
+// edge_detect restricted to vertex v of body b, for callers that spread the vertices of an env over
+// many lanes: the contacts that vertex contributes, in edge order, counted from zero; concatenating
+// the lists in (body, vertex) order and cutting at MAX_CONTACTS reproduces edge_detect.  Returns
+// -1 when the caller has to fall back to edge_detect: the body is not a polygon of at most
+// max_verts vertices (the caller planned one lane per vertex for that many), or the vertex
+// touched `cap` edges or more (the list holds cap records; the last one only signals overflow).
 template <class L>
-MRL_DEV int edge_detect_body(const float *row, const float *shapes, int b, float *contacts) {
-    static_assert(L::MAX_EDGES <= 16, "per-body detection keeps the edge x ranges in registers");
-    int count = 0;
-    const int n_edges = (int)row[L::EDGE_COUNT_OFF];
-    const float *edges = row + L::EDGES_OFF;
-    float ex0[L::MAX_EDGES], ex1[L::MAX_EDGES];
-#pragma unroll
-    for (int e = 0; e < L::MAX_EDGES; ++e) {
-        ex0[e] = edges[e * 6];
-        ex1[e] = edges[e * 6 + 2];
-    }
+MRL_DEV int edge_detect_vertex(const float *row, const float *shapes, int b, int v, int max_verts,
+                               float *contacts, int cap) {
+    static_assert(L::MAX_EDGES <= 32, "one mask word");
     const float *B = row + L::BODIES_OFF + b * BODY_SIZE;
-    const float body_x = B[IDX_X], body_y = B[IDX_Y];
     const float *S = shapes + (int)B[IDX_SHAPE] * SHAPE_SIZE;
-    const int shape_type = (int)S[0];
+    int n_verts = (int)S[1];
+    if (n_verts > MAX_POLY_VERTS) n_verts = MAX_POLY_VERTS;
+    if ((int)S[0] != SHAPE_POLYGON || n_verts > max_verts) return -1;
+    if (v >= n_verts) return 0;
+    int n_edges = (int)row[L::EDGE_COUNT_OFF];
+    const float *edges = row + L::EDGES_OFF;
     float sin_a, cos_a;
     sincos32(B[IDX_ANGLE], sin_a, cos_a);
-    if (shape_type == SHAPE_POLYGON) {
-        int n_verts = (int)S[1];
-        if (n_verts > MAX_POLY_VERTS) n_verts = MAX_POLY_VERTS;
-        for (int v = 0; v < n_verts; ++v) {
-            const float local_x = S[2 + v * 2], local_y = S[3 + v * 2];
-            const float world_x = body_x + local_x * cos_a - local_y * sin_a;
-            const float world_y = body_y + local_x * sin_a + local_y * cos_a;
-            unsigned mask = 0;
+    const float local_x = S[2 + v * 2], local_y = S[3 + v * 2];
+    const float world_x = B[IDX_X] + local_x * cos_a - local_y * sin_a;
+    const float world_y = B[IDX_Y] + local_x * sin_a + local_y * cos_a;
+    unsigned mask = 0;
 #pragma unroll
-            for (int e = 0; e < L::MAX_EDGES; ++e)
-                if (e < n_edges && edge_x_pass(ex0[e], ex1[e], world_x)) mask |= 1u << e;
-            while (mask) {
-                const int e = __ffs((int)mask) - 1;
-                mask &= mask - 1;
-                vertex_edge_test(edges + e * 6, b, world_x, world_y, contacts, count, L::MAX_CONTACTS);
-            }
-        }
-    } else if (shape_type == SHAPE_CIRCLE) {
-        const float radius = S[1], cox = S[2], coy = S[3];
-        const float cwx = body_x + cox * cos_a - coy * sin_a;
-        const float cwy = body_y + cox * sin_a + coy * cos_a;
-        for (int e = 0; e < n_edges; ++e) {
-            const float *E = edges + e * 6;
-            float e_x0 = E[0], e_y0 = E[1], e_x1 = E[2], e_y1 = E[3], e_nx = E[4], e_ny = E[5];
-            float edge_dx = e_x1 - e_x0, edge_dy = e_y1 - e_y0;
-            float edge_len_sq = edge_dx * edge_dx + edge_dy * edge_dy;
-            if (edge_len_sq < 1e-6f) continue;
-            float t = ((cwx - e_x0) * edge_dx + (cwy - e_y0) * edge_dy) / edge_len_sq;
-            if (t < 0.0f) t = 0.0f;
-            if (t > 1.0f) t = 1.0f;
-            float closest_x = e_x0 + t * edge_dx, closest_y = e_y0 + t * edge_dy;
-            float dist_x = cwx - closest_x, dist_y = cwy - closest_y;
-            float dist = sqrtf(dist_x * dist_x + dist_y * dist_y);
-            float penetration = radius - dist;
-            if (penetration > 0.0f && count < L::MAX_CONTACTS) {
-                float cnx = e_nx, cny = e_ny;
-                if (dist > 1e-6f) { cnx = dist_x / dist; cny = dist_y / dist; }
-                put_contact(contacts + count * CONTACT_SIZE, b, closest_x, closest_y, cnx, cny, penetration);
-                count += 1;
-            }
-        }
+    for (int e = 0; e < L::MAX_EDGES; ++e)
+        if (e < n_edges && edge_x_pass(edges[e * 6], edges[e * 6 + 2], world_x)) mask |= 1u << e;
+    int count = 0;
+    while (mask) {
+        const int e = __ffs((int)mask) - 1;
+        mask &= mask - 1;
+        vertex_edge_test(edges + e * 6, b, world_x, world_y, contacts, count, cap);
     }
-    return count;
+    return count >= cap ? -1 : count;
 }
 
 template <class L>
