@@ -34,43 +34,64 @@ struct TileCache {
     int nrow;    // rows of the tile inside the batch
 };
 
-// Hidden stack of one net for the block's 32 rows; leaves act(layer1) in h2[32][H+1].
-// TPW = accumulator tiles (32 columns each) per wavefront: the net is worked on by 2H / TPW
-// threads (threadIdx.x modulo that count picks the role), so TPW = 1 spreads the same MFMA chain
-// over twice the wavefronts.  Everything a later phase needs from global memory and that does not
-// depend on earlier phases (biases, the layer-0 weights) is requested up front, so that a block
-// pays the L2 latency once rather than once per phase.
-template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32)>
-MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
-                          const TileCache tc) {
-    constexpr int T = 2 * H / TPW;
-    constexpr int K0 = PIN_MAX / 2;   // k-steps of layer 0 at the widest input
-    const int t = threadIdx.x % T, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
-    const float *W0 = p, *b0 = p + IN * H;
-    const float *W1 = b0 + H, *b1 = W1 + H * H;
+// Everything the hidden stack of one net needs from global memory that does not depend on the
+// tile's rows: biases, the layer-0 weights, the first block of layer-1 weights.  A kernel issues
+// these loads first thing (before it stages its inputs), so that a block pays the memory latency
+// once rather than once per phase.
+template <int H, int TPW, int KB>
+struct HiddenOperands {
+    static constexpr int K0 = PIN_MAX / 2;   // k-steps of layer 0 at the widest input
     int col[TPW];
     float bias0[TPW], bias1[TPW];
+    float w0[TPW][K0];
+    float bv[TPW][KB];
+
+    MRL_DEV void load(const float *__restrict__ p, int IN) {
+        constexpr int T = 2 * H / TPW;
+        const int t = threadIdx.x % T, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
+        const float *W0 = p, *b0 = p + IN * H;
+        const float *W1 = b0 + H, *b1 = W1 + H * H;
 #pragma unroll
-    for (int q = 0; q < TPW; ++q) {
-        col[q] = 32 * (TPW * w + q) + l31;
-        bias0[q] = b0[col[q]];
-        bias1[q] = b1[col[q]];
-    }
-    float bv[TPW][KB];   // first block of layer-1 weights: on its way while layer 0 runs
-#pragma unroll
-    for (int j = 0; j < KB; ++j) {
-#pragma unroll
-        for (int q = 0; q < TPW; ++q) bv[q][j] = W1[(2 * j + half) * H + col[q]];
-    }
-    {   // layer 0 (K = IN <= 32, padded to even with zeros): all operands first, then the MFMAs
-        float a0[K0], w0[TPW][K0];
+        for (int q = 0; q < TPW; ++q) {
+            col[q] = 32 * (TPW * w + q) + l31;
+            bias0[q] = b0[col[q]];
+            bias1[q] = b1[col[q]];
+        }
 #pragma unroll
         for (int kk = 0; kk < K0; ++kk) {
             const int k = 2 * kk + half;
-            const bool in = k < IN;
-            a0[kk] = in ? xs[l31 * XS_LD + k] : 0.0f;
 #pragma unroll
-            for (int q = 0; q < TPW; ++q) w0[q][kk] = in ? W0[k * H + col[q]] : 0.0f;
+            for (int q = 0; q < TPW; ++q) w0[q][kk] = k < IN ? W0[k * H + col[q]] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < KB; ++j) {
+#pragma unroll
+            for (int q = 0; q < TPW; ++q) bv[q][j] = W1[(2 * j + half) * H + col[q]];
+        }
+    }
+};
+
+// Hidden stack of one net for the block's 32 rows; leaves act(layer1) in h2[32][H+1].
+// TPW = accumulator tiles (32 columns each) per wavefront: the net is worked on by 2H / TPW
+// threads (threadIdx.x modulo that count picks the role), so TPW = 1 spreads the same MFMA chain
+// over twice the wavefronts.  `ops` = the operands loaded ahead by the same thread.
+template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32)>
+MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
+                          const TileCache tc, HiddenOperands<H, TPW, KB> &ops) {
+    constexpr int T = 2 * H / TPW;
+    constexpr int K0 = PIN_MAX / 2;
+    const int t = threadIdx.x % T, lane = t & 63, half = lane >> 5, l31 = lane & 31;
+    const float *W1 = p + IN * H + H;
+    int (&col)[TPW] = ops.col;
+    float (&bias0)[TPW] = ops.bias0, (&bias1)[TPW] = ops.bias1;
+    float (&w0)[TPW][K0] = ops.w0;
+    float (&bv)[TPW][KB] = ops.bv;
+    {   // layer 0 (K = IN <= 32, padded to even with zeros): all operands first, then the MFMAs
+        float a0[K0];
+#pragma unroll
+        for (int kk = 0; kk < K0; ++kk) {
+            const int k = 2 * kk + half;
+            a0[kk] = k < IN ? xs[l31 * XS_LD + k] : 0.0f;
         }
         floatx16 c[TPW];
 #pragma unroll

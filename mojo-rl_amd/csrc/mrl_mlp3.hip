@@ -43,18 +43,28 @@ __global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets
         tc.c1 = cache + (size_t)B * (IN + H);
         tc.c2 = tc.c1 + (size_t)B * 2 * H;
     }
-    for (int i = t; i < PR * IN; i += T) {
-        const int r = i / IN, k = i - r * IN;
-        float v = 0.0f;
-        if (r < nrow) {
-            v = x[row0 * IN + i];
-            if (cache != nullptr) tc.c0[(row0 + r) * (IN + H) + k] = v;
+    // every load that does not depend on an earlier phase goes out first
+    HiddenOperands<H, 1, 32> ops;
+    ops.load(params, IN);
+    constexpr int NX = (PR * PIN_MAX + T - 1) / T;
+    float xv[NX];
+#pragma unroll
+    for (int q = 0; q < NX; ++q) {
+        const int i = t + q * T;
+        xv[q] = (i < PR * IN && i / IN < nrow) ? x[row0 * IN + i] : 0.0f;
+    }
+    stage_head(params + IN * H + H + H * H + H, H, A, GAUSS, w2s, t, T);
+#pragma unroll
+    for (int q = 0; q < NX; ++q) {
+        const int i = t + q * T;
+        if (i < PR * IN) {
+            const int r = i / IN, k = i - r * IN;
+            xs[r * XS_LD + k] = xv[q];
+            if (r < nrow && cache != nullptr) tc.c0[(row0 + r) * (IN + H) + k] = xv[q];
         }
-        xs[r * XS_LD + k] = v;
     }
     __syncthreads();
-    stage_head(params + IN * H + H + H * H + H, H, A, GAUSS, w2s, t, T);
-    hidden_stack<H, ACT, 1>(params, IN, xs, hT, h2, tc);
+    hidden_stack<H, ACT, 1>(params, IN, xs, hT, h2, tc, ops);
     if (t < H) head<H>(w2s, A, h2, ys, PA_MAX + 1);
     __syncthreads();
     const int ld = GAUSS ? 2 * A : A;

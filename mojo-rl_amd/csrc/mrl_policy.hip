@@ -40,21 +40,31 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
     const int row0 = blockIdx.x * PR;
     const int nrow = min(PR, n - row0);
 
-    // observation tile in (rows beyond the batch read as zero), and straight out to rollout[t]
-    for (int i = t; i < PR * IN; i += 2 * TN) {
-        const int r = i / IN, k = i - r * IN;
-        float v = 0.0f;
-        if (r < nrow) {
-            v = obs[(long)row0 * IN + i];
-            r_obs[(long)row0 * IN + i] = v;
+    // every load that does not depend on an earlier phase goes out first: the net's operands, its
+    // head parameters, the observation tile (rows beyond the batch read as zero; the tile also goes
+    // straight out to rollout[t])
+    const float *p = net ? critic_p : actor_p;
+    HiddenOperands<H, TPW, 8> ops;
+    ops.load(p, IN);
+    float xv[(PR * PIN_MAX + 4 * H / TPW - 1) / (4 * H / TPW)];
+#pragma unroll
+    for (int q = 0; q < (int)(sizeof(xv) / sizeof(float)); ++q) {
+        const int i = t + q * 2 * TN;
+        xv[q] = (i < PR * IN && i / IN < nrow) ? obs[(long)row0 * IN + i] : 0.0f;
+    }
+    stage_head(p + IN * H + H + H * H + H, H, net ? 1 : A, GAUSS && net == 0, w2s[net], t % TN, TN);
+#pragma unroll
+    for (int q = 0; q < (int)(sizeof(xv) / sizeof(float)); ++q) {
+        const int i = t + q * 2 * TN;
+        if (i < PR * IN) {
+            const int r = i / IN, k = i - r * IN;
+            xs[r * XS_LD + k] = xv[q];
+            if (r < nrow) r_obs[(long)row0 * IN + i] = xv[q];
         }
-        xs[r * XS_LD + k] = v;
     }
     __syncthreads();
 
-    const float *p = net ? critic_p : actor_p;
-    stage_head(p + IN * H + H + H * H + H, H, net ? 1 : A, GAUSS && net == 0, w2s[net], t % TN, TN);
-    hidden_stack<H, ACT, TPW, 8>(p, IN, xs, hT[net], h2[net], TileCache{});
+    hidden_stack<H, ACT, TPW, 8>(p, IN, xs, hT[net], h2[net], TileCache{}, ops);
     if (t % TN < H) {
         if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1);
         else head<H>(w2s[1], 1, h2[1], vals, 1);

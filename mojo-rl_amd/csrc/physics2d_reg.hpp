@@ -22,6 +22,7 @@
 // all the terrain detectors ever emit.
 #pragma once
 #include <type_traits>
+#include <utility>
 #include "physics2d.hpp"
 
 namespace mrl {
@@ -29,18 +30,37 @@ namespace mrl {
 // floats of LDS scratch per contact: the 9-float record plus two slots for the effective masses
 constexpr int CONTACT_SCRATCH = CONTACT_SIZE + 2;
 
+// Per-body quantities of an env live in short vector values (ext_vector_type), not in arrays:
+// reading or replacing one element of a vector is an operation on the whole value, so the
+// compiler keeps it in registers from the first pass on.  (Arrays indexed inside a loop only get
+// constant indices after unrolling; by then selects of loads have been merged into loads from a
+// computed address, and the whole struct stays in memory.)
 template <int N>
-MRL_DEV float sel(const float (&a)[N], int i) {
+struct BodyVec {
+    static constexpr int W = N <= 2 ? 2 : N <= 4 ? 4 : N <= 8 ? 8 : 16;
+    typedef float type __attribute__((ext_vector_type(W)));
+};
+
+// element i (runtime) of the first N lanes of a body vector, as a select chain
+template <int N, class V, int... K>
+MRL_DEV float sel_impl(const V &a, int i, std::integer_sequence<int, K...>) {
     float r = a[0];
-#pragma unroll
-    for (int k = 1; k < N; ++k) r = (i == k) ? a[k] : r;
+    ((r = (i == K + 1) ? a[K + 1] : r), ...);
     return r;
 }
+template <int N, class V>
+MRL_DEV float sel(const V &a, int i) {
+    return sel_impl<N>(a, i, std::make_integer_sequence<int, N - 1>{});
+}
 
-template <int N>
-MRL_DEV void put(float (&a)[N], int i, float v) {
-#pragma unroll
-    for (int k = 0; k < N; ++k) a[k] = (i == k) ? v : a[k];
+// a[i] = v for runtime i < N
+template <int N, class V, int... K>
+MRL_DEV void put_impl(V &a, int i, float v, std::integer_sequence<int, K...>) {
+    ((a[K] = (i == K) ? v : a[K]), ...);
+}
+template <int N, class V>
+MRL_DEV void put(V &a, int i, float v) {
+    put_impl<N>(a, i, v, std::make_integer_sequence<int, N>{});
 }
 
 // joint j connects bodies a(j) -> b(j); DynamicTopology reads them from the row
@@ -53,7 +73,7 @@ struct DynamicTopology {
 template <class L>
 struct RegBodies {
     static constexpr int NB = L::NUM_BODIES;
-    float x[NB], y[NB], ang[NB], vx[NB], vy[NB], w[NB], im[NB], ii[NB];
+    typename BodyVec<NB>::type x, y, ang, vx, vy, w, im, ii;
 
     MRL_DEV void load(const float *row) {
 #pragma unroll
@@ -121,9 +141,9 @@ MRL_DEV ContactFixed contact_prepare(const RegBodies<L> &B, int ia, float point_
                                      float normal_x, float normal_y) {
     ContactFixed f;
     f.nx = normal_x; f.ny = normal_y;
-    f.inv_mass_a = sel(B.im, ia); f.inv_inertia_a = sel(B.ii, ia);
+    f.inv_mass_a = sel<L::NUM_BODIES>(B.im, ia); f.inv_inertia_a = sel<L::NUM_BODIES>(B.ii, ia);
     const float inv_mass_b = 0.0f, inv_inertia_b = 0.0f;
-    f.ra_x = point_x - sel(B.x, ia); f.ra_y = point_y - sel(B.y, ia);
+    f.ra_x = point_x - sel<L::NUM_BODIES>(B.x, ia); f.ra_y = point_y - sel<L::NUM_BODIES>(B.y, ia);
     const float rb_x = point_x - point_x, rb_y = point_y - point_y;
     const float ra_cross_n = f.ra_x * normal_y - f.ra_y * normal_x;
     const float rb_cross_n = rb_x * normal_y - rb_y * normal_x;
@@ -147,7 +167,7 @@ MRL_DEV void contact_velocity(RegBodies<L> &B, int ia, const ContactFixed &f, fl
                               float friction, float restitution) {
     const float normal_x = f.nx, normal_y = f.ny, ra_x = f.ra_x, ra_y = f.ra_y;
     const float inv_mass_a = f.inv_mass_a, inv_inertia_a = f.inv_inertia_a;
-    float vel_a_x = sel(B.vx, ia), vel_a_y = sel(B.vy, ia), omega_a = sel(B.w, ia);
+    float vel_a_x = sel<L::NUM_BODIES>(B.vx, ia), vel_a_y = sel<L::NUM_BODIES>(B.vy, ia), omega_a = sel<L::NUM_BODIES>(B.w, ia);
     const float vel_b_x = 0.0f, vel_b_y = 0.0f, omega_b = 0.0f, rb_x = 0.0f, rb_y = 0.0f;
     float vel_at_a_x = vel_a_x - omega_a * ra_y, vel_at_a_y = vel_a_y + omega_a * ra_x;
     float vel_at_b_x = vel_b_x - omega_b * rb_y, vel_at_b_y = vel_b_y + omega_b * rb_x;
@@ -180,9 +200,9 @@ MRL_DEV void contact_velocity(RegBodies<L> &B, int ia, const ContactFixed &f, fl
     jt = new_tangent;
     j_tangent = new_tangent - old_tangent;
     const float friction_x = j_tangent * tangent_x, friction_y = j_tangent * tangent_y;
-    put(B.vx, ia, vel_a_x + friction_x * inv_mass_a);
-    put(B.vy, ia, vel_a_y + friction_y * inv_mass_a);
-    put(B.w, ia, omega_a + (ra_x * friction_y - ra_y * friction_x) * inv_inertia_a);
+    put<L::NUM_BODIES>(B.vx, ia, vel_a_x + friction_x * inv_mass_a);
+    put<L::NUM_BODIES>(B.vy, ia, vel_a_y + friction_y * inv_mass_a);
+    put<L::NUM_BODIES>(B.w, ia, omega_a + (ra_x * friction_y - ra_y * friction_x) * inv_inertia_a);
 }
 
 template <class L>
@@ -191,13 +211,13 @@ MRL_DEV void contact_position(RegBodies<L> &B, int ia, float normal_x, float nor
     float correction = depth - slop;
     if (correction <= 0.0f) return;
     correction = baumgarte * correction;
-    const float inv_mass_a = sel(B.im, ia);
+    const float inv_mass_a = sel<L::NUM_BODIES>(B.im, ia);
     const float inv_mass_b = 0.0f;
     const float total = inv_mass_a + inv_mass_b;
     if (total == 0.0f) return;
     const float correction_a = correction * inv_mass_a / total;
-    put(B.x, ia, sel(B.x, ia) + normal_x * correction_a);
-    put(B.y, ia, sel(B.y, ia) + normal_y * correction_a);
+    put<L::NUM_BODIES>(B.x, ia, sel<L::NUM_BODIES>(B.x, ia) + normal_x * correction_a);
+    put<L::NUM_BODIES>(B.y, ia, sel<L::NUM_BODIES>(B.y, ia) + normal_y * correction_a);
 }
 
 // contact list held in registers (short MAX_CONTACTS)
@@ -268,7 +288,7 @@ struct LdsContacts {
             const int ia = (int)C[C_BODY_A];
             ContactFixed f;
             f.nx = C[C_NX]; f.ny = C[C_NY]; f.ra_x = C[C_PX]; f.ra_y = C[C_PY];
-            f.inv_mass_a = sel(B.im, ia); f.inv_inertia_a = sel(B.ii, ia);
+            f.inv_mass_a = sel<L::NUM_BODIES>(B.im, ia); f.inv_inertia_a = sel<L::NUM_BODIES>(B.ii, ia);
             f.k = k_slot(c, 0); f.k_t = k_slot(c, 1);
             float jn = C[C_JN], jt = C[C_JT];
             contact_velocity<L>(B, ia, f, jn, jt, friction, restitution);
@@ -303,8 +323,8 @@ struct RegJoints {
     static MRL_DEV void anchor(const RegBodies<L> &B, const float *J, int a, int b, float &ax, float &ay,
                                float &bx, float &by) {
         float sin_a, cos_a, sin_b, cos_b;
-        sincos32(sel(B.ang, a), sin_a, cos_a);
-        sincos32(sel(B.ang, b), sin_b, cos_b);
+        sincos32(sel<L::NUM_BODIES>(B.ang, a), sin_a, cos_a);
+        sincos32(sel<L::NUM_BODIES>(B.ang, b), sin_b, cos_b);
         const float lax = J[J_AX], lay = J[J_AY], lbx = J[J_BX], lby = J[J_BY];
         ax = lax * cos_a - lay * sin_a; ay = lax * sin_a + lay * cos_a;
         bx = lbx * cos_b - lby * sin_b; by = lbx * sin_b + lby * cos_b;
@@ -325,8 +345,8 @@ struct RegJoints {
             if (!active[j]) continue;
             const int a = ba(j), b = bb(j);
             anchor(B, J, a, b, rax[j], ray[j], rbx[j], rby[j]);
-            const float inv_ma = sel(B.im, a), inv_ia = sel(B.ii, a);
-            const float inv_mb = sel(B.im, b), inv_ib = sel(B.ii, b);
+            const float inv_ma = sel<L::NUM_BODIES>(B.im, a), inv_ia = sel<L::NUM_BODIES>(B.ii, a);
+            const float inv_mb = sel<L::NUM_BODIES>(B.im, b), inv_ib = sel<L::NUM_BODIES>(B.ii, b);
             const float k11 = inv_ma + inv_mb + inv_ia * ray[j] * ray[j] + inv_ib * rby[j] * rby[j];
             const float k12 = -inv_ia * rax[j] * ray[j] - inv_ib * rbx[j] * rby[j];
             const float k22 = inv_ma + inv_mb + inv_ia * rax[j] * rax[j] + inv_ib * rbx[j] * rbx[j];
@@ -335,7 +355,7 @@ struct RegJoints {
             const float inv_det = 1.0f / det;
             inv_k11[j] = k22 * inv_det; inv_k12[j] = -k12 * inv_det; inv_k22[j] = k11 * inv_det;
             eff[j] = inv_ia + inv_ib;
-            const float angle_a = sel(B.ang, a), angle_b = sel(B.ang, b);
+            const float angle_a = sel<L::NUM_BODIES>(B.ang, a), angle_b = sel<L::NUM_BODIES>(B.ang, b);
             const float ref = J[J_REF];
             const float angle_error = (angle_b - angle_a) - ref;
             spring_term[j] = -J[J_STIFF] * angle_error;
@@ -348,20 +368,20 @@ struct RegJoints {
         for (int j = 0; j < MJ; ++j) {
             if (!active[j]) continue;
             const int a = ba(j), b = bb(j);
-            const float vxa = sel(B.vx, a), vya = sel(B.vy, a), wa = sel(B.w, a);
-            const float inv_ma = sel(B.im, a), inv_ia = sel(B.ii, a);
-            const float vxb = sel(B.vx, b), vyb = sel(B.vy, b), wb = sel(B.w, b);
-            const float inv_mb = sel(B.im, b), inv_ib = sel(B.ii, b);
+            const float vxa = sel<L::NUM_BODIES>(B.vx, a), vya = sel<L::NUM_BODIES>(B.vy, a), wa = sel<L::NUM_BODIES>(B.w, a);
+            const float inv_ma = sel<L::NUM_BODIES>(B.im, a), inv_ia = sel<L::NUM_BODIES>(B.ii, a);
+            const float vxb = sel<L::NUM_BODIES>(B.vx, b), vyb = sel<L::NUM_BODIES>(B.vy, b), wb = sel<L::NUM_BODIES>(B.w, b);
+            const float inv_mb = sel<L::NUM_BODIES>(B.im, b), inv_ib = sel<L::NUM_BODIES>(B.ii, b);
             const float r_ax = rax[j], r_ay = ray[j], r_bx = rbx[j], r_by = rby[j];
             const float va_anchor_x = vxa - wa * r_ay, va_anchor_y = vya + wa * r_ax;
             const float vb_anchor_x = vxb - wb * r_by, vb_anchor_y = vyb + wb * r_bx;
             const float cdot_x = vb_anchor_x - va_anchor_x, cdot_y = vb_anchor_y - va_anchor_y;
             const float impulse_x = -(inv_k11[j] * cdot_x + inv_k12[j] * cdot_y);
             const float impulse_y = -(inv_k12[j] * cdot_x + inv_k22[j] * cdot_y);
-            put(B.vx, a, vxa - inv_ma * impulse_x);
-            put(B.vy, a, vya - inv_ma * impulse_y);
-            put(B.vx, b, vxb + inv_mb * impulse_x);
-            put(B.vy, b, vyb + inv_mb * impulse_y);
+            put<L::NUM_BODIES>(B.vx, a, vxa - inv_ma * impulse_x);
+            put<L::NUM_BODIES>(B.vy, a, vya - inv_ma * impulse_y);
+            put<L::NUM_BODIES>(B.vx, b, vxb + inv_mb * impulse_x);
+            put<L::NUM_BODIES>(B.vy, b, vyb + inv_mb * impulse_y);
             float cur_wa = wa - inv_ia * (r_ax * impulse_y - r_ay * impulse_x);
             float cur_wb = wb + inv_ib * (r_bx * impulse_y - r_by * impulse_x);
 
@@ -404,8 +424,8 @@ struct RegJoints {
                     cur_wb = cur_wb + inv_ib * motor_impulse;
                 }
             }
-            put(B.w, a, cur_wa);
-            put(B.w, b, cur_wb);
+            put<L::NUM_BODIES>(B.w, a, cur_wa);
+            put<L::NUM_BODIES>(B.w, b, cur_wb);
         }
     }
 
@@ -415,10 +435,10 @@ struct RegJoints {
             if (!active[j]) continue;
             const float *J = row + L::JOINTS_OFF + j * JOINT_SIZE;
             const int a = ba(j), b = bb(j);
-            const float xa = sel(B.x, a), ya = sel(B.y, a), angle_a = sel(B.ang, a);
-            const float inv_ma = sel(B.im, a), inv_ia = sel(B.ii, a);
-            const float xb = sel(B.x, b), yb = sel(B.y, b), angle_b = sel(B.ang, b);
-            const float inv_mb = sel(B.im, b), inv_ib = sel(B.ii, b);
+            const float xa = sel<L::NUM_BODIES>(B.x, a), ya = sel<L::NUM_BODIES>(B.y, a), angle_a = sel<L::NUM_BODIES>(B.ang, a);
+            const float inv_ma = sel<L::NUM_BODIES>(B.im, a), inv_ia = sel<L::NUM_BODIES>(B.ii, a);
+            const float xb = sel<L::NUM_BODIES>(B.x, b), yb = sel<L::NUM_BODIES>(B.y, b), angle_b = sel<L::NUM_BODIES>(B.ang, b);
+            const float inv_mb = sel<L::NUM_BODIES>(B.im, b), inv_ib = sel<L::NUM_BODIES>(B.ii, b);
             float r_ax, r_ay, r_bx, r_by;
             anchor(B, J, a, b, r_ax, r_ay, r_bx, r_by);
             const float anchor_ax = xa + r_ax, anchor_ay = ya + r_ay;
@@ -435,10 +455,10 @@ struct RegJoints {
             const float ik11 = k22 * inv_det, ik12 = -k12 * inv_det, ik22 = k11 * inv_det;
             const float correction_x = -baumgarte * (ik11 * cx + ik12 * cy);
             const float correction_y = -baumgarte * (ik12 * cx + ik22 * cy);
-            put(B.x, a, xa - inv_ma * correction_x);
-            put(B.y, a, ya - inv_ma * correction_y);
-            put(B.x, b, xb + inv_mb * correction_x);
-            put(B.y, b, yb + inv_mb * correction_y);
+            put<L::NUM_BODIES>(B.x, a, xa - inv_ma * correction_x);
+            put<L::NUM_BODIES>(B.y, a, ya - inv_ma * correction_y);
+            put<L::NUM_BODIES>(B.x, b, xb + inv_mb * correction_x);
+            put<L::NUM_BODIES>(B.y, b, yb + inv_mb * correction_y);
             float cur_a = angle_a - inv_ia * (r_ax * correction_y - r_ay * correction_x);
             float cur_b = angle_b + inv_ib * (r_bx * correction_y - r_by * correction_x);
             if (flags[j] & JF_LIMIT) {
@@ -454,8 +474,8 @@ struct RegJoints {
                     }
                 }
             }
-            put(B.ang, a, cur_a);
-            put(B.ang, b, cur_b);
+            put<L::NUM_BODIES>(B.ang, a, cur_a);
+            put<L::NUM_BODIES>(B.ang, b, cur_b);
         }
     }
 };
