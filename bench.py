@@ -109,6 +109,8 @@ def main():
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="lunarlander")
+    ap.add_argument("--steps-per-launch", type=int, default=250,
+                    help="collection steps per fused launch (where the workload has a fused collection kernel)")
     ap.add_argument("--update-minibatches", type=int, default=200,
                     help="minibatches of 4096 timed for the PPO-update figure")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -144,20 +146,24 @@ def main():
     rb.obs.copy_(rb.states.view(N_ENVS, E.STATE_SIZE)[:, :OBS].reshape(-1))
     desc = rb.descriptor()
 
-    for w in range(args.warmup):
-        mrl.ppo.rollout_step(ctx, desc, w % T, 7 + w, 0, 9000 + w)
+    fused = mrl.ppo.rollout_fused(desc)
+    SPL = max(1, min(args.steps_per_launch, T)) if fused else 1   # collection steps per launch
+    mrl.ppo.rollout_steps(ctx, desc, 0, min(args.warmup, T), 7, 1, 0, 0, 9000, 1)
     ctx.synchronize()
     rb.done_count.zero_()
     ctx.synchronize()
 
-    # ---- timed region: exactly `steps` collection steps
-    # HIP events around the two kernels of every 8th step: an event between two launches costs
-    # device time (about 3 us each here), so timing every step would slow the region it measures
-    ctx.profile_begin(4 * T + 16, sample_every=EVENT_STRIDE)
+    # ---- timed region: exactly `steps` collection steps through mrl_rollout_steps.  Where that is
+    # one fused launch per call, every launch is bracketed by HIP events; where it issues two
+    # kernels per step, the events go around the kernels of every 8th step (an event between two
+    # launches costs device time, about 3 us each here, so timing every step would slow the region
+    # it measures).
+    ctx.profile_begin(4 * T + 16, sample_every=1 if fused else EVENT_STRIDE)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for t in range(T):
-        mrl.ppo.rollout_step(ctx, desc, t, 1000 + t, 0, 50000 + t)
+    for c in range(0, T, SPL if fused else T):
+        n = min(SPL, T - c) if fused else T
+        mrl.ppo.rollout_steps(ctx, desc, c, n, 1000 + c, 1, 0, 0, 50000 + c, 1)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     phases = ctx.profile_end()
@@ -165,24 +171,55 @@ def main():
     episodes = int(rb.done_count.item())
 
     ph_us = {k: (1e3 * v[0] / max(v[1], 1)) for k, v in phases.items()}
-    fwd_us, env_us = ph_us["policy_fwd"], ph_us["env_step"]
+    traffic = measured_traffic() if args.workload == "lunarlander" else {}
+    kernels = {}
+    if fused:
+        # one kernel does everything: its nearest roofline is the fp32 matrix-core peak (the policy
+        # forward is the only throughput-bound part; the env step is a serial chain per wavefront)
+        launch_us = ph_us["collect"]
+        steps_per_launch = T / max(phases["collect"][1], 1)
+        tflops = FWD_FLOPS * N_ENVS * steps_per_launch / (launch_us * 1e-6) / 1e12
+        name = "mrl::collect_kernel<mrl::%s, %d, %d, false>" % (env_name.replace("V2", ""), HIDDEN, 1 if ACT == "relu" else 2)
+        roofline = {"kernel": name + " (policy forward + sampling + env step + auto-reset + rollout stores, %d steps per launch)" % steps_per_launch,
+                    "bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": traffic.get(name),
+                    "avg_launch_us": launch_us, "steps_per_launch": steps_per_launch,
+                    "us_per_step": launch_us / steps_per_launch}
+        kernels["collect_TFLOPs"] = tflops
+        # the same steps issued as two kernels per step (mrl_rollout_step), for comparison
+        T2 = min(T, 200)
+        ctx.profile_begin(4 * T2 + 16, sample_every=EVENT_STRIDE)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for t in range(T2):
+            mrl.ppo.rollout_step(ctx, desc, t, 3000 + t, 0, 70000 + t)
+        torch.cuda.synchronize()
+        dt2 = time.perf_counter() - t2
+        ph2 = ctx.profile_end()
+        ph2_us = {k: (1e3 * v[0] / max(v[1], 1)) for k, v in ph2.items()}
+        two = {"steps": T2, "env_steps_per_s": N_ENVS * T2 / dt2, "us_per_step": 1e6 * dt2 / T2,
+               "policy_kernel_us": ph2_us["policy_fwd"], "env_step_kernel_us": ph2_us["env_step"]}
+        fwd_us, env_us = ph2_us["policy_fwd"], ph2_us["env_step"]
+    else:
+        two = None
+        fwd_us, env_us = ph_us["policy_fwd"], ph_us["env_step"]
     fwd_tflops = FWD_FLOPS * N_ENVS / (fwd_us * 1e-6) / 1e12
     env_gbs = ENV_STEP_BYTES * N_ENVS / (env_us * 1e-6) / 1e9
-    traffic = measured_traffic() if args.workload == "lunarlander" else {}
-    if fwd_us >= env_us:
-        name = "mrl::policy_kernel<%d, %d, %s>" % (HIDDEN, 1 if ACT == "relu" else 2, "true" if continuous else "false")
-        roofline = {"kernel": name + " (actor + critic forward, sampling, stores)", "bound": "mfma",
-                    "achieved": fwd_tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": fwd_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": traffic.get(name),
-                    "avg_launch_us": fwd_us}
-    else:
-        name = {"lunarlander": "mrl::phys_step_kernel<mrl::LunarLander, true>",
-                "bipedal": "mrl::phys_step_kernel<mrl::BipedalWalker, true>",
-                "halfcheetah": "mrl::phys_step_kernel<mrl::HalfCheetah, true>",
-                "cartpole": "mrl::cartpole_step_kernel", "pendulum": "mrl::pendulum_step_kernel"}[args.workload]
-        roofline = {"kernel": name + " (env step + auto-reset + post-step stores)", "bound": "hbm",
-                    "achieved": env_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": env_gbs / HBM_PEAK_GBS,
-                    "traffic": traffic.get(name), "avg_launch_us": env_us}
+    if not fused:
+        if fwd_us >= env_us:
+            name = "mrl::policy_kernel<%d, %d, %s>" % (HIDDEN, 1 if ACT == "relu" else 2, "true" if continuous else "false")
+            roofline = {"kernel": name + " (actor + critic forward, sampling, stores)", "bound": "mfma",
+                        "achieved": fwd_tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                        "frac": fwd_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": traffic.get(name),
+                        "avg_launch_us": fwd_us}
+        else:
+            name = {"lunarlander": "mrl::phys_step_kernel<mrl::LunarLander, true>",
+                    "bipedal": "mrl::phys_step_kernel<mrl::BipedalWalker, true>",
+                    "halfcheetah": "mrl::phys_step_kernel<mrl::HalfCheetah, true>",
+                    "cartpole": "mrl::cartpole_step_kernel", "pendulum": "mrl::pendulum_step_kernel"}[args.workload]
+            roofline = {"kernel": name + " (env step + auto-reset + post-step stores)", "bound": "hbm",
+                        "achieved": env_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": env_gbs / HBM_PEAK_GBS,
+                        "traffic": traffic.get(name), "avg_launch_us": env_us}
 
     # ---- PPO update on the collected batch (minibatch 4096, reference defaults)
     MB = min(4096, N_ENVS * T)
@@ -217,14 +254,17 @@ def main():
         "ppo_update": {"minibatches_timed": n_mb, "ms_per_minibatch": 1e3 * dtu / n_mb,
                        "gae_plus_normalise_ms": gae_ms},
         "episodes_finished": episodes,
-        "phase_us_per_step": ph_us,
-        "phase_events": {"sampled_every_n_steps": EVENT_STRIDE, "launches_timed": phases["env_step"][1]},
-        "kernels": {"policy_fwd_TFLOPs": fwd_tflops, "env_step_GBs": env_gbs,
-                    "env_step_frac_hbm": env_gbs / HBM_PEAK_GBS,
-                    "policy_fwd_frac_mfma": fwd_tflops / MFMA_FP32_PEAK_TFLOPS,
-                    "update_TFLOPs": 3.0 * FWD_FLOPS * update_sps / 1e12},
+        "phase_us": ph_us,
+        "phase_events": ({"launches_timed": phases["collect"][1], "steps_per_launch": SPL} if fused else
+                         {"sampled_every_n_steps": EVENT_STRIDE, "launches_timed": phases["env_step"][1]}),
+        "kernels": dict(kernels, policy_fwd_TFLOPs=fwd_tflops, env_step_GBs=env_gbs,
+                        env_step_frac_hbm=env_gbs / HBM_PEAK_GBS,
+                        policy_fwd_frac_mfma=fwd_tflops / MFMA_FP32_PEAK_TFLOPS,
+                        update_TFLOPs=3.0 * FWD_FLOPS * update_sps / 1e12),
         "roofline": roofline,
     }
+    if two is not None:
+        out["two_kernels_per_step"] = two
     if args.copy_calibration:
         src = torch.ones(16 * 1024 * 1024, device="cuda")
         dst = torch.empty_like(src)

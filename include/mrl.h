@@ -81,7 +81,8 @@ enum {
     MRL_PHASE_SAMPLE = 1,     /* sampling + pre-step stores */
     MRL_PHASE_ENV = 2,        /* env step (+ auto-reset) */
     MRL_PHASE_POST = 3,       /* post-step stores and episode accounting */
-    MRL_PHASE_COUNT = 4
+    MRL_PHASE_COLLECT = 4,    /* a fused launch of mrl_rollout_steps (all of the above, many steps) */
+    MRL_PHASE_COUNT = 5
 };
 int mrl_profile_begin(mrl_ctx *ctx, int max_marks);
 /* Time only every `every`-th call of mrl_rollout_step (1, the default: all of them).  An event
@@ -233,6 +234,24 @@ typedef struct {
 
 int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_seed,
                      uint64_t step_seed, uint64_t reset_seed);
+
+/* The collection loop itself, `for t in range(rollout_len)` of train_gpu (deep_agents/ppo/ppo.mojo:
+ * 2058-2293, ppo_continuous.mojo:2600-2850): steps t0 .. t0 + n_steps - 1 of the rollout, step
+ * t0 + k with the seeds  sample_seed + k * sample_stride (mod 2^32),  step_seed + k * step_stride
+ * and reset_seed + k * reset_stride (mod 2^64) -- the reference derives its per-step seeds from
+ * the step counter in the same affine way.  Buffers end up as after n_steps calls of
+ * mrl_rollout_step with those seeds, except that the order of the finished-episode list
+ * (done_returns / done_lengths) inside the call is unspecified.  Where the env and the networks
+ * allow it (LunarLander, hidden width 256) the whole range is ONE launch: each workgroup keeps its
+ * 32 env rows in LDS and alternates policy forward and env step on them, so states and
+ * observations cross HBM once per call instead of twice per step; otherwise the steps are issued
+ * one by one.  Enqueue only. */
+int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, uint32_t sample_seed,
+                      uint32_t sample_stride, uint64_t step_seed, uint64_t step_stride,
+                      uint64_t reset_seed, uint64_t reset_stride);
+/* 1 when mrl_rollout_steps runs this descriptor as one launch per call, 0 when it issues the
+ * steps one by one (no counterpart in the reference: a caller that times launches asks this). */
+int mrl_rollout_fused(const mrl_rollout *r);
 
 /* ------------------------------------------------------------------ minibatch update
  * The body of train_gpu's minibatch loop (deep_agents/ppo/ppo.mojo:2438-2727 for DeepPPOAgent,

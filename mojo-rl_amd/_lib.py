@@ -100,12 +100,14 @@ SIGNATURES = {
     "mrl_policy_step_discrete": [P, DP, DP, I, P, P, P, U32, P, P, P, P, P],
     "mrl_policy_step_gaussian": [P, DP, DP, I, P, P, P, U32, P, P, P, P, P],
     "mrl_rollout_step": [P, RP, I, U32, U64, U64],
+    "mrl_rollout_steps": [P, RP, I, I, U32, U32, U64, U64, U64, U64],
+    "mrl_rollout_fused": [RP],
     "mrl_ppo_update_minibatch": [P, UP, P, I, I],
     "mrl_ppo_update_epoch": [P, UP, P, I, I, I],
 }
 _SPECIAL = {"mrl_version": (C.c_int, []), "mrl_last_error": (C.c_char_p, [])}
 # size queries return a count, not a status
-_RAW_INT = {"mrl_mlp_param_size", "mrl_mlp_cache_size", "mrl_mlp_out_dim"}
+_RAW_INT = {"mrl_mlp_param_size", "mrl_mlp_cache_size", "mrl_mlp_out_dim", "mrl_rollout_fused"}
 
 
 def exported_names():

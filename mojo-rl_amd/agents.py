@@ -62,12 +62,13 @@ class _PPOAgentBase:
             if max_rollouts is not None and metrics.rollouts >= max_rollouts:
                 break
             rb.done_count.zero_()
-            for t in range(T):
-                ppo.rollout_step(ctx, desc, t,
-                                 (total_steps * 2654435761 + t * 7919) & 0xFFFFFFFF,
-                                 (total_steps * 1103515245 + t * 12345) & (2**64 - 1),
-                                 (total_steps * 1013904223 + t * 2654435761) & (2**64 - 1))
-                total_steps += N
+            # step t of this rollout draws its seeds from the running step count, which grows by N
+            # per step: affine in t, so the whole rollout is one call (one launch where fusable)
+            ppo.rollout_steps(ctx, desc, 0, T,
+                              total_steps * 2654435761, N * 2654435761 + 7919,
+                              total_steps * 1103515245, N * 1103515245 + 12345,
+                              total_steps * 1013904223, N * 1013904223 + 2654435761)
+            total_steps += N * T
             # annealing (ppo.mojo:2385-2406)
             progress = min(1.0, total_steps / float(target_steps))
             if self.anneal_lr:

@@ -41,7 +41,7 @@ class DeviceContext:
     def synchronize(self):
         _lib.call("mrl_ctx_synchronize", self.handle)
 
-    PHASES = ("policy_fwd", "sample_store", "env_step", "post_store")
+    PHASES = ("policy_fwd", "sample_store", "env_step", "post_store", "collect")
 
     def profile_begin(self, max_marks=8192, sample_every=1):
         """Arm per-phase device timing (HIP events on this context's stream); with sample_every = k

@@ -46,9 +46,11 @@ struct HiddenOperands {
     float w0[TPW][K0];
     float bv[TPW][KB];
 
-    MRL_DEV void load(const float *__restrict__ p, int IN) {
+    // tid: the caller's thread index (a caller that loops over many tiles may pass a copy the
+    // optimiser cannot see through, so that nothing derived from it is kept across iterations)
+    MRL_DEV void load(const float *__restrict__ p, int IN, int tid = threadIdx.x) {
         constexpr int T = 2 * H / TPW;
-        const int t = threadIdx.x % T, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
+        const int t = tid % T, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
         const float *W0 = p, *b0 = p + IN * H;
         const float *W1 = b0 + H, *b1 = W1 + H * H;
 #pragma unroll
@@ -75,12 +77,15 @@ struct HiddenOperands {
 // TPW = accumulator tiles (32 columns each) per wavefront: the net is worked on by 2H / TPW
 // threads (threadIdx.x modulo that count picks the role), so TPW = 1 spreads the same MFMA chain
 // over twice the wavefronts.  `ops` = the operands loaded ahead by the same thread.
-template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32)>
+// H2_ON_HT: h2 may share its memory with hT (the block waits until every wavefront has finished
+// reading hT before the first h2 element is written).
+template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32), bool H2_ON_HT = false>
 MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
-                          const TileCache tc, HiddenOperands<H, TPW, KB> &ops) {
+                          const TileCache tc, HiddenOperands<H, TPW, KB> &ops, int tid = threadIdx.x) {
+    static_assert(PR * (H + 1) <= H * HT_LD, "h2 fits into hT");
     constexpr int T = 2 * H / TPW;
     constexpr int K0 = PIN_MAX / 2;
-    const int t = threadIdx.x % T, lane = t & 63, half = lane >> 5, l31 = lane & 31;
+    const int t = tid % T, lane = t & 63, half = lane >> 5, l31 = lane & 31;
     const float *W1 = p + IN * H + H;
     int (&col)[TPW] = ops.col;
     float (&bias0)[TPW] = ops.bias0, (&bias1)[TPW] = ops.bias1;
@@ -153,6 +158,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
                 }
             }
         }
+        if (H2_ON_HT) __syncthreads();
 #pragma unroll
         for (int q = 0; q < TPW; ++q) {
 #pragma unroll
@@ -202,9 +208,9 @@ MRL_DEV void stage_head(const float *__restrict__ W2, int H, int A, bool with_lo
 // wavefront then read distinct LDS banks).  w2s: the head parameters in LDS (stage_head); called
 // by the first H threads of the net.
 template <int H>
-MRL_DEV void head(const float *w2s, int A, const float *h2, float *out, int out_ld) {
+MRL_DEV void head(const float *w2s, int A, const float *h2, float *out, int out_ld, int tid = threadIdx.x) {
     constexpr int TPR = H / PR;
-    const int t = threadIdx.x % H, r = t / TPR, part = t % TPR;
+    const int t = tid % H, r = t / TPR, part = t % TPR;
     float acc[PA_MAX];
 #pragma unroll
     for (int a = 0; a < PA_MAX; ++a) acc[a] = 0.0f;

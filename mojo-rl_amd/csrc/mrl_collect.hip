@@ -1,0 +1,212 @@
+// Fused collection kernel: many rollout steps of a block's envs in ONE launch.
+//
+// Envs do not interact and the policy does not change during a rollout, so a workgroup can take
+// its 32 envs through any number of steps on its own: the env rows stay in LDS from the first step
+// to the last (HBM sees them once in and once out per launch, however many steps), the
+// observation tile feeds the policy straight from those rows, and the sampled actions reach the
+// env step through LDS.  Per step and block:
+//   policy   actor and critic  OBS -> H -> H -> A | 1  on the fp32 matrix cores (the 32 x H tiles
+//            of mlp_tile.hpp, weights streamed from L2), categorical / Gaussian sampling,
+//            rollout row t of obs, action, log-prob and value written;
+//   env      the step of env_block.hpp (wavefront 0 one env per lane, the others contact
+//            detection), reward / done of rollout row t, episode accounting, in-place reset.
+// No workgroup waits for another, so there is nothing between two steps but the block's own
+// barriers; the launch ends when every block has done its n_steps.
+//
+// It gives what n_steps calls of mrl_rollout_step give (same per-env streams: seeds are affine
+// in the step number), except that the finished-episode list is appended in the order in which
+// blocks get there rather than step by step.
+#include "mrl_host.hpp"
+#include "mrl_device.hpp"
+#include "mlp_tile.hpp"
+#include "policy_sample.hpp"
+#include "env_block.hpp"
+
+namespace mrl {
+
+struct CollectArgs {
+    float *states, *obs;                  // [N][STATE], [N][OBS]
+    const float *actor_p, *critic_p, *shapes;
+    int n_envs, A, t0, n_steps;
+    uint32_t sample_seed, sample_stride;
+    uint64_t reset_seed, reset_stride;
+    float *r_obs, *r_actions, *r_logp, *r_values, *r_rewards, *r_dones;   // time-major, row 0
+    Accounting acc;                       // r_rewards / r_dones unused here (set per step)
+};
+
+template <int A, int B>
+constexpr int cmax() { return A > B ? A : B; }
+
+template <class E, int H, int ACT, bool GAUSS>
+__global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
+    using S = Stage<E>;
+    constexpr int TPW = 2, TN = 2 * H / TPW, IN = E::OBS, AW = E::ACT_W;
+    static_assert(E::EPB == PR && E::THREADS == 2 * TN, "one 32-row policy tile per block, both nets side by side");
+    static_assert(IN <= PIN_MAX && AW <= PA_MAX, "policy tile limits");
+    __shared__ float rows[PR * S::STRIDE];
+    __shared__ float xs[PR * XS_LD];
+    __shared__ __align__(16) float w2s[2][HEAD_LDS(H)];
+    __shared__ float logits[PR * (PA_MAX + 1)];
+    __shared__ float vals[PR];
+    __shared__ float act[PR * PA_MAX];
+    __shared__ float shapes[E::NSHAPE];
+    __shared__ unsigned long long was_reset;
+    // the policy's activation tiles and the env step's contact scratch are never live together
+    constexpr int POLICY_F = 2 * H * HT_LD;
+    constexpr int LIST_F = detect_list_floats<E>() + 1;
+    constexpr int ENV_F = PR * S::CSTRIDE + LIST_F + E::DETECT_TASKS * E::EPB + 1;
+    __shared__ float overlay[cmax<POLICY_F, ENV_F>()];
+    float *cts = overlay, *dlist = cts + PR * S::CSTRIDE;
+    int *dcount = reinterpret_cast<int *>(dlist + LIST_F);
+
+    const int t = threadIdx.x, net = t / TN;
+    const int env0 = blockIdx.x * PR;
+    const int nenv = min(PR, a.n_envs - env0);
+    const int N = a.n_envs;
+    float *gbase = a.states + (size_t)env0 * E::STATE;
+    const float *p = net ? a.critic_p : a.actor_p;
+    S::in(rows, gbase, nenv, t);
+    for (int i = t; i < E::NSHAPE; i += E::THREADS) shapes[i] = a.shapes[i];
+    stage_head(p + IN * H + H + H * H + H, H, net ? 1 : a.A, GAUSS && net == 0, w2s[net], t % TN, TN);
+    if (t == 0) was_reset = 0;
+    __syncthreads();
+
+    for (int k = 0; k < a.n_steps; ++k) {
+        // Nothing but the rows is carried from one step to the next: the thread index, the block's
+        // env count and the parameter pointer pass through empty asm statements at the top of each
+        // step, so the optimiser cannot keep what it derives from them (addresses, predicates, the
+        // step-invariant operand values) live through the env step, whose solver needs the registers.
+        int tid = t, ne = __builtin_amdgcn_readfirstlane(nenv), A = __builtin_amdgcn_readfirstlane(a.A);
+        const float *ps = p;
+        asm volatile("" : "+v"(tid), "+v"(ps), "+s"(ne), "+s"(A) : : "memory");
+        const size_t row = (size_t)(a.t0 + k) * N + env0;   // this block's slice of rollout row t
+        const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
+        // ---- policy
+        HiddenOperands<H, TPW, 8> ops;
+        ops.load(ps, IN, tid);
+        for (int i = tid; i < PR * IN; i += E::THREADS) {
+            const int r = i / IN, c = i - r * IN;
+            float v = 0.0f;
+            if (r < ne) {
+                v = rows[r * S::STRIDE + c];
+                a.r_obs[row * IN + i] = v;
+            }
+            xs[r * XS_LD + c] = v;
+        }
+        __syncthreads();
+        float *hT = overlay + (tid / TN) * (H * HT_LD);
+        hidden_stack<H, ACT, TPW, 8, true>(ps, IN, xs, hT, hT, TileCache{}, ops, tid);
+        if (tid < TN) head<H>(w2s[0], A, hT, logits, PA_MAX + 1, tid);
+        else head<H>(w2s[1], 1, hT, vals, 1, tid);
+        __syncthreads();
+        if (tid < ne) {
+            const int i = env0 + tid;
+            float logp;
+            if (GAUSS) {
+                float av[PA_MAX];
+                logp = sample_gaussian(logits + tid * (PA_MAX + 1), w2s[0] + HEAD_LOG_STD(H), A, sseed, i, av);
+                for (int j = 0; j < A; ++j) {
+                    act[tid * AW + j] = av[j];
+                    a.r_actions[(row + tid) * AW + j] = av[j];
+                }
+            } else {
+                int sel;
+                sample_categorical(logits + tid * (PA_MAX + 1), A, sseed, i, sel, logp);
+                act[tid] = (float)sel;
+                a.r_actions[row + tid] = (float)sel;
+            }
+            a.r_logp[row + tid] = logp;
+            a.r_values[row + tid] = vals[tid];
+        }
+        __syncthreads();   // actions visible; the activation tiles are dead from here on
+        // ---- env step
+        Accounting acc = a.acc.at(env0);
+        acc.r_rewards = a.r_rewards + row;
+        acc.r_dones = a.r_dones + row;
+        phys_step_block<E, true>(rows, cts, shapes, dlist, dcount, &was_reset, act, nullptr, nullptr, env0, ne,
+                                 a.reset_seed + (uint64_t)k * a.reset_stride, acc, tid);
+        __syncthreads();
+    }
+
+    for (int i = t; i < nenv * E::OBS; i += E::THREADS) {
+        const int r = i / E::OBS, c = i - r * E::OBS;
+        a.obs[(size_t)env0 * E::OBS + i] = rows[r * S::STRIDE + c];
+    }
+    S::out(rows, gbase, nenv, t, 0, E::STATE);
+}
+
+// true when mrl_rollout_steps can run the descriptor through collect_kernel
+static bool collect_fusable(const mrl_rollout *r, bool gauss, int *act) {
+    if (r->env_id != MRL_ENV_LUNARLANDER || gauss) return false;
+    const mrl_mlp_desc &a = r->actor, &c = r->critic;
+    if (a.n_layers != 3 || c.n_layers != 3) return false;
+    const int k0 = a.layers[0].kind;
+    if (k0 != MRL_LINEAR_RELU && k0 != MRL_LINEAR_TANH) return false;
+    for (const mrl_mlp_desc *d : {&a, &c}) {
+        if (d->layers[0].kind != k0 || d->layers[1].kind != k0) return false;
+        if (d->layers[0].in_dim != LunarLander::OBS || d->layers[0].out_dim != 256 || d->layers[1].out_dim != 256)
+            return false;
+    }
+    if (a.layers[2].kind != MRL_LINEAR || c.layers[2].kind != MRL_LINEAR) return false;
+    if (a.layers[2].out_dim > PA_MAX || c.layers[2].out_dim != 1) return false;
+    *act = (k0 == MRL_LINEAR_RELU) ? 1 : 2;
+    return true;
+}
+
+}  // namespace mrl
+
+using namespace mrl;
+
+extern "C" {
+
+int mrl_rollout_fused(const mrl_rollout *r) {
+    int act = 0;
+    return r != nullptr && collect_fusable(r, r->num_actions == 0, &act) ? 1 : 0;
+}
+
+int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, uint32_t sample_seed,
+                      uint32_t sample_stride, uint64_t step_seed, uint64_t step_stride, uint64_t reset_seed,
+                      uint64_t reset_stride) {
+    MRL_CHECK_ARG(ctx && r, "mrl_rollout_steps: NULL argument");
+    MRL_CHECK_ARG(t0 >= 0 && n_steps >= 0, "mrl_rollout_steps: bad step range");
+    if (n_steps == 0) return MRL_OK;
+    const bool gauss = r->num_actions == 0;
+    int act = 0;
+    if (!collect_fusable(r, gauss, &act)) {
+        for (int k = 0; k < n_steps; ++k) {
+            int rc = mrl_rollout_step(ctx, r, t0 + k, sample_seed + (uint32_t)k * sample_stride,
+                                      step_seed + (uint64_t)k * step_stride, reset_seed + (uint64_t)k * reset_stride);
+            if (rc) return rc;
+        }
+        return MRL_OK;
+    }
+    MRL_CHECK_ARG(r->n_envs > 0, "mrl_rollout_steps: bad sizes");
+    MRL_CHECK_ARG(r->states && r->obs && r->actor_params && r->critic_params && r->r_obs && r->r_actions &&
+                      r->r_log_probs && r->r_values && r->r_rewards && r->r_dones && r->ep_return &&
+                      r->ep_length && r->done_returns && r->done_lengths && r->done_count,
+                  "mrl_rollout_steps: NULL buffer in descriptor");
+    MRL_CHECK_ARG(r->obs_dim == LunarLander::OBS && r->num_actions == 4 && mrl_mlp_out_dim(&r->actor) == 4,
+                  "mrl_rollout_steps: descriptor does not match the env's observation / action space");
+    const float *shapes = ctx->ll_shapes;
+    CollectArgs a{};
+    a.states = r->states; a.obs = r->obs;
+    a.actor_p = r->actor_params; a.critic_p = r->critic_params; a.shapes = shapes;
+    a.n_envs = r->n_envs; a.A = r->num_actions; a.t0 = t0; a.n_steps = n_steps;
+    a.sample_seed = sample_seed; a.sample_stride = sample_stride;
+    a.reset_seed = reset_seed; a.reset_stride = reset_stride;
+    a.r_obs = r->r_obs; a.r_actions = r->r_actions; a.r_logp = r->r_log_probs; a.r_values = r->r_values;
+    a.r_rewards = r->r_rewards; a.r_dones = r->r_dones;
+    a.acc = Accounting{r->r_rewards, r->r_dones, r->ep_return, r->ep_length, r->done_returns, r->done_lengths,
+                       r->done_count, r->done_cap};
+    const dim3 grid(grid_for(r->n_envs, PR)), block(LunarLander::THREADS);
+    profile_step_begin(ctx);
+    profile_mark(ctx, -1);
+    if (act == 1) hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 1, false>), grid, block, 0, ctx->stream, a);
+    else hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 2, false>), grid, block, 0, ctx->stream, a);
+    MRL_CHECK_LAUNCH();
+    profile_mark(ctx, MRL_PHASE_COLLECT);
+    profile_step_end(ctx);
+    return MRL_OK;
+}
+
+}  // extern "C"

@@ -45,6 +45,7 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     c->prof_every = 1;
     c->prof_step = 0;
     c->prof_active = true;
+    c->prof_open_next = false;
     MRL_CHECK_HIP(hipMalloc(&c->ll_shapes, sizeof(mrl::ll::Shapes)));
     mrl::ll::Shapes sh = mrl::ll::make_shapes();
     MRL_CHECK_HIP(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));

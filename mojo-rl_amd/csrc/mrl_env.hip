@@ -9,31 +9,9 @@
 // nothing is re-read.
 #include "mrl_host.hpp"
 #include "env_classic.hpp"
-#include "env_lunar.hpp"
-#include "env_walkers.hpp"
+#include "env_block.hpp"
 
 namespace mrl {
-
-// _store_post_step_kernel (deep_agents/ppo/ppo.mojo:692-708) + accumulate_rewards /
-// increment_steps / extract_completed_episodes (deep_rl/gpu/rl_kernels.mojo:103-200) for one env
-MRL_DEV void account(const Accounting &acc, int i, float r, float d) {
-    if (acc.r_rewards == nullptr) return;
-    acc.r_rewards[i] = r;
-    acc.r_dones[i] = d;
-    float er = acc.ep_return[i] + r;
-    float el = acc.ep_length[i] + 1.0f;
-    if (d > 0.5f) {
-        int slot = atomicAdd(acc.done_count, 1);
-        if (slot < acc.done_cap) {
-            acc.done_returns[slot] = er;
-            acc.done_lengths[slot] = el;
-        }
-        er = 0.0f;
-        el = 0.0f;
-    }
-    acc.ep_return[i] = er;
-    acc.ep_length[i] = el;
-}
 
 // ---------------------------------------------------------------- CartPole / Pendulum
 
@@ -115,184 +93,6 @@ __global__ __launch_bounds__(256) void pendulum_reset_kernel(float *states, floa
     if (selective) dones[i] = 0.0f;
 }
 
-// ---------------------------------------------------------------- physics2d envs
-// Per-env traits of the LDS-staged kernels.  EPB = env rows per workgroup (one wavefront; with
-// 32 rows the upper half of the lanes only helps with the copies), DYN_END = first float of the
-// row that a step never writes (everything before it, plus the metadata, is copied back).
-
-struct LunarLander {
-    using L = ll::L;
-    static constexpr int STATE = ll::STATE, OBS = ll::OBS, ACT_W = 1, EPB = 32, THREADS = 512;
-    static constexpr int DYN_END = L::JOINTS_OFF, NSHAPE = 3 * SHAPE_SIZE;
-    static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
-                             float &r, float &d) {
-        ll::step_row(row, cts, shapes, env, (int)a[0], r, d);
-    }
-    static MRL_DEV void reset(float *row, uint64_t seed, int env) {
-        ll::reset_row(row, ll::combined_seed(seed, env));
-    }
-    static constexpr bool WAVE_RESET = true;
-    static MRL_DEV void reset_wave(float *row, uint64_t seed, int env, int lane) {
-        ll::reset_row_wave(row, ll::combined_seed(seed, env), lane);
-    }
-    // contact detection runs beside the engines of wavefront 0: every half of wavefronts 1 .. 7
-    // takes one (body, vertex) pair of the block's 32 envs -- hull 6 vertices, legs 4 each
-    static constexpr int DETECT_TASKS = 14;
-    static MRL_DEV void detect_task(int k, int &body, int &vertex, int &max_verts) {
-        if (k < 6) { body = 0; vertex = k; max_verts = 6; }
-        else if (k < 10) { body = 1; vertex = k - 6; max_verts = 4; }
-        else { body = 2; vertex = k - 10; max_verts = 4; }
-    }
-    using Carry = ll::StepCarry;
-    static MRL_DEV Carry step_begin(float *row, int env, const float *a) { return ll::step_begin(row, env, (int)a[0]); }
-    static MRL_DEV void step_finish(float *row, float *cts, int n, const float *shapes, const Carry &c, float &r,
-                                    float &d) {
-        ll::step_finish(row, cts, n, shapes, c, r, d);
-    }
-};
-
-struct BipedalWalker {
-    using L = bw::L;
-    static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 32, THREADS = 256;
-    static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = bw::NSHAPE_FLOATS;
-    static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
-                             float &r, float &d) {
-        bw::step_row(row, cts, shapes, env, a, r, d);
-    }
-    static MRL_DEV void reset(float *row, uint64_t seed, int env) { bw::reset_row(row, walker_seed(seed, env)); }
-    static constexpr bool WAVE_RESET = false;
-    static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
-    static constexpr int DETECT_TASKS = 0;
-    static MRL_DEV void detect_task(int, int &, int &, int &) {}
-    struct Carry {};
-    static MRL_DEV Carry step_begin(float *, int, const float *) { return Carry{}; }
-    static MRL_DEV void step_finish(float *, float *, int, const float *, const Carry &, float &, float &) {}
-};
-
-struct HalfCheetah {
-    using L = hc::L;
-    static constexpr int STATE = hc::STATE, OBS = hc::OBS, ACT_W = hc::ACT, EPB = 64, THREADS = 256;
-    static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = hc::NSHAPE_FLOATS;
-    static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
-                             float &r, float &d) {
-        hc::step_row(row, cts, shapes, env, a, r, d);
-    }
-    static MRL_DEV void reset(float *row, uint64_t seed, int env) { hc::reset_row(row, walker_seed(seed, env)); }
-    static constexpr bool WAVE_RESET = false;
-    static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
-    static constexpr int DETECT_TASKS = 0;
-    static MRL_DEV void detect_task(int, int &, int &, int &) {}
-    struct Carry {};
-    static MRL_DEV Carry step_begin(float *, int, const float *) { return Carry{}; }
-    static MRL_DEV void step_finish(float *, float *, int, const float *, const Carry &, float &, float &) {}
-};
-
-constexpr int WAVE = 64;    // the compute phase runs on one wavefront, one lane per env
-
-template <class E>
-struct Stage {
-    static constexpr int STRIDE = E::STATE | 1;                            // odd => conflict-free lane access
-    static constexpr int CSTRIDE = (E::L::MAX_CONTACTS * CONTACT_SCRATCH) | 1;
-
-    // Copies run in batches of UNROLL independent elements per thread (all loads of a batch are
-    // issued before the first store), so a thread waits for memory once per batch and not once
-    // per element.
-    static constexpr int UNROLL = 8;
-
-    static MRL_DEV void in(float *lds, const float *g, int nenv, int lane) {
-        if (E::STATE % 4 == 0) {   // rows are whole float4s, never straddled by a 16-byte load
-            const float4 *src = reinterpret_cast<const float4 *>(g);
-            const int total4 = nenv * (E::STATE / 4);
-            for (int i0 = lane; i0 < total4; i0 += UNROLL * E::THREADS) {
-                float4 v[UNROLL];
-#pragma unroll
-                for (int k = 0; k < UNROLL; ++k)
-                    if (i0 + k * E::THREADS < total4) v[k] = src[i0 + k * E::THREADS];
-#pragma unroll
-                for (int k = 0; k < UNROLL; ++k) {
-                    if (i0 + k * E::THREADS >= total4) continue;
-                    const int f = (i0 + k * E::THREADS) * 4;
-                    const int r = f / E::STATE, c = f - r * E::STATE;
-                    float *d = lds + r * STRIDE + c;
-                    d[0] = v[k].x; d[1] = v[k].y; d[2] = v[k].z; d[3] = v[k].w;
-                }
-            }
-        } else {
-            const int total = nenv * E::STATE;
-            for (int i0 = lane; i0 < total; i0 += UNROLL * E::THREADS) {
-                float v[UNROLL];
-#pragma unroll
-                for (int k = 0; k < UNROLL; ++k)
-                    if (i0 + k * E::THREADS < total) v[k] = g[i0 + k * E::THREADS];
-#pragma unroll
-                for (int k = 0; k < UNROLL; ++k) {
-                    const int i = i0 + k * E::THREADS;
-                    if (i >= total) continue;
-                    const int r = i / E::STATE, c = i - r * E::STATE;
-                    lds[r * STRIDE + c] = v[k];
-                }
-            }
-        }
-    }
-
-    // columns [c0, c1) of every row whose bit is set in `rows` (row r = bit r)
-    static MRL_DEV void out(const float *lds, float *g, int nenv, int lane, int c0, int c1,
-                            unsigned long long rows = ~0ull) {
-        const int w = c1 - c0;
-        const int total = nenv * w;
-        for (int i0 = lane; i0 < total; i0 += UNROLL * E::THREADS) {
-            float v[UNROLL];
-            int at[UNROLL];
-#pragma unroll
-            for (int k = 0; k < UNROLL; ++k) {
-                const int i = i0 + k * E::THREADS;
-                at[k] = -1;
-                if (i >= total) continue;
-                const int r = i / w, c = c0 + (i - r * w);
-                if (!((rows >> r) & 1ull)) continue;
-                v[k] = lds[r * STRIDE + c];
-                at[k] = r * E::STATE + c;
-            }
-#pragma unroll
-            for (int k = 0; k < UNROLL; ++k)
-                if (at[k] >= 0) g[at[k]] = v[k];
-        }
-    }
-
-    // the same for a set of rows that is usually small: a few rows are copied one after the other
-    static MRL_DEV void out_rows(const float *lds, float *g, int nenv, unsigned long long mask, int lane,
-                                 int c0, int c1) {
-        if (__popcll(mask) > 8) {
-            out(lds, g, nenv, lane, c0, c1, mask);
-            return;
-        }
-        while (mask) {
-            const int r = __ffsll((long long)mask) - 1;
-            mask &= mask - 1;
-            for (int c = c0 + lane; c < c1; c += E::THREADS) g[(size_t)r * E::STATE + c] = lds[r * STRIDE + c];
-        }
-    }
-};
-
-// Resets the rows whose bit is set in `mask` (lanes of wavefront 0) and records the mask.  A handful of rows -- the
-// usual case inside a step -- are rebuilt one after the other by all 64 lanes together; many rows
-// (a full reset) are rebuilt by their own lanes in parallel.
-template <class E>
-MRL_DEV void reset_rows(float *rows, unsigned long long *was_reset, unsigned long long mask, uint64_t seed,
-                        int env0, int lane) {
-    using S = Stage<E>;
-    if (lane == 0) *was_reset = mask;
-    if (E::WAVE_RESET && __popcll(mask) <= 8) {
-        while (mask) {
-            const int src = __ffsll((long long)mask) - 1;
-            mask &= mask - 1;
-            E::reset_wave(rows + src * S::STRIDE, seed, env0 + src, lane);
-        }
-    } else if ((mask >> lane) & 1ull) {
-        E::reset(rows + lane * S::STRIDE, seed, env0 + lane);
-    }
-}
-
 // AUTORESET = false: step_kernel_gpu of the trait.  AUTORESET = true: step, then rows that
 // finished are re-initialised in place (selective reset) before the observation is copied out.
 template <class E, bool AUTORESET>
@@ -305,6 +105,8 @@ __global__ __launch_bounds__(E::THREADS) void phys_step_kernel(float *states, co
     __shared__ float cts[E::EPB * S::CSTRIDE];
     __shared__ float shapes[E::NSHAPE];
     __shared__ unsigned long long was_reset;   // rows re-initialised by this launch, one bit each
+    __shared__ float dlist[detect_list_floats<E>() + 1];
+    __shared__ int dcount[E::DETECT_TASKS * E::EPB + 1];
     const int tid = threadIdx.x;
     const int env0 = blockIdx.x * E::EPB;
     const int nenv = min(E::EPB, batch - env0);
@@ -315,71 +117,9 @@ __global__ __launch_bounds__(E::THREADS) void phys_step_kernel(float *states, co
     if (tid == 0) was_reset = 0;
     __syncthreads();
 
-    if constexpr (E::DETECT_TASKS > 0) {
-        // wavefront 0: first half of the step (reads and writes velocities only); the halves of the
-        // other wavefronts: contacts of one (body, vertex) pair each (read positions only), into
-        // lists of their own.  A list holds DCAP records; a vertex that fills it, or a body whose
-        // shape the task table does not cover, sends that env back to detection inside step_finish.
-        constexpr int NT = E::DETECT_TASKS, HALF = WAVE / 2, DCAP = 4;
-        constexpr int LSTRIDE = (DCAP * CONTACT_SIZE) | 1;
-        __shared__ float dlist[NT * E::EPB * LSTRIDE];
-        __shared__ int dcount[NT * E::EPB];
-        static_assert(E::EPB <= HALF && (NT + 1) / 2 < E::THREADS / WAVE, "two tasks per wavefront besides wavefront 0");
-        const int wave = tid / WAVE, lane = tid % WAVE;
-        typename E::Carry carry{};
-        if (wave == 0) {
-            if (lane < nenv)
-                carry = E::step_begin(rows + lane * S::STRIDE, env0 + lane, actions + (size_t)(env0 + lane) * E::ACT_W);
-        } else {
-            const int task = (wave - 1) * 2 + lane / HALF, e = lane % HALF;
-            if (task < NT && e < nenv) {
-                int body, vertex, max_verts;
-                E::detect_task(task, body, vertex, max_verts);
-                dcount[task * E::EPB + e] = edge_detect_vertex<typename E::L>(
-                    rows + e * S::STRIDE, shapes, body, vertex, max_verts, dlist + (task * E::EPB + e) * LSTRIDE, DCAP);
-            }
-        }
-        __syncthreads();
-        if (wave == 0) {
-            bool finished = false;
-            if (lane < nenv) {
-                // concatenate the lists in (body, vertex) order, cut at MAX_CONTACTS
-                float *mine = cts + lane * S::CSTRIDE;
-                int n = 0;
-                bool redo = false;
-                for (int k = 0; k < NT; ++k) {
-                    const float *src = dlist + (k * E::EPB + lane) * LSTRIDE;
-                    const int m = dcount[k * E::EPB + lane];
-                    redo |= m < 0;
-                    for (int c = 0; c < m && n < E::L::MAX_CONTACTS; ++c, ++n)
-                        for (int f = 0; f < CONTACT_SIZE; ++f) mine[n * CONTACT_SIZE + f] = src[c * CONTACT_SIZE + f];
-                }
-                const int env = env0 + lane;
-                float r, d;
-                E::step_finish(rows + lane * S::STRIDE, mine, redo ? -1 : n, shapes, carry, r, d);
-                rewards[env] = r;
-                dones[env] = d;
-                account(acc, env, r, d);
-                finished = d > 0.5f;
-            }
-            if (AUTORESET) reset_rows<E>(rows, &was_reset, __ballot(finished), reset_seed, env0, lane);
-        }
-    } else {
-        if (tid < WAVE) {
-            bool finished = false;
-            if (tid < nenv) {
-                const int env = env0 + tid;
-                float r, d;
-                E::step(rows + tid * S::STRIDE, cts + tid * S::CSTRIDE, shapes, env,
-                        actions + (size_t)env * E::ACT_W, r, d);
-                rewards[env] = r;
-                dones[env] = d;
-                account(acc, env, r, d);
-                finished = d > 0.5f;
-            }
-            if (AUTORESET) reset_rows<E>(rows, &was_reset, __ballot(finished), reset_seed, env0, tid);
-        }
-    }
+    phys_step_block<E, AUTORESET>(rows, cts, shapes, dlist, dcount, &was_reset,
+                                  actions + (size_t)env0 * E::ACT_W, rewards + env0, dones + env0, env0, nenv,
+                                  reset_seed, acc.at(env0));
     __syncthreads();
 
     for (int i = tid; i < nenv * E::OBS; i += E::THREADS) {   // observation out: [nenv, OBS] contiguous

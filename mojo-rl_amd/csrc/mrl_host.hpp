@@ -41,6 +41,7 @@ struct mrl_ctx {
     int prof_every;      // rollout steps between two that are timed (1 = every step)
     long prof_step;      // rollout steps seen since profiling was armed
     bool prof_active;    // marks of the current rollout step are recorded
+    bool prof_open_next; // the current rollout step ends with the event that opens the next one
 };
 
 namespace mrl {
@@ -56,6 +57,14 @@ struct Accounting {
     float *done_returns, *done_lengths;
     int32_t *done_count;
     int32_t done_cap;
+    // the same accounting seen from env i: per-env pointers advanced, the shared list untouched
+    __host__ __device__ Accounting at(int i) const {
+        Accounting a = *this;
+        if (r_rewards != nullptr) {
+            a.r_rewards += i; a.r_dones += i; a.ep_return += i; a.ep_length += i;
+        }
+        return a;
+    }
 };
 
 // mrl_env_step_autoreset with the bookkeeping folded into the same launch
@@ -81,11 +90,27 @@ inline void profile_mark(mrl_ctx *ctx, int tag) {
     ctx->prof_chained = tag >= 0;
 }
 
-// Decides whether the rollout step that starts now is one of the timed ones.
+// Sampled timing (prof_every = k > 1): of every k rollout steps one is timed, and the step before
+// it contributes one event, recorded after its last kernel, that opens the timed step's first
+// phase.  (An opening event recorded straight after kernels that carry no event of their own is
+// not a reliable start: the runtime may resolve it to a time before the last of them ran.)
 inline void profile_step_begin(mrl_ctx *ctx) {
-    ctx->prof_active = !ctx->profiling || ctx->prof_every <= 1 || (ctx->prof_step++ % ctx->prof_every) == 0;
+    ctx->prof_active = true;
+    ctx->prof_open_next = false;
+    if (!ctx->profiling || ctx->prof_every <= 1) return;
+    const long phase = ctx->prof_step++ % ctx->prof_every;
+    ctx->prof_active = phase == 0 && ctx->prof_chained;       // timed only if the step before opened it
+    ctx->prof_open_next = phase == ctx->prof_every - 1;
 }
-inline void profile_step_end(mrl_ctx *ctx) { ctx->prof_active = true; }
+inline void profile_step_end(mrl_ctx *ctx) {
+    if (ctx->profiling && ctx->prof_open_next && ctx->prof_used < ctx->prof_events.size() &&
+        hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream) == hipSuccess) {
+        ctx->prof_tags[ctx->prof_used++] = -1;
+        ctx->prof_chained = true;
+    }
+    ctx->prof_open_next = false;
+    ctx->prof_active = true;
+}
 
 }  // namespace mrl
 

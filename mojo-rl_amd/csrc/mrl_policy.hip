@@ -19,6 +19,7 @@
 #include "mrl_host.hpp"
 #include "mrl_device.hpp"
 #include "mlp_tile.hpp"
+#include "policy_sample.hpp"
 
 namespace mrl {
 
@@ -73,50 +74,23 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
 
     if (t < nrow && !GAUSS) {   // categorical sampling, one lane per env
         const int i = row0 + t;
-        const float *l = logits + t * (PA_MAX + 1);
-        uint32_t rng = seed ^ ((uint32_t)i * 2654435761u);
-        rng = xorshift32(rng);
-        float max_logit = l[0];
-        for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
-        float sum_exp = 0.0f;
-        for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
-        const float u = random_uniform(rng);
-        float cumsum = 0.0f;
-        int sel = 0;
-        for (int a = 0; a < A; ++a) {
-            float prob = expf(l[a] - max_logit) / sum_exp;
-            cumsum = cumsum + prob;
-            if (u < cumsum) { sel = a; break; }
-        }
-        const float pr = expf(l[sel] - max_logit) / sum_exp;
+        int sel;
+        float logp;
+        sample_categorical(logits + t * (PA_MAX + 1), A, seed, i, sel, logp);
         actions[i] = (float)sel;
         r_actions[i] = (float)sel;
-        r_logp[i] = logf(pr + 1e-8f);
+        r_logp[i] = logp;
         r_values[i] = vals[t];
     }
-    if (t < nrow && GAUSS) {    // Gaussian sampling, one lane per env, one Philox stream per (env, j)
+    if (t < nrow && GAUSS) {    // Gaussian sampling, one lane per env
         const int i = row0 + t;
-        const float *mean_row = logits + t * (PA_MAX + 1);
-        const float *log_std_p = w2s[0] + HEAD_LOG_STD(H);
-        const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
-        float total = 0.0f;
+        float act[PA_MAX];
+        const float logp = sample_gaussian(logits + t * (PA_MAX + 1), w2s[0] + HEAD_LOG_STD(H), A, seed, i, act);
         for (int j = 0; j < A; ++j) {
-            const float mean = mean_row[j];
-            float log_std = log_std_p[j];
-            if (log_std < -5.0f) log_std = -5.0f;
-            else if (log_std > 2.0f) log_std = 2.0f;
-            Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j), 0, 0);
-            const float u1 = rv.v[0] + 1e-8f;
-            const float mag = sqrtf(-2.0f * logf(u1));
-            const float noise = mag * cosf(rv.v[1] * (float)6.283185307179586);
-            const float std = expf(log_std);
-            const float action = mean + std * noise;
-            actions[(long)i * A + j] = action;
-            r_actions[(long)i * A + j] = action;
-            const float an = (action - mean) / (std + EPS);
-            total = total + -0.5f * (LOG_2PI + 2.0f * log_std + an * an);
+            actions[(long)i * A + j] = act[j];
+            r_actions[(long)i * A + j] = act[j];
         }
-        r_logp[i] = total;
+        r_logp[i] = logp;
         r_values[i] = vals[t];
     }
 }

@@ -4,6 +4,7 @@
 // a counter instead of being copied to the host after every step.
 #include "mrl_host.hpp"
 #include "mrl_device.hpp"
+#include "policy_sample.hpp"
 
 namespace mrl {
 
@@ -19,25 +20,12 @@ __global__ __launch_bounds__(256) void sample_store_kernel(
     float *__restrict__ r_actions, float *__restrict__ r_logp, float *__restrict__ r_values) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    const float *l = logits + (long)i * A;
-    uint32_t rng = seed ^ ((uint32_t)i * 2654435761u);
-    rng = xorshift32(rng);
-    float max_logit = l[0];
-    for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
-    float sum_exp = 0.0f;
-    for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
-    float u = random_uniform(rng);
-    float cumsum = 0.0f;
-    int sel = 0;
-    for (int a = 0; a < A; ++a) {
-        float prob = expf(l[a] - max_logit) / sum_exp;
-        cumsum = cumsum + prob;
-        if (u < cumsum) { sel = a; break; }
-    }
-    float p = expf(l[sel] - max_logit) / sum_exp;
+    int sel;
+    float logp;
+    sample_categorical(logits + (long)i * A, A, seed, i, sel, logp);
     actions[i] = (float)sel;
     r_actions[i] = (float)sel;
-    r_logp[i] = logf(p + 1e-8f);
+    r_logp[i] = logp;
     r_values[i] = values[i];
     for (int k = 0; k < obs_dim; ++k) r_obs[(long)i * obs_dim + k] = obs[(long)i * obs_dim + k];
 }
@@ -50,23 +38,16 @@ __global__ __launch_bounds__(256) void sample_store_gaussian_kernel(
     float *__restrict__ r_actions, float *__restrict__ r_logp, float *__restrict__ r_values) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
+    float act[16];
+    const float *head = actor_out + (long)i * 2 * A;   // [mean (A) | log_std (A)]
     float total = 0.0f;
-    for (int j = 0; j < A; ++j) {
-        float mean = actor_out[(long)i * 2 * A + j];
-        float log_std = actor_out[(long)i * 2 * A + A + j];
-        if (log_std < -5.0f) log_std = -5.0f;
-        else if (log_std > 2.0f) log_std = 2.0f;
-        Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j), 0, 0);
-        float u1 = rv.v[0] + 1e-8f;
-        float mag = sqrtf(-2.0f * logf(u1));
-        float noise = mag * cosf(rv.v[1] * (float)6.283185307179586);
-        float std = expf(log_std);
-        float action = mean + std * noise;
-        actions[(long)i * A + j] = action;
-        r_actions[(long)i * A + j] = action;
-        float an = (action - mean) / (std + EPS);
-        total = total + -0.5f * (LOG_2PI + 2.0f * log_std + an * an);
+    for (int j0 = 0; j0 < A; j0 += 16) {   // any action width, 16 components at a time
+        const int m = min(16, A - j0);
+        total = total + sample_gaussian_part(head + j0, head + A + j0, m, A, j0, seed, i, act);
+        for (int j = 0; j < m; ++j) {
+            actions[(long)i * A + j0 + j] = act[j];
+            r_actions[(long)i * A + j0 + j] = act[j];
+        }
     }
     r_logp[i] = total;
     r_values[i] = values[i];

@@ -1,0 +1,58 @@
+// Action sampling of one env from its policy head, shared by the fused policy kernel, the fused
+// collection kernel and the stand-alone sampling kernels.
+#pragma once
+#include "mrl_device.hpp"
+
+namespace mrl {
+
+// Categorical sampling from A logits (deep_agents/ppo/ppo.mojo:4064-4123): xorshift32 stream
+// keyed by (seed, env index), inverse-CDF draw, log-probability of the drawn action.
+MRL_DEV void sample_categorical(const float *l, int A, uint32_t seed, int i, int &sel, float &logp) {
+    uint32_t rng = seed ^ ((uint32_t)i * 2654435761u);
+    rng = xorshift32(rng);
+    float max_logit = l[0];
+    for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
+    float sum_exp = 0.0f;
+    for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
+    const float u = random_uniform(rng);
+    float cumsum = 0.0f;
+    sel = 0;
+    for (int a = 0; a < A; ++a) {
+        float prob = expf(l[a] - max_logit) / sum_exp;
+        cumsum = cumsum + prob;
+        if (u < cumsum) { sel = a; break; }
+    }
+    const float pr = expf(l[sel] - max_logit) / sum_exp;
+    logp = logf(pr + 1e-8f);
+}
+
+// Gaussian sampling (deep_agents/ppo/kernels.mojo:12-98) of components j0 .. j0 + m of an action
+// with A components: one Philox stream per (env, component), Box-Muller, clamped log_std;
+// returns the summed log-probability of those components and leaves them in act[0 .. m).
+MRL_DEV float sample_gaussian_part(const float *mean, const float *log_std_p, int m, int A, int j0,
+                                   uint32_t seed, int i, float *act) {
+    const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
+    float total = 0.0f;
+    for (int j = 0; j < m; ++j) {
+        const float mu = mean[j];
+        float log_std = log_std_p[j];
+        if (log_std < -5.0f) log_std = -5.0f;
+        else if (log_std > 2.0f) log_std = 2.0f;
+        Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j0 + j), 0, 0);
+        const float u1 = rv.v[0] + 1e-8f;
+        const float mag = sqrtf(-2.0f * logf(u1));
+        const float noise = mag * cosf(rv.v[1] * (float)6.283185307179586);
+        const float std = expf(log_std);
+        const float action = mu + std * noise;
+        act[j] = action;
+        const float an = (action - mu) / (std + EPS);
+        total = total + -0.5f * (LOG_2PI + 2.0f * log_std + an * an);
+    }
+    return total;
+}
+MRL_DEV float sample_gaussian(const float *mean_row, const float *log_std_p, int A, uint32_t seed, int i,
+                              float *act) {
+    return sample_gaussian_part(mean_row, log_std_p, A, A, 0, seed, i, act);
+}
+
+}  // namespace mrl

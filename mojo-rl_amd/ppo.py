@@ -159,6 +159,21 @@ def rollout_step(ctx, desc, t, sample_seed, step_seed=0, reset_seed=0):
               int(step_seed) & (2**64 - 1), int(reset_seed) & (2**64 - 1))
 
 
+def rollout_steps(ctx, desc, t0, n_steps, sample_seed, sample_stride, step_seed=0, step_stride=0,
+                  reset_seed=0, reset_stride=0):
+    """train_gpu's collection loop over steps t0 .. t0 + n_steps - 1, enqueue only: step t0 + k uses
+    the seeds  seed + k * stride  (sample: mod 2^32, step / reset: mod 2^64).  One launch where the
+    env and the networks allow it (the env rows then stay on chip for the whole range)."""
+    _lib.call("mrl_rollout_steps", ctx.handle, C.byref(desc), t0, n_steps, int(sample_seed) & 0xFFFFFFFF,
+              int(sample_stride) & 0xFFFFFFFF, int(step_seed) & (2**64 - 1), int(step_stride) & (2**64 - 1),
+              int(reset_seed) & (2**64 - 1), int(reset_stride) & (2**64 - 1))
+
+
+def rollout_fused(desc):
+    """True when rollout_steps runs this descriptor as one launch per call."""
+    return bool(_lib.call("mrl_rollout_fused", C.byref(desc)))
+
+
 class PPOUpdate:
     """Phases 2 and 3 of train_gpu (deep_agents/ppo/ppo.mojo:2296-2727 for the discrete agent,
     ppo_continuous.mojo:2852-3260 for the continuous one) on device buffers: bootstrap value,
