@@ -207,6 +207,37 @@ MRL_DEV void reset_rows(float *rows, unsigned long long *was_reset, unsigned lon
     }
 }
 
+// Per-(body, vertex) contact lists of phys_step_block: DCAP records per list (a vertex that fills
+// its list sends the env back to detection inside step_finish), list stride in floats.
+constexpr int DETECT_CAP = 4;
+constexpr int DETECT_STRIDE = (DETECT_CAP * CONTACT_SIZE) | 1;
+
+// task `task` of env slot e: detects into its list and records the count
+template <class E>
+MRL_DEV void detect_vertex_task(const float *rows, const float *shapes, float *dlist, int *dcount, int task, int e) {
+    int body, vertex, max_verts;
+    E::detect_task(task, body, vertex, max_verts);
+    dcount[task * E::EPB + e] = edge_detect_vertex<typename E::L>(
+        rows + e * Stage<E>::STRIDE, shapes, body, vertex, max_verts, dlist + (task * E::EPB + e) * DETECT_STRIDE,
+        DETECT_CAP);
+}
+
+// concatenates env slot e's lists in (body, vertex) order into `mine`, cut at MAX_CONTACTS;
+// returns the contact count, or -1 when some list asks for detection to be redone
+template <class E>
+MRL_DEV int merge_vertex_lists(const float *dlist, const int *dcount, int e, float *mine) {
+    int n = 0;
+    bool redo = false;
+    for (int k = 0; k < E::DETECT_TASKS; ++k) {
+        const float *src = dlist + (k * E::EPB + e) * DETECT_STRIDE;
+        const int m = dcount[k * E::EPB + e];
+        redo |= m < 0;
+        for (int c = 0; c < m && n < E::L::MAX_CONTACTS; ++c, ++n)
+            for (int f = 0; f < CONTACT_SIZE; ++f) mine[n * CONTACT_SIZE + f] = src[c * CONTACT_SIZE + f];
+    }
+    return redo ? -1 : n;
+}
+
 // One step of the block's LDS-resident rows (all threads of the block call it, between two
 // __syncthreads of the caller): wavefront 0 steps one env per lane, the other wavefronts detect
 // contacts where the env splits that off.  `actions` = the actions of the block's envs
@@ -222,10 +253,9 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
     if constexpr (E::DETECT_TASKS > 0) {
         // wavefront 0: first half of the step (reads and writes velocities only); the halves of the
         // other wavefronts: contacts of one (body, vertex) pair each (read positions only), into
-        // lists of their own.  A list holds DCAP records; a vertex that fills it, or a body whose
-        // shape the task table does not cover, sends that env back to detection inside step_finish.
-        constexpr int NT = E::DETECT_TASKS, HALF = WAVE / 2, DCAP = 4;
-        constexpr int LSTRIDE = (DCAP * CONTACT_SIZE) | 1;
+        // lists of their own.  A vertex that fills its list, or a body whose shape the task table
+        // does not cover, sends that env back to detection inside step_finish.
+        constexpr int NT = E::DETECT_TASKS, HALF = WAVE / 2;
         static_assert(E::EPB <= HALF && (NT + 1) / 2 < E::THREADS / WAVE, "two tasks per wavefront besides wavefront 0");
         const int wave = tid / WAVE, lane = tid % WAVE;
         typename E::Carry carry{};
@@ -234,31 +264,17 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
                 carry = E::step_begin(rows + lane * S::STRIDE, env0 + lane, actions + (size_t)lane * E::ACT_W);
         } else {
             const int task = (wave - 1) * 2 + lane / HALF, e = lane % HALF;
-            if (task < NT && e < nenv) {
-                int body, vertex, max_verts;
-                E::detect_task(task, body, vertex, max_verts);
-                dcount[task * E::EPB + e] = edge_detect_vertex<typename E::L>(
-                    rows + e * S::STRIDE, shapes, body, vertex, max_verts, dlist + (task * E::EPB + e) * LSTRIDE, DCAP);
-            }
+            if (task < NT && e < nenv) detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
         }
         __syncthreads();
         if (wave == 0) {
             bool finished = false;
             if (lane < nenv) {
-                // concatenate the lists in (body, vertex) order, cut at MAX_CONTACTS
                 float *mine = cts + lane * S::CSTRIDE;
-                int n = 0;
-                bool redo = false;
-                for (int k = 0; k < NT; ++k) {
-                    const float *src = dlist + (k * E::EPB + lane) * LSTRIDE;
-                    const int m = dcount[k * E::EPB + lane];
-                    redo |= m < 0;
-                    for (int c = 0; c < m && n < E::L::MAX_CONTACTS; ++c, ++n)
-                        for (int f = 0; f < CONTACT_SIZE; ++f) mine[n * CONTACT_SIZE + f] = src[c * CONTACT_SIZE + f];
-                }
+                const int n = merge_vertex_lists<E>(dlist, dcount, lane, mine);
                 const int env = env0 + lane;
                 float r, d;
-                E::step_finish(rows + lane * S::STRIDE, mine, redo ? -1 : n, shapes, carry, r, d);
+                E::step_finish(rows + lane * S::STRIDE, mine, n, shapes, carry, r, d);
                 if (rewards != nullptr) {
                     rewards[env - env0] = r;
                     dones[env - env0] = d;
@@ -290,6 +306,6 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
 
 // LDS floats of the per-task contact lists that phys_step_block needs (0: the env detects inline)
 template <class E>
-constexpr int detect_list_floats() { return E::DETECT_TASKS * E::EPB * ((4 * CONTACT_SIZE) | 1); }
+constexpr int detect_list_floats() { return E::DETECT_TASKS * E::EPB * DETECT_STRIDE; }
 
 }  // namespace mrl

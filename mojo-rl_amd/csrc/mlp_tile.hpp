@@ -79,9 +79,42 @@ struct HiddenOperands {
 // over twice the wavefronts.  `ops` = the operands loaded ahead by the same thread.
 // H2_ON_HT: h2 may share its memory with hT (the block waits until every wavefront has finished
 // reading hT before the first h2 element is written).
-template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32), bool H2_ON_HT = false>
+// `sync` is what the threads working on this net wait at between the phases: the whole block by
+// default; a caller that runs the net on some of its wavefronts only passes their own barrier.
+struct BlockSync {
+    MRL_DEV void operator()() const { __syncthreads(); }
+};
+
+// A barrier among `nwaves` wavefronts of a workgroup (all of them resident, as wavefronts of one
+// workgroup always are), for phases in which the rest of the block does something else: a counter
+// in LDS that only grows; every arrival adds one, and everyone waits until all arrivals of the
+// current round are in.  Every wavefront of the group must call it the same number of times,
+// outside divergent code.  The counter must be zero before the first use.
+struct WaveGroupSync {
+    unsigned *counter;
+    unsigned target;   // arrivals expected by the end of the round in progress
+    unsigned nwaves;
+    MRL_DEV void arrive() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // this wavefront's LDS writes are out
+        if ((threadIdx.x & 63) == 0)
+            __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    MRL_DEV void wait_for(unsigned arrivals) const {
+        while ((int)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - arrivals) < 0)
+            __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+    MRL_DEV void operator()() {
+        target += nwaves;
+        arrive();
+        wait_for(target);
+    }
+};
+
+template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32), bool H2_ON_HT = false, class Sync = BlockSync>
 MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
-                          const TileCache tc, HiddenOperands<H, TPW, KB> &ops, int tid = threadIdx.x) {
+                          const TileCache tc, HiddenOperands<H, TPW, KB> &ops, int tid = threadIdx.x,
+                          Sync &&sync = Sync()) {
     static_assert(PR * (H + 1) <= H * HT_LD, "h2 fits into hT");
     constexpr int T = 2 * H / TPW;
     constexpr int K0 = PIN_MAX / 2;
@@ -124,7 +157,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
             }
         }
     }
-    __syncthreads();
+    sync();
     {   // layer 1 (H x H): weights streamed from L2 one block of KB k-steps ahead of the MFMAs
         floatx16 c[TPW];
 #pragma unroll
@@ -158,7 +191,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
                 }
             }
         }
-        if (H2_ON_HT) __syncthreads();
+        if (H2_ON_HT) sync();
 #pragma unroll
         for (int q = 0; q < TPW; ++q) {
 #pragma unroll
@@ -174,7 +207,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
             }
         }
     }
-    __syncthreads();
+    sync();
 }
 
 // floats of LDS that hold one net's head parameters, every row padded to PA_MAX columns with

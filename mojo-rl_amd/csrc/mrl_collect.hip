@@ -5,11 +5,16 @@
 // to the last (HBM sees them once in and once out per launch, however many steps), the
 // observation tile feeds the policy straight from those rows, and the sampled actions reach the
 // env step through LDS.  Per step and block:
-//   policy   actor and critic  OBS -> H -> H -> A | 1  on the fp32 matrix cores (the 32 x H tiles
-//            of mlp_tile.hpp, weights streamed from L2), categorical / Gaussian sampling,
-//            rollout row t of obs, action, log-prob and value written;
-//   env      the step of env_block.hpp (wavefront 0 one env per lane, the others contact
-//            detection), reward / done of rollout row t, episode accounting, in-place reset.
+//   actor    OBS -> H -> H -> A on the fp32 matrix cores by all eight wavefronts (the 32 x H tiles
+//            of mlp_tile.hpp, weights streamed from L2);
+//   then, side by side,
+//     wavefront 0        categorical / Gaussian sampling, then the env step of env_block.hpp (one
+//                        env per lane), reward / done of rollout row t, episode accounting,
+//                        in-place reset;
+//     wavefronts 1 .. 7  contact detection for that env step;
+//     wavefronts 4 .. 7  then the critic  OBS -> H -> H -> 1  (its value is only stored, so it does
+//                        not hold up the env step; these wavefronts meet at a barrier of their own);
+//   rollout row t of obs, action, log-prob and value written on the way.
 // No workgroup waits for another, so there is nothing between two steps but the block's own
 // barriers; the launch ends when every block has done its n_steps.
 //
@@ -40,9 +45,10 @@ constexpr int cmax() { return A > B ? A : B; }
 template <class E, int H, int ACT, bool GAUSS>
 __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     using S = Stage<E>;
-    constexpr int TPW = 2, TN = 2 * H / TPW, IN = E::OBS, AW = E::ACT_W;
-    static_assert(E::EPB == PR && E::THREADS == 2 * TN, "one 32-row policy tile per block, both nets side by side");
-    static_assert(IN <= PIN_MAX && AW <= PA_MAX, "policy tile limits");
+    constexpr int IN = E::OBS, AW = E::ACT_W, NW = E::THREADS / WAVE;
+    constexpr int CRITIC_WAVE0 = NW / 2, CRITIC_T = E::THREADS / 2;   // the critic's wavefronts: the upper half
+    static_assert(E::EPB == PR && E::THREADS == 2 * H && CRITIC_T == H, "one 32-row policy tile per block");
+    static_assert(IN <= PIN_MAX && AW <= PA_MAX && E::DETECT_TASKS > 0, "policy tile limits; split-off detection");
     __shared__ float rows[PR * S::STRIDE];
     __shared__ float xs[PR * XS_LD];
     __shared__ __align__(16) float w2s[2][HEAD_LDS(H)];
@@ -51,81 +57,124 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     __shared__ float act[PR * PA_MAX];
     __shared__ float shapes[E::NSHAPE];
     __shared__ unsigned long long was_reset;
-    // the policy's activation tiles and the env step's contact scratch are never live together
-    constexpr int POLICY_F = 2 * H * HT_LD;
+    __shared__ unsigned sync_critic, sync_detect;
+    __shared__ float hTc[H * HT_LD];   // the critic's activation tile (live during the env step)
+    // the actor's activation tile and the env step's contact scratch are never live together
     constexpr int LIST_F = detect_list_floats<E>() + 1;
     constexpr int ENV_F = PR * S::CSTRIDE + LIST_F + E::DETECT_TASKS * E::EPB + 1;
-    __shared__ float overlay[cmax<POLICY_F, ENV_F>()];
+    __shared__ float overlay[cmax<H * HT_LD, ENV_F>()];
     float *cts = overlay, *dlist = cts + PR * S::CSTRIDE;
     int *dcount = reinterpret_cast<int *>(dlist + LIST_F);
 
-    const int t = threadIdx.x, net = t / TN;
+    const int t = threadIdx.x;
     const int env0 = blockIdx.x * PR;
     const int nenv = min(PR, a.n_envs - env0);
     const int N = a.n_envs;
     float *gbase = a.states + (size_t)env0 * E::STATE;
-    const float *p = net ? a.critic_p : a.actor_p;
+
     S::in(rows, gbase, nenv, t);
     for (int i = t; i < E::NSHAPE; i += E::THREADS) shapes[i] = a.shapes[i];
-    stage_head(p + IN * H + H + H * H + H, H, net ? 1 : a.A, GAUSS && net == 0, w2s[net], t % TN, TN);
-    if (t == 0) was_reset = 0;
+    {
+        const int net = t / CRITIC_T;
+        const float *p = net ? a.critic_p : a.actor_p;
+        stage_head(p + IN * H + H + H * H + H, H, net ? 1 : a.A, GAUSS && net == 0, w2s[net], t % CRITIC_T, CRITIC_T);
+    }
+    if (t == 0) {
+        was_reset = 0;
+        sync_critic = 0;
+        sync_detect = 0;
+    }
     __syncthreads();
+    WaveGroupSync critic_sync{&sync_critic, 0u, (unsigned)(NW - CRITIC_WAVE0)};
+    WaveGroupSync detect_sync{&sync_detect, 0u, (unsigned)(NW - 1)};
+    static_assert((E::DETECT_TASKS + 1) / 2 <= NW - 1, "two detection tasks per wavefront besides wavefront 0");
 
+    // Per step: every wavefront runs the actor (the action is what the env step waits for); then
+    // wavefront 0 samples and steps the envs, wavefronts 1 .. 7 detect their contacts, and
+    // wavefronts 4 .. 7 go on to run the critic, whose value is only stored -- off the critical path.
     for (int k = 0; k < a.n_steps; ++k) {
         // Nothing but the rows is carried from one step to the next: the thread index, the block's
-        // env count and the parameter pointer pass through empty asm statements at the top of each
+        // env count and the parameter pointers pass through empty asm statements at the top of each
         // step, so the optimiser cannot keep what it derives from them (addresses, predicates, the
         // step-invariant operand values) live through the env step, whose solver needs the registers.
-        int tid = t, ne = __builtin_amdgcn_readfirstlane(nenv), A = __builtin_amdgcn_readfirstlane(a.A);
-        const float *ps = p;
-        asm volatile("" : "+v"(tid), "+v"(ps), "+s"(ne), "+s"(A) : : "memory");
+        int tid = t, ne = __builtin_amdgcn_readfirstlane(nenv), A = __builtin_amdgcn_readfirstlane(a.A), zero = 0;
+        asm volatile("" : "+v"(tid), "+s"(zero), "+s"(ne), "+s"(A) : : "memory");
+        const float *pa = a.actor_p + zero, *pc = a.critic_p + zero;
         const size_t row = (size_t)(a.t0 + k) * N + env0;   // this block's slice of rollout row t
         const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
-        // ---- policy
-        HiddenOperands<H, TPW, 8> ops;
-        ops.load(ps, IN, tid);
-        for (int i = tid; i < PR * IN; i += E::THREADS) {
-            const int r = i / IN, c = i - r * IN;
-            float v = 0.0f;
-            if (r < ne) {
-                v = rows[r * S::STRIDE + c];
-                a.r_obs[row * IN + i] = v;
-            }
-            xs[r * XS_LD + c] = v;
-        }
-        __syncthreads();
-        float *hT = overlay + (tid / TN) * (H * HT_LD);
-        hidden_stack<H, ACT, TPW, 8, true>(ps, IN, xs, hT, hT, TileCache{}, ops, tid);
-        if (tid < TN) head<H>(w2s[0], A, hT, logits, PA_MAX + 1, tid);
-        else head<H>(w2s[1], 1, hT, vals, 1, tid);
-        __syncthreads();
-        if (tid < ne) {
-            const int i = env0 + tid;
-            float logp;
-            if (GAUSS) {
-                float av[PA_MAX];
-                logp = sample_gaussian(logits + tid * (PA_MAX + 1), w2s[0] + HEAD_LOG_STD(H), A, sseed, i, av);
-                for (int j = 0; j < A; ++j) {
-                    act[tid * AW + j] = av[j];
-                    a.r_actions[(row + tid) * AW + j] = av[j];
+        const int wave = tid / WAVE, lane = tid % WAVE;
+        // ---- actor, all wavefronts
+        {
+            HiddenOperands<H, 1, 32> ops;
+            ops.load(pa, IN, tid);
+            for (int i = tid; i < PR * IN; i += E::THREADS) {
+                const int r = i / IN, c = i - r * IN;
+                float v = 0.0f;
+                if (r < ne) {
+                    v = rows[r * S::STRIDE + c];
+                    a.r_obs[row * IN + i] = v;
                 }
-            } else {
-                int sel;
-                sample_categorical(logits + tid * (PA_MAX + 1), A, sseed, i, sel, logp);
-                act[tid] = (float)sel;
-                a.r_actions[row + tid] = (float)sel;
+                xs[r * XS_LD + c] = v;
             }
-            a.r_logp[row + tid] = logp;
-            a.r_values[row + tid] = vals[tid];
+            __syncthreads();
+            hidden_stack<H, ACT, 1, 32, true>(pa, IN, xs, overlay, overlay, TileCache{}, ops, tid);
+            if (tid < H) head<H>(w2s[0], A, overlay, logits, PA_MAX + 1, tid);
+            __syncthreads();   // logits complete; the actor's tile is dead from here on
         }
-        __syncthreads();   // actions visible; the activation tiles are dead from here on
-        // ---- env step
-        Accounting acc = a.acc.at(env0);
-        acc.r_rewards = a.r_rewards + row;
-        acc.r_dones = a.r_dones + row;
-        phys_step_block<E, true>(rows, cts, shapes, dlist, dcount, &was_reset, act, nullptr, nullptr, env0, ne,
-                                 a.reset_seed + (uint64_t)k * a.reset_stride, acc, tid);
-        __syncthreads();
+        if (wave == 0) {
+            // ---- sample, then the env step of env_block.hpp with the contacts of wavefronts 1 .. 3
+            typename E::Carry carry{};
+            if (lane < ne) {
+                const int i = env0 + lane;
+                float logp;
+                if (GAUSS) {
+                    float av[PA_MAX];
+                    logp = sample_gaussian(logits + lane * (PA_MAX + 1), w2s[0] + HEAD_LOG_STD(H), A, sseed, i, av);
+                    for (int j = 0; j < A; ++j) {
+                        act[lane * AW + j] = av[j];
+                        a.r_actions[(row + lane) * AW + j] = av[j];
+                    }
+                } else {
+                    int sel;
+                    sample_categorical(logits + lane * (PA_MAX + 1), A, sseed, i, sel, logp);
+                    act[lane] = (float)sel;
+                    a.r_actions[row + lane] = (float)sel;
+                }
+                a.r_logp[row + lane] = logp;
+                carry = E::step_begin(rows + lane * S::STRIDE, i, act + lane * AW);
+            }
+            detect_sync.target += detect_sync.nwaves;
+            detect_sync.wait_for(detect_sync.target);
+            bool finished = false;
+            if (lane < ne) {
+                float *mine = cts + lane * S::CSTRIDE;
+                const int n = merge_vertex_lists<E>(dlist, dcount, lane, mine);
+                float r, d;
+                E::step_finish(rows + lane * S::STRIDE, mine, n, shapes, carry, r, d);
+                Accounting acc = a.acc.at(env0);
+                acc.r_rewards = a.r_rewards + row;
+                acc.r_dones = a.r_dones + row;
+                account(acc, lane, r, d);
+                finished = d > 0.5f;
+            }
+            reset_rows<E>(rows, &was_reset, __ballot(finished), a.reset_seed + (uint64_t)k * a.reset_stride, env0, lane);
+        } else {
+            // ---- contact detection: one (body, vertex) task per half of wavefronts 1 .. 7
+            const int task = (wave - 1) * 2 + lane / (WAVE / 2), e = lane % (WAVE / 2);
+            if (task < E::DETECT_TASKS && e < ne) detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
+            detect_sync.arrive();
+            if (wave >= CRITIC_WAVE0) {
+                // ---- critic, on its own barrier.  (One wavefront per SIMD here: blocks of 16 k-steps,
+                // so that a block's MFMAs cover the L2 latency of the next block's weights without a
+                // second wavefront's help.)
+                HiddenOperands<H, 2, 16> ops;
+                ops.load(pc, IN, tid);
+                hidden_stack<H, ACT, 2, 16, true>(pc, IN, xs, hTc, hTc, TileCache{}, ops, tid, critic_sync);
+                head<H>(w2s[1], 1, hTc, vals, 1, tid);
+            }
+        }
+        __syncthreads();   // env step done, values complete
+        if (tid < ne) a.r_values[row + tid] = vals[tid];
     }
 
     for (int i = t; i < nenv * E::OBS; i += E::THREADS) {
