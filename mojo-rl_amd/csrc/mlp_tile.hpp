@@ -38,10 +38,15 @@ struct TileCache {
 // tile's rows: biases, the layer-0 weights, the first block of layer-1 weights.  A kernel issues
 // these loads first thing (before it stages its inputs), so that a block pays the memory latency
 // once rather than once per phase.
+// threads that work on one net: one wavefront per TPW column tiles of 32 (the last wavefront's
+// tiles beyond H are computed on repeated columns and dropped)
+constexpr int hidden_threads(int H, int TPW) { return 64 * ((H / 32 + TPW - 1) / TPW); }
+
 template <int H, int TPW, int KB>
 struct HiddenOperands {
     static constexpr int K0 = PIN_MAX / 2;   // k-steps of layer 0 at the widest input
     int col[TPW];
+    int ntile;   // column tiles of this wavefront that exist (TPW, or fewer on the last wavefront)
     float bias0[TPW], bias1[TPW];
     float w0[TPW][K0];
     float bv[TPW][KB];
@@ -49,13 +54,14 @@ struct HiddenOperands {
     // tid: the caller's thread index (a caller that loops over many tiles may pass a copy the
     // optimiser cannot see through, so that nothing derived from it is kept across iterations)
     MRL_DEV void load(const float *__restrict__ p, int IN, int tid = threadIdx.x) {
-        constexpr int T = 2 * H / TPW;
+        constexpr int T = hidden_threads(H, TPW);
         const int t = tid % T, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
         const float *W0 = p, *b0 = p + IN * H;
         const float *W1 = b0 + H, *b1 = W1 + H * H;
+        ntile = (H / 32) % TPW == 0 ? TPW : min(TPW, H / 32 - TPW * w);
 #pragma unroll
         for (int q = 0; q < TPW; ++q) {
-            col[q] = 32 * (TPW * w + q) + l31;
+            col[q] = (TPW * w + q < H / 32 ? 32 * (TPW * w + q) : 0) + l31;
             bias0[q] = b0[col[q]];
             bias1[q] = b1[col[q]];
         }
@@ -116,7 +122,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
                           const TileCache tc, HiddenOperands<H, TPW, KB> &ops, int tid = threadIdx.x,
                           Sync &&sync = Sync()) {
     static_assert(PR * (H + 1) <= H * HT_LD, "h2 fits into hT");
-    constexpr int T = 2 * H / TPW;
+    constexpr int T = hidden_threads(H, TPW);
     constexpr int K0 = PIN_MAX / 2;
     const int t = tid % T, lane = t & 63, half = lane >> 5, l31 = lane & 31;
     const float *W1 = p + IN * H + H;
@@ -144,6 +150,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
         }
 #pragma unroll
         for (int q = 0; q < TPW; ++q) {
+            if (q >= ops.ntile) continue;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = 8 * (v >> 2) + 4 * half + (v & 3);
@@ -194,6 +201,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
         if (H2_ON_HT) sync();
 #pragma unroll
         for (int q = 0; q < TPW; ++q) {
+            if (q >= ops.ntile) continue;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = 8 * (v >> 2) + 4 * half + (v & 3);
@@ -238,35 +246,55 @@ MRL_DEV void stage_head(const float *__restrict__ W2, int H, int A, bool with_lo
 
 // out[r][a] = h2[r] . W2[:, a] + b2[a] for the block's rows; TPR = H/32 lanes cooperate per row,
 // each over 32 consecutive columns that it walks from a different starting point (the lanes of a
-// wavefront then read distinct LDS banks).  w2s: the head parameters in LDS (stage_head); called
-// by the first H threads of the net.
-template <int H>
-MRL_DEV void head(const float *w2s, int A, const float *h2, float *out, int out_ld, int tid = threadIdx.x) {
+// wavefront then read distinct LDS banks).  w2s: the head parameters in LDS (stage_head).
+// NA = outputs carried per lane (1, 4 or 8 >= A): narrower heads read less of each padded row.
+template <int H, int NA>
+MRL_DEV void head_rows(const float *w2s, int A, const float *h2, float *out, int out_ld, int t, int nthreads) {
     constexpr int TPR = H / PR;
-    const int t = tid % H, r = t / TPR, part = t % TPR;
-    float acc[PA_MAX];
-#pragma unroll
-    for (int a = 0; a < PA_MAX; ++a) acc[a] = 0.0f;
-#pragma unroll 8
-    for (int i = 0; i < PR; ++i) {
-        const int n = part * PR + ((i + 4 * part) & (PR - 1));
-        const float hv = h2[r * (H + 1) + n];
-        const float4 wa = *reinterpret_cast<const float4 *>(w2s + n * PA_MAX);
-        const float4 wb = *reinterpret_cast<const float4 *>(w2s + n * PA_MAX + 4);
-        acc[0] = fmaf(hv, wa.x, acc[0]); acc[1] = fmaf(hv, wa.y, acc[1]);
-        acc[2] = fmaf(hv, wa.z, acc[2]); acc[3] = fmaf(hv, wa.w, acc[3]);
-        acc[4] = fmaf(hv, wb.x, acc[4]); acc[5] = fmaf(hv, wb.y, acc[5]);
-        acc[6] = fmaf(hv, wb.z, acc[6]); acc[7] = fmaf(hv, wb.w, acc[7]);
-    }
-    static_assert(PA_MAX == 8, "two float4 per padded row");
+    static_assert(64 % TPR == 0, "the lanes of a row sit in one wavefront");
+    static_assert(PA_MAX == 8 && (NA == 1 || NA == 4 || NA == 8), "one float, one float4 or two per padded row");
     const float *b2 = w2s + HEAD_B2(H);
+    // (row, part) pairs are dealt out PR * TPR = H at a time; nthreads must be a multiple of TPR
+    for (int pair = t; pair < H; pair += nthreads) {
+        const int r = pair / TPR, part = pair % TPR;
+        float acc[NA];
 #pragma unroll
-    for (int a = 0; a < PA_MAX; ++a) {
-        float v = acc[a];
+        for (int a = 0; a < NA; ++a) acc[a] = 0.0f;
+#pragma unroll 8
+        for (int i = 0; i < PR; ++i) {
+            const int n = part * PR + ((i + 4 * part) & (PR - 1));
+            const float hv = h2[r * (H + 1) + n];
+            if (NA == 1) {
+                acc[0] = fmaf(hv, w2s[n * PA_MAX], acc[0]);
+            } else {
+                const float4 wa = *reinterpret_cast<const float4 *>(w2s + n * PA_MAX);
+                acc[0] = fmaf(hv, wa.x, acc[0]); acc[1] = fmaf(hv, wa.y, acc[1]);
+                acc[2] = fmaf(hv, wa.z, acc[2]); acc[3] = fmaf(hv, wa.w, acc[3]);
+                if (NA == 8) {
+                    const float4 wb = *reinterpret_cast<const float4 *>(w2s + n * PA_MAX + 4);
+                    acc[4] = fmaf(hv, wb.x, acc[4]); acc[5] = fmaf(hv, wb.y, acc[5]);
+                    acc[6] = fmaf(hv, wb.z, acc[6]); acc[7] = fmaf(hv, wb.w, acc[7]);
+                }
+            }
+        }
 #pragma unroll
-        for (int off = TPR / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-        if (part == 0 && a < A) out[r * out_ld + a] = v + b2[a];
+        for (int a = 0; a < NA; ++a) {
+            float v = acc[a];
+#pragma unroll
+            for (int off = TPR / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+            if (part == 0 && a < A) out[r * out_ld + a] = v + b2[a];
+        }
     }
+}
+
+// t = index of the calling thread among the `nthreads` (a multiple of H / 32) that share the work;
+// by default the first H threads of the net call it, one (row, part) pair each
+template <int H>
+MRL_DEV void head(const float *w2s, int A, const float *h2, float *out, int out_ld, int t = threadIdx.x % H,
+                  int nthreads = H) {
+    if (A == 1) head_rows<H, 1>(w2s, A, h2, out, out_ld, t, nthreads);
+    else if (A <= 4) head_rows<H, 4>(w2s, A, h2, out, out_ld, t, nthreads);
+    else head_rows<H, 8>(w2s, A, h2, out, out_ld, t, nthreads);
 }
 
 }  // namespace mrl

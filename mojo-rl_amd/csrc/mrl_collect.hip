@@ -12,7 +12,7 @@
 //                        env per lane), reward / done of rollout row t, episode accounting,
 //                        in-place reset;
 //     wavefronts 1 .. 7  contact detection for that env step;
-//     wavefronts 4 .. 7  then the critic  OBS -> H -> H -> 1  (its value is only stored, so it does
+//     wavefronts 5 .. 7  then the critic  OBS -> H -> H -> 1  (its value is only stored, so it does
 //                        not hold up the env step; these wavefronts meet at a barrier of their own);
 //   rollout row t of obs, action, log-prob and value written on the way.
 // No workgroup waits for another, so there is nothing between two steps but the block's own
@@ -46,8 +46,11 @@ template <class E, int H, int ACT, bool GAUSS>
 __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     using S = Stage<E>;
     constexpr int IN = E::OBS, AW = E::ACT_W, NW = E::THREADS / WAVE;
-    constexpr int CRITIC_WAVE0 = NW / 2, CRITIC_T = E::THREADS / 2;   // the critic's wavefronts: the upper half
-    static_assert(E::EPB == PR && E::THREADS == 2 * H && CRITIC_T == H, "one 32-row policy tile per block");
+    // the critic's wavefronts: the last three, so that none of them shares a SIMD with wavefront 0
+    // (wavefronts of a workgroup go round the four SIMDs) and its solver keeps that SIMD's issue
+    // slots to itself
+    constexpr int CRITIC_TPW = 3, CRITIC_T = hidden_threads(H, CRITIC_TPW), CRITIC_WAVE0 = NW - CRITIC_T / WAVE;
+    static_assert(E::EPB == PR && E::THREADS == 2 * H && NW == 8 && CRITIC_WAVE0 == 5, "one 32-row policy tile per block");
     static_assert(IN <= PIN_MAX && AW <= PA_MAX && E::DETECT_TASKS > 0, "policy tile limits; split-off detection");
     __shared__ float rows[PR * S::STRIDE];
     __shared__ float xs[PR * XS_LD];
@@ -75,9 +78,9 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     S::in(rows, gbase, nenv, t);
     for (int i = t; i < E::NSHAPE; i += E::THREADS) shapes[i] = a.shapes[i];
     {
-        const int net = t / CRITIC_T;
+        const int net = t / H;
         const float *p = net ? a.critic_p : a.actor_p;
-        stage_head(p + IN * H + H + H * H + H, H, net ? 1 : a.A, GAUSS && net == 0, w2s[net], t % CRITIC_T, CRITIC_T);
+        stage_head(p + IN * H + H + H * H + H, H, net ? 1 : a.A, GAUSS && net == 0, w2s[net], t % H, H);
     }
     if (t == 0) {
         was_reset = 0;
@@ -91,7 +94,7 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
 
     // Per step: every wavefront runs the actor (the action is what the env step waits for); then
     // wavefront 0 samples and steps the envs, wavefronts 1 .. 7 detect their contacts, and
-    // wavefronts 4 .. 7 go on to run the critic, whose value is only stored -- off the critical path.
+    // wavefronts 5 .. 7 go on to run the critic, whose value is only stored -- off the critical path.
     for (int k = 0; k < a.n_steps; ++k) {
         // Nothing but the rows is carried from one step to the next: the thread index, the block's
         // env count and the parameter pointers pass through empty asm statements at the top of each
@@ -167,10 +170,11 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
                 // ---- critic, on its own barrier.  (One wavefront per SIMD here: blocks of 16 k-steps,
                 // so that a block's MFMAs cover the L2 latency of the next block's weights without a
                 // second wavefront's help.)
-                HiddenOperands<H, 2, 16> ops;
-                ops.load(pc, IN, tid);
-                hidden_stack<H, ACT, 2, 16, true>(pc, IN, xs, hTc, hTc, TileCache{}, ops, tid, critic_sync);
-                head<H>(w2s[1], 1, hTc, vals, 1, tid);
+                const int tl = tid - CRITIC_WAVE0 * WAVE;   // index among the critic's threads
+                HiddenOperands<H, CRITIC_TPW, 16> ops;
+                ops.load(pc, IN, tl);
+                hidden_stack<H, ACT, CRITIC_TPW, 16, true>(pc, IN, xs, hTc, hTc, TileCache{}, ops, tl, critic_sync);
+                head<H>(w2s[1], 1, hTc, vals, 1, tl, CRITIC_T);
             }
         }
         __syncthreads();   // env step done, values complete
