@@ -10,12 +10,19 @@ namespace mrl {
 
 // _store_post_step_kernel (deep_agents/ppo/ppo.mojo:692-708) + accumulate_rewards /
 // increment_steps / extract_completed_episodes (deep_rl/gpu/rl_kernels.mojo:103-200) for one env
-MRL_DEV void account(const Accounting &acc, int i, float r, float d) {
+// `before` = env i's running (return, length) as they stood before the step; a caller with a long
+// step reads them ahead of it (account_before) so that the step does not end on a memory round trip
+struct EpisodeSums { float ret, len; };
+MRL_DEV EpisodeSums account_before(const Accounting &acc, int i) {
+    if (acc.r_rewards == nullptr) return EpisodeSums{0.0f, 0.0f};
+    return EpisodeSums{acc.ep_return[i], acc.ep_length[i]};
+}
+MRL_DEV void account(const Accounting &acc, int i, float r, float d, const EpisodeSums &before) {
     if (acc.r_rewards == nullptr) return;
     acc.r_rewards[i] = r;
     acc.r_dones[i] = d;
-    float er = acc.ep_return[i] + r;
-    float el = acc.ep_length[i] + 1.0f;
+    float er = before.ret + r;
+    float el = before.len + 1.0f;
     if (d > 0.5f) {
         int slot = atomicAdd(acc.done_count, 1);
         if (slot < acc.done_cap) {
@@ -28,6 +35,7 @@ MRL_DEV void account(const Accounting &acc, int i, float r, float d) {
     acc.ep_return[i] = er;
     acc.ep_length[i] = el;
 }
+MRL_DEV void account(const Accounting &acc, int i, float r, float d) { account(acc, i, r, d, account_before(acc, i)); }
 
 // ---------------------------------------------------------------- physics2d envs
 // Per-env traits of the LDS-staged kernels.  EPB = env rows per workgroup (one wavefront; with
@@ -259,7 +267,9 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
         static_assert(E::EPB <= HALF && (NT + 1) / 2 < E::THREADS / WAVE, "two tasks per wavefront besides wavefront 0");
         const int wave = tid / WAVE, lane = tid % WAVE;
         typename E::Carry carry{};
+        EpisodeSums sums{0.0f, 0.0f};
         if (wave == 0) {
+            if (lane < nenv) sums = account_before(acc, lane);
             if (lane < nenv)
                 carry = E::step_begin(rows + lane * S::STRIDE, env0 + lane, actions + (size_t)lane * E::ACT_W);
         } else {
@@ -279,7 +289,7 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
                     rewards[env - env0] = r;
                     dones[env - env0] = d;
                 }
-                account(acc, env - env0, r, d);
+                account(acc, env - env0, r, d, sums);
                 finished = d > 0.5f;
             }
             if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, lane);
@@ -289,6 +299,7 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
             bool finished = false;
             if (tid < nenv) {
                 const int env = env0 + tid;
+                const EpisodeSums sums = account_before(acc, tid);
                 float r, d;
                 E::step(rows + tid * S::STRIDE, cts + tid * S::CSTRIDE, shapes, env,
                         actions + (size_t)tid * E::ACT_W, r, d);
@@ -296,7 +307,7 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
                     rewards[env - env0] = r;
                     dones[env - env0] = d;
                 }
-                account(acc, env - env0, r, d);
+                account(acc, env - env0, r, d, sums);
                 finished = d > 0.5f;
             }
             if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, tid);

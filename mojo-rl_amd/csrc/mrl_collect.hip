@@ -88,6 +88,10 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
         sync_detect = 0;
     }
     __syncthreads();
+    // wavefront 0, lane = env slot: the env's running episode return and length stay in registers
+    const bool owner = t < nenv;
+    float ep_return = owner ? a.acc.ep_return[env0 + t] : 0.0f;
+    float ep_length = owner ? a.acc.ep_length[env0 + t] : 0.0f;
     WaveGroupSync critic_sync{&sync_critic, 0u, (unsigned)(NW - CRITIC_WAVE0)};
     WaveGroupSync detect_sync{&sync_detect, 0u, (unsigned)(NW - 1)};
     static_assert((E::DETECT_TASKS + 1) / 2 <= NW - 1, "two detection tasks per wavefront besides wavefront 0");
@@ -154,11 +158,22 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
                 const int n = merge_vertex_lists<E>(dlist, dcount, lane, mine);
                 float r, d;
                 E::step_finish(rows + lane * S::STRIDE, mine, n, shapes, carry, r, d);
-                Accounting acc = a.acc.at(env0);
-                acc.r_rewards = a.r_rewards + row;
-                acc.r_dones = a.r_dones + row;
-                account(acc, lane, r, d);
+                // rollout row t and the episode accounting of account(), on the running sums that
+                // this lane carries for its env
+                a.r_rewards[row + lane] = r;
+                a.r_dones[row + lane] = d;
+                ep_return = ep_return + r;
+                ep_length = ep_length + 1.0f;
                 finished = d > 0.5f;
+                if (finished) {
+                    const int slot = atomicAdd(a.acc.done_count, 1);
+                    if (slot < a.acc.done_cap) {
+                        a.acc.done_returns[slot] = ep_return;
+                        a.acc.done_lengths[slot] = ep_length;
+                    }
+                    ep_return = 0.0f;
+                    ep_length = 0.0f;
+                }
             }
             reset_rows<E>(rows, &was_reset, __ballot(finished), a.reset_seed + (uint64_t)k * a.reset_stride, env0, lane);
         } else {
@@ -181,6 +196,10 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
         if (tid < ne) a.r_values[row + tid] = vals[tid];
     }
 
+    if (owner) {
+        a.acc.ep_return[env0 + t] = ep_return;
+        a.acc.ep_length[env0 + t] = ep_length;
+    }
     for (int i = t; i < nenv * E::OBS; i += E::THREADS) {
         const int r = i / E::OBS, c = i - r * E::OBS;
         a.obs[(size_t)env0 * E::OBS + i] = rows[r * S::STRIDE + c];
