@@ -275,7 +275,9 @@ typedef struct {
     float *actor_grads, *critic_grads;
     float *actor_state, *critic_state;       /* Adam (m, v) interleaved, [P, 2] */
     const float *r_obs, *r_actions, *r_log_probs, *r_values, *advantages, *returns; /* [T*N, ...] */
-    float *mb_obs, *mb_actions, *mb_adv, *mb_ret, *mb_logp, *mb_val;                /* [MB, ...] */
+    float *mb_obs, *mb_actions, *mb_adv, *mb_ret, *mb_logp, *mb_val;                /* [MB, ...] scratch: the gathered
+                                                 minibatch when the nets run layer by layer, untouched when the fused
+                                                 forward reads the rollout rows itself */
     float *actor_out, *values, *g_actor_out, *g_values, *kl;
     float *actor_cache, *critic_cache;       /* [MB * CACHE_SIZE] */
     int32_t *kl_flag;                        /* [4], may be NULL when target_kl <= 0 */

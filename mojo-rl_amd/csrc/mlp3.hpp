@@ -16,11 +16,30 @@ struct Mlp3Net {
 };
 struct Mlp3Nets { Mlp3Net n[2]; };
 
+// PPO tail of a paired forward (net 0 = actor, net 1 = critic) over minibatch rows that are still
+// where the rollout left them: the forward reads its input rows through `idx`, and every row tile
+// goes straight on to its loss gradients (deep_agents/ppo/ppo.mojo:285-378, 538-633;
+// kernels.mojo:230-486) and to its share of the KL early-stop test, so that neither a gather nor a
+// loss launch is needed.  enabled = 0: plain forward.
+struct FwdLoss {
+    int enabled;
+    const int32_t *idx;                                   // [mb] rollout rows of the minibatch
+    const float *r_obs, *r_act, *r_adv, *r_ret, *r_logp, *r_val;
+    const float *adv_stats;                               // {mean, std} of the minibatch's advantages; null: as they are
+    float *g_actor_out, *g_values, *kl;                   // [mb, head], [mb], [mb]
+    float *kl_part;                                       // [row tiles]
+    int *arrived;                                         // zero between launches
+    int32_t *kl_flag;                                     // null: no test
+    int mb, A, continuous, clip_value;                    // A = actions (discrete) or action width (continuous)
+    float clip_eps, ent_coef, value_coef, target_kl;
+};
+
 bool mlp3_fusable(const mrl_mlp_desc &d, int *H, int *act, bool *gauss);
 bool mlp3_pair_fusable(const mrl_mlp_desc &a, const mrl_mlp_desc &b);
 int mlp3_forward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *in, const float *params,
                  float *out, float *cache);
-int mlp3_forward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io);
+int mlp3_forward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io,
+                   const FwdLoss *loss = nullptr);
 size_t mlp3_backward_ws(const mrl_mlp_desc *const *descs, int n_nets, int batch);
 int mlp3_backward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *grad_out, const float *params,
                   const float *cache, float *grads, float *ws);

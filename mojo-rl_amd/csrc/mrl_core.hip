@@ -60,8 +60,8 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     }
     MRL_CHECK_HIP(hipMalloc(&c->reduce_scratch, sizeof(float) * c->reduce_scratch_floats));
     c->upd_scratch = nullptr;
-    MRL_CHECK_HIP(hipMalloc(&c->upd_scratch, sizeof(float) * 4096));
-    MRL_CHECK_HIP(hipMemset(c->upd_scratch, 0, sizeof(float) * 4096));
+    MRL_CHECK_HIP(hipMalloc(&c->upd_scratch, sizeof(float) * 8192));
+    MRL_CHECK_HIP(hipMemset(c->upd_scratch, 0, sizeof(float) * 8192));
     *out = c;
     return MRL_OK;
 }

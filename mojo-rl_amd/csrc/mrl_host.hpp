@@ -30,7 +30,8 @@ struct mrl_ctx {
     float *rollout_ws;
     size_t rollout_ws_floats;
     // scratch of the minibatch update: per-block KL partials [0, 1024), their arrival counter
-    // (int, at float index 1024; zero between launches), sum-of-squares partials [2048, 4096)
+    // (int, at float index 1024; zero between launches), sum-of-squares partials [2048, 4096),
+    // advantage {mean, std} of up to 2048 minibatches [4096, 8192)
     float *upd_scratch;
     // phase timing: events recorded on `stream` at phase boundaries while armed
     bool profiling;

@@ -14,13 +14,14 @@
 #include "mrl_device.hpp"
 #include "mlp_tile.hpp"
 #include "mlp3.hpp"
+#include "ppo_grads.hpp"
 
 namespace mrl {
 
 // grid = (row tiles, nets): blockIdx.y picks the net, so that an actor and a critic that read the
 // same inputs go through the chip side by side
 template <int H, int ACT>
-__global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets nets) {
+__global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets nets, FwdLoss fl) {
     constexpr int T = 2 * H;   // one 32-column accumulator tile per wavefront
     __shared__ float xs[PR * XS_LD];
     __shared__ float hT[H * HT_LD];
@@ -51,7 +52,11 @@ __global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets
 #pragma unroll
     for (int q = 0; q < NX; ++q) {
         const int i = t + q * T;
-        xv[q] = (i < PR * IN && i / IN < nrow) ? x[row0 * IN + i] : 0.0f;
+        xv[q] = 0.0f;
+        if (i < PR * IN && i / IN < nrow) {
+            const int r = i / IN;
+            xv[q] = fl.enabled ? fl.r_obs[(size_t)fl.idx[row0 + r] * IN + (i - r * IN)] : x[row0 * IN + i];
+        }
     }
     stage_head(params + IN * H + H + H * H + H, H, A, GAUSS, w2s, t, T);
 #pragma unroll
@@ -79,6 +84,70 @@ __global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets
             else if (v > 2.0f) v = 2.0f;
         }
         out[(row0 + r) * ld + a] = v;
+    }
+    if (!fl.enabled) return;
+    // ---- loss gradients of the tile's rows, one lane per row (wavefront 0)
+    if (t >= 64) return;
+    const int b = (int)row0 + t;
+    const bool mine = t < nrow;
+    const long src = mine ? fl.idx[b] : 0;
+    if (blockIdx.y == 1) {   // critic
+        if (mine)
+            fl.g_values[b] = critic_grad_value(ys[t * (PA_MAX + 1)], fl.clip_value ? fl.r_val[src] : 0.0f, fl.r_ret[src],
+                                               fl.mb, fl.continuous, fl.clip_value, fl.value_coef, fl.clip_eps);
+        return;
+    }
+    float kl = 0.0f;
+    if (mine) {
+        float adv = fl.r_adv[src];
+        if (fl.adv_stats != nullptr) adv = (adv - fl.adv_stats[0]) / (fl.adv_stats[1] + 1e-8f);
+        const float old_logp = fl.r_logp[src];
+        float o[2 * PA_MAX], g[2 * PA_MAX];
+#pragma unroll
+        for (int a = 0; a < PA_MAX; ++a) {
+            o[a] = ys[t * (PA_MAX + 1) + a];
+            float ls = w2s[HEAD_LOG_STD(H) + a];
+            o[PA_MAX + a] = ls;
+        }
+        if (fl.continuous) {
+            float oo[2 * PA_MAX], act[PA_MAX];
+            for (int j = 0; j < A; ++j) {
+                oo[j] = o[j];
+                oo[A + j] = o[PA_MAX + j];   // clamped inside the gradient, as in the stored output
+                act[j] = fl.r_act[src * A + j];
+            }
+            kl = actor_grad_gaussian_row(oo, act, adv, old_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
+            for (int j = 0; j < 2 * A; ++j) fl.g_actor_out[(size_t)b * 2 * A + j] = g[j];
+        } else {
+            kl = actor_grad_discrete_row(o, (int)fl.r_act[src], adv, old_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
+            for (int a = 0; a < A; ++a) fl.g_actor_out[(size_t)b * A + a] = g[a];
+        }
+        fl.kl[b] = kl;
+    }
+    if (fl.kl_flag == nullptr) return;
+    // KL test: every actor tile leaves the sum of its rows' estimates; the last one to arrive adds
+    // the tiles up in order, compares the mean with target_kl and re-arms the counter
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) kl += __shfl_xor(kl, off, 64);
+    int last = 0;
+    if (t == 0) {
+        __hip_atomic_store(&fl.kl_part[blockIdx.x], kl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence();
+        last = atomicAdd(fl.arrived, 1) == (int)gridDim.x - 1;
+    }
+    last = __shfl(last, 0, 64);
+    if (!last) return;
+    __threadfence();
+    float sum = 0.0f;
+    for (int i = t; i < (int)gridDim.x; i += 64)
+        sum += __hip_atomic_load(&fl.kl_part[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (t == 0) {
+        const float mean = sum / (float)fl.mb;
+        fl.kl_flag[1] = __float_as_int(mean);
+        if (mean > fl.target_kl) fl.kl_flag[0] = 1;
+        *fl.arrived = 0;
     }
 }
 
@@ -455,9 +524,9 @@ bool mlp3_pair_fusable(const mrl_mlp_desc &a, const mrl_mlp_desc &b) {
 }
 
 template <int H, int ACT>
-static void launch_fwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, int n_nets) {
+static void launch_fwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, int n_nets, const FwdLoss &fl) {
     dim3 grid((batch + PR - 1) / PR, n_nets);
-    hipLaunchKernelGGL((mlp3_fwd_kernel<H, ACT>), grid, dim3(2 * H), 0, ctx->stream, batch, IN, nets);
+    hipLaunchKernelGGL((mlp3_fwd_kernel<H, ACT>), grid, dim3(2 * H), 0, ctx->stream, batch, IN, nets, fl);
 }
 template <int H, int ACT>
 static void launch_bwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, int n_nets) {
@@ -466,7 +535,8 @@ static void launch_bwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, 
 }
 
 // forward of one or two nets (descs[i], io.n[i]) in one launch
-int mlp3_forward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io) {
+int mlp3_forward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io,
+                   const FwdLoss *loss) {
     int H = 0, act = 0;
     bool gauss = false;
     for (int i = 0; i < n_nets; ++i) {
@@ -476,10 +546,16 @@ int mlp3_forward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, i
     }
     if (n_nets == 2 && !mlp3_pair_fusable(*descs[0], *descs[1])) return MRL_E_UNSUPPORTED;
     const int IN = descs[0]->layers[0].in_dim;
-    if (H == 256 && act == 1) launch_fwd_t<256, 1>(ctx, batch, IN, io, n_nets);
-    else if (H == 256) launch_fwd_t<256, 2>(ctx, batch, IN, io, n_nets);
-    else if (act == 1) launch_fwd_t<64, 1>(ctx, batch, IN, io, n_nets);
-    else launch_fwd_t<64, 2>(ctx, batch, IN, io, n_nets);
+    FwdLoss fl{};
+    if (loss != nullptr) {
+        if (n_nets != 2 || (batch + PR - 1) / PR > 1024) return MRL_E_UNSUPPORTED;   // one KL partial per row tile
+        fl = *loss;
+        fl.enabled = 1;
+    }
+    if (H == 256 && act == 1) launch_fwd_t<256, 1>(ctx, batch, IN, io, n_nets, fl);
+    else if (H == 256) launch_fwd_t<256, 2>(ctx, batch, IN, io, n_nets, fl);
+    else if (act == 1) launch_fwd_t<64, 1>(ctx, batch, IN, io, n_nets, fl);
+    else launch_fwd_t<64, 2>(ctx, batch, IN, io, n_nets, fl);
     MRL_CHECK_LAUNCH();
     return MRL_OK;
 }

@@ -115,6 +115,53 @@ __global__ __launch_bounds__(UTPB) void gather_norm_kernel(GatherArgs g) {
     }
 }
 
+// Mean and standard deviation of the advantages of minibatch blockIdx.x (rows idx[k * mb ..]), with
+// the arithmetic of the normalising workgroup of gather_norm_kernel: stats[2k] = mean,
+// stats[2k + 1] = sqrt(variance + 1e-8).  The fused forward normalises with them on the fly.
+__global__ __launch_bounds__(UTPB) void adv_stats_kernel(const int32_t *__restrict__ idx,
+                                                         const float *__restrict__ r_adv, int mb,
+                                                         float *__restrict__ stats) {
+    __shared__ float smem[4];
+    constexpr int PER = 32;
+    const int32_t *my = idx + (size_t)blockIdx.x * mb;
+    float mean, variance;
+    if (mb <= PER * UTPB) {
+        float v[PER];
+        bool in[PER];
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const int i = threadIdx.x + k * UTPB;
+            in[k] = i < mb;
+            v[k] = in[k] ? r_adv[my[i]] : 0.0f;
+        }
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) s += v[k];
+        mean = u_block_sum<4>(s, smem) / (float)mb;
+        float q = 0.0f;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const float d = v[k] - mean;
+            q += in[k] ? d * d : 0.0f;
+        }
+        variance = u_block_sum<4>(q, smem) / (float)mb;
+    } else {
+        float s = 0.0f;
+        for (int i = threadIdx.x; i < mb; i += UTPB) s += r_adv[my[i]];
+        mean = u_block_sum<4>(s, smem) / (float)mb;
+        float q = 0.0f;
+        for (int i = threadIdx.x; i < mb; i += UTPB) {
+            const float d = r_adv[my[i]] - mean;
+            q += d * d;
+        }
+        variance = u_block_sum<4>(q, smem) / (float)mb;
+    }
+    if (threadIdx.x == 0) {
+        stats[2 * blockIdx.x] = mean;
+        stats[2 * blockIdx.x + 1] = sqrtf(variance + 1e-8f);
+    }
+}
+
 // Actor and critic loss gradients in one launch (grid.y = 0: actor, 1: critic) and the KL test:
 // every actor workgroup leaves the sum of its samples' KL estimates, the last one to arrive adds
 // them up in workgroup order, compares the mean with target_kl and re-arms the counter.
@@ -257,18 +304,32 @@ static int update_check(const mrl_update *u, const char *who) {
     return MRL_OK;
 }
 
-int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int actor_t,
-                             int critic_t) {
-    MRL_CHECK_ARG(ctx != nullptr, "mrl_ppo_update_minibatch: ctx is NULL");
-    int rc = update_check(u, "mrl_ppo_update_minibatch");
-    if (rc) return rc;
-    MRL_CHECK_ARG(indices != nullptr && actor_t >= 1 && critic_t >= 1,
-                  "mrl_ppo_update_minibatch: need indices and step counts >= 1");
+// floats of ctx->upd_scratch: KL partials, their arrival counter, sum-of-squares partials, and the
+// advantage statistics of up to STATS_MAX minibatches
+constexpr int SCR_KL = 0, SCR_ARRIVED = 1024, SCR_SQ = 2048, SCR_STATS = 4096, STATS_MAX = 2048;
+
+static bool update_paired(const mrl_update *u) {
+    return mlp3_pair_fusable(u->actor, u->critic) && reinterpret_cast<uintptr_t>(u->actor_params) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(u->critic_params) % 16 == 0 && (u->minibatch + 31) / 32 <= 1024;
+}
+
+// stats: {mean, std} of this minibatch's advantages on the device, already enqueued (paired nets
+// only); null: worked out here
+static int update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int actor_t, int critic_t,
+                            const float *stats) {
+    int rc;
     const int mb = u->minibatch, head = mrl_mlp_out_dim(&u->actor);
     const int Pa = mrl_mlp_param_size(&u->actor), Pc = mrl_mlp_param_size(&u->critic);
     const bool cont = u->continuous != 0;
+    const bool paired = update_paired(u);
 
-    {
+    if (paired && u->norm_adv_per_minibatch && stats == nullptr) {
+        float *st = ctx->upd_scratch + SCR_STATS;
+        hipLaunchKernelGGL(adv_stats_kernel, dim3(1), dim3(UTPB), 0, ctx->stream, indices, u->advantages, mb, st);
+        MRL_CHECK_LAUNCH();
+        stats = st;
+    }
+    if (!paired) {
         GatherArgs g{indices, u->r_obs, u->r_actions, u->advantages, u->returns, u->r_log_probs, u->r_values,
                      u->mb_obs, u->mb_actions, u->mb_adv, u->mb_ret, u->mb_logp, u->mb_val,
                      mb, u->obs_dim, u->act_width, u->norm_adv_per_minibatch};
@@ -279,14 +340,25 @@ int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *i
     }
 
     const mrl_mlp_desc *descs[2] = {&u->actor, &u->critic};
-    const bool paired = mlp3_pair_fusable(u->actor, u->critic) &&
-                        reinterpret_cast<uintptr_t>(u->actor_params) % 16 == 0 &&
-                        reinterpret_cast<uintptr_t>(u->critic_params) % 16 == 0;
     Mlp3Nets io{};
     io.n[0].x = u->mb_obs; io.n[0].params = u->actor_params; io.n[0].out = u->actor_out; io.n[0].cache = u->actor_cache;
     io.n[1].x = u->mb_obs; io.n[1].params = u->critic_params; io.n[1].out = u->values; io.n[1].cache = u->critic_cache;
     if (paired) {
-        rc = mlp3_forward_n(ctx, descs, 2, mb, io);
+        // forward of both nets straight from the rollout rows, loss gradients and KL test in its tail
+        FwdLoss fl{};
+        fl.idx = indices;
+        fl.r_obs = u->r_obs; fl.r_act = u->r_actions; fl.r_adv = u->advantages; fl.r_ret = u->returns;
+        fl.r_logp = u->r_log_probs; fl.r_val = u->r_values;
+        fl.adv_stats = u->norm_adv_per_minibatch ? stats : nullptr;
+        fl.g_actor_out = u->g_actor_out; fl.g_values = u->g_values; fl.kl = u->kl;
+        fl.kl_part = ctx->upd_scratch + SCR_KL;
+        fl.arrived = reinterpret_cast<int *>(ctx->upd_scratch + SCR_ARRIVED);
+        fl.kl_flag = u->target_kl > 0.0f ? u->kl_flag : nullptr;
+        fl.mb = mb; fl.A = cont ? u->act_width : head; fl.continuous = cont ? 1 : 0;
+        fl.clip_value = u->clip_value ? 1 : 0;
+        fl.clip_eps = u->clip_epsilon; fl.ent_coef = u->entropy_coef; fl.value_coef = u->value_loss_coef;
+        fl.target_kl = u->target_kl;
+        rc = mlp3_forward_n(ctx, descs, 2, mb, io, &fl);
         if (rc) return rc;
     } else {
         rc = mrl_mlp_forward(ctx, &u->actor, mb, u->mb_obs, u->actor_params, u->actor_out, u->actor_cache);
@@ -295,7 +367,7 @@ int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *i
         if (rc) return rc;
     }
 
-    {
+    if (!paired) {
         const int nblk = grid_for(mb, UTPB);
         const bool test = u->target_kl > 0.0f && nblk <= 1024;
         LossArgs a{u->actor_out, u->mb_logp, u->mb_adv, u->mb_actions, u->values, u->mb_val, u->mb_ret,
@@ -359,14 +431,37 @@ int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *i
     return MRL_OK;
 }
 
+int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int actor_t,
+                             int critic_t) {
+    MRL_CHECK_ARG(ctx != nullptr, "mrl_ppo_update_minibatch: ctx is NULL");
+    int rc = update_check(u, "mrl_ppo_update_minibatch");
+    if (rc) return rc;
+    MRL_CHECK_ARG(indices != nullptr && actor_t >= 1 && critic_t >= 1,
+                  "mrl_ppo_update_minibatch: need indices and step counts >= 1");
+    return update_minibatch(ctx, u, indices, actor_t, critic_t, nullptr);
+}
+
 int mrl_ppo_update_epoch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int n_minibatches,
                          int actor_t0, int critic_t0) {
-    MRL_CHECK_ARG(ctx != nullptr && u != nullptr, "mrl_ppo_update_epoch: NULL argument");
+    MRL_CHECK_ARG(ctx != nullptr, "mrl_ppo_update_epoch: ctx is NULL");
+    int rc = update_check(u, "mrl_ppo_update_epoch");
+    if (rc) return rc;
     MRL_CHECK_ARG(n_minibatches >= 0 && actor_t0 >= 0 && critic_t0 >= 0, "mrl_ppo_update_epoch: negative count");
-    for (int k = 0; k < n_minibatches; ++k) {
-        int rc = mrl_ppo_update_minibatch(ctx, u, indices + (size_t)k * u->minibatch, actor_t0 + k + 1,
-                                          critic_t0 + k + 1);
-        if (rc) return rc;
+    MRL_CHECK_ARG(n_minibatches == 0 || indices != nullptr, "mrl_ppo_update_epoch: indices is NULL");
+    const bool ahead = update_paired(u) && u->norm_adv_per_minibatch;
+    for (int k0 = 0; k0 < n_minibatches; k0 += STATS_MAX) {
+        const int n = std::min(STATS_MAX, n_minibatches - k0);
+        float *stats = ctx->upd_scratch + SCR_STATS;
+        if (ahead) {   // the advantage statistics of all these minibatches in one launch
+            hipLaunchKernelGGL(adv_stats_kernel, dim3(n), dim3(UTPB), 0, ctx->stream,
+                               indices + (size_t)k0 * u->minibatch, u->advantages, u->minibatch, stats);
+            MRL_CHECK_LAUNCH();
+        }
+        for (int k = k0; k < k0 + n; ++k) {
+            rc = update_minibatch(ctx, u, indices + (size_t)k * u->minibatch, actor_t0 + k + 1, critic_t0 + k + 1,
+                                  ahead ? stats + 2 * (k - k0) : nullptr);
+            if (rc) return rc;
+        }
     }
     return MRL_OK;
 }

@@ -5,13 +5,10 @@
 
 namespace mrl {
 
-// deep_agents/ppo/ppo.mojo:285-378; returns the sample's KL estimate (old - new log-prob)
-MRL_DEV float actor_grad_discrete_one(int b, const float *__restrict__ logits, const float *__restrict__ old_logp,
-                                      const float *__restrict__ adv, const float *__restrict__ actions, int mb,
-                                      int A, float clip_eps, float ent_coef, float *__restrict__ grad_logits) {
-    const float *l = logits + (long)b * A;
-    int action = (int)actions[b];
-    float advantage = adv[b];
+// deep_agents/ppo/ppo.mojo:285-378 for one sample: l = its A logits, g = its A gradient slots;
+// returns the sample's KL estimate (old - new log-prob)
+MRL_DEV float actor_grad_discrete_row(const float *l, int action, float advantage, float old, int mb, int A,
+                                      float clip_eps, float ent_coef, float *g_row) {
     float max_logit = l[0];
     for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
     float sum_exp = 0.0f;
@@ -22,7 +19,6 @@ MRL_DEV float actor_grad_discrete_one(int b, const float *__restrict__ logits, c
         if (a == action) p_action = p;
     }
     float new_logp = logf(p_action + 1e-8f);
-    float old = old_logp[b];
     float ratio = expf(new_logp - old);
     bool clipped = (ratio < 1.0f - clip_eps) || (ratio > 1.0f + clip_eps);
     for (int a = 0; a < A; ++a) {
@@ -34,19 +30,23 @@ MRL_DEV float actor_grad_discrete_one(int b, const float *__restrict__ logits, c
             float d_entropy = -p * (1.0f + log_prob_ent);
             g = (-advantage * ratio * d_log_prob - ent_coef * d_entropy) / (float)mb;
         }
-        grad_logits[(long)b * A + a] = g;
+        g_row[a] = g;
     }
     return old - new_logp;
 }
-
-// deep_agents/ppo/kernels.mojo:230-412; returns the sample's KL estimate ((ratio - 1) - diff, clamped)
-MRL_DEV float actor_grad_gaussian_one(int b, const float *__restrict__ actor_out, const float *__restrict__ old_logp,
+MRL_DEV float actor_grad_discrete_one(int b, const float *__restrict__ logits, const float *__restrict__ old_logp,
                                       const float *__restrict__ adv, const float *__restrict__ actions, int mb,
-                                      int A, float clip_eps, float ent_coef, float *__restrict__ grad_out) {
+                                      int A, float clip_eps, float ent_coef, float *__restrict__ grad_logits) {
+    return actor_grad_discrete_row(logits + (long)b * A, (int)actions[b], adv[b], old_logp[b], mb, A, clip_eps,
+                                   ent_coef, grad_logits + (long)b * A);
+}
+
+// deep_agents/ppo/kernels.mojo:230-412 for one sample: o = [mean (A) | log_std (A)], act = its A
+// action components, g = its 2A gradient slots; returns the sample's KL estimate
+// ((ratio - 1) - diff, clamped)
+MRL_DEV float actor_grad_gaussian_row(const float *o, const float *act, float advantage, float old_log_prob,
+                                      int mb, int A, float clip_eps, float ent_coef, float *g) {
     const float eps = 1e-6f, log_2pi = (float)1.8378770664093453;
-    const float *o = actor_out + (long)b * 2 * A;
-    const float *act = actions + (long)b * A;
-    float advantage = adv[b], old_log_prob = old_logp[b];
     float new_log_prob = 0.0f;
     for (int j = 0; j < A; ++j) {
         float log_std = o[A + j];
@@ -68,7 +68,6 @@ MRL_DEV float actor_grad_gaussian_one(int b, const float *__restrict__ actor_out
     if (clipped_ratio < 1.0f - clip_eps) clipped_ratio = 1.0f - clip_eps;
     else if (clipped_ratio > 1.0f + clip_eps) clipped_ratio = 1.0f + clip_eps;
     bool is_clipped = clipped_ratio * advantage < ratio * advantage;
-    float *g = grad_out + (long)b * 2 * A;
     for (int j = 0; j < A; ++j) {
         float gm = 0.0f, gs = 0.0f;
         if (!is_clipped) {
@@ -91,18 +90,21 @@ MRL_DEV float actor_grad_gaussian_one(int b, const float *__restrict__ actor_out
     }
     return kl;
 }
+MRL_DEV float actor_grad_gaussian_one(int b, const float *__restrict__ actor_out, const float *__restrict__ old_logp,
+                                      const float *__restrict__ adv, const float *__restrict__ actions, int mb,
+                                      int A, float clip_eps, float ent_coef, float *__restrict__ grad_out) {
+    return actor_grad_gaussian_row(actor_out + (long)b * 2 * A, actions + (long)b * A, adv[b], old_logp[b], mb, A,
+                                   clip_eps, ent_coef, grad_out + (long)b * 2 * A);
+}
 
 // ppo.mojo:538-633 (convention 0) and kernels.mojo:416-486 (convention 1)
-MRL_DEV float critic_grad_one(int b, const float *__restrict__ values, const float *__restrict__ old_values,
-                              const float *__restrict__ returns, int mb, int convention, int clipped,
-                              float value_coef, float clip_eps) {
-    float v = values[b], ret = returns[b];
+MRL_DEV float critic_grad_value(float v, float v_old, float ret, int mb, int convention, int clipped,
+                                float value_coef, float clip_eps) {
     float out;
     if (convention == 0) {
         if (!clipped) {
             out = 2.0f * value_coef * (v - ret) / (float)mb;
         } else {
-            float v_old = old_values[b];
             float v_diff = v - v_old;
             float v_clipped;
             if (v_diff > clip_eps) v_clipped = v_old + clip_eps;
@@ -120,7 +122,7 @@ MRL_DEV float critic_grad_one(int b, const float *__restrict__ values, const flo
         if (!clipped) {
             out = (v - ret) / (float)mb;
         } else {
-            float old_value = old_values[b];
+            float old_value = v_old;
             float d = v - old_value;
             float mn = d < clip_eps ? d : clip_eps;
             float mx = mn > -clip_eps ? mn : -clip_eps;
@@ -138,6 +140,13 @@ MRL_DEV float critic_grad_one(int b, const float *__restrict__ values, const flo
         }
     }
     return out;
+}
+
+MRL_DEV float critic_grad_one(int b, const float *__restrict__ values, const float *__restrict__ old_values,
+                              const float *__restrict__ returns, int mb, int convention, int clipped,
+                              float value_coef, float clip_eps) {
+    return critic_grad_value(values[b], clipped ? old_values[b] : 0.0f, returns[b], mb, convention, clipped, value_coef,
+                             clip_eps);
 }
 
 }  // namespace mrl
