@@ -45,8 +45,11 @@ int mlp3_backward(mrl_ctx *ctx, const mrl_mlp_desc &d, int batch, const float *g
                   const float *cache, float *grads, float *ws);
 // sq_part (nullable): receives per-block sums of squares of the gradients, [net * 1024 + block];
 // *sq_blocks = number of blocks written (0 when none were)
+// fused (nullable): the nets have not gone forward yet -- one kernel per row tile runs forward
+// (inputs read through fused->idx, io.n[i].out written, h1 into the cache's c1 rows), loss
+// gradients and the way back, in place of a forward launch, a loss launch and the dx launch
 int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io,
-                    float *const *grads, float *ws, float *sq_part, int *sq_blocks);
+                    float *const *grads, float *ws, float *sq_part, int *sq_blocks, const FwdLoss *fused = nullptr);
 // grows the context's MLP workspace to at least `floats`
 int mlp_ensure_ws(mrl_ctx *ctx, size_t floats, float **out);
 

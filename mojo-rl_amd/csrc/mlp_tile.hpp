@@ -26,8 +26,8 @@ MRL_DEV float activate(float x) {
 
 // Where a tile's forward leaves the reference's per-layer cache (deep_rl/model/sequential.mojo:
 // 104-133, blocked per layer): c0 rows [x (IN) | layer-0 pre-activation or tanh output (H)],
-// c1 rows [h1 (H) | layer-1 pre-activation or tanh output (H)], c2 rows [h2 (H)].  c0 == nullptr:
-// nothing is cached.
+// c1 rows [h1 (H) | layer-1 pre-activation or tanh output (H)], c2 rows [h2 (H)].  All null:
+// nothing is cached; c1 alone: only h1 is stored (what the H x H weight gradient reads).
 struct TileCache {
     float *c0, *c1, *c2;
     long row0;   // first batch row of the tile
@@ -157,8 +157,8 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
                 const float pre = c[q][v] + bias0[q];
                 const float y = activate<ACT>(pre);
                 hT[col[q] * HT_LD + row] = y;
-                if (tc.c0 != nullptr && row < tc.nrow) {
-                    tc.c0[(tc.row0 + row) * (IN + H) + IN + col[q]] = ACT == 1 ? pre : y;
+                if (tc.c1 != nullptr && row < tc.nrow) {
+                    if (tc.c0 != nullptr) tc.c0[(tc.row0 + row) * (IN + H) + IN + col[q]] = ACT == 1 ? pre : y;
                     tc.c1[(tc.row0 + row) * (2 * H) + col[q]] = y;
                 }
             }
@@ -208,7 +208,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
                 const float pre = c[q][v] + bias1[q];
                 const float y = activate<ACT>(pre);
                 h2[row * (H + 1) + col[q]] = y;
-                if (tc.c0 != nullptr && row < tc.nrow) {
+                if (tc.c2 != nullptr && row < tc.nrow) {
                     tc.c1[(tc.row0 + row) * (2 * H) + H + col[q]] = ACT == 1 ? pre : y;
                     tc.c2[(tc.row0 + row) * H + col[q]] = y;
                 }

@@ -336,6 +336,250 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
     }
 }
 
+// ---------------------------------------------------------------- forward + loss + backward of a tile
+// The PPO minibatch never needs the activations outside the workgroup that made them: a row tile
+// goes forward (as mlp3_fwd_kernel with its loss tail), and while h1 and h2 are still in LDS the
+// same workgroup takes the loss gradient back through the three layers (as mlp3_bwd_dx_kernel).
+// Only what the H x H weight gradient needs leaves the chip -- h1 (into the cache's c1 rows) and
+// g1 -- next to the per-tile bias / thin-layer partials.  act' comes from the activation's output
+// (y > 0 for ReLU, 1 - y^2 for tanh), which is what the cached entries decide as well.
+template <int ACT>
+MRL_DEV float act_deriv_out(float y) {
+    if (ACT == 1) return y > 0.0f ? 1.0f : 0.0f;
+    if (ACT == 2) return 1.0f - y * y;
+    return 1.0f;
+}
+
+template <int H, int ACT>
+__global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets nets, FwdLoss fl) {
+    constexpr int T = 2 * H, KCH = 64;
+    static_assert(KCH * (H + 1) <= H * HT_LD + PR * (H + 1), "the W1 staging buffer fits over the two activation tiles");
+    __shared__ float xs[PR * XS_LD];
+    __shared__ float big[H * HT_LD + PR * (H + 1)];   // hT | h2 going forward, W1 chunks going back
+    __shared__ float ys[PR * (PA_MAX + 1)];
+    __shared__ __align__(16) float w2s[HEAD_LDS(H)];
+    __shared__ float g2s[PR * (2 * PA_MAX + 1)];
+    __shared__ float gT[H * HT_LD];                   // g1 of the tile, k-major
+    float *hT = big, *h2 = big + H * HT_LD, *wT = big;
+    const Mlp3Net &nn = nets.n[blockIdx.y];
+    const float *__restrict__ params = nn.params;
+    float *__restrict__ out = nn.out;
+    float *__restrict__ g1 = nn.g1;
+    float *__restrict__ ls_part = nn.ls_part;
+    float *__restrict__ db_part = nn.db_part + (size_t)blockIdx.x * (2 * H + PA_MAX);
+    const int A = nn.A;
+    float *__restrict__ thin_part = nn.thin_part + (size_t)blockIdx.x * ((size_t)IN * H + (size_t)H * A);
+    const bool GAUSS = nn.gauss != 0;
+    const int ld = GAUSS ? 2 * A : A;
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
+    const long row0 = (long)blockIdx.x * PR;
+    const int nrow = (int)min((long)PR, B - row0);
+    const float *W1 = params + IN * H + H;
+    TileCache tc{nullptr, nn.cache + (size_t)B * (IN + H), nullptr, row0, nrow};   // h1 only
+
+    // ---- forward
+    HiddenOperands<H, 1, 32> ops;
+    ops.load(params, IN);
+    constexpr int NX = (PR * PIN_MAX + T - 1) / T;
+    float xv[NX];
+#pragma unroll
+    for (int q = 0; q < NX; ++q) {
+        const int i = t + q * T;
+        xv[q] = 0.0f;
+        if (i < PR * IN && i / IN < nrow) {
+            const int r = i / IN;
+            xv[q] = fl.r_obs[(size_t)fl.idx[row0 + r] * IN + (i - r * IN)];
+        }
+    }
+    stage_head(params + IN * H + H + H * H + H, H, A, GAUSS, w2s, t, T);
+    for (int i = t; i < PR * (2 * PA_MAX + 1); i += T) g2s[i] = 0.0f;
+#pragma unroll
+    for (int q = 0; q < NX; ++q) {
+        const int i = t + q * T;
+        if (i < PR * IN) xs[(i / IN) * XS_LD + (i % IN)] = xv[q];
+    }
+    __syncthreads();
+    hidden_stack<H, ACT, 1>(params, IN, xs, hT, h2, tc, ops);
+    if (t < H) head<H>(w2s, A, h2, ys, PA_MAX + 1);
+    __syncthreads();
+    for (int i = t; i < nrow * ld; i += T) {
+        const int r = i / ld, a = i - r * ld;
+        float v;
+        if (a < A) {
+            v = ys[r * (PA_MAX + 1) + a];
+        } else {   // state-independent log_std, clamped (deep_rl/model/stochastic_actor.mojo:260-275)
+            v = w2s[HEAD_LOG_STD(H) + (a - A)];
+            if (v < -5.0f) v = -5.0f;
+            else if (v > 2.0f) v = 2.0f;
+        }
+        out[(row0 + r) * ld + a] = v;
+    }
+    // what the way back needs from the forward tiles before their memory is reused: act'(h1) at
+    // this lane's accumulator positions; and the first chunk of W1
+    const int col = 32 * w + l31;
+    float d0[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) d0[v] = act_deriv_out<ACT>(hT[col * HT_LD + 8 * (v >> 2) + 4 * half + (v & 3)]);
+    const int wrow = t % H, wseg = (t / H) * (KCH / 2);   // thread copies W1[wrow][o0 + wseg .. + KCH / 2)
+    float4 nxt[KCH / 8];
+    auto fetch = [&](int o0) {
+        const float4 *src = reinterpret_cast<const float4 *>(W1 + (size_t)wrow * H + o0 + wseg);
+#pragma unroll
+        for (int q = 0; q < KCH / 8; ++q) nxt[q] = src[q];
+    };
+    fetch(0);
+
+    // ---- loss gradients of the tile's rows, one lane per row (wavefront 0), into g2s and out
+    float kl = 0.0f;
+    if (t < nrow) {
+        const int b = (int)row0 + t;
+        const long src = fl.idx[b];
+        float *g2row = g2s + t * (2 * PA_MAX + 1);
+        if (blockIdx.y == 1) {   // critic
+            const float g = critic_grad_value(ys[t * (PA_MAX + 1)], fl.clip_value ? fl.r_val[src] : 0.0f, fl.r_ret[src],
+                                              fl.mb, fl.continuous, fl.clip_value, fl.value_coef, fl.clip_eps);
+            g2row[0] = g;
+            fl.g_values[b] = g;
+        } else {
+            float adv = fl.r_adv[src];
+            if (fl.adv_stats != nullptr) adv = (adv - fl.adv_stats[0]) / (fl.adv_stats[1] + 1e-8f);
+            const float old_logp = fl.r_logp[src];
+            float o[2 * PA_MAX], g[2 * PA_MAX];
+            for (int a = 0; a < A; ++a) o[a] = ys[t * (PA_MAX + 1) + a];
+            if (fl.continuous) {
+                float act[PA_MAX];
+                for (int j = 0; j < A; ++j) {
+                    o[A + j] = w2s[HEAD_LOG_STD(H) + j];   // clamped inside the gradient, as in the stored output
+                    act[j] = fl.r_act[src * A + j];
+                }
+                kl = actor_grad_gaussian_row(o, act, adv, old_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
+            } else {
+                kl = actor_grad_discrete_row(o, (int)fl.r_act[src], adv, old_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
+            }
+            for (int j = 0; j < ld; ++j) {
+                g2row[j] = g[j];
+                fl.g_actor_out[(size_t)b * ld + j] = g[j];
+            }
+            fl.kl[b] = kl;
+        }
+    }
+    if (fl.kl_flag != nullptr && blockIdx.y == 0 && t < 64) {
+        // KL test: every actor tile leaves the sum of its rows' estimates; the last one to arrive
+        // adds the tiles up in order, compares the mean with target_kl and re-arms the counter
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) kl += __shfl_xor(kl, off, 64);
+        int last = 0;
+        if (t == 0) {
+            __hip_atomic_store(&fl.kl_part[blockIdx.x], kl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __threadfence();
+            last = atomicAdd(fl.arrived, 1) == (int)gridDim.x - 1;
+        }
+        last = __shfl(last, 0, 64);
+        if (last) {
+            __threadfence();
+            float sum = 0.0f;
+            for (int i = t; i < (int)gridDim.x; i += 64)
+                sum += __hip_atomic_load(&fl.kl_part[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+            if (t == 0) {
+                const float mean = sum / (float)fl.mb;
+                fl.kl_flag[1] = __float_as_int(mean);
+                if (mean > fl.target_kl) fl.kl_flag[0] = 1;
+                *fl.arrived = 0;
+            }
+        }
+    }
+    __syncthreads();   // g2s complete
+
+    // ---- back through the head and layer 1's activation
+    if (t < H) {   // g1[r][n] = (sum_a g2[r][a] W2[n][a]) * act'(layer 1); thread t owns column n = t
+        float w2row[PA_MAX];
+#pragma unroll
+        for (int a = 0; a < PA_MAX; ++a) w2row[a] = w2s[t * PA_MAX + a];   // zero beyond A
+        float colsum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < PR; ++r) {
+            float s = 0.0f;
+#pragma unroll
+            for (int a = 0; a < PA_MAX; ++a)
+                if (a < A) s = fmaf(g2s[r * (2 * PA_MAX + 1) + a], w2row[a], s);
+            float g = 0.0f;
+            if (r < nrow) {
+                g = s * act_deriv_out<ACT>(h2[r * (H + 1) + t]);
+                g1[(row0 + r) * H + t] = g;
+            }
+            gT[t * HT_LD + r] = g;
+            colsum += g;
+        }
+        db_part[H + t] = colsum;   // bias gradient of layer 1, this tile's rows
+    } else {       // meanwhile the other half of the block: dW2[n][a] of the tile = sum_r h2[r][n] g2[r][a]
+        const int n = t - H;
+        float s[PA_MAX];
+#pragma unroll
+        for (int a = 0; a < PA_MAX; ++a) s[a] = 0.0f;
+#pragma unroll
+        for (int r = 0; r < PR; ++r) {
+            const float h = r < nrow ? h2[r * (H + 1) + n] : 0.0f;
+#pragma unroll
+            for (int a = 0; a < PA_MAX; ++a)
+                if (a < A) s[a] = fmaf(h, g2s[r * (2 * PA_MAX + 1) + a], s[a]);
+        }
+        float *o2 = thin_part + (size_t)IN * H + (size_t)n * A;
+#pragma unroll
+        for (int a = 0; a < PA_MAX; ++a)
+            if (a < A) o2[a] = s[a];
+        if (n < ld) {   // column sums of the tile: bias gradient of the head, log_std gradient
+            float cs2 = 0.0f;
+            for (int r = 0; r < PR; ++r) cs2 += g2s[r * (2 * PA_MAX + 1) + n];
+            if (n < A) db_part[2 * H + n] = cs2;
+            else ls_part[(long)blockIdx.x * A + (n - A)] = cs2;
+        }
+    }
+    // ---- dh1 = g1 W1^T: wavefront w owns input columns [32w, 32w + 32); the next chunk of W1 is
+    // fetched into registers while the matrix cores work on the current one
+    floatx16 acc = {0};
+    for (int o0 = 0; o0 < H; o0 += KCH) {
+        __syncthreads();   // gT complete and the activation tiles read (first round) / previous chunk consumed
+#pragma unroll
+        for (int q = 0; q < KCH / 8; ++q) {
+            wT[(wseg + 4 * q + 0) * (H + 1) + wrow] = nxt[q].x;
+            wT[(wseg + 4 * q + 1) * (H + 1) + wrow] = nxt[q].y;
+            wT[(wseg + 4 * q + 2) * (H + 1) + wrow] = nxt[q].z;
+            wT[(wseg + 4 * q + 3) * (H + 1) + wrow] = nxt[q].w;
+        }
+        __syncthreads();
+        if (o0 + KCH < H) fetch(o0 + KCH);
+        __builtin_amdgcn_sched_barrier(0);   // keep the loads ahead of the MFMAs that hide them
+#pragma unroll
+        for (int kk = 0; kk < KCH / 2; ++kk) {
+            const int k = 2 * kk + half;
+            const float a = gT[(o0 + k) * HT_LD + l31];
+            const float b = wT[k * (H + 1) + col];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+        }
+    }
+    float cs = 0.0f;
+    float gv[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int row = 8 * (v >> 2) + 4 * half + (v & 3);
+        gv[v] = row < nrow ? acc[v] * d0[v] : 0.0f;
+        cs += gv[v];
+    }
+    // the two halves of the wavefront hold the other 16 rows of the same column
+    cs += __shfl_xor(cs, 32, 64);
+    if (half == 0) db_part[col] = cs;   // bias gradient of layer 0, this tile's rows
+    // dW0[i][col] of the tile = sum_r x[r][i] g0[r][col]
+    for (int i = 0; i < IN; ++i) {
+        float s = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s = fmaf(xs[(8 * (v >> 2) + 4 * half + (v & 3)) * XS_LD + i], gv[v], s);
+        s += __shfl_xor(s, 32, 64);
+        if (half == 0) thin_part[(size_t)i * H + col] = s;
+    }
+}
+
 // ---------------------------------------------------------------- [dW | db] of the three layers
 constexpr int DBM = 64, DBN = 64, DKC = 32, DLD = 65;
 
@@ -529,9 +773,12 @@ static void launch_fwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, 
     hipLaunchKernelGGL((mlp3_fwd_kernel<H, ACT>), grid, dim3(2 * H), 0, ctx->stream, batch, IN, nets, fl);
 }
 template <int H, int ACT>
-static void launch_bwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, int n_nets) {
+static void launch_bwd_t(mrl_ctx *ctx, int batch, int IN, const Mlp3Nets &nets, int n_nets, const FwdLoss *fused) {
     dim3 grid((batch + PR - 1) / PR, n_nets);
-    hipLaunchKernelGGL((mlp3_bwd_dx_kernel<H, ACT>), grid, dim3(2 * H), 0, ctx->stream, batch, IN, nets);
+    if (fused != nullptr)
+        hipLaunchKernelGGL((mlp3_fb_kernel<H, ACT>), grid, dim3(2 * H), 0, ctx->stream, batch, IN, nets, *fused);
+    else
+        hipLaunchKernelGGL((mlp3_bwd_dx_kernel<H, ACT>), grid, dim3(2 * H), 0, ctx->stream, batch, IN, nets);
 }
 
 // forward of one or two nets (descs[i], io.n[i]) in one launch
@@ -584,7 +831,8 @@ size_t mlp3_backward_ws(const mrl_mlp_desc *const *descs, int n_nets, int batch)
 // backward (parameter gradients only) of one or two nets: io.n[i].grad_out / params / cache in,
 // grads[i] out; ws as sized by mlp3_backward_ws
 int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, int batch, Mlp3Nets io,
-                    float *const *grads, float *ws, float *sq_part, int *sq_blocks) {
+                    float *const *grads, float *ws, float *sq_part, int *sq_blocks, const FwdLoss *fused) {
+    if (fused != nullptr && (n_nets != 2 || (batch + PR - 1) / PR > 1024)) return MRL_E_UNSUPPORTED;
     int H = 0, act = 0;
     bool gauss = false;
     for (int i = 0; i < n_nets; ++i) {
@@ -612,10 +860,16 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
         io.n[i].thin_part = w; w += (size_t)tiles * ((size_t)IN * H + (size_t)H * descs[i]->layers[2].out_dim);
     }
     float *partial = w;
-    if (H == 256 && act == 1) launch_bwd_t<256, 1>(ctx, batch, IN, io, n_nets);
-    else if (H == 256) launch_bwd_t<256, 2>(ctx, batch, IN, io, n_nets);
-    else if (act == 1) launch_bwd_t<64, 1>(ctx, batch, IN, io, n_nets);
-    else launch_bwd_t<64, 2>(ctx, batch, IN, io, n_nets);
+    FwdLoss fl{};
+    if (fused != nullptr) {
+        fl = *fused;
+        fl.enabled = 1;
+        fused = &fl;
+    }
+    if (H == 256 && act == 1) launch_bwd_t<256, 1>(ctx, batch, IN, io, n_nets, fused);
+    else if (H == 256) launch_bwd_t<256, 2>(ctx, batch, IN, io, n_nets, fused);
+    else if (act == 1) launch_bwd_t<64, 1>(ctx, batch, IN, io, n_nets, fused);
+    else launch_bwd_t<64, 2>(ctx, batch, IN, io, n_nets, fused);
     MRL_CHECK_LAUNCH();
     DwSet dw;
     dw.n = n_nets;   // the H x H layer of each net; the thin layers come out of the dx kernel

@@ -343,9 +343,10 @@ static int update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *in
     Mlp3Nets io{};
     io.n[0].x = u->mb_obs; io.n[0].params = u->actor_params; io.n[0].out = u->actor_out; io.n[0].cache = u->actor_cache;
     io.n[1].x = u->mb_obs; io.n[1].params = u->critic_params; io.n[1].out = u->values; io.n[1].cache = u->critic_cache;
+    FwdLoss fl{};
     if (paired) {
-        // forward of both nets straight from the rollout rows, loss gradients and KL test in its tail
-        FwdLoss fl{};
+        // both nets go forward straight from the rollout rows, on to their loss gradients and the KL
+        // test and back again in one launch per row tile (mlp3_backward_n below)
         fl.idx = indices;
         fl.r_obs = u->r_obs; fl.r_act = u->r_actions; fl.r_adv = u->advantages; fl.r_ret = u->returns;
         fl.r_logp = u->r_log_probs; fl.r_val = u->r_values;
@@ -358,8 +359,6 @@ static int update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *in
         fl.clip_value = u->clip_value ? 1 : 0;
         fl.clip_eps = u->clip_epsilon; fl.ent_coef = u->entropy_coef; fl.value_coef = u->value_loss_coef;
         fl.target_kl = u->target_kl;
-        rc = mlp3_forward_n(ctx, descs, 2, mb, io, &fl);
-        if (rc) return rc;
     } else {
         rc = mrl_mlp_forward(ctx, &u->actor, mb, u->mb_obs, u->actor_params, u->actor_out, u->actor_cache);
         if (rc) return rc;
@@ -392,7 +391,7 @@ static int update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *in
         rc = mlp_ensure_ws(ctx, mlp3_backward_ws(descs, 2, mb), &ws);
         if (rc) return rc;
         rc = mlp3_backward_n(ctx, descs, 2, mb, io, grads, ws,
-                             u->max_grad_norm > 0.0f ? ctx->upd_scratch + 2048 : nullptr, &sq_blocks);
+                             u->max_grad_norm > 0.0f ? ctx->upd_scratch + SCR_SQ : nullptr, &sq_blocks, &fl);
         if (rc) return rc;
     } else {
         rc = mrl_mlp_backward(ctx, &u->actor, mb, u->g_actor_out, u->actor_params, u->actor_cache, u->actor_grads,
