@@ -393,6 +393,29 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
     }
     stage_head(params + IN * H + H + H * H + H, H, A, GAUSS, w2s, t, T);
     for (int i = t; i < PR * (2 * PA_MAX + 1); i += T) g2s[i] = 0.0f;
+    // the loss lane of row t (wavefront 0) asks for its row's rollout entries now
+    const bool loss_lane = t < nrow;
+    const long src = loss_lane ? fl.idx[row0 + t] : 0;
+    float l_adv = 0.0f, l_logp = 0.0f, l_ret = 0.0f, l_val = 0.0f, l_mean = 0.0f, l_std = 1.0f, l_act[PA_MAX];
+#pragma unroll
+    for (int j = 0; j < PA_MAX; ++j) l_act[j] = 0.0f;
+    if (loss_lane) {
+        if (blockIdx.y == 1) {
+            l_ret = fl.r_ret[src];
+            if (fl.clip_value) l_val = fl.r_val[src];
+        } else {
+            l_adv = fl.r_adv[src];
+            l_logp = fl.r_logp[src];
+            if (fl.adv_stats != nullptr) { l_mean = fl.adv_stats[0]; l_std = fl.adv_stats[1]; }
+            if (fl.continuous) {
+#pragma unroll
+                for (int j = 0; j < PA_MAX; ++j)
+                    if (j < A) l_act[j] = fl.r_act[src * A + j];
+            } else {
+                l_act[0] = fl.r_act[src];
+            }
+        }
+    }
 #pragma unroll
     for (int q = 0; q < NX; ++q) {
         const int i = t + q * T;
@@ -431,30 +454,24 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
 
     // ---- loss gradients of the tile's rows, one lane per row (wavefront 0), into g2s and out
     float kl = 0.0f;
-    if (t < nrow) {
+    if (loss_lane) {
         const int b = (int)row0 + t;
-        const long src = fl.idx[b];
         float *g2row = g2s + t * (2 * PA_MAX + 1);
         if (blockIdx.y == 1) {   // critic
-            const float g = critic_grad_value(ys[t * (PA_MAX + 1)], fl.clip_value ? fl.r_val[src] : 0.0f, fl.r_ret[src],
-                                              fl.mb, fl.continuous, fl.clip_value, fl.value_coef, fl.clip_eps);
+            const float g = critic_grad_value(ys[t * (PA_MAX + 1)], l_val, l_ret, fl.mb, fl.continuous, fl.clip_value,
+                                              fl.value_coef, fl.clip_eps);
             g2row[0] = g;
             fl.g_values[b] = g;
         } else {
-            float adv = fl.r_adv[src];
-            if (fl.adv_stats != nullptr) adv = (adv - fl.adv_stats[0]) / (fl.adv_stats[1] + 1e-8f);
-            const float old_logp = fl.r_logp[src];
+            float adv = l_adv;
+            if (fl.adv_stats != nullptr) adv = (adv - l_mean) / (l_std + 1e-8f);
             float o[2 * PA_MAX], g[2 * PA_MAX];
             for (int a = 0; a < A; ++a) o[a] = ys[t * (PA_MAX + 1) + a];
             if (fl.continuous) {
-                float act[PA_MAX];
-                for (int j = 0; j < A; ++j) {
-                    o[A + j] = w2s[HEAD_LOG_STD(H) + j];   // clamped inside the gradient, as in the stored output
-                    act[j] = fl.r_act[src * A + j];
-                }
-                kl = actor_grad_gaussian_row(o, act, adv, old_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
+                for (int j = 0; j < A; ++j) o[A + j] = w2s[HEAD_LOG_STD(H) + j];   // clamped inside the gradient, as in the stored output
+                kl = actor_grad_gaussian_row(o, l_act, adv, l_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
             } else {
-                kl = actor_grad_discrete_row(o, (int)fl.r_act[src], adv, old_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
+                kl = actor_grad_discrete_row(o, (int)l_act[0], adv, l_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
             }
             for (int j = 0; j < ld; ++j) {
                 g2row[j] = g[j];
@@ -492,49 +509,52 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
     }
     __syncthreads();   // g2s complete
 
-    // ---- back through the head and layer 1's activation
-    if (t < H) {   // g1[r][n] = (sum_a g2[r][a] W2[n][a]) * act'(layer 1); thread t owns column n = t
-        float w2row[PA_MAX];
+    // ---- back through the head and layer 1's activation, on the matrix cores; wavefront w owns
+    // columns [32w, 32w + 32) of the hidden layers throughout
+    {   // g1[r][n] = (sum_a g2[r][a] W2[n][a]) * act'(layer 1): K = PA_MAX (W2 rows are zero beyond A)
+        floatx16 c = {0};
 #pragma unroll
-        for (int a = 0; a < PA_MAX; ++a) w2row[a] = w2s[t * PA_MAX + a];   // zero beyond A
+        for (int kk = 0; kk < PA_MAX / 2; ++kk) {
+            const int k = 2 * kk + half;
+            c = __builtin_amdgcn_mfma_f32_32x32x2f32(g2s[l31 * (2 * PA_MAX + 1) + k], w2s[col * PA_MAX + k], c, 0, 0, 0);
+        }
         float colsum = 0.0f;
 #pragma unroll
-        for (int r = 0; r < PR; ++r) {
-            float s = 0.0f;
-#pragma unroll
-            for (int a = 0; a < PA_MAX; ++a)
-                if (a < A) s = fmaf(g2s[r * (2 * PA_MAX + 1) + a], w2row[a], s);
+        for (int v = 0; v < 16; ++v) {
+            const int row = 8 * (v >> 2) + 4 * half + (v & 3);
             float g = 0.0f;
-            if (r < nrow) {
-                g = s * act_deriv_out<ACT>(h2[r * (H + 1) + t]);
-                g1[(row0 + r) * H + t] = g;
+            if (row < nrow) {
+                g = c[v] * act_deriv_out<ACT>(h2[row * (H + 1) + col]);
+                g1[(row0 + row) * H + col] = g;
             }
-            gT[t * HT_LD + r] = g;
+            gT[col * HT_LD + row] = g;
             colsum += g;
         }
-        db_part[H + t] = colsum;   // bias gradient of layer 1, this tile's rows
-    } else {       // meanwhile the other half of the block: dW2[n][a] of the tile = sum_r h2[r][n] g2[r][a]
-        const int n = t - H;
-        float s[PA_MAX];
+        colsum += __shfl_xor(colsum, 32, 64);
+        if (half == 0) db_part[H + col] = colsum;   // bias gradient of layer 1, this tile's rows
+    }
+    {   // dW2[n][a] of the tile = sum_r h2[r][n] g2[r][a]: K = the tile's 32 rows (g2 rows beyond nrow are zero)
+        floatx16 c = {0};
 #pragma unroll
-        for (int a = 0; a < PA_MAX; ++a) s[a] = 0.0f;
-#pragma unroll
-        for (int r = 0; r < PR; ++r) {
-            const float h = r < nrow ? h2[r * (H + 1) + n] : 0.0f;
-#pragma unroll
-            for (int a = 0; a < PA_MAX; ++a)
-                if (a < A) s[a] = fmaf(h, g2s[r * (2 * PA_MAX + 1) + a], s[a]);
+        for (int kk = 0; kk < PR / 2; ++kk) {
+            const int r = 2 * kk + half;
+            const float gb = l31 < 2 * PA_MAX ? g2s[r * (2 * PA_MAX + 1) + l31] : 0.0f;
+            c = __builtin_amdgcn_mfma_f32_32x32x2f32(h2[r * (H + 1) + col], gb, c, 0, 0, 0);
         }
-        float *o2 = thin_part + (size_t)IN * H + (size_t)n * A;
+        if (l31 < A) {
+            float *o2 = thin_part + (size_t)IN * H + l31;
 #pragma unroll
-        for (int a = 0; a < PA_MAX; ++a)
-            if (a < A) o2[a] = s[a];
-        if (n < ld) {   // column sums of the tile: bias gradient of the head, log_std gradient
-            float cs2 = 0.0f;
-            for (int r = 0; r < PR; ++r) cs2 += g2s[r * (2 * PA_MAX + 1) + n];
-            if (n < A) db_part[2 * H + n] = cs2;
-            else ls_part[(long)blockIdx.x * A + (n - A)] = cs2;
+            for (int v = 0; v < 16; ++v) {
+                const int n = 32 * w + 8 * (v >> 2) + 4 * half + (v & 3);
+                o2[(size_t)n * A] = c[v];
+            }
         }
+    }
+    if (t < ld) {   // column sums of the tile: bias gradient of the head, log_std gradient
+        float cs2 = 0.0f;
+        for (int r = 0; r < PR; ++r) cs2 += g2s[r * (2 * PA_MAX + 1) + t];
+        if (t < A) db_part[2 * H + t] = cs2;
+        else ls_part[(long)blockIdx.x * A + (t - A)] = cs2;
     }
     // ---- dh1 = g1 W1^T: wavefront w owns input columns [32w, 32w + 32); the next chunk of W1 is
     // fetched into registers while the matrix cores work on the current one
@@ -551,12 +571,28 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
         __syncthreads();
         if (o0 + KCH < H) fetch(o0 + KCH);
         __builtin_amdgcn_sched_barrier(0);   // keep the loads ahead of the MFMAs that hide them
+        // operands of eight k-steps are read from LDS while the previous eight are multiplied
+        constexpr int G = 8;
+        float a[G], b[G], na[G], nb[G];
 #pragma unroll
-        for (int kk = 0; kk < KCH / 2; ++kk) {
-            const int k = 2 * kk + half;
-            const float a = gT[(o0 + k) * HT_LD + l31];
-            const float b = wT[k * (H + 1) + col];
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+        for (int j = 0; j < G; ++j) {
+            a[j] = gT[(o0 + 2 * j + half) * HT_LD + l31];
+            b[j] = wT[(2 * j + half) * (H + 1) + col];
+        }
+#pragma unroll
+        for (int g = 0; g < KCH / 2 / G; ++g) {
+            if (g + 1 < KCH / 2 / G) {
+#pragma unroll
+                for (int j = 0; j < G; ++j) {
+                    const int k = 2 * ((g + 1) * G + j) + half;
+                    na[j] = gT[(o0 + k) * HT_LD + l31];
+                    nb[j] = wT[k * (H + 1) + col];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < G; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[j], acc, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < G; ++j) { a[j] = na[j]; b[j] = nb[j]; }
         }
     }
     float cs = 0.0f;
