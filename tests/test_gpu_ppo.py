@@ -576,3 +576,81 @@ def test_update_driver_runs_epochs_and_stops_on_kl(mrl, ctx):
     upd2.minibatch_step(upd2.indices[:MB])
     ctx.synchronize()
     assert torch.equal(frozen, anet.params)
+
+
+@pytest.mark.parametrize("env_name,kind,MB", [("LunarLanderV2", "relu", 4096), ("LunarLanderV2", "tanh", 1000),
+                                              ("HalfCheetahPlanarV2", "tanh", 777)])
+def test_fused_update_minibatch_equals_its_parts(mrl, ctx, env_name, kind, MB):
+    """mrl_ppo_update_minibatch on nets of hidden width 256 (one kernel takes a row tile forward,
+    through the loss and back) against the same minibatch issued call by call: gather,
+    normalise, forward with cache, loss gradients, backward, clip, Adam.  The fused kernel sums
+    in a different order, hence MLP tolerances on the gradients."""
+    say("case", env_name, kind, MB)
+    E = getattr(mrl, env_name)
+    cont = E.NUM_ACTIONS == 0
+    lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
+    A = E.ACTION_DIM if cont else E.NUM_ACTIONS
+    head = mrl.StochasticActor(256, A) if cont else mrl.Linear(256, A)
+    actor = mrl.seq(lin(E.OBS_DIM, 256), lin(256, 256), head)
+    critic = mrl.seq(lin(E.OBS_DIM, 256), lin(256, 256), mrl.Linear(256, 1))
+    N, T = 512, 8
+    g = torch.Generator(device="cuda").manual_seed(11)
+    rnd = lambda n, s=1.0: (torch.rand(n, device="cuda", generator=g) - 0.5) * 2 * s
+    rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N, T)
+    rb.actor_params, rb.critic_params = rnd(actor.PARAM_SIZE, 0.15), rnd(critic.PARAM_SIZE, 0.15)
+    total, aw = N * T, rb.act_width
+    rb.r_obs.copy_(rnd(total * E.OBS_DIM))
+    rb.r_actions.copy_(rnd(total * aw) if cont else torch.randint(0, A, (total,), device="cuda", generator=g).float())
+    rb.r_log_probs.copy_(rnd(total, 0.3) - (2.0 if cont else 1.2))
+    rb.r_values.copy_(rnd(total))
+    aopt, copt = mrl.Adam(lr=3e-4), mrl.Adam(lr=1e-3)
+    cls = mrl.ppo.ContinuousUpdate if cont else mrl.ppo.DiscreteUpdate
+    upd = cls(ctx, rb, MB, aopt, copt, target_kl=0.0)
+    upd.advantages.copy_(rnd(total, 2.0) + 0.3)
+    upd.returns.copy_(rnd(total))
+    idx = torch.randperm(total, device="cuda", generator=g)[:MB].to(torch.int32)
+    ap0, cp0 = rb.actor_params.clone(), rb.critic_params.clone()
+    upd.minibatch_step(idx)
+    ctx.synchronize()
+
+    # ---- the same minibatch, call by call, on copies
+    z = lambda n: torch.zeros(n, device="cuda")
+    hd = actor.OUT_DIM
+    mb = (z(MB * E.OBS_DIM), z(MB * aw), z(MB), z(MB), z(MB), z(MB))
+    mrl.ppo.gather_minibatch(ctx, idx, (rb.r_obs, rb.r_actions, upd.advantages, upd.returns, rb.r_log_probs, rb.r_values),
+                             mb, E.OBS_DIM, aw)
+    m_obs, m_act, m_adv, m_ret, m_lp, m_val = mb
+    mrl.ppo.normalize_advantages(ctx, m_adv)
+    a_out, vals = z(MB * hd), z(MB)
+    a_cache, c_cache = z(MB * actor.CACHE_SIZE), z(MB * critic.CACHE_SIZE)
+    actor.forward_gpu_ws(ctx, a_out, m_obs, ap0, a_cache)
+    critic.forward_gpu_ws(ctx, vals, m_obs, cp0, c_cache)
+    g_out, kl, g_val = z(MB * hd), z(MB), z(MB)
+    if cont:
+        mrl.ppo.ppo_continuous_actor_grad(ctx, g_out, kl, a_out, m_lp, m_adv, m_act, 0.2, 0.01)
+    else:
+        mrl.ppo.ppo_actor_grad_with_kl(ctx, g_out, kl, a_out, m_lp, m_adv, m_act, 0.2, 0.01)
+    mrl.ppo.ppo_critic_grad(ctx, g_val, vals, m_ret, 0.5, old_values=m_val, clip_epsilon=0.2, continuous=cont)
+    ga, gc = z(actor.PARAM_SIZE), z(critic.PARAM_SIZE)
+    actor.backward_gpu_ws(ctx, None, g_out, ap0, a_cache, ga)
+    critic.backward_gpu_ws(ctx, None, g_val, cp0, c_cache, gc)
+    mrl.ppo.clip_grad_norm(ctx, ga, 0.5)
+    mrl.ppo.clip_grad_norm(ctx, gc, 0.5)
+    ap1, cp1 = ap0.clone(), cp0.clone()
+    mrl.Adam(lr=3e-4).step_gpu(ctx, ap1, ga, z(2 * actor.PARAM_SIZE))
+    mrl.Adam(lr=1e-3).step_gpu(ctx, cp1, gc, z(2 * critic.PARAM_SIZE))
+    if cont:
+        mrl.ppo.clamp_log_std_params(ctx, ap1, actor.PARAM_SIZE - A, A)
+    ctx.synchronize()
+
+    torch.testing.assert_close(upd.actor_out, a_out, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(upd.values, vals, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(upd.kl, kl, rtol=1e-3, atol=1e-5)
+    torch.testing.assert_close(upd.g_actor_out, g_out, rtol=1e-3, atol=1e-7)
+    torch.testing.assert_close(upd.g_values, g_val, rtol=1e-3, atol=1e-8)
+    scale = lambda t: float(t.abs().max())
+    torch.testing.assert_close(upd.actor_grads, ga, rtol=2e-3, atol=2e-4 * scale(ga))
+    torch.testing.assert_close(upd.critic_grads, gc, rtol=2e-3, atol=2e-4 * scale(gc))
+    # Adam's first step moves every parameter by about lr; both paths must agree on the sign and size
+    torch.testing.assert_close(rb.actor_params - ap0, ap1 - ap0, rtol=0.0, atol=0.05 * 3e-4)
+    torch.testing.assert_close(rb.critic_params - cp0, cp1 - cp0, rtol=0.0, atol=0.05 * 1e-3)
