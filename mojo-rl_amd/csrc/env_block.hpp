@@ -50,6 +50,8 @@ struct LunarLander {
                              float &r, float &d) {
         ll::step_row(row, cts, shapes, env, (int)a[0], r, d);
     }
+    static constexpr int POST_TASKS = 0;
+    static MRL_DEV void post_task(float *, int) {}
     static MRL_DEV void reset(float *row, uint64_t seed, int env) {
         ll::reset_row(row, ll::combined_seed(seed, env));
     }
@@ -77,13 +79,19 @@ struct BipedalWalker {
     using L = bw::L;
     static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 32, THREADS = 256;
     static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = bw::NSHAPE_FLOATS;
+    // the ten lidar rays of the observation are left out of the step and run afterwards, spread
+    // over all wavefronts of the block (task k = ray k)
+    static constexpr int POST_TASKS = 10;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
-        bw::step_row(row, cts, shapes, env, a, r, d);
+        bw::step_row<false>(row, cts, shapes, env, a, r, d);
     }
+    static MRL_DEV void post_task(float *row, int task) { row[14 + task] = bw::lidar_value(row, task, nullptr); }
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { bw::reset_row(row, walker_seed(seed, env)); }
-    static constexpr bool WAVE_RESET = false;
-    static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
+    static constexpr bool WAVE_RESET = true;
+    static MRL_DEV void reset_wave(float *row, uint64_t seed, int env, int lane) {
+        bw::reset_row_wave(row, walker_seed(seed, env), lane);
+    }
     static constexpr int DETECT_TASKS = 0;
     static MRL_DEV void detect_task(int, int &, int &, int &) {}
     struct Carry {};
@@ -99,6 +107,8 @@ struct HalfCheetah {
                              float &r, float &d) {
         hc::step_row(row, cts, shapes, env, a, r, d);
     }
+    static constexpr int POST_TASKS = 0;
+    static MRL_DEV void post_task(float *, int) {}
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { hc::reset_row(row, walker_seed(seed, env)); }
     static constexpr bool WAVE_RESET = false;
     static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
@@ -215,6 +225,26 @@ MRL_DEV void reset_rows(float *rows, unsigned long long *was_reset, unsigned lon
     }
 }
 
+// The same with every wavefront of the block taking part (all threads call it): wavefront w
+// rebuilds the rows whose rank among the set bits is w modulo the number of wavefronts.
+template <class E>
+MRL_DEV void reset_rows_block(float *rows, unsigned long long mask, uint64_t seed, int env0, int tid) {
+    using S = Stage<E>;
+    constexpr int NW = E::THREADS / 64;
+    const int wave = tid / 64, lane = tid % 64;
+    if (E::WAVE_RESET && __popcll(mask) <= 8 * NW) {
+        int rank = 0;
+        while (mask) {
+            const int src = __ffsll((long long)mask) - 1;
+            mask &= mask - 1;
+            if (rank % NW == wave) E::reset_wave(rows + src * S::STRIDE, seed, env0 + src, lane);
+            ++rank;
+        }
+    } else if (wave == 0 && ((mask >> lane) & 1ull)) {
+        E::reset(rows + lane * S::STRIDE, seed, env0 + lane);
+    }
+}
+
 // Per-(body, vertex) contact lists of phys_step_block: DCAP records per list (a vertex that fills
 // its list sends the env back to detection inside step_finish), list stride in floats.
 constexpr int DETECT_CAP = 4;
@@ -310,7 +340,23 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
                 account(acc, env - env0, r, d, sums);
                 finished = d > 0.5f;
             }
-            if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, tid);
+            if (E::POST_TASKS > 0) {
+                const unsigned long long fin = __ballot(finished);
+                if (tid == 0) *was_reset = AUTORESET ? fin : 0ull;
+            } else if (AUTORESET) {
+                reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, tid);
+            }
+        }
+        if constexpr (E::POST_TASKS > 0) {
+            // what the step left for afterwards (rows that finished get it from their reset instead),
+            // then the resets, both by all wavefronts
+            __syncthreads();
+            const unsigned long long fin = *was_reset;
+            constexpr int SLOTS = E::THREADS / E::EPB;   // tasks in flight per env
+            const int e = tid % E::EPB;
+            if (e < nenv && !((fin >> e) & 1ull))
+                for (int task = tid / E::EPB; task < E::POST_TASKS; task += SLOTS) E::post_task(rows + e * S::STRIDE, task);
+            if (AUTORESET) reset_rows_block<E>(rows, fin, reset_seed, env0, tid);
         }
     }
 }

@@ -81,10 +81,10 @@ inline Shapes make_shapes() {
     return s;
 }
 
-MRL_DEV void observe(float *row) {
+// observation entries 0 .. 13: hull and joint state, leg contact flags
+MRL_DEV void observe_state(const float *row, float *o) {
     const float *B = row + L::BODIES_OFF;
     double hull_angle = B[IDX_ANGLE], hull_omega = B[IDX_OMEGA], hull_vx = B[IDX_VX], hull_vy = B[IDX_VY];
-    float o[OBS];
     o[0] = (float)hull_angle;
     o[1] = (float)(hull_omega / 5.0);
     o[2] = (float)(hull_vx * (600.0 / SCALE) / FPS);
@@ -100,20 +100,33 @@ MRL_DEV void observe(float *row) {
         q[3] = (float)((lo - uo) / 10.0);
         q[4] = row[L::META_OFF + (leg ? META_RIGHT : META_LEFT)] > 0.5f ? 1.0f : 0.0f;
     }
+}
+
+// observation entry 14 + i: lidar ray i of ten.  near != nullptr: the edges within lidar range of
+// the hull in x, selected by the caller once for all its rays (every ray stays within that range)
+MRL_DEV float lidar_value(const float *row, int i, const EdgeMask<L> *near) {
+    const float *B = row + L::BODIES_OFF;
     const float hull_x = B[IDX_X], hull_y = B[IDX_Y], hull_angle_rad = B[IDX_ANGLE];
     const float lidar_range = (float)LIDAR_RANGE;
-    // every ray stays within lidar_range of the hull in x: select those edges once for the ten rays
+    float local_angle = (float)i * 1.5f / (float)9;
+    float world_angle = hull_angle_rad - local_angle - (float)(3.14159265358979323846 / 2.0);
+    float sn, cs;
+    sincos32(world_angle, sn, cs);
+    if (!(hull_x == hull_x)) return lidar_ray<L>(row, hull_x, hull_y, cs * lidar_range, sn * lidar_range);
+    if (near != nullptr) return lidar_ray_near<L>(row, *near, hull_x, hull_y, cs * lidar_range, sn * lidar_range);
+    EdgeMask<L> mine;
+    edges_near<L>(row, hull_x - lidar_range, hull_x + lidar_range, 0.02f, mine);
+    return lidar_ray_near<L>(row, mine, hull_x, hull_y, cs * lidar_range, sn * lidar_range);
+}
+
+MRL_DEV void observe(float *row) {
+    float o[OBS];
+    observe_state(row, o);
+    const float hull_x = row[L::BODIES_OFF + IDX_X], lidar_range = (float)LIDAR_RANGE;
     EdgeMask<L> near;
     const bool plain = !(hull_x == hull_x);
     if (!plain) edges_near<L>(row, hull_x - lidar_range, hull_x + lidar_range, 0.02f, near);
-    for (int i = 0; i < 10; ++i) {
-        float local_angle = (float)i * 1.5f / (float)9;
-        float world_angle = hull_angle_rad - local_angle - (float)(3.14159265358979323846 / 2.0);
-        float sn, cs;
-        sincos32(world_angle, sn, cs);
-        o[14 + i] = plain ? lidar_ray<L>(row, hull_x, hull_y, cs * lidar_range, sn * lidar_range)
-                          : lidar_ray_near<L>(row, near, hull_x, hull_y, cs * lidar_range, sn * lidar_range);
-    }
+    for (int i = 0; i < 10; ++i) o[14 + i] = lidar_value(row, i, &near);
 #pragma unroll
     for (int k = 0; k < OBS; ++k) row[k] = o[k];
 }
@@ -167,6 +180,101 @@ MRL_DEV void reset_row(float *row, uint64_t cseed) {
     row[L::META_OFF + META_PREV_SHAPING] = (float)(130.0 * hull_x / SCALE);
 }
 
+MRL_DEV void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// reset_row by the 64 lanes of a wavefront together (all lanes call it with the same row): the
+// Philox draws of the terrain walk, the edges, the bodies / joints and the observation's lidar
+// rays are spread over the lanes; the walk itself, a recursion through sign(height - y), stays on
+// one lane.  Every value comes from the expressions of reset_row, so the row is bit-identical.
+MRL_DEV void reset_row_wave(float *row, uint64_t cseed, int lane) {
+    for (int k = lane; k < STATE; k += 64) row[k] = 0.0f;
+    wave_sync();
+    // parked in the (still unused) edge area: the noise of terrain step i at [i], the height y_i at [YS + i]
+    float *tmp = row + L::EDGES_OFF;
+    constexpr int YS = 200;
+    static_assert(YS + N_EDGES + 1 <= N_EDGES * 6 && N_EDGES + 1 <= YS, "scratch inside the edge area");
+    for (int i = TERRAIN_STARTPAD + 1 + lane; i <= N_EDGES; i += 64) {
+        Uniform4 rv = philox_uniform4(cseed + 1000ull, 0, (uint64_t)(i - TERRAIN_STARTPAD - 1));
+        tmp[i] = (rv.v[0] * 2.0f - 1.0f) / (float)SCALE;
+    }
+    wave_sync();
+    if (lane == 0) {
+        float y = (float)TERRAIN_HEIGHT, velocity = 0.0f;
+        for (int i = 0; i <= N_EDGES; ++i) {
+            const float terrain_height = (float)TERRAIN_HEIGHT;
+            velocity = 0.8f * velocity + 0.01f * (terrain_height > y ? 1.0f : -1.0f);
+            if (i > TERRAIN_STARTPAD) velocity = velocity + tmp[i];
+            y = y + velocity;
+            tmp[YS + i] = y;
+        }
+    }
+    wave_sync();
+    float ya[2], yb[2];   // this lane's edges lane and lane + 64: heights at both ends
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int i = lane + 64 * q + 1;
+        ya[q] = tmp[YS + i - 1];
+        yb[q] = tmp[YS + i];
+    }
+    wave_sync();   // all heights read before the first edge overwrites the scratch
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int i = lane + 64 * q + 1;
+        float x0 = (float)(i - 1) * (float)TERRAIN_STEP, x1 = (float)i * (float)TERRAIN_STEP;
+        float y0 = ya[q], y1 = yb[q];
+        float dx = x1 - x0, dy = y1 - y0;
+        float length = sqrtf(dx * dx + dy * dy);
+        float nx = -dy / length, ny = dx / length;
+        if (ny < 0.0f) { nx = -nx; ny = -ny; }
+        float *E = row + L::EDGES_OFF + (i - 1) * 6;
+        E[0] = x0; E[1] = y0; E[2] = x1; E[3] = y1; E[4] = nx; E[5] = ny;
+    }
+    static_assert(N_EDGES == 128, "two edges per lane");
+    Uniform4 rv = philox_uniform4(cseed, 0, 0);
+    const double init_x = (double)TERRAIN_STARTPAD * TERRAIN_STEP;
+    const double init_y = TERRAIN_HEIGHT + 2.0 * LEG_H;
+    const double init_vx = ((double)rv.v[0] * 2.0 - 1.0) * 0.1, init_vy = ((double)rv.v[1] * 2.0 - 1.0) * 0.1;
+    float *B = row + L::BODIES_OFF;
+    if (lane == 0) {
+        row[L::EDGE_COUNT_OFF] = (float)N_EDGES;
+        row[L::JOINT_COUNT_OFF] = 4.0f;
+        w_set_body(B, init_x, init_y, init_vx, init_vy, 1.0 / 5.0, 1.0 / 2.0, 0);
+    }
+    if (lane == 1 || lane == 2) {
+        const int leg = lane - 1;
+        double upper_y = init_y + LEG_DOWN - UPPER_H / 2;
+        w_set_body(B + (2 * leg + 1) * BODY_SIZE, init_x, upper_y, init_vx, init_vy, 1.0 / 0.8, 1.0 / 0.1, 2 * leg + 1);
+        double lower_y = upper_y - UPPER_H / 2 - LOWER_H / 2;
+        w_set_body(B + (2 * leg + 2) * BODY_SIZE, init_x, lower_y, init_vx, init_vy, 1.0 / 0.5, 1.0 / 0.05, 2 * leg + 2);
+    }
+    if (lane == 3 || lane == 4) {
+        const int leg = lane - 3;
+        float *J = row + L::JOINTS_OFF + (2 * leg) * JOINT_SIZE;
+        w_set_motor_joint(J, 0, 2 * leg + 1, 0.0, LEG_DOWN, 0.0, UPPER_H / 2, -0.8, 1.1, MOTORS_TORQUE);
+        w_set_motor_joint(J + JOINT_SIZE, 2 * leg + 1, 2 * leg + 2, 0.0, -UPPER_H / 2, 0.0, LOWER_H / 2, -1.6, -0.1,
+                          MOTORS_TORQUE);
+    }
+    wave_sync();
+    // observation: lanes 0 .. 9 one lidar ray each, lane 10 the rest
+    if (lane < 10) {
+        row[14 + lane] = lidar_value(row, lane, nullptr);
+    } else if (lane == 10) {
+        float o[14];
+        observe_state(row, o);
+#pragma unroll
+        for (int k = 0; k < 14; ++k) row[k] = o[k];
+        double hull_x = B[IDX_X];
+        row[L::META_OFF + META_PREV_SHAPING] = (float)(130.0 * hull_x / SCALE);
+    }
+    wave_sync();
+}
+
+// LIDAR = false: the lidar entries of the observation (14 .. 23) are left to the caller
+template <bool LIDAR = true>
 MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env, const float *action,
                       float &reward, float &done) {
     (void)env;
@@ -197,7 +305,14 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
     if (hull) M[META_GAME_OVER] = 1.0f;
     const float *B = row + L::BODIES_OFF;
     M[META_SCROLL] = B[IDX_X] - (float)(600.0 / SCALE / 5.0);
-    observe(row);
+    if (LIDAR) {
+        observe(row);
+    } else {
+        float o[14];
+        observe_state(row, o);
+#pragma unroll
+        for (int k = 0; k < 14; ++k) row[k] = o[k];
+    }
 
     int step_count = (int)M[META_STEP] + 1;
     double hull_x = B[IDX_X], hull_y = B[IDX_Y], hull_angle = B[IDX_ANGLE];
