@@ -132,38 +132,39 @@ struct Stage {
     static constexpr int UNROLL = 8;
 
     static MRL_DEV void in(float *lds, const float *g, int nenv, int lane) {
-        if (E::STATE % 4 == 0) {   // rows are whole float4s, never straddled by a 16-byte load
-            const float4 *src = reinterpret_cast<const float4 *>(g);
-            const int total4 = nenv * (E::STATE / 4);
-            for (int i0 = lane; i0 < total4; i0 += UNROLL * E::THREADS) {
-                float4 v[UNROLL];
+        // The block's rows are one contiguous run that starts on a 16-byte boundary (EPB rows are a
+        // multiple of 16 bytes), so it is read with 16-byte loads whatever STATE is; a load may
+        // straddle two rows, each float finds its own (row, column).
+        static_assert((E::EPB * E::STATE) % 4 == 0, "a block's rows start 16-byte aligned");
+        const int total = nenv * E::STATE;
+        const int total4 = total / 4;
+        const float4 *src = reinterpret_cast<const float4 *>(g);
+        for (int i0 = lane; i0 < total4; i0 += UNROLL * E::THREADS) {
+            float4 v[UNROLL];
 #pragma unroll
-                for (int k = 0; k < UNROLL; ++k)
-                    if (i0 + k * E::THREADS < total4) v[k] = src[i0 + k * E::THREADS];
+            for (int k = 0; k < UNROLL; ++k)
+                if (i0 + k * E::THREADS < total4) v[k] = src[i0 + k * E::THREADS];
 #pragma unroll
-                for (int k = 0; k < UNROLL; ++k) {
-                    if (i0 + k * E::THREADS >= total4) continue;
-                    const int f = (i0 + k * E::THREADS) * 4;
+            for (int k = 0; k < UNROLL; ++k) {
+                if (i0 + k * E::THREADS >= total4) continue;
+                const int f = (i0 + k * E::THREADS) * 4;
+                const float e[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+                if (E::STATE % 4 == 0) {   // never straddles
                     const int r = f / E::STATE, c = f - r * E::STATE;
                     float *d = lds + r * STRIDE + c;
-                    d[0] = v[k].x; d[1] = v[k].y; d[2] = v[k].z; d[3] = v[k].w;
+                    d[0] = e[0]; d[1] = e[1]; d[2] = e[2]; d[3] = e[3];
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int r = (f + j) / E::STATE, c = (f + j) - r * E::STATE;
+                        lds[r * STRIDE + c] = e[j];
+                    }
                 }
             }
-        } else {
-            const int total = nenv * E::STATE;
-            for (int i0 = lane; i0 < total; i0 += UNROLL * E::THREADS) {
-                float v[UNROLL];
-#pragma unroll
-                for (int k = 0; k < UNROLL; ++k)
-                    if (i0 + k * E::THREADS < total) v[k] = g[i0 + k * E::THREADS];
-#pragma unroll
-                for (int k = 0; k < UNROLL; ++k) {
-                    const int i = i0 + k * E::THREADS;
-                    if (i >= total) continue;
-                    const int r = i / E::STATE, c = i - r * E::STATE;
-                    lds[r * STRIDE + c] = v[k];
-                }
-            }
+        }
+        for (int i = total4 * 4 + lane; i < total; i += E::THREADS) {   // at most three floats
+            const int r = i / E::STATE, c = i - r * E::STATE;
+            lds[r * STRIDE + c] = g[i];
         }
     }
 
