@@ -3,9 +3,13 @@
 // call that only enqueues: gather, per-minibatch advantage normalisation, actor and critic
 // forward, loss gradients, KL test, backward, global-norm clip, Adam (and the log_std clamp).
 // The actor and the critic do not depend on each other inside a minibatch, so when both have one
-// of the fused shapes every stage runs them side by side in ONE launch: 7 launches per
-// minibatch (gather + normalise, forward, loss gradients + KL test, backward dx, dW, sum,
-// clip + Adam) instead of about 40, and twice the workgroups per launch.
+// of the fused shapes they run side by side in every launch, and a row tile never leaves its
+// workgroup between the forward pass and the way back: 4 launches per minibatch (forward + loss
+// gradients + KL test + backward dx; dW; sum; clip + Adam) instead of about 40.  The minibatch is
+// not gathered: the forward reads its rows from the rollout through the indices and the loss
+// normalises the advantage with statistics computed ahead (once per epoch for all minibatches).
+// Other net shapes go layer by layer: gather + normalise, forward, loss gradients + KL test,
+// backward, clip + Adam.
 //
 // KL early stop: the reference copies the per-sample KL to the host after the actor's loss
 // gradient and breaks out of the minibatch and epoch loops when its mean exceeds target_kl.
