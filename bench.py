@@ -179,7 +179,10 @@ def main():
         launch_us = ph_us["collect"]
         steps_per_launch = T / max(phases["collect"][1], 1)
         tflops = FWD_FLOPS * N_ENVS * steps_per_launch / (launch_us * 1e-6) / 1e12
-        name = "mrl::collect_kernel<mrl::%s, %d, %d, false>" % (env_name.replace("V2", ""), HIDDEN, 1 if ACT == "relu" else 2)
+        act_id = 1 if ACT == "relu" else 2
+        name = {"lunarlander": "mrl::collect_kernel<mrl::LunarLander, %d, %d, false>" % (HIDDEN, act_id),
+                "cartpole": "mrl::collect_classic_kernel<mrl::CartPoleSlot, %d, false>" % act_id,
+                "pendulum": "mrl::collect_classic_kernel<mrl::PendulumSlot, %d, true>" % act_id}[args.workload]
         roofline = {"kernel": name + " (policy forward + sampling + env step + auto-reset + rollout stores, %d steps per launch)" % steps_per_launch,
                     "bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": traffic.get(name),

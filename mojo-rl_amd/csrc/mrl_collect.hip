@@ -26,6 +26,7 @@
 #include "mlp_tile.hpp"
 #include "policy_sample.hpp"
 #include "env_block.hpp"
+#include "env_classic.hpp"
 
 namespace mrl {
 
@@ -207,19 +208,158 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     S::out(rows, gbase, nenv, t, 0, E::STATE);
 }
 
+// ---------------------------------------------------------------- CartPole / Pendulum
+// The same idea for the envs whose state is a handful of floats: a workgroup of two wavefronts
+// (actor on one, critic on the other, hidden width 64) takes its 32 envs through all the steps
+// of the launch; lanes 0 .. 31 of wavefront 0 carry one env each in registers -- state, step
+// counter, episode sums -- and do sampling, step, accounting and reset in place.
+struct CartPoleSlot {
+    static constexpr int OBS = cartpole::OBS, ACT_W = 1;
+    float s[4];
+    int32_t steps;
+    MRL_DEV void load(const float *states, const int32_t *side, int i) {
+        const float4 v = reinterpret_cast<const float4 *>(states)[i];
+        s[0] = v.x; s[1] = v.y; s[2] = v.z; s[3] = v.w;
+        steps = side[i];
+    }
+    MRL_DEV void store(float *states, int32_t *side, int i) const {
+        reinterpret_cast<float4 *>(states)[i] = make_float4(s[0], s[1], s[2], s[3]);
+        side[i] = steps;
+    }
+    MRL_DEV float obs(int k) const { return s[k]; }
+    MRL_DEV void step(const float *act, float &r, float &d) { cartpole::step(s, steps, (int)act[0], r, d); }
+    MRL_DEV void reset(int i, uint64_t seed) { cartpole::reset(s, steps, i, (uint32_t)seed); }
+};
+struct PendulumSlot {
+    static constexpr int OBS = pendulum::OBS, ACT_W = 1;
+    float s[8];
+    MRL_DEV void load(const float *states, const int32_t *, int i) {
+        const float4 *row = reinterpret_cast<const float4 *>(states) + 2 * (size_t)i;
+        const float4 a = row[0], b = row[1];
+        s[0] = a.x; s[1] = a.y; s[2] = a.z; s[3] = a.w; s[4] = b.x; s[5] = b.y; s[6] = b.z; s[7] = b.w;
+    }
+    MRL_DEV void store(float *states, int32_t *, int i) const {
+        float4 *row = reinterpret_cast<float4 *>(states) + 2 * (size_t)i;
+        row[0] = make_float4(s[0], s[1], s[2], s[3]);
+        row[1] = make_float4(s[4], s[5], s[6], s[7]);
+    }
+    MRL_DEV float obs(int k) const { return s[k]; }
+    MRL_DEV void step(const float *act, float &r, float &d) { pendulum::step(s, act[0], r, d); }
+    MRL_DEV void reset(int i, uint64_t seed) { pendulum::reset(s, i, seed); }
+};
+
+template <class C, int ACT, bool GAUSS>
+__global__ __launch_bounds__(128) void collect_classic_kernel(CollectArgs a, int32_t *side) {
+    constexpr int H = 64, TPW = 2, TN = hidden_threads(H, TPW), IN = C::OBS, AW = C::ACT_W;
+    static_assert(TN == 64 && IN <= PIN_MAX, "one wavefront per net");
+    __shared__ float xs[PR * XS_LD];
+    __shared__ float hT[2][H * HT_LD];
+    __shared__ float h2[2][PR * (H + 1)];
+    __shared__ float logits[PR * (PA_MAX + 1)];
+    __shared__ float vals[PR];
+    __shared__ __align__(16) float w2s[2][HEAD_LDS(H)];
+    const int t = threadIdx.x;
+    const int env0 = blockIdx.x * PR;
+    const int nenv = min(PR, a.n_envs - env0);
+    const int N = a.n_envs;
+    const bool owner = t < nenv;   // lanes 0 .. nenv - 1 of wavefront 0: one env each
+    C slot{};
+    float ep_return = 0.0f, ep_length = 0.0f;
+    if (owner) {
+        slot.load(a.states, side, env0 + t);
+        ep_return = a.acc.ep_return[env0 + t];
+        ep_length = a.acc.ep_length[env0 + t];
+    }
+    {
+        const int net = t / TN;
+        const float *p = net ? a.critic_p : a.actor_p;
+        stage_head(p + IN * H + H + H * H + H, H, net ? 1 : a.A, GAUSS && net == 0, w2s[net], t % TN, TN);
+    }
+    for (int i = t; i < PR * XS_LD; i += 128) xs[i] = 0.0f;
+    __syncthreads();
+
+    for (int k = 0; k < a.n_steps; ++k) {
+        // (the empty asm keeps what the optimiser derives from these values inside the step)
+        int tid = t, ne = __builtin_amdgcn_readfirstlane(nenv), A = __builtin_amdgcn_readfirstlane(a.A), zero = 0;
+        asm volatile("" : "+v"(tid), "+s"(zero), "+s"(ne), "+s"(A) : : "memory");
+        const int net = tid / TN;
+        const float *p = (net ? a.critic_p : a.actor_p) + zero;
+        const size_t row = (size_t)(a.t0 + k) * N + env0;   // this block's slice of rollout row t
+        const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
+        HiddenOperands<H, TPW, 8> ops;
+        ops.load(p, IN, tid);
+        if (tid < ne) {
+#pragma unroll
+            for (int c = 0; c < IN; ++c) {
+                const float v = slot.obs(c);
+                xs[tid * XS_LD + c] = v;
+                a.r_obs[(row + tid) * IN + c] = v;
+            }
+        }
+        __syncthreads();
+        hidden_stack<H, ACT, TPW, 8>(p, IN, xs, hT[net], h2[net], TileCache{}, ops, tid);
+        if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1, tid % H);
+        else head<H>(w2s[1], 1, h2[1], vals, 1, tid % H);
+        __syncthreads();
+        if (tid < ne) {
+            const int i = env0 + tid;
+            float av[PA_MAX], logp;
+            if (GAUSS) {
+                logp = sample_gaussian(logits + tid * (PA_MAX + 1), w2s[0] + HEAD_LOG_STD(H), A, sseed, i, av);
+                for (int j = 0; j < A; ++j) a.r_actions[(row + tid) * AW + j] = av[j];
+            } else {
+                int sel;
+                sample_categorical(logits + tid * (PA_MAX + 1), A, sseed, i, sel, logp);
+                av[0] = (float)sel;
+                a.r_actions[row + tid] = av[0];
+            }
+            a.r_logp[row + tid] = logp;
+            a.r_values[row + tid] = vals[tid];
+            float r, d;
+            slot.step(av, r, d);
+            a.r_rewards[row + tid] = r;
+            a.r_dones[row + tid] = d;
+            ep_return = ep_return + r;
+            ep_length = ep_length + 1.0f;
+            if (d > 0.5f) {
+                const int s = atomicAdd(a.acc.done_count, 1);
+                if (s < a.acc.done_cap) {
+                    a.acc.done_returns[s] = ep_return;
+                    a.acc.done_lengths[s] = ep_length;
+                }
+                ep_return = 0.0f;
+                ep_length = 0.0f;
+                slot.reset(i, a.reset_seed + (uint64_t)k * a.reset_stride);
+            }
+        }
+    }
+    if (owner) {
+        slot.store(a.states, side, env0 + t);
+#pragma unroll
+        for (int c = 0; c < IN; ++c) a.obs[(size_t)(env0 + t) * IN + c] = slot.obs(c);
+        a.acc.ep_return[env0 + t] = ep_return;
+        a.acc.ep_length[env0 + t] = ep_length;
+    }
+}
+
 // true when mrl_rollout_steps can run the descriptor through collect_kernel
+// (the wide kernel: LunarLander with hidden width 256; the two-wavefront kernel: CartPole and
+// Pendulum with hidden width 64)
 static bool collect_fusable(const mrl_rollout *r, bool gauss, int *act) {
-    if (r->env_id != MRL_ENV_LUNARLANDER || gauss) return false;
+    int obs, hidden;
+    if (r->env_id == MRL_ENV_LUNARLANDER && !gauss) { obs = LunarLander::OBS; hidden = 256; }
+    else if (r->env_id == MRL_ENV_CARTPOLE && !gauss) { obs = cartpole::OBS; hidden = 64; }
+    else if (r->env_id == MRL_ENV_PENDULUM && gauss) { obs = pendulum::OBS; hidden = 64; }
+    else return false;
     const mrl_mlp_desc &a = r->actor, &c = r->critic;
     if (a.n_layers != 3 || c.n_layers != 3) return false;
     const int k0 = a.layers[0].kind;
     if (k0 != MRL_LINEAR_RELU && k0 != MRL_LINEAR_TANH) return false;
     for (const mrl_mlp_desc *d : {&a, &c}) {
         if (d->layers[0].kind != k0 || d->layers[1].kind != k0) return false;
-        if (d->layers[0].in_dim != LunarLander::OBS || d->layers[0].out_dim != 256 || d->layers[1].out_dim != 256)
-            return false;
+        if (d->layers[0].in_dim != obs || d->layers[0].out_dim != hidden || d->layers[1].out_dim != hidden) return false;
     }
-    if (a.layers[2].kind != MRL_LINEAR || c.layers[2].kind != MRL_LINEAR) return false;
+    if (a.layers[2].kind != (gauss ? MRL_STOCHASTIC_ACTOR : MRL_LINEAR) || c.layers[2].kind != MRL_LINEAR) return false;
     if (a.layers[2].out_dim > PA_MAX || c.layers[2].out_dim != 1) return false;
     *act = (k0 == MRL_LINEAR_RELU) ? 1 : 2;
     return true;
@@ -257,24 +397,42 @@ int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, u
                       r->r_log_probs && r->r_values && r->r_rewards && r->r_dones && r->ep_return &&
                       r->ep_length && r->done_returns && r->done_lengths && r->done_count,
                   "mrl_rollout_steps: NULL buffer in descriptor");
-    MRL_CHECK_ARG(r->obs_dim == LunarLander::OBS && r->num_actions == 4 && mrl_mlp_out_dim(&r->actor) == 4,
+    int ss, od, na, ad;
+    int rc = mrl_env_dims(r->env_id, &ss, &od, &na, &ad);
+    if (rc) return rc;
+    MRL_CHECK_ARG(od == r->obs_dim && (gauss ? (ad > 0 && mrl_mlp_out_dim(&r->actor) == 2 * ad)
+                                             : (na == r->num_actions && mrl_mlp_out_dim(&r->actor) == na)),
                   "mrl_rollout_steps: descriptor does not match the env's observation / action space");
     const float *shapes = ctx->ll_shapes;
     CollectArgs a{};
     a.states = r->states; a.obs = r->obs;
     a.actor_p = r->actor_params; a.critic_p = r->critic_params; a.shapes = shapes;
-    a.n_envs = r->n_envs; a.A = r->num_actions; a.t0 = t0; a.n_steps = n_steps;
+    a.n_envs = r->n_envs; a.A = gauss ? ad : na; a.t0 = t0; a.n_steps = n_steps;
     a.sample_seed = sample_seed; a.sample_stride = sample_stride;
     a.reset_seed = reset_seed; a.reset_stride = reset_stride;
     a.r_obs = r->r_obs; a.r_actions = r->r_actions; a.r_logp = r->r_log_probs; a.r_values = r->r_values;
     a.r_rewards = r->r_rewards; a.r_dones = r->r_dones;
     a.acc = Accounting{r->r_rewards, r->r_dones, r->ep_return, r->ep_length, r->done_returns, r->done_lengths,
                        r->done_count, r->done_cap};
-    const dim3 grid(grid_for(r->n_envs, PR)), block(LunarLander::THREADS);
+    const dim3 grid(grid_for(r->n_envs, PR));
+    int32_t *side = nullptr;
+    if (r->env_id == MRL_ENV_CARTPOLE) {
+        rc = cartpole_side(ctx, r->states, r->n_envs, &side);
+        if (rc) return rc;
+    }
     profile_step_begin(ctx);
     profile_mark(ctx, -1);
-    if (act == 1) hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 1, false>), grid, block, 0, ctx->stream, a);
-    else hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 2, false>), grid, block, 0, ctx->stream, a);
+    if (r->env_id == MRL_ENV_LUNARLANDER) {
+        const dim3 block(LunarLander::THREADS);
+        if (act == 1) hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 1, false>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 2, false>), grid, block, 0, ctx->stream, a);
+    } else if (r->env_id == MRL_ENV_CARTPOLE) {
+        if (act == 1) hipLaunchKernelGGL((collect_classic_kernel<CartPoleSlot, 1, false>), grid, dim3(128), 0, ctx->stream, a, side);
+        else hipLaunchKernelGGL((collect_classic_kernel<CartPoleSlot, 2, false>), grid, dim3(128), 0, ctx->stream, a, side);
+    } else {
+        if (act == 1) hipLaunchKernelGGL((collect_classic_kernel<PendulumSlot, 1, true>), grid, dim3(128), 0, ctx->stream, a, side);
+        else hipLaunchKernelGGL((collect_classic_kernel<PendulumSlot, 2, true>), grid, dim3(128), 0, ctx->stream, a, side);
+    }
     MRL_CHECK_LAUNCH();
     profile_mark(ctx, MRL_PHASE_COLLECT);
     profile_step_end(ctx);

@@ -172,7 +172,7 @@ static int launch_phys_step(mrl_ctx *ctx, int batch, float *states, const float 
     return MRL_OK;
 }
 
-static int cartpole_side(mrl_ctx *ctx, const float *states, int batch, int32_t **out) {
+int cartpole_side(mrl_ctx *ctx, const float *states, int batch, int32_t **out) {
     auto it = ctx->cartpole_steps.find(states);
     if (it != ctx->cartpole_steps.end() && it->second.batch >= batch) {
         *out = it->second.steps;

@@ -73,6 +73,9 @@ int env_step_accounting(mrl_ctx *ctx, int env_id, int batch, float *states, cons
                         float *rewards, float *dones, float *obs, uint64_t step_seed, uint64_t reset_seed,
                         const Accounting &acc);
 
+// CartPole's per-env step counters for the rows at `states` (created zeroed on first use)
+int cartpole_side(mrl_ctx *ctx, const float *states, int batch, int32_t **out);
+
 inline int grid_for(long n, int block) { return (int)((n + block - 1) / block); }
 
 // Records a phase boundary: the time since the previous mark is charged to `tag`; tag < 0 opens

@@ -18,11 +18,12 @@ def ctx(mrl):
     return mrl.DeviceContext("cuda:0")
 
 
-def _pair(mrl, ctx, N, T, hidden, kind):
-    E = mrl.LunarLanderV2
+def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
+    E = {"lunar": mrl.LunarLanderV2, "cartpole": mrl.CartPoleEnv, "pendulum": mrl.PendulumV2}[env]
     lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
-    actor = mrl.seq(lin(8, hidden), lin(hidden, hidden), mrl.Linear(hidden, 4))
-    critic = mrl.seq(lin(8, hidden), lin(hidden, hidden), mrl.Linear(hidden, 1))
+    head = mrl.StochasticActor(hidden, E.ACTION_DIM) if E.ACTION_DIM else mrl.Linear(hidden, E.NUM_ACTIONS)
+    actor = mrl.seq(lin(E.OBS_DIM, hidden), lin(hidden, hidden), head)
+    critic = mrl.seq(lin(E.OBS_DIM, hidden), lin(hidden, hidden), mrl.Linear(hidden, 1))
     g = torch.Generator(device="cuda").manual_seed(5)
     ap = (torch.rand(actor.PARAM_SIZE, device="cuda", generator=g) - 0.5) * 0.3
     cp = (torch.rand(critic.PARAM_SIZE, device="cuda", generator=g) - 0.5) * 0.3
@@ -32,17 +33,29 @@ def _pair(mrl, ctx, N, T, hidden, kind):
         rb.actor_params, rb.critic_params = ap, cp
         E.reset_kernel_gpu(ctx, rb.states, 3)
         # some episodes end inside the range, so that in-place resets and the accounting are covered
-        rb.states.view(N, 192)[::3, 188] = 995.0
-        rb.obs.copy_(rb.states.view(N, 192)[:, :8].reshape(-1))
+        rows = rb.states.view(N, E.STATE_SIZE)
+        if env == "lunar":
+            rows[::3, 188] = 995.0    # step counter close to the limit
+        elif env == "cartpole":
+            rows[::3, 0] = 2.39       # cart next to the edge of the track, moving outwards
+            rows[::3, 1] = 2.0
+        else:
+            rows[::3, 4] = 197.0      # step counter close to the limit
+        rb.obs.copy_(rows[:, :E.OBS_DIM].reshape(-1))
         out.append(rb)
     return out
 
 
-@pytest.mark.parametrize("N,T,hidden,kind", [(8192, 12, 256, "relu"), (1000, 9, 256, "tanh"), (77, 5, 256, "relu"),
-                                             (300, 6, 64, "relu")])
-def test_rollout_steps_equals_single_steps(mrl, ctx, N, T, hidden, kind):
-    print("case", N, T, hidden, kind, flush=True)
-    one, many = _pair(mrl, ctx, N, T, hidden, kind)
+@pytest.mark.parametrize("env,N,T,hidden,kind", [
+    ("lunar", 8192, 12, 256, "relu"), ("lunar", 1000, 9, 256, "tanh"), ("lunar", 77, 5, 256, "relu"),
+    ("lunar", 300, 6, 64, "relu"),            # not fusable: the loop of single steps behind the same call
+    ("cartpole", 8192, 12, 64, "relu"), ("cartpole", 77, 7, 64, "tanh"),
+    ("pendulum", 8192, 12, 64, "tanh"), ("pendulum", 1000, 9, 64, "relu"),
+    ("cartpole", 300, 6, 256, "relu"),        # not fusable
+])
+def test_rollout_steps_equals_single_steps(mrl, ctx, env, N, T, hidden, kind):
+    print("case", env, N, T, hidden, kind, flush=True)
+    one, many = _pair(mrl, ctx, N, T, hidden, kind, env)
     s0, ss, r0, rs = 1234567, 2654435761 * N + 7919, 99, 0x9E3779B97F4A7C15
     d1, d2 = one.descriptor(), many.descriptor()
     for t in range(T):
