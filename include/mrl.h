@@ -242,10 +242,11 @@ int mrl_rollout_step(mrl_ctx *ctx, const mrl_rollout *r, int t, uint32_t sample_
  * the step counter in the same affine way.  Buffers end up as after n_steps calls of
  * mrl_rollout_step with those seeds, except that the order of the finished-episode list
  * (done_returns / done_lengths) inside the call is unspecified.  Where the env and the networks
- * allow it (LunarLander, hidden width 256) the whole range is ONE launch: each workgroup keeps its
- * 32 env rows in LDS and alternates policy forward and env step on them, so states and
- * observations cross HBM once per call instead of twice per step; otherwise the steps are issued
- * one by one.  Enqueue only. */
+ * allow it (LunarLander with hidden width 256; CartPole and Pendulum with hidden width 64) the
+ * whole range is ONE launch: each workgroup keeps its 32 envs on the chip (rows in LDS, or state
+ * in registers for the two small envs) and alternates policy forward and env step on them, so
+ * states and observations cross HBM once per call instead of twice per step; otherwise the
+ * steps are issued one by one.  Enqueue only. */
 int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, uint32_t sample_seed,
                       uint32_t sample_stride, uint64_t step_seed, uint64_t step_stride,
                       uint64_t reset_seed, uint64_t reset_stride);

@@ -209,10 +209,14 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
 }
 
 // ---------------------------------------------------------------- CartPole / Pendulum
-// The same idea for the envs whose state is a handful of floats: a workgroup of two wavefronts
-// (actor on one, critic on the other, hidden width 64) takes its 32 envs through all the steps
-// of the launch; lanes 0 .. 31 of wavefront 0 carry one env each in registers -- state, step
-// counter, episode sums -- and do sampling, step, accounting and reset in place.
+// The same idea for the envs whose state is a handful of floats: a workgroup of four wavefronts
+// (two on the actor, two on the critic, hidden width 64, one 32-column tile each) takes its 32
+// envs through all the steps of the launch.  Each wavefront's share of the hidden layers' weights
+// is loaded into registers once, before the first step; lanes 0 .. 31 of wavefront 0 carry one
+// env each in registers -- state, step counter, episode sums -- and do sampling, step,
+// accounting and reset in place.  A step is one dependent chain (observation -> two layers on
+// the matrix cores -> head -> sample -> env step), so the time of a step does not depend on the
+// number of envs until there are more workgroups than the chip holds at once.
 struct CartPoleSlot {
     static constexpr int OBS = cartpole::OBS, ACT_W = 1;
     float s[4];
@@ -248,10 +252,14 @@ struct PendulumSlot {
     MRL_DEV void reset(int i, uint64_t seed) { pendulum::reset(s, i, seed); }
 };
 
+constexpr int CLASSIC_TPW = 1;   // accumulator tiles per wavefront: 1 = two wavefronts per net
+constexpr int CLASSIC_THREADS = 2 * hidden_threads(64, CLASSIC_TPW);
+
 template <class C, int ACT, bool GAUSS>
-__global__ __launch_bounds__(128) void collect_classic_kernel(CollectArgs a, int32_t *side) {
-    constexpr int H = 64, TPW = 2, TN = hidden_threads(H, TPW), IN = C::OBS, AW = C::ACT_W;
-    static_assert(TN == 64 && IN <= PIN_MAX, "one wavefront per net");
+__global__ __launch_bounds__(CLASSIC_THREADS) void collect_classic_kernel(CollectArgs a, int32_t *side) {
+    constexpr int H = 64, TPW = CLASSIC_TPW, TN = hidden_threads(H, TPW), IN = C::OBS, AW = C::ACT_W;
+    constexpr int KB = H / 2;   // all of layer 1 in one block of k-steps: its weights stay in registers
+    static_assert(IN <= PIN_MAX, "observation fits the input tile");
     __shared__ float xs[PR * XS_LD];
     __shared__ float hT[2][H * HT_LD];
     __shared__ float h2[2][PR * (H + 1)];
@@ -275,7 +283,10 @@ __global__ __launch_bounds__(128) void collect_classic_kernel(CollectArgs a, int
         const float *p = net ? a.critic_p : a.actor_p;
         stage_head(p + IN * H + H + H * H + H, H, net ? 1 : a.A, GAUSS && net == 0, w2s[net], t % TN, TN);
     }
-    for (int i = t; i < PR * XS_LD; i += 128) xs[i] = 0.0f;
+    for (int i = t; i < PR * XS_LD; i += CLASSIC_THREADS) xs[i] = 0.0f;
+    // the hidden layers' weights of this wavefront's column tiles, loaded once for all the steps
+    HiddenOperands<H, TPW, KB> ops;
+    ops.load(t / TN ? a.critic_p : a.actor_p, IN, t);
     __syncthreads();
 
     for (int k = 0; k < a.n_steps; ++k) {
@@ -286,8 +297,6 @@ __global__ __launch_bounds__(128) void collect_classic_kernel(CollectArgs a, int
         const float *p = (net ? a.critic_p : a.actor_p) + zero;
         const size_t row = (size_t)(a.t0 + k) * N + env0;   // this block's slice of rollout row t
         const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
-        HiddenOperands<H, TPW, 8> ops;
-        ops.load(p, IN, tid);
         if (tid < ne) {
 #pragma unroll
             for (int c = 0; c < IN; ++c) {
@@ -297,9 +306,11 @@ __global__ __launch_bounds__(128) void collect_classic_kernel(CollectArgs a, int
             }
         }
         __syncthreads();
-        hidden_stack<H, ACT, TPW, 8>(p, IN, xs, hT[net], h2[net], TileCache{}, ops, tid);
-        if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1, tid % H);
-        else head<H>(w2s[1], 1, h2[1], vals, 1, tid % H);
+        hidden_stack<H, ACT, TPW, KB>(p, IN, xs, hT[net], h2[net], TileCache{}, ops, tid);
+        if (tid % TN < H) {
+            if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1, tid % H);
+            else head<H>(w2s[1], 1, h2[1], vals, 1, tid % H);
+        }
         __syncthreads();
         if (tid < ne) {
             const int i = env0 + tid;
@@ -427,11 +438,11 @@ int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, u
         if (act == 1) hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 1, false>), grid, block, 0, ctx->stream, a);
         else hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 2, false>), grid, block, 0, ctx->stream, a);
     } else if (r->env_id == MRL_ENV_CARTPOLE) {
-        if (act == 1) hipLaunchKernelGGL((collect_classic_kernel<CartPoleSlot, 1, false>), grid, dim3(128), 0, ctx->stream, a, side);
-        else hipLaunchKernelGGL((collect_classic_kernel<CartPoleSlot, 2, false>), grid, dim3(128), 0, ctx->stream, a, side);
+        if (act == 1) hipLaunchKernelGGL((collect_classic_kernel<CartPoleSlot, 1, false>), grid, dim3(CLASSIC_THREADS), 0, ctx->stream, a, side);
+        else hipLaunchKernelGGL((collect_classic_kernel<CartPoleSlot, 2, false>), grid, dim3(CLASSIC_THREADS), 0, ctx->stream, a, side);
     } else {
-        if (act == 1) hipLaunchKernelGGL((collect_classic_kernel<PendulumSlot, 1, true>), grid, dim3(128), 0, ctx->stream, a, side);
-        else hipLaunchKernelGGL((collect_classic_kernel<PendulumSlot, 2, true>), grid, dim3(128), 0, ctx->stream, a, side);
+        if (act == 1) hipLaunchKernelGGL((collect_classic_kernel<PendulumSlot, 1, true>), grid, dim3(CLASSIC_THREADS), 0, ctx->stream, a, side);
+        else hipLaunchKernelGGL((collect_classic_kernel<PendulumSlot, 2, true>), grid, dim3(CLASSIC_THREADS), 0, ctx->stream, a, side);
     }
     MRL_CHECK_LAUNCH();
     profile_mark(ctx, MRL_PHASE_COLLECT);
