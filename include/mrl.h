@@ -137,6 +137,13 @@ int mrl_sample_categorical(mrl_ctx *ctx, const float *logits, int n, int num_act
 /* _sample_continuous_actions_kernel, deep_agents/ppo/kernels.mojo:12-98 */
 int mrl_sample_gaussian(mrl_ctx *ctx, const float *actor_out, int n, int action_dim, uint32_t seed,
                         float *actions, float *log_probs);
+/* The action of the evaluation policies without sampling.  continuous != 0: the mean of the
+ * Gaussian head, actions[i, j] = actor_out[i, j] with actor_out rows [mean (A) | log_std (A)]
+ * (extract_deterministic_actions in evaluate_gpu, deep_agents/ppo/ppo_continuous.mojo:807-822).
+ * continuous == 0: the first index of the largest logit as a float, which is the argmax of the
+ * softmax probabilities that select_action(training=False) takes (ppo.mojo:988-1027). */
+int mrl_greedy_actions(mrl_ctx *ctx, const float *actor_out, int n, int num_actions, int continuous,
+                       float *actions);
 /* host GAE loop of train_gpu, deep_agents/ppo/ppo.mojo:2317-2353 (time-major, idx = t*N + env) */
 int mrl_gae(mrl_ctx *ctx, int T, int N, const float *rewards, const float *values,
             const float *dones, const float *bootstrap, double gamma, double lam, float *adv,

@@ -14,12 +14,12 @@ from .envs import CartPoleEnv, PendulumV2, LunarLanderV2, BipedalWalkerV2, HalfC
 from .model import Model, Linear, LinearReLU, LinearTanh, StochasticActor, seq  # noqa: E402
 from .optimizer import Adam  # noqa: E402
 from .training import Network, Xavier, Kaiming, init_params_small  # noqa: E402
-from . import ppo  # noqa: E402
+from . import ppo, checkpoint  # noqa: E402
 from .agents import DeepPPOAgent, DeepPPOContinuousAgent, TrainingMetrics  # noqa: E402
 
 __all__ = ["DeviceContext", "CartPoleEnv", "PendulumV2", "LunarLanderV2", "BipedalWalkerV2",
            "HalfCheetahPlanarV2", "MrlError", "Model",
            "Linear", "LinearReLU", "LinearTanh", "StochasticActor", "seq", "Adam", "ppo",
-           "Network", "Xavier", "Kaiming", "init_params_small",
+           "Network", "Xavier", "Kaiming", "init_params_small", "checkpoint",
            "DeepPPOAgent", "DeepPPOContinuousAgent", "TrainingMetrics",
            "LINEAR", "LINEAR_RELU", "LINEAR_TANH", "STOCHASTIC_ACTOR"]

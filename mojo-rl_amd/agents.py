@@ -11,7 +11,7 @@ rollout / epoch.  Network sizes, hyper-parameter names and defaults are the refe
 """
 import torch
 
-from . import ppo
+from . import checkpoint, ppo
 from .model import Linear, LinearReLU, LinearTanh, StochasticActor, seq
 from .optimizer import Adam
 from .training import Network, Xavier, Kaiming, init_params_small
@@ -80,13 +80,98 @@ class _PPOAgentBase:
             cnt = min(int(rb.done_count.item()), rb.done_cap)
             if cnt:
                 metrics.log_episodes(rb.done_returns[:cnt].tolist(), rb.done_lengths[:cnt].tolist())
+            # auto-checkpoint whenever the episode count passes a multiple of checkpoint_every
+            # (ppo.mojo:2228-2255; the parameters only change between rollouts)
+            if (self.checkpoint_every > 0 and self.checkpoint_path != ""
+                    and (completed + cnt) // self.checkpoint_every > completed // self.checkpoint_every):
+                self.save_checkpoint(self.checkpoint_path)
+                if verbose:
+                    print("  [Checkpoint saved at episode %d ]" % (completed + cnt), flush=True)
             completed += cnt
             metrics.rollouts += 1
             metrics.total_steps = total_steps
             if verbose and metrics.rollouts % print_every == 0:
                 print("rollout %d  steps %d  episodes %d  mean return (last 100) %.2f" % (
                     metrics.rollouts, total_steps, completed, metrics.mean_reward()), flush=True)
+        if self.continuous:
+            self.train_step_count += total_steps   # ppo_continuous.mojo:3328
         return metrics
+
+    def evaluate_gpu(self, ctx, env, num_episodes=100, max_steps=1000, verbose=False, stochastic=True,
+                     steps_per_readback=32):
+        """DeepPPOContinuousAgent.evaluate_gpu (deep_agents/ppo/ppo_continuous.mojo:703-975): run the
+        policy on `n_envs` device envs until `num_episodes` episodes have finished or `max_steps`
+        steps have been taken; returns the mean return of the first `num_episodes` finished
+        episodes (steps in order, envs in index order within a step), 0.0 if none finished.
+        Step `s` samples with seed s * 2654435761 (or takes the mean action when `stochastic` is
+        false), steps the envs with seed s and re-initialises finished envs with seed s, as there.
+
+        The discrete agent has no GPU evaluation in the reference; here it gets the same loop with
+        categorical sampling or, when `stochastic` is false, the greedy action of its CPU
+        `evaluate` (ppo.mojo:1487-1556).
+
+        Rewards and done flags are read back every `steps_per_readback` steps instead of every
+        step; the steps issued past the last counted episode do not change the result."""
+        if env.OBS_DIM != self.obs_dim:
+            raise ValueError("env OBS_DIM %d != agent obs_dim %d" % (env.OBS_DIM, self.obs_dim))
+        self.build_networks(ctx)
+        N, dev = self.n_envs, ctx.device
+        aw = env.ACTION_DIM if self.continuous else 1
+        states = torch.zeros(N * env.STATE_SIZE, device=dev)
+        obs = torch.zeros(N * env.OBS_DIM, device=dev)
+        actions = torch.zeros(N * aw, device=dev)
+        log_probs = torch.zeros(N, device=dev)
+        actor_out = torch.zeros(N * self.actor.model.OUT_DIM, device=dev)
+        K = max(1, int(steps_per_readback))
+        rewards = torch.zeros(K * N, device=dev)
+        dones = torch.zeros(K * N, device=dev)
+        env.reset_kernel_gpu(ctx, states, 0)
+        obs.copy_(states.view(N, env.STATE_SIZE)[:, :env.OBS_DIM].reshape(-1))
+        if verbose:
+            print("Running GPU evaluation with", N, "parallel envs...", flush=True)
+        current = [0.0] * N
+        episode_rewards = []
+        step = 0
+        while len(episode_rewards) < num_episodes and step < max_steps:
+            k = min(K, max_steps - step)
+            for j in range(k):
+                s = step + j
+                self.actor.model.forward_gpu_no_cache_ws(ctx, actor_out, obs, self.actor.params)
+                if not stochastic:
+                    ppo.greedy_actions(ctx, actor_out, actions, N, self.continuous)
+                elif self.continuous:
+                    ppo.sample_continuous_actions(ctx, actor_out, actions, log_probs, s * 2654435761)
+                else:
+                    ppo.sample_actions(ctx, actor_out, actions, log_probs, s * 2654435761)
+                env.step_autoreset_kernel_gpu(ctx, states, actions, rewards[j * N:(j + 1) * N],
+                                              dones[j * N:(j + 1) * N], obs, s, s)
+            ctx.synchronize()
+            r_host = rewards[:k * N].view(k, N).tolist()
+            d_host = dones[:k * N].view(k, N).tolist()
+            for j in range(k):
+                rj, dj = r_host[j], d_host[j]
+                for i in range(N):
+                    current[i] += rj[i]
+                    if dj[i] > 0:
+                        episode_rewards.append(current[i])
+                        current[i] = 0.0
+                        if len(episode_rewards) >= num_episodes:
+                            break
+                step += 1
+                if len(episode_rewards) >= num_episodes:
+                    break
+        if not episode_rewards:
+            if verbose:
+                print("Warning: No episodes completed!")
+            return 0.0
+        avg = sum(episode_rewards) / float(len(episode_rewards))
+        if verbose:
+            print("GPU EVALUATION SUMMARY (%s Actions)" % ("Continuous" if self.continuous else "Discrete"))
+            print("Episodes completed:", len(episode_rewards))
+            print("Average reward:", avg)
+            print("Min reward:", min(episode_rewards))
+            print("Max reward:", max(episode_rewards))
+        return avg
 
 
 class DeepPPOAgent(_PPOAgentBase):
@@ -98,7 +183,7 @@ class DeepPPOAgent(_PPOAgentBase):
                  critic_lr=0.001, entropy_coef=0.01, value_loss_coef=0.5, num_epochs=4,
                  normalize_advantages=True, target_kl=0.015, max_grad_norm=0.5, anneal_lr=True,
                  anneal_entropy=False, target_total_steps=0, clip_value=True, norm_adv_per_minibatch=True,
-                 init_seed=0):
+                 init_seed=0, minibatch_size=64, checkpoint_every=0, checkpoint_path=""):
         self.obs_dim, self.num_actions, self.hidden_dim = obs_dim, num_actions, hidden_dim
         self.rollout_len, self.n_envs, self.gpu_minibatch_size = rollout_len, n_envs, gpu_minibatch_size
         self.gamma, self.gae_lambda, self.clip_epsilon = gamma, gae_lambda, clip_epsilon
@@ -107,6 +192,9 @@ class DeepPPOAgent(_PPOAgentBase):
         self.normalize_advantages, self.target_kl, self.max_grad_norm = normalize_advantages, target_kl, max_grad_norm
         self.anneal_lr, self.anneal_entropy, self.target_total_steps = anneal_lr, anneal_entropy, target_total_steps
         self.clip_value, self.norm_adv_per_minibatch, self.init_seed = clip_value, norm_adv_per_minibatch, init_seed
+        # minibatch_size is the CPU trainer's; it is carried for the checkpoint metadata only
+        self.minibatch_size, self.checkpoint_every, self.checkpoint_path = minibatch_size, checkpoint_every, checkpoint_path
+        self.train_step_count = 0
         self.actor = self.critic = self.rb = self.upd = None
 
     def _nets(self):
@@ -114,11 +202,30 @@ class DeepPPOAgent(_PPOAgentBase):
         return (seq(LinearReLU(self.obs_dim, H), LinearReLU(H, H), Linear(H, self.num_actions)),
                 seq(LinearReLU(self.obs_dim, H), LinearReLU(H, H), Linear(H, 1)))
 
-    def _build(self, ctx, env):
+    def build_networks(self, ctx):
+        """Create and initialise actor and critic on `ctx` (a no-op once they exist)."""
         if self.actor is None:
             am, cm = self._nets()
             self.actor = Network(ctx, am, Adam(lr=self.actor_lr), Xavier(seed=2 * self.init_seed + 1))
             self.critic = Network(ctx, cm, Adam(lr=self.critic_lr), Xavier(seed=2 * self.init_seed + 2))
+
+    def save_checkpoint(self, filepath):
+        """ppo.mojo:3926-3980."""
+        checkpoint.save_ppo_agent(self, filepath)
+
+    def load_checkpoint(self, filepath, ctx=None):
+        """ppo.mojo:3982-4055.  `ctx` is needed when the networks have not been built yet."""
+        self._networks_for_load(ctx)
+        checkpoint.load_ppo_agent(self, filepath)
+
+    def _networks_for_load(self, ctx):
+        if self.actor is None:
+            if ctx is None:
+                raise ValueError("load_checkpoint: pass the DeviceContext, the networks do not exist yet")
+            self.build_networks(ctx)
+
+    def _build(self, ctx, env):
+        self.build_networks(ctx)
         self.rb = ppo.RolloutBuffers(ctx, env, self.actor.model, self.critic.model, self.n_envs, self.rollout_len,
                                      done_cap=max(1024, 2 * self.n_envs * self.rollout_len // 8),
                                      continuous=self.continuous)
@@ -153,13 +260,20 @@ class DeepPPOContinuousAgent(DeepPPOAgent):
         return (seq(LinearTanh(self.obs_dim, H), LinearTanh(H, H), StochasticActor(H, self.action_dim)),
                 seq(LinearTanh(self.obs_dim, H), LinearTanh(H, H), Linear(H, 1)))
 
-    def _build(self, ctx, env):
-        fresh = self.actor is None
-        if fresh:
+    def build_networks(self, ctx):
+        if self.actor is None:
             am, cm = self._nets()
             self.actor = Network(ctx, am, Adam(lr=self.actor_lr), Kaiming(seed=2 * self.init_seed + 1))
             self.critic = Network(ctx, cm, Adam(lr=self.critic_lr), Kaiming(seed=2 * self.init_seed + 2))
             H = self.hidden_dim
             init_params_small(ctx, self.actor.params, self.obs_dim * H + H + H * H + H, H, self.action_dim,
                               seed=2 * self.init_seed + 3)
-        super()._build(ctx, env)
+
+    def save_checkpoint(self, filepath):
+        """ppo_continuous.mojo:493-523."""
+        checkpoint.save_ppo_continuous_agent(self, filepath)
+
+    def load_checkpoint(self, filepath, ctx=None):
+        """ppo_continuous.mojo:525-604."""
+        self._networks_for_load(ctx)
+        checkpoint.load_ppo_continuous_agent(self, filepath)

@@ -445,6 +445,37 @@ int mrl_sample_gaussian(mrl_ctx *ctx, const float *actor_out, int n, int action_
     return MRL_OK;
 }
 
+__global__ __launch_bounds__(256) void greedy_actions_kernel(const float *__restrict__ actor_out, int n, int A,
+                                                             int continuous, float *__restrict__ actions) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (continuous) {
+        if (i >= n * A) return;
+        const int row = i / A, j = i - row * A;
+        actions[i] = actor_out[(size_t)row * 2 * A + j];
+    } else {
+        if (i >= n) return;
+        const float *l = actor_out + (size_t)i * A;
+        int best = 0;
+        float top = l[0];
+        for (int a = 1; a < A; ++a)
+            if (l[a] > top) { top = l[a]; best = a; }
+        actions[i] = (float)best;
+    }
+}
+
+int mrl_greedy_actions(mrl_ctx *ctx, const float *actor_out, int n, int num_actions, int continuous,
+                       float *actions) {
+    MRL_CHECK_ARG(ctx, "mrl_greedy_actions: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0 && num_actions > 0, "mrl_greedy_actions: bad sizes");
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(actor_out && actions, "mrl_greedy_actions: NULL buffer");
+    const long work = continuous ? (long)n * num_actions : (long)n;
+    hipLaunchKernelGGL(greedy_actions_kernel, dim3(grid_for(work, 256)), dim3(256), 0, ctx->stream, actor_out, n,
+                       num_actions, continuous, actions);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
 int mrl_gae(mrl_ctx *ctx, int T, int N, const float *rewards, const float *values,
             const float *dones, const float *bootstrap, double gamma, double lam, float *adv,
             float *ret) {

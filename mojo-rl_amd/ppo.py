@@ -22,6 +22,16 @@ def sample_continuous_actions(ctx, actor_output, actions, log_probs, seed):
               int(seed) & 0xFFFFFFFF, _ptr(actions), _ptr(log_probs))
 
 
+def greedy_actions(ctx, actor_output, actions, n, continuous):
+    """The actions of `n` rows without sampling: the Gaussian head's mean
+    (extract_deterministic_actions, deep_agents/ppo/ppo_continuous.mojo:807-822; rows of
+    actor_output are [mean | log_std]) or the argmax of the logits (select_action with
+    training=False, ppo.mojo:988-1027)."""
+    width = actor_output.numel() // max(n, 1)
+    _lib.call("mrl_greedy_actions", ctx.handle, _ptr(actor_output), n, width // 2 if continuous else width,
+              1 if continuous else 0, _ptr(actions))
+
+
 def compute_gae(ctx, rewards, values, dones, bootstrap, gamma, gae_lambda, advantages, returns):
     """GAE over time-major [T*N] buffers (index t*N + env); ppo.mojo:2317-2353."""
     n = bootstrap.numel()

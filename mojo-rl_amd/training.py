@@ -12,7 +12,7 @@ import math
 
 import torch
 
-from . import _lib
+from . import _lib, checkpoint
 from .context import _ptr
 
 
@@ -77,3 +77,11 @@ class Network:
 
     def update_gpu(self):
         self.optimizer.step_gpu(self.ctx, self.params, self.grads, self.optimizer_state)
+
+    def save_checkpoint(self, filepath):
+        """deep_rl/training/network.mojo:774-798."""
+        checkpoint.save_network(self, filepath)
+
+    def load_checkpoint(self, filepath):
+        """deep_rl/training/network.mojo:800-835."""
+        checkpoint.load_network(self, filepath)
