@@ -34,7 +34,11 @@ enum mrl_env_id {
     MRL_ENV_PENDULUM = 1,    /* envs/pendulum/pendulum_v2.mojo:57 PendulumV2 */
     MRL_ENV_LUNARLANDER = 2, /* envs/lunar_lander/lunar_lander_v2.mojo:123 LunarLanderV2 */
     MRL_ENV_BIPEDAL = 3,     /* envs/bipedal_walker/bipedal_walker_v2.mojo:103 BipedalWalkerV2 */
-    MRL_ENV_HALFCHEETAH = 4  /* envs/half_cheetah/cheetah_planar_v2.mojo:91 HalfCheetahPlanarV2 */
+    MRL_ENV_HALFCHEETAH = 4, /* envs/half_cheetah/cheetah_planar_v2.mojo:91 HalfCheetahPlanarV2 */
+    /* LunarLanderV2 as a GPUContinuousEnv: the step_kernel_gpu overload with ACTION_DIM = 2
+     * (lunar_lander_v2.mojo:1520-1588); rows, reset and selective reset are those of
+     * MRL_ENV_LUNARLANDER */
+    MRL_ENV_LUNARLANDER_CONTINUOUS = 5
 };
 
 /* layer kinds of an MLP description; deep_rl/model/{linear,linear_relu,linear_tanh,stochastic_actor}.mojo */

@@ -10,14 +10,15 @@ from ._lib import MrlError, LINEAR, LINEAR_RELU, LINEAR_TANH, STOCHASTIC_ACTOR
 _lib.lib()  # load now: a missing or unloadable HIP library is an import error, not a fallback
 
 from .context import DeviceContext  # noqa: E402
-from .envs import CartPoleEnv, PendulumV2, LunarLanderV2, BipedalWalkerV2, HalfCheetahPlanarV2  # noqa: E402
+from .envs import (CartPoleEnv, PendulumV2, LunarLanderV2, LunarLanderV2Continuous, BipedalWalkerV2,  # noqa: E402
+                   HalfCheetahPlanarV2)
 from .model import Model, Linear, LinearReLU, LinearTanh, StochasticActor, seq  # noqa: E402
 from .optimizer import Adam  # noqa: E402
 from .training import Network, Xavier, Kaiming, init_params_small  # noqa: E402
 from . import ppo, checkpoint  # noqa: E402
 from .agents import DeepPPOAgent, DeepPPOContinuousAgent, TrainingMetrics  # noqa: E402
 
-__all__ = ["DeviceContext", "CartPoleEnv", "PendulumV2", "LunarLanderV2", "BipedalWalkerV2",
+__all__ = ["DeviceContext", "CartPoleEnv", "PendulumV2", "LunarLanderV2", "LunarLanderV2Continuous", "BipedalWalkerV2",
            "HalfCheetahPlanarV2", "MrlError", "Model",
            "Linear", "LinearReLU", "LinearTanh", "StochasticActor", "seq", "Adam", "ppo",
            "Network", "Xavier", "Kaiming", "init_params_small", "checkpoint",

@@ -17,6 +17,7 @@ LIB_PATH = os.environ.get("MRL_HIP_LIB") or os.path.join(HERE, "libmrl_hip.so")
 MAX_LAYERS = 8
 LINEAR, LINEAR_RELU, LINEAR_TANH, STOCHASTIC_ACTOR = 0, 1, 2, 3
 ENV_CARTPOLE, ENV_PENDULUM, ENV_LUNARLANDER, ENV_BIPEDAL, ENV_HALFCHEETAH = 0, 1, 2, 3, 4
+ENV_LUNARLANDER_CONTINUOUS = 5
 
 
 class Layer(C.Structure):

@@ -75,6 +75,21 @@ struct LunarLander {
     }
 };
 
+// LunarLanderV2 behind the continuous-action trait (the reference overloads step_kernel_gpu on
+// the same struct, lunar_lander_v2.mojo:1520-1588): same rows, resets and contact detection,
+// two action components per env
+struct LunarLanderContinuous : LunarLander {
+    static constexpr int ACT_W = 2;
+    static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
+                             float &r, float &d) {
+        const Carry c = ll::step_begin_continuous(row, env, a);
+        ll::step_finish(row, cts, -1, shapes, c, r, d);
+    }
+    static MRL_DEV Carry step_begin(float *row, int env, const float *a) {
+        return ll::step_begin_continuous(row, env, a);
+    }
+};
+
 struct BipedalWalker {
     using L = bw::L;
     static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 32, THREADS = 256;

@@ -311,6 +311,27 @@ MRL_DEV StepCarry step_begin(float *row, int env, int action) {
     return c;
 }
 
+// The continuous-action overload (step_continuous_vec, lunar_lander_v2.mojo:1329-1383, decoded in
+// fp64 like the rest of the engine arithmetic): a[0] in [-1, 1] is the main throttle, remapped to
+// (a0 + 1) / 2 and clipped to [0, 1]; a[1] clipped to [-1, 1] fires the left (< -0.5) or right
+// (> 0.5) engine with power (|a1| - 0.5) * 2.  Both engines can fire in one step.
+MRL_DEV StepCarry step_begin_continuous(float *row, int env, const float *a) {
+    StepCarry c;
+    c.skip = row[L::META_OFF + META_DONE] > 0.5f;
+    c.step_count = (int)row[L::META_OFF + META_STEP];
+    double m_power = ((double)a[0] + 1.0) * 0.5;
+    if (m_power < 0.0) m_power = 0.0;
+    if (m_power > 1.0) m_power = 1.0;
+    double side_action = (double)a[1], s_power = 0.0, direction = 0.0;
+    if (side_action < -1.0) side_action = -1.0;
+    if (side_action > 1.0) side_action = 1.0;
+    if (side_action < -0.5) { direction = -1.0; s_power = (-side_action - 0.5) * 2.0; }
+    else if (side_action > 0.5) { direction = 1.0; s_power = (side_action - 0.5) * 2.0; }
+    c.m_power = m_power; c.s_power = s_power;
+    if (!c.skip) apply_engines(row, env, c.step_count, m_power, s_power, direction);
+    return c;
+}
+
 MRL_DEV void step_finish(float *row, float *contacts, int n_given, const float *shapes, const StepCarry &c,
                          float &reward, float &done) {
     if (c.skip) {

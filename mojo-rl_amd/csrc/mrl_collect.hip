@@ -359,6 +359,7 @@ __global__ __launch_bounds__(CLASSIC_THREADS) void collect_classic_kernel(Collec
 static bool collect_fusable(const mrl_rollout *r, bool gauss, int *act) {
     int obs, hidden;
     if (r->env_id == MRL_ENV_LUNARLANDER && !gauss) { obs = LunarLander::OBS; hidden = 256; }
+    else if (r->env_id == MRL_ENV_LUNARLANDER_CONTINUOUS && gauss) { obs = LunarLander::OBS; hidden = 256; }
     else if (r->env_id == MRL_ENV_CARTPOLE && !gauss) { obs = cartpole::OBS; hidden = 64; }
     else if (r->env_id == MRL_ENV_PENDULUM && gauss) { obs = pendulum::OBS; hidden = 64; }
     else return false;
@@ -437,6 +438,10 @@ int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, u
         const dim3 block(LunarLander::THREADS);
         if (act == 1) hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 1, false>), grid, block, 0, ctx->stream, a);
         else hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 2, false>), grid, block, 0, ctx->stream, a);
+    } else if (r->env_id == MRL_ENV_LUNARLANDER_CONTINUOUS) {
+        const dim3 block(LunarLander::THREADS);
+        if (act == 1) hipLaunchKernelGGL((collect_kernel<LunarLanderContinuous, 256, 1, true>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((collect_kernel<LunarLanderContinuous, 256, 2, true>), grid, block, 0, ctx->stream, a);
     } else if (r->env_id == MRL_ENV_CARTPOLE) {
         if (act == 1) hipLaunchKernelGGL((collect_classic_kernel<CartPoleSlot, 1, false>), grid, dim3(CLASSIC_THREADS), 0, ctx->stream, a, side);
         else hipLaunchKernelGGL((collect_classic_kernel<CartPoleSlot, 2, false>), grid, dim3(CLASSIC_THREADS), 0, ctx->stream, a, side);

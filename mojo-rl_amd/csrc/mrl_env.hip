@@ -203,6 +203,7 @@ int mrl_env_dims(int env_id, int *state_size, int *obs_dim, int *num_actions, in
         case MRL_ENV_CARTPOLE: s = 4; o = 4; na = 2; ad = 0; break;
         case MRL_ENV_PENDULUM: s = 8; o = 3; na = 0; ad = 1; break;
         case MRL_ENV_LUNARLANDER: s = ll::STATE; o = ll::OBS; na = 4; ad = 0; break;
+        case MRL_ENV_LUNARLANDER_CONTINUOUS: s = ll::STATE; o = ll::OBS; na = 0; ad = 2; break;
         case MRL_ENV_BIPEDAL: s = bw::STATE; o = bw::OBS; na = 0; ad = bw::ACT; break;
         case MRL_ENV_HALFCHEETAH: s = hc::STATE; o = hc::OBS; na = 0; ad = hc::ACT; break;
         default: return set_error(MRL_E_UNSUPPORTED, "mrl_env_dims: env_id %d is not built", env_id);
@@ -237,7 +238,10 @@ static int env_reset_impl(mrl_ctx *ctx, int env_id, int batch, float *states, fl
             hipLaunchKernelGGL(pendulum_reset_kernel, dim3(grid_for(batch, 256)), dim3(256), 0,
                                ctx->stream, states, dones, batch, seed, selective);
             break;
-        case MRL_ENV_LUNARLANDER: launch_phys_reset<LunarLander>(ctx, batch, states, dones, seed, selective); break;
+        case MRL_ENV_LUNARLANDER:
+        case MRL_ENV_LUNARLANDER_CONTINUOUS:
+            launch_phys_reset<LunarLander>(ctx, batch, states, dones, seed, selective);
+            break;
         case MRL_ENV_BIPEDAL: launch_phys_reset<BipedalWalker>(ctx, batch, states, dones, seed, selective); break;
         case MRL_ENV_HALFCHEETAH: launch_phys_reset<HalfCheetah>(ctx, batch, states, dones, seed, selective); break;
         default:
@@ -282,6 +286,10 @@ static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, con
         case MRL_ENV_LUNARLANDER:
             launch_phys_step<LunarLander>(ctx, batch, states, actions, rewards, dones, obs, ctx->ll_shapes,
                                           autoreset, reset_seed, acc);
+            break;
+        case MRL_ENV_LUNARLANDER_CONTINUOUS:
+            launch_phys_step<LunarLanderContinuous>(ctx, batch, states, actions, rewards, dones, obs, ctx->ll_shapes,
+                                                    autoreset, reset_seed, acc);
             break;
         case MRL_ENV_BIPEDAL:
             launch_phys_step<BipedalWalker>(ctx, batch, states, actions, rewards, dones, obs, ctx->bw_shapes,

@@ -77,6 +77,13 @@ class LunarLanderV2(_GPUEnv):         # envs/lunar_lander/lunar_lander_v2.mojo:1
     ENV_ID, STATE_SIZE, OBS_DIM, NUM_ACTIONS = _lib.ENV_LUNARLANDER, 192, 8, 4
 
 
+class LunarLanderV2Continuous(_GPUEnv):
+    """LunarLanderV2 as a GPUContinuousEnv (the reference overloads step_kernel_gpu on the one
+    struct by ACTION_DIM, lunar_lander_v2.mojo:1520-1588; here the overload is a class of its
+    own): action[0] main throttle in [-1, 1], action[1] side control in [-1, 1]."""
+    ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_LUNARLANDER_CONTINUOUS, 192, 8, 2
+
+
 class BipedalWalkerV2(_GPUEnv):       # envs/bipedal_walker/bipedal_walker_v2.mojo:103
     ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_BIPEDAL, 950, 24, 4
 

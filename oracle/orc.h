@@ -114,6 +114,11 @@ void orc_ll_reset(float *row, uint64_t combined_seed);
 /* contacts_out (8*9 floats) and n_contacts_out may be NULL */
 void orc_ll_step(float *row, int env, int action, float *reward, float *done,
                  float *contacts_out, int *n_contacts_out);
+/* the continuous-action overload: a0 = main throttle in [-1, 1], a1 = side control in [-1, 1] */
+void orc_ll_step_continuous(float *row, int env, float a0, float a1, float *reward, float *done,
+                            float *contacts_out, int *n_contacts_out);
+void orc_ll_step_continuous_batch(float *states, const float *actions, float *rewards, float *dones,
+                                  float *obs, int batch);
 void orc_ll_reset_batch(float *states, int batch, uint64_t seed);
 void orc_ll_selective_reset_batch(float *states, const float *dones, int batch, uint64_t seed);
 void orc_ll_step_batch(float *states, const float *actions, float *rewards, float *dones,

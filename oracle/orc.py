@@ -75,6 +75,8 @@ def load():
         "orc_ll_combined_seed": (C.c_uint64, [C.c_uint64, C.c_int]),
         "orc_ll_reset": (None, [f32p, C.c_uint64]),
         "orc_ll_step": (None, [f32p, C.c_int, C.c_int, f32p, f32p, C.c_void_p, C.c_void_p]),
+        "orc_ll_step_continuous": (None, [f32p, C.c_int, C.c_float, C.c_float, f32p, f32p, C.c_void_p, C.c_void_p]),
+        "orc_ll_step_continuous_batch": (None, [f32p, f32p, f32p, f32p, f32p, C.c_int]),
         "orc_ll_reset_batch": (None, [f32p, C.c_int, C.c_uint64]),
         "orc_ll_selective_reset_batch": (None, [f32p, f32p, C.c_int, C.c_uint64]),
         "orc_ll_step_batch": (None, [f32p, f32p, f32p, f32p, f32p, C.c_int, C.c_int]),

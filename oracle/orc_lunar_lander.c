@@ -8,6 +8,8 @@
  *   reset                lunar_lander_v2.mojo:443-634 (_reset_cpu), row writes as
  *                        :1709-1966 (_reset_env_gpu), seed combination :1618-1638
  *   engines              lunar_lander_v2.mojo:1025-1095 (_apply_engines, Float64)
+ *   continuous actions   lunar_lander_v2.mojo:1329-1383 (step_continuous_vec: throttle and side
+ *                        control decoded in Float64) + :1385-1436 (_step_cpu_continuous)
  *   physics step         lunar_lander_v2.mojo:1097-1168 (_step_physics_cpu)
  *   observation          lunar_lander_v2.mojo:699-775 + envs/lunar_lander/helpers.mojo:10-64
  *   reward / termination lunar_lander_v2.mojo:1192-1255 + helpers.mojo:92-133
@@ -223,8 +225,36 @@ static void apply_engines(const orc_layout *L, float *row, int env, int step_cou
     B[ORC_IDX_OMEGA] = (float)(omega + domega);
 }
 
+static void step_powers(float *row, int env, double m_power, double s_power, double direction, float *reward,
+                        float *done, float *contacts_out, int *n_contacts_out);
+
 void orc_ll_step(float *row, int env, int action, float *reward, float *done, float *contacts_out,
                  int *n_contacts_out) {
+    double m_power = 0.0, s_power = 0.0, direction = 0.0;
+    if (action == 2) m_power = 1.0;
+    else if (action == 1) { s_power = 1.0; direction = -1.0; }
+    else if (action == 3) { s_power = 1.0; direction = 1.0; }
+    step_powers(row, env, m_power, s_power, direction, reward, done, contacts_out, n_contacts_out);
+}
+
+/* step_continuous_vec, lunar_lander_v2.mojo:1329-1383: a0 in [-1, 1] -> throttle (a0 + 1) / 2
+ * clipped to [0, 1]; a1 clipped to [-1, 1], the side engine fires beyond +-0.5 with power
+ * (|a1| - 0.5) * 2 */
+void orc_ll_step_continuous(float *row, int env, float a0, float a1, float *reward, float *done,
+                            float *contacts_out, int *n_contacts_out) {
+    double m_power = ((double)a0 + 1.0) * 0.5;
+    if (m_power < 0.0) m_power = 0.0;
+    if (m_power > 1.0) m_power = 1.0;
+    double side_action = (double)a1, s_power = 0.0, direction = 0.0;
+    if (side_action < -1.0) side_action = -1.0;
+    if (side_action > 1.0) side_action = 1.0;
+    if (side_action < -0.5) { direction = -1.0; s_power = (-side_action - 0.5) * 2.0; }
+    else if (side_action > 0.5) { direction = 1.0; s_power = (side_action - 0.5) * 2.0; }
+    step_powers(row, env, m_power, s_power, direction, reward, done, contacts_out, n_contacts_out);
+}
+
+static void step_powers(float *row, int env, double m_power, double s_power, double direction, float *reward,
+                        float *done, float *contacts_out, int *n_contacts_out) {
     orc_layout L; orc_ll_layout(&L);
     float shapes[60]; orc_ll_shapes(shapes);
     float contacts[8 * ORC_CONTACT_SIZE];
@@ -237,10 +267,6 @@ void orc_ll_step(float *row, int env, int action, float *reward, float *done, fl
     }
 
     int step_count = (int)row[L.meta_off + META_STEP];
-    double m_power = 0.0, s_power = 0.0, direction = 0.0;
-    if (action == 2) m_power = 1.0;
-    else if (action == 1) { s_power = 1.0; direction = -1.0; }
-    else if (action == 3) { s_power = 1.0; direction = 1.0; }
 
     apply_engines(&L, row, env, step_count, m_power, s_power, direction);
 
@@ -298,6 +324,15 @@ void orc_ll_reset_batch(float *states, int batch, uint64_t seed) {
 void orc_ll_selective_reset_batch(float *states, const float *dones, int batch, uint64_t seed) {
     for (int i = 0; i < batch; ++i)
         if (dones[i] > 0.5f) orc_ll_reset(states + (long)i * ORC_LL_STATE, orc_ll_combined_seed(seed, i));
+}
+
+void orc_ll_step_continuous_batch(float *states, const float *actions, float *rewards, float *dones,
+                                  float *obs, int batch) {
+    for (int i = 0; i < batch; ++i) {
+        float *row = states + (long)i * ORC_LL_STATE;
+        orc_ll_step_continuous(row, i, actions[2 * i], actions[2 * i + 1], rewards + i, dones + i, 0, 0);
+        memcpy(obs + (long)i * 8, row, sizeof(float) * 8);
+    }
 }
 
 void orc_ll_step_batch(float *states, const float *actions, float *rewards, float *dones,

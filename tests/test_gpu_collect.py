@@ -19,7 +19,8 @@ def ctx(mrl):
 
 
 def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
-    E = {"lunar": mrl.LunarLanderV2, "cartpole": mrl.CartPoleEnv, "pendulum": mrl.PendulumV2}[env]
+    E = {"lunar": mrl.LunarLanderV2, "lunarc": mrl.LunarLanderV2Continuous, "cartpole": mrl.CartPoleEnv,
+         "pendulum": mrl.PendulumV2}[env]
     lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
     head = mrl.StochasticActor(hidden, E.ACTION_DIM) if E.ACTION_DIM else mrl.Linear(hidden, E.NUM_ACTIONS)
     actor = mrl.seq(lin(E.OBS_DIM, hidden), lin(hidden, hidden), head)
@@ -34,7 +35,7 @@ def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
         E.reset_kernel_gpu(ctx, rb.states, 3)
         # some episodes end inside the range, so that in-place resets and the accounting are covered
         rows = rb.states.view(N, E.STATE_SIZE)
-        if env == "lunar":
+        if env in ("lunar", "lunarc"):
             rows[::3, 188] = 995.0    # step counter close to the limit
         elif env == "cartpole":
             rows[::3, 0] = 2.39       # cart next to the edge of the track, moving outwards
@@ -52,6 +53,7 @@ def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
     ("cartpole", 8192, 12, 64, "relu"), ("cartpole", 77, 7, 64, "tanh"),
     ("pendulum", 8192, 12, 64, "tanh"), ("pendulum", 1000, 9, 64, "relu"),
     ("cartpole", 300, 6, 256, "relu"),        # not fusable
+    ("lunarc", 8192, 12, 256, "tanh"), ("lunarc", 77, 6, 256, "relu"), ("lunarc", 300, 6, 64, "tanh"),
 ])
 def test_rollout_steps_equals_single_steps(mrl, ctx, env, N, T, hidden, kind):
     print("case", env, N, T, hidden, kind, flush=True)

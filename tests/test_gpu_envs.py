@@ -196,6 +196,74 @@ def test_lunar_lander_contacts_and_reset_cycle(mrl, orc, ctx):
     assert crashes > 50 and lands > 500
 
 
+def llc_policy(rng, obs):
+    """Continuous stand-in policy: throttle and side control beyond [-1, 1] now and then, the dead
+    band of the side engines, and full throttle when falling fast."""
+    n = obs.shape[0]
+    a = rng.uniform(-1.4, 1.4, (n, 2)).astype(np.float32)
+    a[rng.random(n) < 0.2, 1] = 0.5           # edge of the dead band
+    a[obs[:, 3] < -0.3, 0] = 1.0
+    return a
+
+
+@pytest.mark.parametrize("batch,seed,low", [(1, 3, False), (65, 4, False), (8192, 5, False), (2048, 6, True)])
+def test_lunar_lander_continuous_rollout_parity(mrl, orc, ctx, batch, seed, low):
+    say("lunar continuous batch", batch, "low start", low)
+    E = mrl.LunarLanderV2Continuous
+    s_h = np.zeros((batch, 192), np.float32)
+    orc.orc_ll_reset_batch(s_h, batch, seed)
+    rng = np.random.default_rng(seed)
+    if low:   # start low over the pad: contacts, crashes and landings within the 64 steps
+        b = s_h[:, 8:47].reshape(batch, 3, 13)
+        b[:, :, 1] -= rng.uniform(7.5, 9.4, batch).astype(np.float32)[:, None]
+        b[:, :, 0] += rng.uniform(-6, 6, batch).astype(np.float32)[:, None]
+    s = torch.full((batch * 192,), 7.0, device="cuda")
+    E.reset_kernel_gpu(ctx, s, seed)
+    ctx.synchronize()
+    if low:
+        s.copy_(dev(s_h.reshape(-1)))
+    else:
+        close(s.cpu().numpy().reshape(batch, 192), s_h)
+        s_h[:] = s.cpu().numpy().reshape(batch, 192)
+    a = torch.zeros(batch * 2, device="cuda")
+    r, d, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch * 8))
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 8), np.float32)
+    n_done = 0
+    for t in range(64):
+        act = llc_policy(rng, s_h[:, :8])
+        a.copy_(dev(act.reshape(-1)))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_ll_step_continuous_batch(s_h, act, r_h, d_h, o_h, batch)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 192)
+        close(sg, s_h)
+        close(o.cpu().numpy().reshape(batch, 8), o_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        np.testing.assert_array_equal(r.cpu().numpy(), r_h)   # reward exact
+        n_done += int(d_h.sum())
+        s_h[:] = sg
+    say("  finished rows seen:", n_done)
+    assert not low or n_done > 100
+
+
+def test_lunar_lander_continuous_corners_equal_discrete_actions(mrl, ctx):
+    batch = 512
+    D, Cn = mrl.LunarLanderV2, mrl.LunarLanderV2Continuous
+    s1 = torch.zeros(batch * 192, device="cuda")
+    D.reset_kernel_gpu(ctx, s1, 8)
+    s2 = s1.clone()
+    g = torch.Generator(device="cuda").manual_seed(3)
+    table = torch.tensor([[-1.0, 0.0], [-1.0, -1.0], [1.0, 0.25], [-1.0, 1.0]], device="cuda")
+    bufs = lambda: tuple(torch.zeros(n, device="cuda") for n in (batch, batch, batch * 8))
+    r1, d1, o1 = bufs(); r2, d2, o2 = bufs()
+    for t in range(30):
+        a = torch.randint(0, 4, (batch,), device="cuda", generator=g)
+        D.step_autoreset_kernel_gpu(ctx, s1, a.float(), r1, d1, o1, t, 70 + t)
+        Cn.step_autoreset_kernel_gpu(ctx, s2, table[a].reshape(-1).contiguous(), r2, d2, o2, t, 70 + t)
+        ctx.synchronize()
+        assert torch.equal(s1, s2) and torch.equal(r1, r2) and torch.equal(d1, d2) and torch.equal(o1, o2)
+
+
 def test_lunar_lander_autoreset_equals_step_then_selective_reset(mrl, ctx):
     batch = 1000
     E = mrl.LunarLanderV2
@@ -313,7 +381,8 @@ def test_half_cheetah_rollout_parity(mrl, orc, ctx, batch, seed):
     assert d_h.sum() == 0 or True
 
 
-@pytest.mark.parametrize("name", ["CartPoleEnv", "PendulumV2", "BipedalWalkerV2", "HalfCheetahPlanarV2"])
+@pytest.mark.parametrize("name", ["CartPoleEnv", "PendulumV2", "BipedalWalkerV2", "HalfCheetahPlanarV2",
+                                  "LunarLanderV2Continuous"])
 def test_autoreset_equals_step_then_selective_reset(mrl, ctx, name):
     E = getattr(mrl, name)
     batch = 777
@@ -334,6 +403,8 @@ def test_autoreset_equals_step_then_selective_reset(mrl, ctx, name):
             a = (torch.rand(batch * aw, device="cuda", generator=g) * 2 - 1) * 1.2
         if name == "PendulumV2" and t == 0:
             s1.view(batch, 8)[:, 4] = 170; s2.view(batch, 8)[:, 4] = 170
+        if name == "LunarLanderV2Continuous" and t == 0:
+            s1.view(batch, 192)[:, 188] = 970; s2.view(batch, 192)[:, 188] = 970
         E.step_kernel_gpu(ctx, s1, a, r1, d1, o1, t)
         dstep = d1.clone()
         E.selective_reset_kernel_gpu(ctx, s1, d1, 50 + t)

@@ -41,3 +41,19 @@ def test_continuous_agent_improves_pendulum(mrl):
     # the log_std clamp holds
     ls = agent.actor.params[-1:]
     assert (ls >= -5.0).all() and (ls <= 2.0).all()
+
+
+def test_continuous_agent_runs_on_the_continuous_lunar_lander(mrl):
+    """The continuous-action LunarLander overload behind the continuous agent: the fused collection
+    kernel (hidden width 256), GAE and the update run and keep every buffer finite."""
+    ctx = mrl.DeviceContext("cuda:0")
+    agent = mrl.DeepPPOContinuousAgent(obs_dim=8, action_dim=2, hidden_dim=256, rollout_len=64, n_envs=512,
+                                       gpu_minibatch_size=4096, num_epochs=2, target_kl=0.0, init_seed=3)
+    m = agent.train_gpu(ctx, mrl.LunarLanderV2Continuous, num_episodes=10**9, max_rollouts=3, seed=2)
+    assert mrl.ppo.rollout_fused(agent.rb.descriptor())
+    assert m.rollouts == 3 and m.total_steps == 3 * 64 * 512
+    assert len(m.episode_rewards) > 0 and all(np.isfinite(m.episode_rewards))
+    assert torch.isfinite(agent.actor.params).all() and torch.isfinite(agent.critic.params).all()
+    assert torch.isfinite(agent.rb.states).all()
+    got = agent.evaluate_gpu(ctx, mrl.LunarLanderV2Continuous, num_episodes=64, max_steps=400)
+    assert np.isfinite(got) and got < 0.0     # three rollouts do not make a pilot

@@ -207,3 +207,84 @@ def test_batch_matches_single(orc):
     s2 = s.copy()
     orc.orc_ll_selective_reset_batch(s2, dn, n, 78)
     assert np.array_equal(s2[np.arange(n) != 3], s[np.arange(n) != 3]) and s2[3, META] == 0
+
+
+# ---------------------------------------------------------------- continuous-action overload
+
+def step_c(orc, row, a0, a1, env=0):
+    r, d = np.zeros(1, np.float32), np.zeros(1, np.float32)
+    orc.orc_ll_step_continuous(row, env, a0, a1, r, d, None, None)
+    return float(r[0]), float(d[0])
+
+
+def test_continuous_corner_actions_are_the_discrete_actions(orc):
+    """Full throttle / full side control / nothing decode to the powers of the four discrete
+    actions, so the whole step (state, reward, done) must agree bit for bit -- also beyond the
+    clipping range and for several steps in a row."""
+    table = {0: (-1.0, 0.0), 2: (1.0, 0.3), 1: (-1.0, -1.0), 3: (-1.0, 1.0)}
+    beyond = {0: (-3.0, -0.5), 2: (7.0, 0.5), 1: (-1.5, -4.0), 3: (-2.0, 9.0)}
+    for tab in (table, beyond):
+        for action, (a0, a1) in tab.items():
+            a, b = fresh(orc, 13, env=3), fresh(orc, 13, env=3)
+            for _ in range(5):
+                ra, da, _, _ = step(orc, a, action, env=3)
+                rb, db = step_c(orc, b, a0, a1, env=3)
+                assert (ra, da) == (rb, db)
+                assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_continuous_powers_scale_the_engine_impulse_and_the_fuel_cost(orc):
+    base = fresh(orc, 17)
+    vy0 = {}
+    # main engine: the velocity change of the hull against the unpowered step is linear in the throttle
+    noop = base.copy(); step_c(orc, noop, -1.0, 0.0)
+    full = base.copy(); step_c(orc, full, 1.0, 0.0)
+    for a0 in (-0.5, 0.0, 0.5):
+        p = (a0 + 1.0) / 2.0
+        row = base.copy()
+        prev = float(row[META + 2])
+        r, _ = step_c(orc, row, a0, 0.0)
+        for k in (3, 4, 5):
+            want = noop[BOD + k] + p * (full[BOD + k] - noop[BOD + k])
+            assert abs(row[BOD + k] - want) < 2e-5, (a0, k)
+        o = row[:8]
+        sh = (-100 * math.hypot(o[0], o[1]) - 100 * math.hypot(o[2], o[3]) - 100 * abs(o[4]) + 10 * o[6] + 10 * o[7])
+        assert abs(r - (sh - prev - 0.30 * p)) < 2e-3
+    # side engine: dead band up to |a1| = 0.5, then power (|a1| - 0.5) * 2 with the sign as direction
+    for a1 in (-0.5, -0.2, 0.0, 0.5):
+        row = base.copy(); step_c(orc, row, -1.0, a1)
+        assert np.array_equal(row.view(np.uint32), noop.view(np.uint32))
+    left = base.copy(); step_c(orc, left, -1.0, -1.0)
+    right = base.copy(); step_c(orc, right, -1.0, 1.0)
+    for a1, ref in ((-0.75, left), (0.75, right), (0.9, right)):
+        s = (abs(a1) - 0.5) * 2.0
+        row = base.copy()
+        prev = float(row[META + 2])
+        r, _ = step_c(orc, row, -1.0, a1)
+        for k in (3, 4, 5):
+            want = noop[BOD + k] + s * (ref[BOD + k] - noop[BOD + k])
+            assert abs(row[BOD + k] - want) < 2e-5, (a1, k)
+        o = row[:8]
+        sh = (-100 * math.hypot(o[0], o[1]) - 100 * math.hypot(o[2], o[3]) - 100 * abs(o[4]) + 10 * o[6] + 10 * o[7])
+        assert abs(r - (sh - prev - 0.03 * s)) < 2e-3
+    # both engines at once: the impulses add
+    both = base.copy(); step_c(orc, both, 0.0, 0.75)
+    half = base.copy(); step_c(orc, half, 0.0, 0.0)
+    side = base.copy(); step_c(orc, side, -1.0, 0.75)
+    for k in (3, 4, 5):
+        assert abs(both[BOD + k] - (half[BOD + k] + side[BOD + k] - noop[BOD + k])) < 2e-5
+
+
+def test_continuous_batch_matches_single(orc):
+    n = 6
+    states = np.zeros((n, 192), np.float32)
+    orc.orc_ll_reset_batch(states, n, 21)
+    singles = states.copy()
+    g = np.random.default_rng(2)
+    acts = g.uniform(-1.3, 1.3, size=(n, 2)).astype(np.float32)
+    rew, don, obs = np.zeros(n, np.float32), np.zeros(n, np.float32), np.zeros((n, 8), np.float32)
+    orc.orc_ll_step_continuous_batch(states, acts, rew, don, obs, n)
+    for i in range(n):
+        r, d = step_c(orc, singles[i], float(acts[i, 0]), float(acts[i, 1]), env=i)
+        assert r == rew[i] and d == don[i]
+    assert np.array_equal(states, singles) and np.array_equal(obs, states[:, :8])
