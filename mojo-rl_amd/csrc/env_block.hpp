@@ -92,26 +92,45 @@ struct LunarLanderContinuous : LunarLander {
 
 struct BipedalWalker {
     using L = bw::L;
-    static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 32, THREADS = 256;
+    static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 16, THREADS = 512;
     static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = bw::NSHAPE_FLOATS;
     // the ten lidar rays of the observation are left out of the step and run afterwards, spread
-    // over all wavefronts of the block (task k = ray k)
-    static constexpr int POST_TASKS = 10;
+    // over all wavefronts of the block: task k = half k % 2 of the edges for ray k / 2.  The two
+    // halves of a ray sit EPB lanes apart in one wavefront and exchange their minima there.
+    static constexpr int POST_TASKS = 20;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
         bw::step_row<false>(row, cts, shapes, env, a, r, d);
     }
-    static MRL_DEV void post_task(float *row, int task) { row[14 + task] = bw::lidar_value(row, task, nullptr); }
+    static MRL_DEV void post_task(float *row, int task) {
+        static_assert(2 * EPB <= 64 && (THREADS / EPB) % 2 == 0 && POST_TASKS % 2 == 0, "both halves of a ray in one wavefront, in the same pass");
+        float t = bw::lidar_value_part(row, task >> 1, task & 1, 2);
+        const float other = __shfl_xor(t, EPB, 64);
+        t = other < t ? other : t;
+        if ((task & 1) == 0) row[14 + (task >> 1)] = t;
+    }
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { bw::reset_row(row, walker_seed(seed, env)); }
     static constexpr bool WAVE_RESET = true;
     static MRL_DEV void reset_wave(float *row, uint64_t seed, int env, int lane) {
         bw::reset_row_wave(row, walker_seed(seed, env), lane);
     }
-    static constexpr int DETECT_TASKS = 0;
-    static MRL_DEV void detect_task(int, int &, int &, int &) {}
-    struct Carry {};
-    static MRL_DEV Carry step_begin(float *, int, const float *) { return Carry{}; }
-    static MRL_DEV void step_finish(float *, float *, int, const float *, const Carry &, float &, float &) {}
+    // contact detection ahead of the step, spread over all wavefronts: one (body, vertex) pair of
+    // one env per lane -- hull 5 vertices, the four leg segments 4 each, against the 128 edges
+    static constexpr int DETECT_TASKS = 21;
+    static MRL_DEV void detect_task(int k, int &body, int &vertex, int &max_verts) {
+        if (k < 5) { body = 0; vertex = k; max_verts = 5; }
+        else { body = 1 + (k - 5) / 4; vertex = (k - 5) % 4; max_verts = 4; }
+    }
+    struct Carry { float act[bw::ACT]; };
+    static MRL_DEV Carry step_begin(float *row, int, const float *a) {
+        Carry c;
+        bw::step_motors(row, a, c.act);
+        return c;
+    }
+    static MRL_DEV void step_finish(float *row, float *cts, int n, const float *shapes, const Carry &c, float &r,
+                                    float &d) {
+        bw::step_finish<false>(row, cts, n, shapes, c.act, r, d);
+    }
 };
 
 struct HalfCheetah {
@@ -304,7 +323,7 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
                              float *dones, int env0, int nenv, uint64_t reset_seed, const Accounting &acc,
                              int tid = threadIdx.x) {
     using S = Stage<E>;
-    if constexpr (E::DETECT_TASKS > 0) {
+    if constexpr (E::DETECT_TASKS > 0 && E::POST_TASKS == 0) {
         // wavefront 0: first half of the step (reads and writes velocities only); the halves of the
         // other wavefronts: contacts of one (body, vertex) pair each (read positions only), into
         // lists of their own.  A vertex that fills its list, or a body whose shape the task table
@@ -341,14 +360,34 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
             if (AUTORESET) reset_rows<E>(rows, was_reset, __ballot(finished), reset_seed, env0, lane);
         }
     } else {
+        typename E::Carry carry{};
+        if constexpr (E::DETECT_TASKS > 0) {
+            // first the contacts, by every wavefront: EPB lanes per (body, vertex) pair, as many
+            // pairs at a time as the block has such lane groups; the lanes that will step the envs
+            // put the action into the joint motors first (detection does not read the joints)
+            static_assert(WAVE % E::EPB == 0 && E::EPB <= WAVE, "lane groups of EPB inside a wavefront");
+            constexpr int SLOTS = E::THREADS / E::EPB;
+            const int e = tid % E::EPB;
+            if (tid < nenv) carry = E::step_begin(rows + tid * S::STRIDE, env0 + tid, actions + (size_t)tid * E::ACT_W);
+            if (e < nenv)
+                for (int task = tid / E::EPB; task < E::DETECT_TASKS; task += SLOTS)
+                    detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
+            __syncthreads();
+        }
         if (tid < WAVE) {
             bool finished = false;
             if (tid < nenv) {
                 const int env = env0 + tid;
                 const EpisodeSums sums = account_before(acc, tid);
                 float r, d;
-                E::step(rows + tid * S::STRIDE, cts + tid * S::CSTRIDE, shapes, env,
-                        actions + (size_t)tid * E::ACT_W, r, d);
+                if constexpr (E::DETECT_TASKS > 0) {
+                    float *mine = cts + tid * S::CSTRIDE;
+                    const int n = merge_vertex_lists<E>(dlist, dcount, tid, mine);
+                    E::step_finish(rows + tid * S::STRIDE, mine, n, shapes, carry, r, d);
+                } else {
+                    E::step(rows + tid * S::STRIDE, cts + tid * S::CSTRIDE, shapes, env,
+                            actions + (size_t)tid * E::ACT_W, r, d);
+                }
                 if (rewards != nullptr) {
                     rewards[env - env0] = r;
                     dones[env - env0] = d;

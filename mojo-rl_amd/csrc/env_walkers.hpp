@@ -119,6 +119,30 @@ MRL_DEV float lidar_value(const float *row, int i, const EdgeMask<L> *near) {
     return lidar_ray_near<L>(row, mine, hull_x, hull_y, cs * lidar_range, sn * lidar_range);
 }
 
+// Lidar ray i against a share of the edges only: part `part` of `nparts` takes the edges of the
+// mask words [part * WORDS / nparts, (part + 1) * WORDS / nparts); the ray's value is the minimum
+// over the parts (every part starts from 1, the value of a ray that hits nothing, and a hit
+// replaces it only by something smaller: the minimum over all edges, however they are grouped).
+// The edge set is picked for the ray's own x extent.
+MRL_DEV float lidar_value_part(const float *row, int i, int part, int nparts) {
+    const float *B = row + L::BODIES_OFF;
+    const float hull_x = B[IDX_X], hull_y = B[IDX_Y], hull_angle_rad = B[IDX_ANGLE];
+    const float lidar_range = (float)LIDAR_RANGE;
+    float local_angle = (float)i * 1.5f / (float)9;
+    float world_angle = hull_angle_rad - local_angle - (float)(3.14159265358979323846 / 2.0);
+    float sn, cs;
+    sincos32(world_angle, sn, cs);
+    const float rdx = cs * lidar_range, rdy = sn * lidar_range;
+    if (!(hull_x == hull_x)) return part == 0 ? lidar_ray<L>(row, hull_x, hull_y, rdx, rdy) : 1.0f;
+    const float end_x = hull_x + rdx;
+    const float lo = hull_x < end_x ? hull_x : end_x, hi = hull_x < end_x ? end_x : hull_x;
+    if (!(lo == lo && hi == hi)) return part == 0 ? lidar_ray<L>(row, hull_x, hull_y, rdx, rdy) : 1.0f;
+    constexpr int W = EdgeMask<L>::WORDS;
+    EdgeMask<L> mine;
+    edges_near<L>(row, lo, hi, 0.02f, mine, part * W / nparts, (part + 1) * W / nparts);
+    return lidar_ray_near<L>(row, mine, hull_x, hull_y, rdx, rdy);
+}
+
 MRL_DEV void observe(float *row) {
     float o[OBS];
     observe_state(row, o);
@@ -273,12 +297,13 @@ MRL_DEV void reset_row_wave(float *row, uint64_t cseed, int lane) {
     wave_sync();
 }
 
+// An env step in two halves, so that contact detection (which reads body positions, shapes and
+// edges only) can run on other lanes beside the first:
+//   step_motors   the action into the joint motors (writes joints only); act = the raw action
+//   step_finish   physics with the `n_given` contacts in `contacts` (n_given < 0: detect here),
+//                 contact flags, observation, reward, termination.
 // LIDAR = false: the lidar entries of the observation (14 .. 23) are left to the caller
-template <bool LIDAR = true>
-MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env, const float *action,
-                      float &reward, float &done) {
-    (void)env;
-    float act[ACT];
+MRL_DEV void step_motors(float *row, const float *action, float *act) {
 #pragma unroll
     for (int j = 0; j < ACT; ++j) {
         act[j] = action[j];
@@ -290,8 +315,13 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
         J[J_MOTOR_SPEED] = sign * (float)((j & 1) ? 6.0 : 4.0);
         J[J_MAX_TORQUE] = (float)MOTORS_TORQUE * fabsf(a);
     }
+}
+
+template <bool LIDAR = true>
+MRL_DEV void step_finish(float *row, float *contacts, int n_given, const float *shapes, const float *act,
+                         float &reward, float &done) {
     int n = reg_physics_substep<L, Topology, false, false>(row, shapes, contacts, (float)0.0, (float)-10.0, (float)(1.0 / FPS),
-                                      (float)2.5, (float)0.0, (float)0.2, (float)0.005, 6, 2);
+                                      (float)2.5, (float)0.0, (float)0.2, (float)0.005, 6, 2, n_given);
     bool left = false, right = false, hull = false;
     for (int c = 0; c < n; ++c) {
         int b = (int)contacts[c * CONTACT_SIZE + C_BODY_A];
@@ -338,6 +368,15 @@ MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env,
     M[META_DONE] = terminated ? 1.0f : 0.0f;
     reward = r;
     done = terminated ? 1.0f : 0.0f;
+}
+
+template <bool LIDAR = true>
+MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env, const float *action,
+                      float &reward, float &done) {
+    (void)env;
+    float act[ACT];
+    step_motors(row, action, act);
+    step_finish<LIDAR>(row, contacts, -1, shapes, act, reward, done);
 }
 }  // namespace bw
 

@@ -120,6 +120,10 @@ MRL_DEV bool edge_x_pass(float e_x0, float e_x1, float world_x) {
     return !(world_x < x_min || world_x > x_max);
 }
 
+// bits [0, n) of a 32-bit word, n clamped to [0, 32]: the edges of mask word q that exist are
+// word_bits(n_edges - 32 q)
+MRL_DEV unsigned word_bits(int n) { return n >= 32 ? 0xffffffffu : (n <= 0 ? 0u : (1u << n) - 1u); }
+
 // Bit e of a mask is set when terrain edge e can matter for an x interval.
 template <class L>
 struct EdgeMask {
@@ -129,26 +133,36 @@ struct EdgeMask {
 
 // Edges whose x-range pre-check (edge_x_pass) can succeed for some x in [xlo, xhi]: a superset of
 // the edges any such vertex passes, decided with the same fp32 bounds the pre-check uses.
-// widen = 0 gives exactly that; lidar passes its own safety margin on top.
+// widen = 0 gives exactly that; lidar passes its own safety margin on top.  Only the mask words
+// [q0, q1) are worked out (a caller that splits the edges over several lanes); the rest is zero.
 template <class L>
-MRL_DEV void edges_near(const float *row, float xlo, float xhi, float widen, EdgeMask<L> &m) {
+MRL_DEV void edges_near(const float *row, float xlo, float xhi, float widen, EdgeMask<L> &m, int q0 = 0,
+                        int q1 = EdgeMask<L>::WORDS) {
     int n_edges = (int)row[L::EDGE_COUNT_OFF];
     if (n_edges > L::MAX_EDGES) n_edges = L::MAX_EDGES;
     const float *edges = row + L::EDGES_OFF;
 #pragma unroll
     for (int q = 0; q < EdgeMask<L>::WORDS; ++q) {
+        if (q < q0 || q >= q1) { m.w[q] = 0; continue; }
+        // every slot of the word is tested, whether the edge exists or not (the slots are inside the
+        // row), and the word is cut to the existing edges afterwards: no test depends on n_edges, so
+        // the loads of a round go out together instead of one by one behind a branch each
         unsigned bits = 0;
         const int e0 = q * 32;
-        for (int k = 0; k < 32; ++k) {
-            const int e = e0 + k;
-            if (e >= n_edges) break;
-            const float e_x0 = edges[e * 6], e_x1 = edges[e * 6 + 2];
-            const float margin = 0.1f;
-            float x_min = e_x0 - margin, x_max = e_x1 + margin;
-            if (e_x0 > e_x1) { x_min = e_x1 - margin; x_max = e_x0 + margin; }
-            if (!(xhi < x_min - widen || xlo > x_max + widen)) bits |= 1u << k;
+#pragma unroll 1
+        for (int k0 = 0; k0 < 32; k0 += 8) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int k = k0 + j, e = e0 + k;
+                if (e >= L::MAX_EDGES) continue;
+                const float e_x0 = edges[e * 6], e_x1 = edges[e * 6 + 2];
+                const float margin = 0.1f;
+                float x_min = e_x0 - margin, x_max = e_x1 + margin;
+                if (e_x0 > e_x1) { x_min = e_x1 - margin; x_max = e_x0 + margin; }
+                bits |= (unsigned)!(xhi < x_min - widen || xlo > x_max + widen) << k;
+            }
         }
-        m.w[q] = bits;
+        m.w[q] = bits & word_bits(n_edges - e0);
     }
 }
 
@@ -279,7 +293,6 @@ MRL_DEV int edge_detect(const float *row, const float *shapes, float *contacts) 
 template <class L>
 MRL_DEV int edge_detect_vertex(const float *row, const float *shapes, int b, int v, int max_verts,
                                float *contacts, int cap) {
-    static_assert(L::MAX_EDGES <= 32, "one mask word");
     const float *B = row + L::BODIES_OFF + b * BODY_SIZE;
     const float *S = shapes + (int)B[IDX_SHAPE] * SHAPE_SIZE;
     int n_verts = (int)S[1];
@@ -293,15 +306,24 @@ MRL_DEV int edge_detect_vertex(const float *row, const float *shapes, int b, int
     const float local_x = S[2 + v * 2], local_y = S[3 + v * 2];
     const float world_x = B[IDX_X] + local_x * cos_a - local_y * sin_a;
     const float world_y = B[IDX_Y] + local_x * sin_a + local_y * cos_a;
-    unsigned mask = 0;
-#pragma unroll
-    for (int e = 0; e < L::MAX_EDGES; ++e)
-        if (e < n_edges && edge_x_pass(edges[e * 6], edges[e * 6 + 2], world_x)) mask |= 1u << e;
+    // the x-range pre-check of 32 edges at a time into a bit mask, then the full test of the
+    // survivors in ascending order (the order edge_detect visits them in)
     int count = 0;
-    while (mask) {
-        const int e = __ffs((int)mask) - 1;
-        mask &= mask - 1;
-        vertex_edge_test(edges + e * 6, b, world_x, world_y, contacts, count, cap);
+#pragma unroll
+    for (int q = 0; q < (L::MAX_EDGES + 31) / 32; ++q) {
+        // (all slots tested, the word cut to the existing edges afterwards: see edges_near)
+        unsigned mask = 0;
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+            const int e = q * 32 + k;
+            if (e < L::MAX_EDGES) mask |= (unsigned)edge_x_pass(edges[e * 6], edges[e * 6 + 2], world_x) << k;
+        }
+        mask &= word_bits(n_edges - q * 32);
+        while (mask) {
+            const int e = q * 32 + __ffs((int)mask) - 1;
+            mask &= mask - 1;
+            vertex_edge_test(edges + e * 6, b, world_x, world_y, contacts, count, cap);
+        }
     }
     return count >= cap ? -1 : count;
 }
