@@ -52,16 +52,20 @@ struct HiddenOperands {
     float bv[TPW][KB];
 
     // tid: the caller's thread index (a caller that loops over many tiles may pass a copy the
-    // optimiser cannot see through, so that nothing derived from it is kept across iterations)
-    MRL_DEV void load(const float *__restrict__ p, int IN, int tid = threadIdx.x) {
+    // optimiser cannot see through, so that nothing derived from it is kept across iterations).
+    // tile0 / tiles: the column tiles of this wavefront when the caller deals them out itself
+    // (tiles <= TPW of them from tile0 on); by default wavefront w takes tiles TPW w .. TPW w + TPW - 1.
+    MRL_DEV void load(const float *__restrict__ p, int IN, int tid = threadIdx.x, int tile0 = -1, int tiles = 0) {
         constexpr int T = hidden_threads(H, TPW);
-        const int t = tid % T, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
+        const int t = tid % T, lane = tid & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
         const float *W0 = p, *b0 = p + IN * H;
         const float *W1 = b0 + H, *b1 = W1 + H * H;
         ntile = (H / 32) % TPW == 0 ? TPW : min(TPW, H / 32 - TPW * w);
+        if (tile0 < 0) tile0 = TPW * w;
+        else ntile = tiles;
 #pragma unroll
         for (int q = 0; q < TPW; ++q) {
-            col[q] = (TPW * w + q < H / 32 ? 32 * (TPW * w + q) : 0) + l31;
+            col[q] = (q < ntile && tile0 + q < H / 32 ? 32 * (tile0 + q) : 0) + l31;
             bias0[q] = b0[col[q]];
             bias1[q] = b1[col[q]];
         }
@@ -117,10 +121,11 @@ struct WaveGroupSync {
     }
 };
 
-template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32), bool H2_ON_HT = false, class Sync = BlockSync>
-MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
-                          const TileCache tc, HiddenOperands<H, TPW, KB> &ops, int tid = threadIdx.x,
-                          Sync &&sync = Sync()) {
+// NT = the column tiles this wavefront really has (ops.ntile, known at compile time here): the
+// MFMAs, weight loads and epilogues of the other TPW - NT slots are left out.
+template <int H, int ACT, int TPW, int KB, bool H2_ON_HT, int NT, class Sync>
+MRL_DEV void hidden_stack_tiles(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
+                                const TileCache tc, HiddenOperands<H, TPW, KB> &ops, int tid, Sync &sync) {
     static_assert(PR * (H + 1) <= H * HT_LD, "h2 fits into hT");
     constexpr int T = hidden_threads(H, TPW);
     constexpr int K0 = PIN_MAX / 2;
@@ -139,18 +144,17 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
         }
         floatx16 c[TPW];
 #pragma unroll
-        for (int q = 0; q < TPW; ++q) c[q] = floatx16{0};
+        for (int q = 0; q < NT; ++q) c[q] = floatx16{0};
 #pragma unroll
         for (int kk = 0; kk < K0; ++kk) {
             if (2 * kk < IN) {
 #pragma unroll
-                for (int q = 0; q < TPW; ++q)
+                for (int q = 0; q < NT; ++q)
                     c[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[kk], w0[q][kk], c[q], 0, 0, 0);
             }
         }
 #pragma unroll
-        for (int q = 0; q < TPW; ++q) {
-            if (q >= ops.ntile) continue;
+        for (int q = 0; q < NT; ++q) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = 8 * (v >> 2) + 4 * half + (v & 3);
@@ -168,7 +172,7 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
     {   // layer 1 (H x H): weights streamed from L2 one block of KB k-steps ahead of the MFMAs
         floatx16 c[TPW];
 #pragma unroll
-        for (int q = 0; q < TPW; ++q) c[q] = floatx16{0};
+        for (int q = 0; q < NT; ++q) c[q] = floatx16{0};
         float a[KB], na[KB], nb[TPW][KB];
 #pragma unroll
         for (int j = 0; j < KB; ++j) a[j] = hT[(2 * j + half) * HT_LD + l31];
@@ -180,13 +184,13 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
                     const int k = 2 * ((blk + 1) * KB + j) + half;
                     na[j] = hT[k * HT_LD + l31];
 #pragma unroll
-                    for (int q = 0; q < TPW; ++q) nb[q][j] = W1[k * H + col[q]];
+                    for (int q = 0; q < NT; ++q) nb[q][j] = W1[k * H + col[q]];
                 }
             }
 #pragma unroll
             for (int j = 0; j < KB; ++j) {
 #pragma unroll
-                for (int q = 0; q < TPW; ++q)
+                for (int q = 0; q < NT; ++q)
                     c[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], bv[q][j], c[q], 0, 0, 0);
             }
             if (more) {
@@ -194,14 +198,13 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
                 for (int j = 0; j < KB; ++j) {
                     a[j] = na[j];
 #pragma unroll
-                    for (int q = 0; q < TPW; ++q) bv[q][j] = nb[q][j];
+                    for (int q = 0; q < NT; ++q) bv[q][j] = nb[q][j];
                 }
             }
         }
         if (H2_ON_HT) sync();
 #pragma unroll
-        for (int q = 0; q < TPW; ++q) {
-            if (q >= ops.ntile) continue;
+        for (int q = 0; q < NT; ++q) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = 8 * (v >> 2) + 4 * half + (v & 3);
@@ -216,6 +219,22 @@ MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, 
         }
     }
     sync();
+}
+
+template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32), bool H2_ON_HT = false, class Sync = BlockSync>
+MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
+                          const TileCache tc, HiddenOperands<H, TPW, KB> &ops, int tid = threadIdx.x,
+                          Sync &&sync = Sync()) {
+    // ops.ntile is the same for all lanes of a wavefront; a wavefront with fewer tiles than slots
+    // runs the variant without the spare slots' work (every variant meets the same barriers)
+    if (ops.ntile >= TPW) return hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, TPW>(p, IN, xs, hT, h2, tc, ops, tid, sync);
+    if constexpr (TPW >= 3) {
+        if (ops.ntile == 2) return hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, 2>(p, IN, xs, hT, h2, tc, ops, tid, sync);
+    }
+    if constexpr (TPW >= 2) {
+        if (ops.ntile == 1) return hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, 1>(p, IN, xs, hT, h2, tc, ops, tid, sync);
+    }
+    hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, 0>(p, IN, xs, hT, h2, tc, ops, tid, sync);
 }
 
 // floats of LDS that hold one net's head parameters, every row padded to PA_MAX columns with

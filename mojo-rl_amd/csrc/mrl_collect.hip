@@ -50,8 +50,11 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     // the critic's wavefronts: the last three, so that none of them shares a SIMD with wavefront 0
     // (wavefronts of a workgroup go round the four SIMDs) and its solver keeps that SIMD's issue
     // slots to itself
-    constexpr int CRITIC_TPW = 3, CRITIC_T = hidden_threads(H, CRITIC_TPW), CRITIC_WAVE0 = NW - CRITIC_T / WAVE;
-    static_assert(E::EPB == PR && E::THREADS == 2 * H && NW == 8 && CRITIC_WAVE0 == 5, "one 32-row policy tile per block");
+    // the critic runs on the six wavefronts that do not share a SIMD with wavefront 0 (1, 2, 3, 5, 6,
+    // 7: two per SIMD, so that one's MFMAs cover the other's loads and epilogues); its eight column
+    // tiles are dealt out 3 / 3 / 2 per SIMD
+    constexpr int CRITIC_TPW = 2, CRITIC_WAVES = 6, CRITIC_T = CRITIC_WAVES * WAVE;
+    static_assert(E::EPB == PR && E::THREADS == 2 * H && NW == 8 && H == 256, "one 32-row policy tile per block");
     static_assert(IN <= PIN_MAX && AW <= PA_MAX && E::DETECT_TASKS > 0, "policy tile limits; split-off detection");
     __shared__ float rows[PR * S::STRIDE];
     __shared__ float xs[PR * XS_LD];
@@ -93,13 +96,13 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     const bool owner = t < nenv;
     float ep_return = owner ? a.acc.ep_return[env0 + t] : 0.0f;
     float ep_length = owner ? a.acc.ep_length[env0 + t] : 0.0f;
-    WaveGroupSync critic_sync{&sync_critic, 0u, (unsigned)(NW - CRITIC_WAVE0)};
+    WaveGroupSync critic_sync{&sync_critic, 0u, (unsigned)CRITIC_WAVES};
     WaveGroupSync detect_sync{&sync_detect, 0u, (unsigned)(NW - 1)};
     static_assert((E::DETECT_TASKS + 1) / 2 <= NW - 1, "two detection tasks per wavefront besides wavefront 0");
 
     // Per step: every wavefront runs the actor (the action is what the env step waits for); then
-    // wavefront 0 samples and steps the envs, wavefronts 1 .. 7 detect their contacts, and
-    // wavefronts 5 .. 7 go on to run the critic, whose value is only stored -- off the critical path.
+    // wavefront 0 samples and steps the envs, wavefronts 1 .. 7 detect their contacts, and all of
+    // these but wavefront 4 go on to run the critic, whose value is only stored -- off the critical path.
     for (int k = 0; k < a.n_steps; ++k) {
         // Nothing but the rows is carried from one step to the next: the thread index, the block's
         // env count and the parameter pointers pass through empty asm statements at the top of each
@@ -182,13 +185,14 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
             const int task = (wave - 1) * 2 + lane / (WAVE / 2), e = lane % (WAVE / 2);
             if (task < E::DETECT_TASKS && e < ne) detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
             detect_sync.arrive();
-            if (wave >= CRITIC_WAVE0) {
-                // ---- critic, on its own barrier.  (One wavefront per SIMD here: blocks of 16 k-steps,
-                // so that a block's MFMAs cover the L2 latency of the next block's weights without a
-                // second wavefront's help.)
-                const int tl = tid - CRITIC_WAVE0 * WAVE;   // index among the critic's threads
+            if (wave != 4) {
+                // ---- critic, on its own barrier: member g = 0 .. 5 of the group is wavefront g + 1
+                // (g < 3) or g + 2; members g and g + 3 share a SIMD and take tiles {2, 1}, {2, 1}, {1, 1}
+                const int g = wave < 4 ? wave - 1 : wave - 2;
+                const int tl = g * WAVE + lane;   // index among the critic's threads
+                const int tile0 = g < 2 ? 2 * g : g + 2, tiles = g < 2 ? 2 : 1;
                 HiddenOperands<H, CRITIC_TPW, 16> ops;
-                ops.load(pc, IN, tl);
+                ops.load(pc, IN, tl, tile0, tiles);
                 hidden_stack<H, ACT, CRITIC_TPW, 16, true>(pc, IN, xs, hTc, hTc, TileCache{}, ops, tl, critic_sync);
                 head<H>(w2s[1], 1, hTc, vals, 1, tl, CRITIC_T);
             }
