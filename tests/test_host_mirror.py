@@ -57,7 +57,8 @@ def test_bad_descriptions_raise(mrl):
 
 def test_env_constants_match_the_library_and_the_oracle_layouts(mrl, orc, orcmod):
     want = {"CartPoleEnv": (4, 4, 2, 0), "PendulumV2": (8, 3, 0, 1), "LunarLanderV2": (192, 8, 4, 0),
-            "BipedalWalkerV2": (950, 24, 0, 4), "HalfCheetahPlanarV2": (253, 17, 0, 6)}
+            "LunarLanderV2Continuous": (192, 8, 0, 2), "BipedalWalkerV2": (950, 24, 0, 4),
+            "HalfCheetahPlanarV2": (253, 17, 0, 6)}
     for name, (ss, od, na, ad) in want.items():
         E = getattr(mrl, name)
         assert (E.STATE_SIZE, E.OBS_DIM, E.NUM_ACTIONS, E.ACTION_DIM) == (ss, od, na, ad)
@@ -77,6 +78,10 @@ def test_null_context_is_an_error_not_a_crash(mrl):
         mrl._lib.call("mrl_gae", None, 1, 1, None, None, None, None, 0.99, 0.95, None, None)
     with pytest.raises(mrl.MrlError):
         mrl._lib.call("mrl_permutation", None, None, 10, 1)
+    with pytest.raises(mrl.MrlError, match="ctx"):
+        mrl._lib.call("mrl_greedy_actions", None, None, 4, 2, 0, None)
+    with pytest.raises(mrl.MrlError, match="NULL"):
+        mrl._lib.call("mrl_rollout_steps", None, None, 0, 1, 0, 0, 0, 0, 0, 0)
     assert b"" != mrl._lib.lib().mrl_last_error()
 
 
