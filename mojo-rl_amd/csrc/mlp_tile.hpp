@@ -263,25 +263,28 @@ MRL_DEV void stage_head(const float *__restrict__ W2, int H, int A, bool with_lo
     }
 }
 
-// out[r][a] = h2[r] . W2[:, a] + b2[a] for the block's rows; TPR = H/32 lanes cooperate per row,
-// each over 32 consecutive columns that it walks from a different starting point (the lanes of a
-// wavefront then read distinct LDS banks).  w2s: the head parameters in LDS (stage_head).
+// out[r][a] = h2[r] . W2[:, a] + b2[a] for the block's rows; TPR = H/16 lanes cooperate per row,
+// each over 16 consecutive columns that it walks from a different starting point (the lanes of a
+// wavefront then spread over the LDS banks, for the activations and for the padded weight rows
+// alike), and add their sums up in a butterfly.  The result does not depend on how many threads
+// share the work: the 2 H (row, part) pairs are dealt out nthreads at a time.
+// w2s: the head parameters in LDS (stage_head).
 // NA = outputs carried per lane (1, 4 or 8 >= A): narrower heads read less of each padded row.
 template <int H, int NA>
 MRL_DEV void head_rows(const float *w2s, int A, const float *h2, float *out, int out_ld, int t, int nthreads) {
-    constexpr int TPR = H / PR;
+    constexpr int CP = 16, TPR = H / CP;
     static_assert(64 % TPR == 0, "the lanes of a row sit in one wavefront");
     static_assert(PA_MAX == 8 && (NA == 1 || NA == 4 || NA == 8), "one float, one float4 or two per padded row");
     const float *b2 = w2s + HEAD_B2(H);
-    // (row, part) pairs are dealt out PR * TPR = H at a time; nthreads must be a multiple of TPR
-    for (int pair = t; pair < H; pair += nthreads) {
+    // nthreads must be a multiple of TPR
+    for (int pair = t; pair < PR * TPR; pair += nthreads) {
         const int r = pair / TPR, part = pair % TPR;
         float acc[NA];
 #pragma unroll
         for (int a = 0; a < NA; ++a) acc[a] = 0.0f;
 #pragma unroll 8
-        for (int i = 0; i < PR; ++i) {
-            const int n = part * PR + ((i + 4 * part) & (PR - 1));
+        for (int i = 0; i < CP; ++i) {
+            const int n = part * CP + ((i + part) & (CP - 1));
             const float hv = h2[r * (H + 1) + n];
             if (NA == 1) {
                 acc[0] = fmaf(hv, w2s[n * PA_MAX], acc[0]);
@@ -306,8 +309,8 @@ MRL_DEV void head_rows(const float *w2s, int A, const float *h2, float *out, int
     }
 }
 
-// t = index of the calling thread among the `nthreads` (a multiple of H / 32) that share the work;
-// by default the first H threads of the net call it, one (row, part) pair each
+// t = index of the calling thread among the `nthreads` (a multiple of H / 16) that share the work;
+// by default the first H threads of the net call it, two (row, part) pairs each
 template <int H>
 MRL_DEV void head(const float *w2s, int A, const float *h2, float *out, int out_ld, int t = threadIdx.x % H,
                   int nthreads = H) {

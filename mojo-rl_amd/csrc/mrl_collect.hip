@@ -129,7 +129,7 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
             }
             __syncthreads();
             hidden_stack<H, ACT, 1, 32, true>(pa, IN, xs, overlay, overlay, TileCache{}, ops, tid);
-            if (tid < H) head<H>(w2s[0], A, overlay, logits, PA_MAX + 1, tid);
+            head<H>(w2s[0], A, overlay, logits, PA_MAX + 1, tid, E::THREADS);
             __syncthreads();   // logits complete; the actor's tile is dead from here on
         }
         if (wave == 0) {
@@ -311,10 +311,8 @@ __global__ __launch_bounds__(CLASSIC_THREADS) void collect_classic_kernel(Collec
         }
         __syncthreads();
         hidden_stack<H, ACT, TPW, KB>(p, IN, xs, hT[net], h2[net], TileCache{}, ops, tid);
-        if (tid % TN < H) {
-            if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1, tid % H);
-            else head<H>(w2s[1], 1, h2[1], vals, 1, tid % H);
-        }
+        if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1, tid % TN, TN);
+        else head<H>(w2s[1], 1, h2[1], vals, 1, tid % TN, TN);
         __syncthreads();
         if (tid < ne) {
             const int i = env0 + tid;

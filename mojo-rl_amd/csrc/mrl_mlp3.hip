@@ -70,7 +70,7 @@ __global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets
     }
     __syncthreads();
     hidden_stack<H, ACT, 1>(params, IN, xs, hT, h2, tc, ops);
-    if (t < H) head<H>(w2s, A, h2, ys, PA_MAX + 1);
+    head<H>(w2s, A, h2, ys, PA_MAX + 1, t, 2 * H);
     __syncthreads();
     const int ld = GAUSS ? 2 * A : A;
     for (int i = t; i < nrow * ld; i += T) {
@@ -423,7 +423,7 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
     }
     __syncthreads();
     hidden_stack<H, ACT, 1>(params, IN, xs, hT, h2, tc, ops);
-    if (t < H) head<H>(w2s, A, h2, ys, PA_MAX + 1);
+    head<H>(w2s, A, h2, ys, PA_MAX + 1, t, 2 * H);
     __syncthreads();
     for (int i = t; i < nrow * ld; i += T) {
         const int r = i / ld, a = i - r * ld;

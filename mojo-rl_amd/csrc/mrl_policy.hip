@@ -66,10 +66,8 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
     __syncthreads();
 
     hidden_stack<H, ACT, TPW, 8>(p, IN, xs, hT[net], h2[net], TileCache{}, ops);
-    if (t % TN < H) {
-        if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1);
-        else head<H>(w2s[1], 1, h2[1], vals, 1);
-    }
+    if (net == 0) head<H>(w2s[0], A, h2[0], logits, PA_MAX + 1, t % TN, TN);
+    else head<H>(w2s[1], 1, h2[1], vals, 1, t % TN, TN);
     __syncthreads();
 
     if (t < nrow && !GAUSS) {   // categorical sampling, one lane per env
