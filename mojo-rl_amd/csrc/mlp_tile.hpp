@@ -187,6 +187,9 @@ MRL_DEV void hidden_stack_tiles(const float *__restrict__ p, int IN, const float
                     for (int q = 0; q < NT; ++q) nb[q][j] = W1[k * H + col[q]];
                 }
             }
+            // the next block's loads stay ahead of this block's MFMAs (left alone, the scheduler moves
+            // them behind the MFMAs, next to their first use, and their latency is no longer hidden)
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < KB; ++j) {
 #pragma unroll
