@@ -6,12 +6,11 @@
 // LDS (staged there with coalesced loads, lane stride odd so that lanes hit distinct
 // banks); `contacts` is this lane's [MAX_CONTACTS][9] scratch, also in LDS.
 //
-// Arithmetic follows the CPU statement of the reference line by line
-// (integrators/euler.mojo:82-183, collision/edge_terrain.mojo:174-408,
-// collision/flat_terrain.mojo:69-204, solvers/impulse.mojo:94-402,
-// joints/revolute.mojo:69-495, lidar/lidar.mojo:25-141); the one restructuring is that
-// the joint anchors' world offsets are computed once per phase in which the angles
-// cannot change (the velocity iterations), which yields the same values.
+// This file: the row layout, contact detection against the terrain (collision/edge_terrain.mojo:
+// 174-408, collision/flat_terrain.mojo:69-204) and the lidar ray test (lidar/lidar.mojo:25-141),
+// arithmetic as in the CPU statement of the reference line by line.  The integrators and the
+// Gauss-Seidel sweeps (integrators/euler.mojo, solvers/impulse.mojo, joints/revolute.mojo) run on
+// registers: physics2d_reg.hpp.
 #pragma once
 #include "mrl_device.hpp"
 
@@ -47,44 +46,6 @@ struct Layout {
 using LunarLanderLayout = Layout<3, 8, 2, 16, 8, 4, 3>;      // physics2d/layout.mojo:247-255
 using BipedalWalkerLayout = Layout<5, 20, 4, 128, 24, 8, 5>; // :280-288
 using HalfCheetahLayout = Layout<7, 14, 6, 2, 17, 8, 7>;     // :291-299
-
-template <class L>
-MRL_DEV void integrate_velocities(float *row, float gx, float gy, float dt) {
-    for (int b = 0; b < L::NUM_BODIES; ++b) {
-        float *B = row + L::BODIES_OFF + b * BODY_SIZE;
-        float inv_mass = B[IDX_INV_MASS], inv_inertia = B[IDX_INV_INERTIA];
-        if (inv_mass == 0.0f) continue;
-        const float *F = row + L::FORCES_OFF + b * 3;
-        float vx = B[IDX_VX], vy = B[IDX_VY], omega = B[IDX_OMEGA];
-        vx = vx + (F[0] * inv_mass + gx) * dt;
-        vy = vy + (F[1] * inv_mass + gy) * dt;
-        omega = omega + F[2] * inv_inertia * dt;
-        B[IDX_VX] = vx; B[IDX_VY] = vy; B[IDX_OMEGA] = omega;
-    }
-}
-
-template <class L>
-MRL_DEV void integrate_positions(float *row, float dt) {
-    const float pi_val = (float)3.14159265358979323846;
-    const float two_pi = (float)(2.0 * 3.14159265358979323846);
-    for (int b = 0; b < L::NUM_BODIES; ++b) {
-        float *B = row + L::BODIES_OFF + b * BODY_SIZE;
-        if (B[IDX_INV_MASS] == 0.0f) continue;
-        float x = B[IDX_X] + B[IDX_VX] * dt;
-        float y = B[IDX_Y] + B[IDX_VY] * dt;
-        float angle = B[IDX_ANGLE] + B[IDX_OMEGA] * dt;
-        if (angle > 100.0f || angle < -100.0f) {
-            angle = 0.0f;
-        } else if (angle > pi_val) {
-            angle = angle - two_pi;
-            if (angle > pi_val) angle = angle - two_pi;
-        } else if (angle < -pi_val) {
-            angle = angle + two_pi;
-            if (angle < -pi_val) angle = angle + two_pi;
-        }
-        B[IDX_X] = x; B[IDX_Y] = y; B[IDX_ANGLE] = angle;
-    }
-}
 
 MRL_DEV void put_contact(float *c, int body, float px, float py, float nx, float ny, float depth) {
     c[C_BODY_A] = (float)body; c[C_BODY_B] = -1.0f;
@@ -365,278 +326,6 @@ MRL_DEV int flat_detect(const float *row, const float *shapes, float ground_y, f
         }
     }
     return count;
-}
-
-// one Gauss-Seidel sweep over the contact list (body B is always the ground in these envs;
-// the body-B branch is kept for contacts between two bodies)
-template <class L>
-MRL_DEV void contact_solve_velocity(float *row, float *contacts, int count, float friction,
-                                    float restitution) {
-    for (int c = 0; c < count; ++c) {
-        float *C = contacts + c * CONTACT_SIZE;
-        int ia = (int)C[C_BODY_A], ib = (int)C[C_BODY_B];
-        float point_x = C[C_PX], point_y = C[C_PY], normal_x = C[C_NX], normal_y = C[C_NY];
-        float *A = row + L::BODIES_OFF + ia * BODY_SIZE;
-        float *Bb = row + L::BODIES_OFF + (ib >= 0 ? ib : 0) * BODY_SIZE;
-        const bool hasb = ib >= 0;
-        float pos_a_x = A[IDX_X], pos_a_y = A[IDX_Y];
-        float vel_a_x = A[IDX_VX], vel_a_y = A[IDX_VY], omega_a = A[IDX_OMEGA];
-        float inv_mass_a = A[IDX_INV_MASS], inv_inertia_a = A[IDX_INV_INERTIA];
-        float inv_mass_b = 0.0f, inv_inertia_b = 0.0f, vel_b_x = 0.0f, vel_b_y = 0.0f, omega_b = 0.0f;
-        float pos_b_x = point_x, pos_b_y = point_y;
-        if (hasb) {
-            pos_b_x = Bb[IDX_X]; pos_b_y = Bb[IDX_Y];
-            vel_b_x = Bb[IDX_VX]; vel_b_y = Bb[IDX_VY]; omega_b = Bb[IDX_OMEGA];
-            inv_mass_b = Bb[IDX_INV_MASS]; inv_inertia_b = Bb[IDX_INV_INERTIA];
-        }
-        float ra_x = point_x - pos_a_x, ra_y = point_y - pos_a_y;
-        float rb_x = point_x - pos_b_x, rb_y = point_y - pos_b_y;
-        float vel_at_a_x = vel_a_x - omega_a * ra_y, vel_at_a_y = vel_a_y + omega_a * ra_x;
-        float vel_at_b_x = vel_b_x - omega_b * rb_y, vel_at_b_y = vel_b_y + omega_b * rb_x;
-        float rel_vel_x = vel_at_a_x - vel_at_b_x, rel_vel_y = vel_at_a_y - vel_at_b_y;
-        float vel_normal = rel_vel_x * normal_x + rel_vel_y * normal_y;
-        if (!(vel_normal < 0.0f)) continue;
-
-        float ra_cross_n = ra_x * normal_y - ra_y * normal_x;
-        float rb_cross_n = rb_x * normal_y - rb_y * normal_x;
-        float k = inv_mass_a + inv_mass_b;
-        k = k + inv_inertia_a * ra_cross_n * ra_cross_n;
-        k = k + inv_inertia_b * rb_cross_n * rb_cross_n;
-        float j_normal = -(1.0f + restitution) * vel_normal / k;
-        float old_impulse = C[C_JN];
-        float new_impulse = old_impulse + j_normal;
-        if (new_impulse < 0.0f) new_impulse = 0.0f;
-        C[C_JN] = new_impulse;
-        j_normal = new_impulse - old_impulse;
-        float impulse_x = j_normal * normal_x, impulse_y = j_normal * normal_y;
-        vel_a_x = vel_a_x + impulse_x * inv_mass_a;
-        vel_a_y = vel_a_y + impulse_y * inv_mass_a;
-        omega_a = omega_a + (ra_x * impulse_y - ra_y * impulse_x) * inv_inertia_a;
-        if (hasb) {
-            vel_b_x = vel_b_x - impulse_x * inv_mass_b;
-            vel_b_y = vel_b_y - impulse_y * inv_mass_b;
-            omega_b = omega_b - (rb_x * impulse_y - rb_y * impulse_x) * inv_inertia_b;
-        }
-        vel_at_a_x = vel_a_x - omega_a * ra_y; vel_at_a_y = vel_a_y + omega_a * ra_x;
-        vel_at_b_x = vel_b_x - omega_b * rb_y; vel_at_b_y = vel_b_y + omega_b * rb_x;
-        rel_vel_x = vel_at_a_x - vel_at_b_x; rel_vel_y = vel_at_a_y - vel_at_b_y;
-
-        float tangent_x = -normal_y, tangent_y = normal_x;
-        float vel_tangent = rel_vel_x * tangent_x + rel_vel_y * tangent_y;
-        float ra_cross_t = ra_x * tangent_y - ra_y * tangent_x;
-        float rb_cross_t = rb_x * tangent_y - rb_y * tangent_x;
-        float k_t = inv_mass_a + inv_mass_b;
-        k_t = k_t + inv_inertia_a * ra_cross_t * ra_cross_t;
-        k_t = k_t + inv_inertia_b * rb_cross_t * rb_cross_t;
-        float j_tangent = -vel_tangent / k_t;
-        float max_friction = friction * new_impulse;
-        float old_tangent = C[C_JT];
-        float new_tangent = old_tangent + j_tangent;
-        if (new_tangent > max_friction) new_tangent = max_friction;
-        else if (new_tangent < -max_friction) new_tangent = -max_friction;
-        C[C_JT] = new_tangent;
-        j_tangent = new_tangent - old_tangent;
-        float friction_x = j_tangent * tangent_x, friction_y = j_tangent * tangent_y;
-        A[IDX_VX] = vel_a_x + friction_x * inv_mass_a;
-        A[IDX_VY] = vel_a_y + friction_y * inv_mass_a;
-        A[IDX_OMEGA] = omega_a + (ra_x * friction_y - ra_y * friction_x) * inv_inertia_a;
-        if (hasb) {
-            Bb[IDX_VX] = vel_b_x - friction_x * inv_mass_b;
-            Bb[IDX_VY] = vel_b_y - friction_y * inv_mass_b;
-            Bb[IDX_OMEGA] = omega_b - (rb_x * friction_y - rb_y * friction_x) * inv_inertia_b;
-        }
-    }
-}
-
-template <class L>
-MRL_DEV void contact_solve_position(float *row, const float *contacts, int count, float baumgarte,
-                                    float slop) {
-    for (int c = 0; c < count; ++c) {
-        const float *C = contacts + c * CONTACT_SIZE;
-        int ia = (int)C[C_BODY_A], ib = (int)C[C_BODY_B];
-        float normal_x = C[C_NX], normal_y = C[C_NY], penetration = C[C_DEPTH];
-        float correction = penetration - slop;
-        if (correction <= 0.0f) continue;
-        correction = baumgarte * correction;
-        float *A = row + L::BODIES_OFF + ia * BODY_SIZE;
-        float *Bb = row + L::BODIES_OFF + (ib >= 0 ? ib : 0) * BODY_SIZE;
-        float inv_mass_a = A[IDX_INV_MASS];
-        float inv_mass_b = (ib >= 0) ? Bb[IDX_INV_MASS] : 0.0f;
-        float total = inv_mass_a + inv_mass_b;
-        if (total == 0.0f) continue;
-        float correction_a = correction * inv_mass_a / total;
-        float correction_b = correction * inv_mass_b / total;
-        A[IDX_X] = A[IDX_X] + normal_x * correction_a;
-        A[IDX_Y] = A[IDX_Y] + normal_y * correction_a;
-        if (ib >= 0) {
-            Bb[IDX_X] = Bb[IDX_X] - normal_x * correction_b;
-            Bb[IDX_Y] = Bb[IDX_Y] - normal_y * correction_b;
-        }
-    }
-}
-
-// world-space anchor offsets of every joint (r_a, r_b), valid while the angles do not change
-template <class L>
-struct JointAnchors { float rax[L::MAX_JOINTS], ray[L::MAX_JOINTS], rbx[L::MAX_JOINTS], rby[L::MAX_JOINTS]; };
-
-template <class L>
-MRL_DEV void joint_anchor(const float *row, const float *J, float &rax, float &ray, float &rbx,
-                          float &rby) {
-    const float *A = row + L::BODIES_OFF + (int)J[J_BODY_A] * BODY_SIZE;
-    const float *B = row + L::BODIES_OFF + (int)J[J_BODY_B] * BODY_SIZE;
-    float sin_a, cos_a, sin_b, cos_b;
-    sincos32(A[IDX_ANGLE], sin_a, cos_a);
-    sincos32(B[IDX_ANGLE], sin_b, cos_b);
-    float local_ax = J[J_AX], local_ay = J[J_AY], local_bx = J[J_BX], local_by = J[J_BY];
-    rax = local_ax * cos_a - local_ay * sin_a; ray = local_ax * sin_a + local_ay * cos_a;
-    rbx = local_bx * cos_b - local_by * sin_b; rby = local_bx * sin_b + local_by * cos_b;
-}
-
-template <class L>
-MRL_DEV void joint_anchors_all(const float *row, JointAnchors<L> &an) {
-    int n_joints = (int)row[L::JOINT_COUNT_OFF];
-#pragma unroll
-    for (int j = 0; j < L::MAX_JOINTS; ++j) {
-        an.rax[j] = an.ray[j] = an.rbx[j] = an.rby[j] = 0.0f;
-        if (j < n_joints) {
-            const float *J = row + L::JOINTS_OFF + j * JOINT_SIZE;
-            if ((int)J[J_TYPE] == 0) joint_anchor<L>(row, J, an.rax[j], an.ray[j], an.rbx[j], an.rby[j]);
-        }
-    }
-}
-
-template <class L>
-MRL_DEV void joint_solve_velocity(float *row, const JointAnchors<L> &an, float dt) {
-    int n_joints = (int)row[L::JOINT_COUNT_OFF];
-#pragma unroll
-    for (int j = 0; j < L::MAX_JOINTS; ++j) {
-        if (j >= n_joints) break;
-        const float *J = row + L::JOINTS_OFF + j * JOINT_SIZE;
-        if ((int)J[J_TYPE] != 0) continue;
-        float *A = row + L::BODIES_OFF + (int)J[J_BODY_A] * BODY_SIZE;
-        float *B = row + L::BODIES_OFF + (int)J[J_BODY_B] * BODY_SIZE;
-        float angle_a = A[IDX_ANGLE], vxa = A[IDX_VX], vya = A[IDX_VY], wa = A[IDX_OMEGA];
-        float inv_ma = A[IDX_INV_MASS], inv_ia = A[IDX_INV_INERTIA];
-        float angle_b = B[IDX_ANGLE], vxb = B[IDX_VX], vyb = B[IDX_VY], wb = B[IDX_OMEGA];
-        float inv_mb = B[IDX_INV_MASS], inv_ib = B[IDX_INV_INERTIA];
-        float rax = an.rax[j], ray = an.ray[j], rbx = an.rbx[j], rby = an.rby[j];
-        float va_anchor_x = vxa - wa * ray, va_anchor_y = vya + wa * rax;
-        float vb_anchor_x = vxb - wb * rby, vb_anchor_y = vyb + wb * rbx;
-        float cdot_x = vb_anchor_x - va_anchor_x, cdot_y = vb_anchor_y - va_anchor_y;
-        float k11 = inv_ma + inv_mb + inv_ia * ray * ray + inv_ib * rby * rby;
-        float k12 = -inv_ia * rax * ray - inv_ib * rbx * rby;
-        float k22 = inv_ma + inv_mb + inv_ia * rax * rax + inv_ib * rbx * rbx;
-        float det = k11 * k22 - k12 * k12;
-        if (det < 1e-10f) det = 1e-10f;
-        float inv_det = 1.0f / det;
-        float inv_k11 = k22 * inv_det, inv_k12 = -k12 * inv_det, inv_k22 = k11 * inv_det;
-        float impulse_x = -(inv_k11 * cdot_x + inv_k12 * cdot_y);
-        float impulse_y = -(inv_k12 * cdot_x + inv_k22 * cdot_y);
-        A[IDX_VX] = vxa - inv_ma * impulse_x;
-        A[IDX_VY] = vya - inv_ma * impulse_y;
-        B[IDX_VX] = vxb + inv_mb * impulse_x;
-        B[IDX_VY] = vyb + inv_mb * impulse_y;
-        float cur_wa = wa - inv_ia * (rax * impulse_y - ray * impulse_x);
-        float cur_wb = wb + inv_ib * (rbx * impulse_y - rby * impulse_x);
-
-        int flags = (int)J[J_FLAGS];
-        float eff = inv_ia + inv_ib;
-        if (flags & JF_SPRING) {
-            float angle_error = (angle_b - angle_a) - J[J_REF];
-            float rel_omega = wb - wa;  // angular velocities from before the point impulse
-            float spring_torque = -J[J_STIFF] * angle_error - J[J_DAMP] * rel_omega;
-            float angular_impulse = spring_torque * dt;
-            if (eff > 1e-10f) {
-                cur_wa = cur_wa - inv_ia * angular_impulse / eff;
-                cur_wb = cur_wb + inv_ib * angular_impulse / eff;
-            }
-        }
-        if (flags & JF_LIMIT) {
-            float relative_angle = angle_b - angle_a - J[J_REF];
-            float rel_omega = cur_wb - cur_wa;
-            if (eff > 1e-10f) {
-                float limit_impulse = 0.0f;
-                if (relative_angle <= J[J_LO]) {
-                    if (rel_omega < 0.0f) limit_impulse = -rel_omega / eff;
-                } else if (relative_angle >= J[J_HI]) {
-                    if (rel_omega > 0.0f) limit_impulse = -rel_omega / eff;
-                }
-                if (limit_impulse != 0.0f) {
-                    cur_wa = cur_wa - inv_ia * limit_impulse;
-                    cur_wb = cur_wb + inv_ib * limit_impulse;
-                }
-            }
-        }
-        if (flags & JF_MOTOR) {
-            float rel_omega = cur_wb - cur_wa;
-            float speed_error = J[J_MOTOR_SPEED] - rel_omega;
-            if (eff > 1e-10f) {
-                float motor_impulse = speed_error / eff;
-                float max_impulse = J[J_MAX_TORQUE] * dt;
-                if (motor_impulse > max_impulse) motor_impulse = max_impulse;
-                if (motor_impulse < -max_impulse) motor_impulse = -max_impulse;
-                cur_wa = cur_wa - inv_ia * motor_impulse;
-                cur_wb = cur_wb + inv_ib * motor_impulse;
-            }
-        }
-        A[IDX_OMEGA] = cur_wa;
-        B[IDX_OMEGA] = cur_wb;
-    }
-}
-
-template <class L>
-MRL_DEV void joint_solve_position(float *row, float baumgarte, float slop) {
-    int n_joints = (int)row[L::JOINT_COUNT_OFF];
-    for (int j = 0; j < n_joints; ++j) {
-        if (j >= L::MAX_JOINTS) break;
-        const float *J = row + L::JOINTS_OFF + j * JOINT_SIZE;
-        if ((int)J[J_TYPE] != 0) continue;
-        float *A = row + L::BODIES_OFF + (int)J[J_BODY_A] * BODY_SIZE;
-        float *B = row + L::BODIES_OFF + (int)J[J_BODY_B] * BODY_SIZE;
-        float xa = A[IDX_X], ya = A[IDX_Y], angle_a = A[IDX_ANGLE];
-        float inv_ma = A[IDX_INV_MASS], inv_ia = A[IDX_INV_INERTIA];
-        float xb = B[IDX_X], yb = B[IDX_Y], angle_b = B[IDX_ANGLE];
-        float inv_mb = B[IDX_INV_MASS], inv_ib = B[IDX_INV_INERTIA];
-        float rax, ray, rbx, rby;
-        joint_anchor<L>(row, J, rax, ray, rbx, rby);
-        float anchor_ax = xa + rax, anchor_ay = ya + ray;
-        float anchor_bx = xb + rbx, anchor_by = yb + rby;
-        float cx = anchor_bx - anchor_ax, cy = anchor_by - anchor_ay;
-        float error = sqrtf(cx * cx + cy * cy);
-        if (error < slop) continue;
-        float k11 = inv_ma + inv_mb + inv_ia * ray * ray + inv_ib * rby * rby;
-        float k12 = -inv_ia * rax * ray - inv_ib * rbx * rby;
-        float k22 = inv_ma + inv_mb + inv_ia * rax * rax + inv_ib * rbx * rbx;
-        float det = k11 * k22 - k12 * k12;
-        if (det < 1e-10f) det = 1e-10f;
-        float inv_det = 1.0f / det;
-        float inv_k11 = k22 * inv_det, inv_k12 = -k12 * inv_det, inv_k22 = k11 * inv_det;
-        float correction_x = -baumgarte * (inv_k11 * cx + inv_k12 * cy);
-        float correction_y = -baumgarte * (inv_k12 * cx + inv_k22 * cy);
-        A[IDX_X] = xa - inv_ma * correction_x;
-        A[IDX_Y] = ya - inv_ma * correction_y;
-        B[IDX_X] = xb + inv_mb * correction_x;
-        B[IDX_Y] = yb + inv_mb * correction_y;
-        float cur_a = angle_a - inv_ia * (rax * correction_y - ray * correction_x);
-        float cur_b = angle_b + inv_ib * (rbx * correction_y - rby * correction_x);
-        int flags = (int)J[J_FLAGS];
-        if (flags & JF_LIMIT) {
-            float relative_angle = cur_b - cur_a - J[J_REF];
-            float eff = inv_ia + inv_ib;
-            if (eff > 1e-10f) {
-                float angle_correction = 0.0f;
-                float lower = J[J_LO], upper = J[J_HI];
-                if (relative_angle < lower) angle_correction = baumgarte * (lower - relative_angle);
-                else if (relative_angle > upper) angle_correction = baumgarte * (upper - relative_angle);
-                if (angle_correction != 0.0f) {
-                    cur_a = cur_a - inv_ia * angle_correction / eff;
-                    cur_b = cur_b + inv_ib * angle_correction / eff;
-                }
-            }
-        }
-        A[IDX_ANGLE] = cur_a;
-        B[IDX_ANGLE] = cur_b;
-    }
 }
 
 // ray / edge test of physics2d/lidar/lidar.mojo:25-141 for one edge
