@@ -414,3 +414,80 @@ def test_autoreset_equals_step_then_selective_reset(mrl, ctx, name):
         assert torch.equal(o2.view(batch, E.OBS_DIM), s2.view(batch, E.STATE_SIZE)[:, :E.OBS_DIM])
         ended += int(d2.sum().item())
     assert ended > 0 or name == "HalfCheetahPlanarV2"
+
+
+def _crowd_edges(rows, edges_off, first, count, x_center, y):
+    """Rewrites `count` consecutive terrain edges of every row into a staircase of tiny flat edges
+    around x_center at height y: a vertex above them passes the x-range pre-check of all of them."""
+    for k in range(count):
+        e = rows[:, edges_off + 6 * (first + k): edges_off + 6 * (first + k + 1)]
+        x0 = x_center - 0.02 + 0.01 * k
+        e[:, 0], e[:, 1], e[:, 2], e[:, 3], e[:, 4], e[:, 5] = x0, y, x0 + 0.01, y, 0.0, 1.0
+
+
+def test_walker_vertex_over_many_edges_takes_the_serial_detector(mrl, orc, ctx):
+    """A vertex that touches four or more edges overflows its per-task contact list; the env then
+    falls back to the one-lane detector inside the step.  Terrain with a cluster of tiny edges under
+    the feet forces that path (and the MAX_CONTACTS cut-off of the merged list)."""
+    batch = 96
+    E = mrl.BipedalWalkerV2
+    s_h = np.zeros((batch, 950), np.float32)
+    orc.orc_bw_reset_batch(s_h, None, batch, 4)
+    hull_x = float(s_h[0, 24])
+    foot_y = float(s_h[:, 24 + 13 * 4 + 1].min()) - 34.0 / 30.0 / 2
+    assert abs(hull_x - 20 * 14.0 / 30.0) < 1e-3
+    # edges start after obs 24, bodies 5*13, forces 5*3, joints 4*17, joint count 1
+    edges_off = 24 + 65 + 15 + 68 + 1
+    assert abs(s_h[0, edges_off + 6 * 19 + 2] - hull_x) < 1e-3      # edge 19 ends under the hull
+    _crowd_edges(s_h[::2], edges_off, 17, 6, hull_x, foot_y + 0.05)   # every other env
+    s = dev(s_h.reshape(-1))
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch * 4, batch, batch, batch * 24))
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 24), np.float32)
+    rng = np.random.default_rng(4)
+    touched = 0
+    for t in range(12):
+        act = rng.uniform(-1.0, 1.0, (batch, 4)).astype(np.float32)
+        a.copy_(dev(act.reshape(-1)))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_bw_step_batch(s_h, act, r_h, d_h, o_h, batch, 8)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 950)
+        close(sg, s_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        np.testing.assert_allclose(r.cpu().numpy(), r_h, rtol=1e-5, atol=2e-5)
+        touched += int((o_h[::2, 8] + o_h[::2, 13] > 0).sum())
+        s_h[:] = sg
+    say("  leg-contact observations on the crowded terrain:", touched)
+    assert touched > 100
+
+
+def test_lander_vertex_over_many_edges_takes_the_serial_detector(mrl, orc, ctx):
+    batch = 64
+    E = mrl.LunarLanderV2
+    s_h = np.zeros((batch, 192), np.float32)
+    orc.orc_ll_reset_batch(s_h, batch, 6)
+    b = s_h[:, 8:47].reshape(batch, 3, 13)
+    edges_off = 91
+    pad_y = float(s_h[0, edges_off + 6 * 5 + 1])           # the helipad edges are flat
+    b[:, :, 1] -= (b[:, 0, 1] - pad_y - 0.9)[:, None]       # hull 0.9 above the pad: legs reach it in a few steps
+    b[:, :, 0] += (10.0 - b[:, 0, 0])[:, None]
+    leg_x = float(b[0, 1, 0])
+    _crowd_edges(s_h[::2], edges_off, 4, 6, leg_x, pad_y)
+    s = dev(s_h.reshape(-1))
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch, batch * 8))
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 8), np.float32)
+    legs = 0
+    for t in range(30):
+        act = np.zeros(batch, np.float32)
+        a.copy_(dev(act))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_ll_step_batch(s_h, act, r_h, d_h, o_h, batch, 8)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 192)
+        close(sg, s_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        np.testing.assert_array_equal(r.cpu().numpy(), r_h)
+        legs += int((o_h[::2, 6] + o_h[::2, 7] > 0).sum())
+        s_h[:] = sg
+    say("  leg contacts on the crowded pad:", legs)
+    assert legs > 20
