@@ -36,8 +36,11 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
     __shared__ float vals[PR];
     __shared__ __align__(16) float w2s[2][HEAD_LDS(H)];
     constexpr int TN = 2 * H / TPW;          // threads per net
-    const int t = threadIdx.x;
-    const int net = t / TN;                  // 0 = actor, 1 = critic
+    // a block works on both nets (2 TN threads) or, launched with TN threads and grid.y = 2, on the
+    // net blockIdx.y alone: a batch of few row tiles then spreads over twice as many CUs
+    const int t = threadIdx.x, nthr = blockDim.x;
+    const int net = t / TN + blockIdx.y;     // 0 = actor, 1 = critic
+    const bool has_actor = blockIdx.y == 0, has_critic = nthr > TN || blockIdx.y == 1;
     const int row0 = blockIdx.x * PR;
     const int nrow = min(PR, n - row0);
 
@@ -47,20 +50,20 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
     const float *p = net ? critic_p : actor_p;
     HiddenOperands<H, TPW, 8> ops;
     ops.load(p, IN);
-    float xv[(PR * PIN_MAX + 4 * H / TPW - 1) / (4 * H / TPW)];
+    float xv[(PR * PIN_MAX + TN - 1) / TN];
 #pragma unroll
     for (int q = 0; q < (int)(sizeof(xv) / sizeof(float)); ++q) {
-        const int i = t + q * 2 * TN;
+        const int i = t + q * nthr;
         xv[q] = (i < PR * IN && i / IN < nrow) ? obs[(long)row0 * IN + i] : 0.0f;
     }
     stage_head(p + IN * H + H + H * H + H, H, net ? 1 : A, GAUSS && net == 0, w2s[net], t % TN, TN);
 #pragma unroll
     for (int q = 0; q < (int)(sizeof(xv) / sizeof(float)); ++q) {
-        const int i = t + q * 2 * TN;
+        const int i = t + q * nthr;
         if (i < PR * IN) {
             const int r = i / IN, k = i - r * IN;
             xs[r * XS_LD + k] = xv[q];
-            if (r < nrow) r_obs[(long)row0 * IN + i] = xv[q];
+            if (r < nrow && has_actor) r_obs[(long)row0 * IN + i] = xv[q];
         }
     }
     __syncthreads();
@@ -70,7 +73,8 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
     else head<H>(w2s[1], 1, h2[1], vals, 1, t % TN, TN);
     __syncthreads();
 
-    if (t < nrow && !GAUSS) {   // categorical sampling, one lane per env
+    if (t < nrow && has_critic) r_values[row0 + t] = vals[t];
+    if (t < nrow && !GAUSS && has_actor) {   // categorical sampling, one lane per env
         const int i = row0 + t;
         int sel;
         float logp;
@@ -78,9 +82,8 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
         actions[i] = (float)sel;
         r_actions[i] = (float)sel;
         r_logp[i] = logp;
-        r_values[i] = vals[t];
     }
-    if (t < nrow && GAUSS) {    // Gaussian sampling, one lane per env
+    if (t < nrow && GAUSS && has_actor) {    // Gaussian sampling, one lane per env
         const int i = row0 + t;
         float act[PA_MAX];
         const float logp = sample_gaussian(logits + t * (PA_MAX + 1), w2s[0] + HEAD_LOG_STD(H), A, seed, i, act);
@@ -89,12 +92,12 @@ __global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
             r_actions[(long)i * A + j] = act[j];
         }
         r_logp[i] = logp;
-        r_values[i] = vals[t];
     }
 }
 
 // true when the pair (actor, critic) has the shape this kernel is specialised for
 constexpr int PTPW = 2;   // accumulator tiles per wavefront in the policy kernel (1 measured no faster)
+constexpr int POLICY_SPLIT_BELOW = 256;   // CUs of the MI355X: up to this many workgroups run side by side
 
 bool policy_fusable(const mrl_mlp_desc &a, const mrl_mlp_desc &c, bool gauss, int *H, int *act) {
     if (a.n_layers != 3 || c.n_layers != 3) return false;
@@ -122,10 +125,13 @@ int launch_policy(mrl_ctx *ctx, const mrl_mlp_desc &a, const mrl_mlp_desc &c, bo
     int H = 0, act = 0;
     if (!policy_fusable(a, c, gauss, &H, &act)) return MRL_E_UNSUPPORTED;
     const int IN = a.layers[0].in_dim, A = a.layers[2].out_dim;
-    dim3 grid((n + PR - 1) / PR);
+    // few row tiles: actor and critic of a tile go to workgroups of their own (twice the CUs at work)
+    const int tiles = (n + PR - 1) / PR;
+    const bool split = 2 * tiles <= POLICY_SPLIT_BELOW;
+    dim3 grid(tiles, split ? 2 : 1);
 #define MRL_LAUNCH(HH, AA, GG)                                                                         \
-    hipLaunchKernelGGL((policy_kernel<HH, AA, GG, PTPW>), grid, dim3(4 * HH / PTPW), 0, ctx->stream, obs, n, IN, A, ap, \
-                       cp, seed, actions, r_obs, r_actions, r_logp, r_values)
+    hipLaunchKernelGGL((policy_kernel<HH, AA, GG, PTPW>), grid, dim3((split ? 2 : 4) * HH / PTPW), 0, ctx->stream, obs, \
+                       n, IN, A, ap, cp, seed, actions, r_obs, r_actions, r_logp, r_values)
     if (gauss) {
         if (H == 256 && act == 1) MRL_LAUNCH(256, 1, true);
         else if (H == 256 && act == 2) MRL_LAUNCH(256, 2, true);
