@@ -24,7 +24,7 @@
 namespace mrl {
 
 template <int H, int ACT, bool GAUSS, int TPW>
-__global__ __launch_bounds__(4 * H / TPW) void policy_kernel(
+__global__ __launch_bounds__(TPW == 1 ? 2 * H : 4 * H / TPW) void policy_kernel(
     const float *__restrict__ obs, int n, int IN, int A, const float *__restrict__ actor_p,
     const float *__restrict__ critic_p, uint32_t seed, float *__restrict__ actions,
     float *__restrict__ r_obs, float *__restrict__ r_actions, float *__restrict__ r_logp,
@@ -125,13 +125,19 @@ int launch_policy(mrl_ctx *ctx, const mrl_mlp_desc &a, const mrl_mlp_desc &c, bo
     int H = 0, act = 0;
     if (!policy_fusable(a, c, gauss, &H, &act)) return MRL_E_UNSUPPORTED;
     const int IN = a.layers[0].in_dim, A = a.layers[2].out_dim;
-    // few row tiles: actor and critic of a tile go to workgroups of their own (twice the CUs at work)
+    // few row tiles: actor and critic of a tile go to workgroups of their own (twice the CUs at work),
+    // at hidden width 256 with one column tile per wavefront (eight wavefronts per net: two per SIMD,
+    // where a workgroup of four would leave each SIMD a single wavefront with nothing to overlap)
     const int tiles = (n + PR - 1) / PR;
     const bool split = 2 * tiles <= POLICY_SPLIT_BELOW;
     dim3 grid(tiles, split ? 2 : 1);
 #define MRL_LAUNCH(HH, AA, GG)                                                                         \
-    hipLaunchKernelGGL((policy_kernel<HH, AA, GG, PTPW>), grid, dim3((split ? 2 : 4) * HH / PTPW), 0, ctx->stream, obs, \
-                       n, IN, A, ap, cp, seed, actions, r_obs, r_actions, r_logp, r_values)
+    if (split && HH == 256)                                                                             \
+        hipLaunchKernelGGL((policy_kernel<HH, AA, GG, 1>), grid, dim3(2 * HH), 0, ctx->stream, obs,     \
+                           n, IN, A, ap, cp, seed, actions, r_obs, r_actions, r_logp, r_values);        \
+    else                                                                                                \
+        hipLaunchKernelGGL((policy_kernel<HH, AA, GG, PTPW>), grid, dim3((split ? 2 : 4) * HH / PTPW), 0, ctx->stream, obs, \
+                           n, IN, A, ap, cp, seed, actions, r_obs, r_actions, r_logp, r_values)
     if (gauss) {
         if (H == 256 && act == 1) MRL_LAUNCH(256, 1, true);
         else if (H == 256 && act == 2) MRL_LAUNCH(256, 2, true);
