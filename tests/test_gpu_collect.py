@@ -75,3 +75,96 @@ def test_rollout_steps_equals_single_steps(mrl, ctx, env, N, T, hidden, kind):
     assert cnt == int(many.done_count.item()) and cnt > 0
     key = lambda rb: sorted(zip(rb.done_returns[:cnt].tolist(), rb.done_lengths[:cnt].tolist()))
     assert key(one) == key(many)
+
+
+def _low_start(E, N, seed, orc):
+    """Rows reset by the oracle, then lowered to just above the terrain with a sideways offset and a
+    tilt, so that leg contacts, lander-body crashes, landings and in-place resets all happen within
+    a few dozen steps (envs/lunar_lander/lunar_lander_v2.mojo:1097-1255)."""
+    import numpy as np
+    s_h = np.zeros((N, E.STATE_SIZE), np.float32)
+    orc.orc_ll_reset_batch(s_h, N, seed)
+    rng = np.random.default_rng(seed)
+    b = s_h[:, 8:47].reshape(N, 3, 13)
+    b[:, :, 1] -= rng.uniform(7.5, 9.4, N).astype(np.float32)[:, None]
+    b[:, :, 0] += rng.uniform(-6, 6, N).astype(np.float32)[:, None]
+    b[:, 0, 2] = rng.uniform(-0.4, 0.4, N).astype(np.float32)
+    return s_h
+
+
+@pytest.mark.parametrize("env,kind,N", [("lunar", "relu", 2048), ("lunarc", "tanh", 2048), ("lunar", "tanh", 77)])
+def test_fused_collection_through_contacts(mrl, ctx, orc, env, kind, N):
+    """The fused collection kernel with the envs on the ground: contact detection on the other
+    wavefronts, list merge, solver with contacts, crash / landing terminations and resets inside the
+    launch.  (1) one-step launches against the oracle fed the kernel's own actions; (2) a 64-step range
+    in two launches against the same steps issued one by one, bit for bit."""
+    import numpy as np
+    print("case contacts", env, kind, N, flush=True)
+    T = 64
+    E = mrl.LunarLanderV2 if env == "lunar" else mrl.LunarLanderV2Continuous
+    cont = env == "lunarc"
+    lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
+    head = mrl.StochasticActor(256, 2) if cont else mrl.Linear(256, 4)
+    actor = mrl.seq(lin(8, 256), lin(256, 256), head)
+    critic = mrl.seq(lin(8, 256), lin(256, 256), mrl.Linear(256, 1))
+    g = torch.Generator(device="cuda").manual_seed(9)
+    ap = (torch.rand(actor.PARAM_SIZE, device="cuda", generator=g) - 0.5) * 0.3
+    cp = (torch.rand(critic.PARAM_SIZE, device="cuda", generator=g) - 0.5) * 0.3
+    s0_h = _low_start(E, N, 21, orc)
+    rbs = []
+    for _ in range(3):
+        rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N, T)
+        rb.actor_params, rb.critic_params = ap, cp
+        rb.states.copy_(torch.from_numpy(s0_h.reshape(-1)).cuda())
+        rb.obs.copy_(rb.states.view(N, 192)[:, :8].reshape(-1))
+        rbs.append(rb)
+    single, fused1, fused = rbs
+    assert mrl.ppo.rollout_fused(fused.descriptor()) == 1
+    # reset seeds stay below 2^63: the reset rounds the seed through fp32 and converts it back to
+    # a signed integer (lunar_lander_v2.mojo:1638), which is only defined in that range
+    s0, ss, r0, rs = 424242, 2654435761 * N + 7919, 5, 0x9E3779B97F
+
+    # (1) launches of one step each, checked against the oracle after every step
+    s_h = s0_h.copy()
+    r_h, d_h, o_h = np.zeros(N, np.float32), np.zeros(N, np.float32), np.zeros((N, 8), np.float32)
+    d1 = fused1.descriptor()
+    crashes = leg_obs = landed = resets = 0
+    aw = 2 if cont else 1
+    for t in range(T):
+        mrl.ppo.rollout_steps(ctx, d1, t, 1, (s0 + t * ss) & 0xFFFFFFFF, 0, 0, 0, (r0 + t * rs) & (2**64 - 1), 0)
+        ctx.synchronize()
+        acts = fused1.r_actions[t * N * aw:(t + 1) * N * aw].cpu().numpy()
+        if cont:
+            orc.orc_ll_step_continuous_batch(s_h, np.ascontiguousarray(acts.reshape(N, 2)), r_h, d_h, o_h, N)
+        else:
+            orc.orc_ll_step_batch(s_h, acts, r_h, d_h, o_h, N, 1)
+        np.testing.assert_array_equal(fused1.r_rewards[t * N:(t + 1) * N].cpu().numpy(), r_h, err_msg="reward, step %d" % t)
+        np.testing.assert_array_equal(fused1.r_dones[t * N:(t + 1) * N].cpu().numpy(), d_h, err_msg="done, step %d" % t)
+        crashes += int((r_h == -100).sum())
+        landed += int(((d_h > 0) & (r_h > 50)).sum())
+        leg_obs += int((o_h[:, 6] + o_h[:, 7] > 0).sum())
+        resets += int(d_h.sum())
+        orc.orc_ll_selective_reset_batch(s_h, d_h, N, (r0 + t * rs) & (2**64 - 1))
+        sg = fused1.states.cpu().numpy().reshape(N, 192)
+        np.testing.assert_allclose(sg, s_h, rtol=1e-5, atol=1e-6, err_msg="state, step %d" % t)
+        np.testing.assert_allclose(fused1.obs.cpu().numpy().reshape(N, 8), s_h[:, :8], rtol=1e-5, atol=1e-6)
+        s_h[:] = sg
+    print("  crashes", crashes, "landings", landed, "leg-contact observations", leg_obs, "resets", resets, flush=True)
+    assert crashes > N // 40 and leg_obs > N // 4 and resets >= crashes
+
+    # (2) the same range as two launches, against single steps
+    dsingle, dfused = single.descriptor(), fused.descriptor()
+    for t in range(T):
+        mrl.ppo.rollout_step(ctx, dsingle, t, (s0 + t * ss) & 0xFFFFFFFF, 0, (r0 + t * rs) & (2**64 - 1))
+    k = 23
+    mrl.ppo.rollout_steps(ctx, dfused, 0, k, s0, ss & 0xFFFFFFFF, 0, 0, r0, rs)
+    mrl.ppo.rollout_steps(ctx, dfused, k, T - k, (s0 + k * ss) & 0xFFFFFFFF, ss & 0xFFFFFFFF, 0, 0,
+                          (r0 + k * rs) & (2**64 - 1), rs)
+    ctx.synchronize()
+    for name in ("r_obs", "r_actions", "r_log_probs", "r_values", "r_rewards", "r_dones", "states", "obs",
+                 "ep_return", "ep_length"):
+        a, b, c = getattr(single, name), getattr(fused, name), getattr(fused1, name)
+        assert torch.equal(a, b), "%s: fused range differs from single steps in %d places" % (name, int((a != b).sum()))
+        assert torch.equal(a, c), "%s: one-step launches differ from single steps in %d places" % (name, int((a != c).sum()))
+    cnt = int(single.done_count.item())
+    assert cnt == int(fused.done_count.item()) == resets

@@ -541,6 +541,160 @@ def test_continuous_update_minibatch_against_oracle(mrl, orc, orcmod, ctx, H):
     np.testing.assert_allclose(h(rb.critic_params), cp2, rtol=1e-5, atol=0.03 * 1e-3)
 
 
+def _f64_param_grads(spec, params, x, g_out):
+    """Parameter gradients of sum(out * g_out) for an MLP given as [(kind, in, out)] (kinds as
+    mrl_layer_kind) with params [W | b] per layer (+ log_std), evaluated by torch autograd in
+    float64 on the CPU: the value both fp32 summation orders (the oracle's serial loops, the
+    kernels' tiles) are rounding errors away from."""
+    p = torch.tensor(params, dtype=torch.float64, requires_grad=True)
+    cur, off = torch.tensor(x, dtype=torch.float64), 0
+    for kind, i, o in spec:
+        W = p[off:off + i * o].view(i, o); off += i * o
+        b = p[off:off + o]; off += o
+        cur = cur @ W + b
+        if kind == 1:
+            cur = torch.relu(cur)
+        elif kind == 2:
+            cur = torch.tanh(cur)
+        elif kind == 3:
+            ls = p[off:off + o]; off += o
+            cur = torch.cat([cur, torch.clamp(ls, -5.0, 2.0).expand(cur.shape[0], o)], 1)
+    (cur * torch.tensor(g_out, dtype=torch.float64)).sum().backward()
+    return p.grad.numpy()
+
+
+def _clip64(g, max_norm):
+    n = np.sqrt((g * g).sum())
+    return g * (max_norm / (n + 1e-8)) if n > max_norm else g
+
+
+@pytest.mark.parametrize("env_name,kind", [("LunarLanderV2", "relu"), ("HalfCheetahPlanarV2", "tanh")])
+def test_fused_update_minibatch_against_oracle_at_bench_size(mrl, orc, orcmod, ctx, env_name, kind):
+    """mrl_ppo_update_minibatch at the sizes bench.py times (hidden width 256, minibatch 4096; the
+    discrete 8-256-256-4 ReLU nets of the LunarLander agent and the Gaussian 17-256-256-6 tanh nets of
+    the HalfCheetah agent) against the oracle's sequence forward -> loss gradient -> backward -> clip
+    -> Adam (-> log_std clamp), deep_agents/ppo/ppo.mojo:2438-2727 and ppo_continuous.mojo:3000-3260.
+    Bar: KL, loss gradients and parameter gradients within 1e-4 of the tensor's scale.  The float64
+    value of the parameter gradients is evaluated as well, so that the test states how far each
+    fp32 summation order is from it."""
+    say("case", env_name, kind)
+    rng = np.random.default_rng(23)
+    E = getattr(mrl, env_name)
+    cont = E.NUM_ACTIONS == 0
+    od = E.OBS_DIM
+    A = E.ACTION_DIM if cont else E.NUM_ACTIONS
+    H, MB, N, T = 256, 4096, 1024, 8
+    hk = 1 if kind == "relu" else 2
+    lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
+    head = mrl.StochasticActor(H, A) if cont else mrl.Linear(H, A)
+    actor = mrl.seq(lin(od, H), lin(H, H), head)
+    critic = mrl.seq(lin(od, H), lin(H, H), mrl.Linear(H, 1))
+    spec_a = [(hk, od, H), (hk, H, H), (3 if cont else 0, H, A)]
+    spec_c = [(hk, od, H), (hk, H, H), (0, H, 1)]
+    la, lc = orcmod.layers(spec_a), orcmod.layers(spec_c)
+    hd = actor.OUT_DIM
+    # the reference's initialisation scales: Kaiming U(+-sqrt(2/fan_in)) / Xavier over the net's dims
+    bound = (2.0 / od) ** 0.5 if cont else (2.0 / (od + A)) ** 0.5
+    ap = rng.uniform(-bound, bound, actor.PARAM_SIZE).astype(np.float32) * 0.5
+    cp = rng.uniform(-bound, bound, critic.PARAM_SIZE).astype(np.float32) * 0.5
+    if cont:
+        ap[-A:] = -0.5
+    total, aw = N * T, (A if cont else 1)
+    r_obs = rng.normal(size=(total, od)).astype(np.float32)
+    out0 = np.zeros((total, hd), np.float32)
+    orc.orc_mlp_forward(la, 3, total, r_obs, ap, out0, None)
+    r_lp = np.zeros(total, np.float32)
+    if cont:
+        r_act = np.zeros((total, A), np.float32)
+        orc.orc_sample_gaussian(out0, total, A, 5, r_act, r_lp)
+    else:
+        r_act = np.zeros(total, np.float32)
+        orc.orc_sample_categorical(out0, total, A, 5, r_act, r_lp)
+    r_lp += rng.normal(size=total).astype(np.float32) * 0.1      # ratios on both sides of the clip range
+    r_val = rng.normal(size=total).astype(np.float32)
+    adv = (rng.normal(size=total) * 2.0 + 0.3).astype(np.float32)
+    ret = (r_val + rng.normal(size=total) * 0.5).astype(np.float32)
+    rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N, T)
+    rb.actor_params, rb.critic_params = d(ap), d(cp)
+    rb.r_obs.copy_(d(r_obs.reshape(-1))); rb.r_actions.copy_(d(r_act.reshape(-1)))
+    rb.r_log_probs.copy_(d(r_lp)); rb.r_values.copy_(d(r_val))
+    a_lr, c_lr = 3e-4, 1e-3
+    max_norm = 0.5 if cont else 0.1          # below the raw gradient norm: the clip is active
+    cls = mrl.ppo.ContinuousUpdate if cont else mrl.ppo.DiscreteUpdate
+    upd = cls(ctx, rb, MB, mrl.Adam(lr=a_lr), mrl.Adam(lr=c_lr), target_kl=0.0, max_grad_norm=max_norm)
+    upd.advantages.copy_(d(adv)); upd.returns.copy_(d(ret))
+    idx = rng.permutation(total)[:MB].astype(np.int32)
+    upd.minibatch_step(d(idx))
+    ctx.synchronize()
+
+    # ---- the oracle's sequence
+    mo, ma, madv = np.ascontiguousarray(r_obs[idx]), np.ascontiguousarray(r_act[idx]), adv[idx].copy()
+    orc.orc_normalize_minibatch_host(madv, MB)
+    cache = np.zeros(MB * actor.CACHE_SIZE, np.float32)
+    out = np.zeros((MB, hd), np.float32)
+    orc.orc_mlp_forward(la, 3, MB, mo, ap, out, cache.ctypes.data)
+    g_out, kl = np.zeros((MB, hd), np.float32), np.zeros(MB, np.float32)
+    if cont:
+        orc.orc_ppo_actor_grad_gaussian(out, r_lp[idx], madv, ma, MB, A, 0.2, 0.01, g_out, kl)
+    else:
+        orc.orc_ppo_actor_grad_discrete(out, r_lp[idx], madv, ma, MB, A, 0.2, 0.01, g_out, kl)
+    ga = np.zeros(actor.PARAM_SIZE, np.float32)
+    orc.orc_mlp_backward(la, 3, MB, g_out, ap, cache, ga, None)
+    ga_raw = ga.copy()
+    orc.orc_clip_grad_norm(ga, ga.size, max_norm)
+    ap2, st = ap.copy(), np.zeros(2 * ga.size, np.float32)
+    orc.orc_adam_step(ap2, ga, st, ga.size, 1, a_lr, 0.9, 0.999, 1e-8)
+    if cont:
+        orc.orc_clamp_log_std(ap2, ap2.size - A, A)
+    ccache = np.zeros(MB * critic.CACHE_SIZE, np.float32)
+    v = np.zeros((MB, 1), np.float32)
+    orc.orc_mlp_forward(lc, 3, MB, mo, cp, v, ccache.ctypes.data)
+    gv = np.zeros(MB, np.float32)
+    orc.orc_ppo_critic_grad(v.reshape(-1), r_val[idx], ret[idx], MB, 1 if cont else 0, 1, 0.5, 0.2, gv)
+    gc = np.zeros(critic.PARAM_SIZE, np.float32)
+    orc.orc_mlp_backward(lc, 3, MB, gv.reshape(MB, 1), cp, ccache, gc, None)
+    orc.orc_clip_grad_norm(gc, gc.size, max_norm)
+    cp2, st = cp.copy(), np.zeros(2 * gc.size, np.float32)
+    orc.orc_adam_step(cp2, gc, st, gc.size, 1, c_lr, 0.9, 0.999, 1e-8)
+
+    def rel(a, b):          # largest difference in units of the tensor's scale
+        return float(np.abs(a.astype(np.float64) - b).max() / np.abs(b).max())
+
+    clipped_rows = int((np.abs(g_out).sum(1) == 0).sum()) if not cont else -1
+    say("  rows with the ratio outside the clip range (discrete):", clipped_rows, "of", MB)
+    assert rel(h(upd.actor_out).reshape(MB, hd), out) < 1e-4
+    assert rel(h(upd.values), v.reshape(-1)) < 1e-4
+    assert rel(h(upd.kl), kl) < 1e-4
+    assert rel(h(upd.g_actor_out).reshape(MB, hd), g_out) < 1e-4
+    assert rel(h(upd.g_values), gv) < 1e-4
+    # parameter gradients: GPU vs oracle, and both against float64 autograd fed the oracle's loss gradients
+    ga64 = _clip64(_f64_param_grads(spec_a, ap, mo, g_out), max_norm)
+    gc64 = _clip64(_f64_param_grads(spec_c, cp, mo, gv.reshape(MB, 1)), max_norm)
+    e = {"actor gpu-oracle": rel(h(upd.actor_grads), ga), "actor gpu-f64": rel(h(upd.actor_grads), ga64),
+         "actor oracle-f64": rel(ga, ga64), "critic gpu-oracle": rel(h(upd.critic_grads), gc),
+         "critic gpu-f64": rel(h(upd.critic_grads), gc64), "critic oracle-f64": rel(gc, gc64)}
+    say("  parameter-gradient error / tensor scale:", {k: "%.2e" % x for k, x in e.items()})
+    assert all(x < 1e-4 for x in e.values()), e
+    # per layer block as well (a thin layer's error must not hide behind a wide layer's scale)
+    off = 0
+    for kind_, i, o in spec_a:
+        n = i * o + o + (o if kind_ == 3 else 0)
+        assert rel(h(upd.actor_grads)[off:off + n], ga[off:off + n]) < 1e-4, ("actor layer", i, o)
+        off += n
+    off = 0
+    for kind_, i, o in spec_c:
+        n = i * o + o
+        assert rel(h(upd.critic_grads)[off:off + n], gc[off:off + n]) < 1e-4, ("critic layer", i, o)
+        off += n
+    assert float(np.sqrt((ga_raw.astype(np.float64) ** 2).sum())) > max_norm
+    # Adam's first step is lr * g / (|g| + eps): entries near eps follow their own rounding error, so
+    # the step is compared to 3 % of lr and, for entries that are not tiny, to 1e-3 of lr
+    for got, want, p0, g, lr in ((h(rb.actor_params), ap2, ap, ga, a_lr), (h(rb.critic_params), cp2, cp, gc, c_lr)):
+        np.testing.assert_allclose(got, want, rtol=0, atol=0.03 * lr)
+        big = np.abs(g) > 1e-5
+        np.testing.assert_allclose((got - p0)[big], (want - p0)[big], rtol=0, atol=1e-3 * lr + 1e-7)
+
+
 def test_update_driver_runs_epochs_and_stops_on_kl(mrl, ctx):
     """PPOUpdate.update end to end on a small LunarLander rollout: permutation drawn on the device,
     the KL flag raised on the device stops the epochs, parameters stay finite."""
