@@ -23,48 +23,44 @@ int mrl_version(void) { return 100; }
 
 const char *mrl_last_error(void) { return mrl::g_error; }
 
+// a failed set-up step releases what the steps before it obtained
+#define CTX_TRY(expr)                                                                             \
+    do {                                                                                          \
+        hipError_t _e = (expr);                                                                   \
+        if (_e != hipSuccess) {                                                                   \
+            mrl_ctx_destroy(c);                                                                   \
+            return mrl::set_error(MRL_E_HIP, "mrl_ctx_create: %s failed: %s", #expr, hipGetErrorString(_e)); \
+        }                                                                                         \
+    } while (0)
+
 int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     MRL_CHECK_ARG(out != nullptr, "mrl_ctx_create: out is NULL");
     int count = 0;
     hipError_t e = hipGetDeviceCount(&count);
     if (e != hipSuccess || count == 0)
         return mrl::set_error(MRL_E_HIP, "mrl_ctx_create: no HIP device (%s)", hipGetErrorString(e));
-    mrl_ctx *c = new mrl_ctx();
+    mrl_ctx *c = new mrl_ctx();        // value-initialised: every pointer starts out null
     c->stream = (hipStream_t)hip_stream;
-    MRL_CHECK_HIP(hipGetDevice(&c->device));
-    c->ll_shapes = nullptr;
-    c->reduce_scratch = nullptr;
     c->reduce_scratch_floats = 4096;
-    c->mlp_ws = nullptr;
-    c->mlp_ws_floats = 0;
-    c->rollout_ws = nullptr;
-    c->rollout_ws_floats = 0;
-    c->profiling = false;
-    c->prof_used = 0;
-    c->prof_chained = false;
     c->prof_every = 1;
-    c->prof_step = 0;
     c->prof_active = true;
-    c->prof_open_next = false;
-    MRL_CHECK_HIP(hipMalloc(&c->ll_shapes, sizeof(mrl::ll::Shapes)));
+    CTX_TRY(hipGetDevice(&c->device));
     mrl::ll::Shapes sh = mrl::ll::make_shapes();
-    MRL_CHECK_HIP(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));
-    c->bw_shapes = c->hc_shapes = nullptr;
-    {
-        mrl::bw::Shapes bs = mrl::bw::make_shapes();
-        MRL_CHECK_HIP(hipMalloc(&c->bw_shapes, sizeof(bs)));
-        MRL_CHECK_HIP(hipMemcpy(c->bw_shapes, &bs, sizeof(bs), hipMemcpyHostToDevice));
-        mrl::hc::Shapes hs = mrl::hc::make_shapes();
-        MRL_CHECK_HIP(hipMalloc(&c->hc_shapes, sizeof(hs)));
-        MRL_CHECK_HIP(hipMemcpy(c->hc_shapes, &hs, sizeof(hs), hipMemcpyHostToDevice));
-    }
-    MRL_CHECK_HIP(hipMalloc(&c->reduce_scratch, sizeof(float) * c->reduce_scratch_floats));
-    c->upd_scratch = nullptr;
-    MRL_CHECK_HIP(hipMalloc(&c->upd_scratch, sizeof(float) * 8192));
-    MRL_CHECK_HIP(hipMemset(c->upd_scratch, 0, sizeof(float) * 8192));
+    CTX_TRY(hipMalloc(&c->ll_shapes, sizeof(sh)));
+    CTX_TRY(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));
+    mrl::bw::Shapes bs = mrl::bw::make_shapes();
+    CTX_TRY(hipMalloc(&c->bw_shapes, sizeof(bs)));
+    CTX_TRY(hipMemcpy(c->bw_shapes, &bs, sizeof(bs), hipMemcpyHostToDevice));
+    mrl::hc::Shapes hs = mrl::hc::make_shapes();
+    CTX_TRY(hipMalloc(&c->hc_shapes, sizeof(hs)));
+    CTX_TRY(hipMemcpy(c->hc_shapes, &hs, sizeof(hs), hipMemcpyHostToDevice));
+    CTX_TRY(hipMalloc(&c->reduce_scratch, sizeof(float) * c->reduce_scratch_floats));
+    CTX_TRY(hipMalloc(&c->upd_scratch, sizeof(float) * 8192));
+    CTX_TRY(hipMemset(c->upd_scratch, 0, sizeof(float) * 8192));
     *out = c;
     return MRL_OK;
 }
+#undef CTX_TRY
 
 int mrl_ctx_destroy(mrl_ctx *ctx) {
     if (!ctx) return MRL_OK;
