@@ -196,6 +196,16 @@ int mrl_ppo_critic_grad(mrl_ctx *ctx, const float *values, const float *old_valu
                         float clip_eps, float *grad_values);
 /* gradient_norm_kernel + reduce + apply, ppo.mojo:382-534 / kernels.mojo:603-805; in place */
 int mrl_clip_grad_norm(mrl_ctx *ctx, float *grads, int n, float max_norm);
+/* mrl_clip_grad_norm for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * per-block partial sums live in a file-scope device array of 1 KiB that every device holds from
+ * library load to process end, instead of in memory obtained from hipMalloc; its address is looked
+ * up by mrl_ctx_create.  The call allocates and frees nothing, and gives the results of
+ * mrl_clip_grad_norm bit for bit.  n is limited to MRL_CLIP_STATIC_MAX_N elements; a larger n is
+ * rejected with MRL_E_ARG.  All calls on one device share that device's array: calls that overlap
+ * on one device (two streams, two threads) race. */
+#define MRL_CLIP_STATIC_MAX_N (1 << 24)
+int mrl_clip_grad_norm_static(mrl_ctx *ctx, float *grads, int n, float max_norm);
 /* Adam.step_gpu, deep_rl/optimizer/adam.mojo:52-105, :162-247.  t is the optimiser's step count
  * AFTER the increment (1 on the first call); state is [n, 2] interleaved (m, v). */
 int mrl_adam_step(mrl_ctx *ctx, float *params, const float *grads, float *state, int n, int t,

@@ -92,6 +92,7 @@ SIGNATURES = {
     "mrl_ppo_actor_grad_gaussian": [P, P, P, P, P, I, I, F, F, P, P],
     "mrl_ppo_critic_grad": [P, P, P, P, I, I, I, F, F, P],
     "mrl_clip_grad_norm": [P, P, I, F],
+    "mrl_clip_grad_norm_static": [P, P, I, F],
     "mrl_adam_step": [P, P, P, P, I, I, D, D, D, D],
     "mrl_clamp_log_std": [P, P, I, I],
     "mrl_rms_update": [P, P, P, I],

@@ -57,6 +57,10 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     CTX_TRY(hipMalloc(&c->reduce_scratch, sizeof(float) * c->reduce_scratch_floats));
     CTX_TRY(hipMalloc(&c->upd_scratch, sizeof(float) * 8192));
     CTX_TRY(hipMemset(c->upd_scratch, 0, sizeof(float) * 8192));
+    {
+        int rc = mrl::clip_static_setup(c->device);
+        if (rc != MRL_OK) { mrl_ctx_destroy(c); return rc; }
+    }
     *out = c;
     return MRL_OK;
 }

@@ -76,6 +76,10 @@ int env_step_accounting(mrl_ctx *ctx, int env_id, int batch, float *states, cons
 // CartPole's per-env step counters for the rows at `states` (created zeroed on first use)
 int cartpole_side(mrl_ctx *ctx, const float *states, int batch, int32_t **out);
 
+// resolves the device address of the file-scope scratch of mrl_clip_grad_norm_static for `device`
+// (the current device); idempotent
+int clip_static_setup(int device);
+
 inline int grid_for(long n, int block) { return (int)((n + block - 1) / block); }
 
 // Records a phase boundary: the time since the previous mark is charged to `tag`; tag < 0 opens

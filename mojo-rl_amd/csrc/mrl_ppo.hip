@@ -419,6 +419,32 @@ __global__ void clamp_log_std_kernel(float *params, int offset, int A) {
 
 using namespace mrl;
 
+// ---------------------------------------------------------------- allocation-free clip
+// Scratch of mrl_clip_grad_norm_static: the per-block partial sums of squares live in this
+// file-scope array instead of memory obtained from hipMalloc (each device the library runs on holds
+// its own 1 KiB copy until the process ends).  In host code the array's name is only a handle for the
+// symbol: the device address is looked up once per device and kept in g_clip_scratch_ptr.
+constexpr int CLIP_STATIC_PARTIALS = 256;
+constexpr int CLIP_STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) float g_clip_scratch[CLIP_STATIC_PARTIALS];
+static float *g_clip_scratch_ptr[CLIP_STATIC_MAX_DEVICES] = {};
+
+namespace mrl {
+// Looks the address of this device's copy of the scratch array up; `device` must be the current
+// device.  Called by mrl_ctx_create, and again (a no-op then) by the entry point itself.
+int clip_static_setup(int device) {
+    if (device < 0 || device >= CLIP_STATIC_MAX_DEVICES)
+        return set_error(MRL_E_ARG, "clip_static_setup: device %d outside 0..%d", device, CLIP_STATIC_MAX_DEVICES - 1);
+    if (g_clip_scratch_ptr[device] != nullptr) return MRL_OK;
+    float *p = nullptr;
+    hipError_t e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(g_clip_scratch));
+    if (e != hipSuccess || p == nullptr)
+        return set_error(MRL_E_HIP, "hipGetSymbolAddress(g_clip_scratch) failed: %s", hipGetErrorString(e));
+    g_clip_scratch_ptr[device] = p;
+    return MRL_OK;
+}
+}  // namespace mrl
+
 extern "C" {
 
 int mrl_sample_categorical(mrl_ctx *ctx, const float *logits, int n, int num_actions, uint32_t seed,
@@ -645,6 +671,29 @@ int mrl_clip_grad_norm(mrl_ctx *ctx, float *grads, int n, float max_norm) {
     MRL_CHECK_ARG(grads, "mrl_clip_grad_norm: NULL buffer");
     int nb = std::min(256, grid_for(n, TPB));
     float *part = ctx->reduce_scratch + 1024;
+    hipLaunchKernelGGL(sq_partial_kernel, dim3(nb), dim3(TPB), 0, ctx->stream, grads, n, part);
+    hipLaunchKernelGGL(clip_apply_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream, grads, n,
+                       part, nb, max_norm);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_clip_grad_norm_static(mrl_ctx *ctx, float *grads, int n, float max_norm) {
+    MRL_CHECK_ARG(ctx, "mrl_clip_grad_norm_static: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0, "mrl_clip_grad_norm_static: negative size");
+    MRL_CHECK_ARG(n <= MRL_CLIP_STATIC_MAX_N,
+                  "mrl_clip_grad_norm_static: n = %d exceeds the limit of %d elements of the allocation-free "
+                  "variant (use mrl_clip_grad_norm)", n, MRL_CLIP_STATIC_MAX_N);
+    if (n == 0) return MRL_OK;
+    MRL_CHECK_ARG(grads, "mrl_clip_grad_norm_static: NULL buffer");
+    int dev = -1;
+    MRL_CHECK_HIP(hipGetDevice(&dev));
+    int rc = mrl::clip_static_setup(dev);          // resolved by mrl_ctx_create; a lookup, no allocation
+    if (rc != MRL_OK) return rc;
+    float *part = g_clip_scratch_ptr[dev];
+    // same kernels and block count as mrl_clip_grad_norm: the results are the same bit for bit.
+    // Every partial that the second kernel reads has been written by the first: nothing to clear.
+    int nb = std::min(CLIP_STATIC_PARTIALS, grid_for(n, TPB));
     hipLaunchKernelGGL(sq_partial_kernel, dim3(nb), dim3(TPB), 0, ctx->stream, grads, n, part);
     hipLaunchKernelGGL(clip_apply_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx->stream, grads, n,
                        part, nb, max_norm);

@@ -85,6 +85,16 @@ def clip_grad_norm(ctx, grads, max_grad_norm):
     _lib.call("mrl_clip_grad_norm", ctx.handle, _ptr(grads), grads.numel(), float(max_grad_norm))
 
 
+CLIP_STATIC_MAX_N = 1 << 24
+
+
+def clip_grad_norm_static(ctx, grads, max_grad_norm):
+    """clip_grad_norm for callers that must not allocate device memory: the partial sums live in a
+    file-scope device array of the library.  Same results; at most CLIP_STATIC_MAX_N elements; calls
+    that overlap on one device race on that array."""
+    _lib.call("mrl_clip_grad_norm_static", ctx.handle, _ptr(grads), grads.numel(), float(max_grad_norm))
+
+
 def clamp_log_std_params(ctx, params, log_std_offset, action_dim):
     """clamp_log_std_params_kernel, kernels.mojo:842-873."""
     _lib.call("mrl_clamp_log_std", ctx.handle, _ptr(params), log_std_offset, action_dim)
