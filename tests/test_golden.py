@@ -91,18 +91,15 @@ def test_hip_path_reproduces_golden_trajectories(mrl, traj, name, cls):
     T, N = R.shape
     s = torch.from_numpy(traj["%s_state0" % name].copy()).cuda().reshape(-1)
     r, d, o = torch.zeros(N, device="cuda"), torch.zeros(N, device="cuda"), torch.zeros(O[0].size, device="cuda")
-    exact_reward = name in ("pendulum", "lunar")
     for t in range(T):
         print(name, "step", t, flush=True)
         a = torch.from_numpy(np.ascontiguousarray(A[t].reshape(-1))).cuda()
         E.step_kernel_gpu(ctx, s, a, r, d, o, t)
         ctx.synchronize()
-        np.testing.assert_allclose(o.cpu().numpy().reshape(O[t].shape), O[t], rtol=1e-5, atol=1e-6)
-        if exact_reward:
-            np.testing.assert_array_equal(r.cpu().numpy(), R[t])
-        else:
-            np.testing.assert_allclose(r.cpu().numpy(), R[t], rtol=1e-5, atol=1e-5)
+        # no resynchronisation between steps: the whole trajectory has to stay on the oracle's bits
+        np.testing.assert_array_equal(o.cpu().numpy().reshape(O[t].shape), O[t])
+        np.testing.assert_array_equal(r.cpu().numpy(), R[t])
         np.testing.assert_array_equal(d.cpu().numpy(), D[t])
         E.selective_reset_kernel_gpu(ctx, s, d, 1000 + t)
     ctx.synchronize()
-    np.testing.assert_allclose(s.cpu().numpy().reshape(N, -1), traj["%s_state_end" % name], rtol=1e-5, atol=1e-6)
+    np.testing.assert_array_equal(s.cpu().numpy().reshape(N, -1), traj["%s_state_end" % name])
