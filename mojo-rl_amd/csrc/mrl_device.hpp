@@ -6,6 +6,8 @@
 //     unless fmaf() is written out;
 //   * fp32 sin/cos of an fp32 angle are the correctly rounded values, computed through
 //     the fp64 routine and rounded once;
+//   * fp32 exp/log where an index or a branch depends on the last bit (action sampling, the PPO
+//     ratio and its clip test) are the correctly rounded values as well;
 //   * fp32 divide and sqrt are IEEE (hipcc default for gfx9).
 #pragma once
 #include <hip/hip_runtime.h>
@@ -17,6 +19,8 @@ namespace mrl {
 
 MRL_DEV float sin32(float x) { return (float)::sin((double)x); }
 MRL_DEV float cos32(float x) { return (float)::cos((double)x); }
+MRL_DEV float exp32(float x) { return (float)::exp((double)x); }
+MRL_DEV float log32(float x) { return (float)::log((double)x); }
 MRL_DEV void sincos32(float x, float &s, float &c) {
     double ds, dc;
     ::sincos((double)x, &ds, &dc);

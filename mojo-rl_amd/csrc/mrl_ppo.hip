@@ -4,6 +4,7 @@
 #include "mrl_host.hpp"
 #include "mrl_device.hpp"
 #include "ppo_grads.hpp"
+#include "policy_sample.hpp"
 
 namespace mrl {
 
@@ -39,24 +40,11 @@ __global__ __launch_bounds__(TPB) void sample_categorical_kernel(const float *__
                                                                  float *__restrict__ log_probs) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    const float *l = logits + (long)i * A;
-    uint32_t rng = seed ^ ((uint32_t)i * 2654435761u);
-    rng = xorshift32(rng);
-    float max_logit = l[0];
-    for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
-    float sum_exp = 0.0f;
-    for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
-    float u = random_uniform(rng);
-    float cumsum = 0.0f;
-    int sel = 0;
-    for (int a = 0; a < A; ++a) {
-        float prob = expf(l[a] - max_logit) / sum_exp;
-        cumsum = cumsum + prob;
-        if (u < cumsum) { sel = a; break; }
-    }
+    int sel;
+    float logp;
+    sample_categorical(logits + (long)i * A, A, seed, i, sel, logp);
     actions[i] = (float)sel;
-    float p = expf(l[sel] - max_logit) / sum_exp;
-    log_probs[i] = logf(p + 1e-8f);
+    log_probs[i] = logp;
 }
 
 // deep_agents/ppo/kernels.mojo:12-98
@@ -66,25 +54,8 @@ __global__ __launch_bounds__(TPB) void sample_gaussian_kernel(const float *__res
                                                               float *__restrict__ log_probs) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
-    float total = 0.0f;
-    for (int j = 0; j < A; ++j) {
-        float mean = actor_out[(long)i * 2 * A + j];
-        float log_std = actor_out[(long)i * 2 * A + A + j];
-        if (log_std < -5.0f) log_std = -5.0f;
-        else if (log_std > 2.0f) log_std = 2.0f;
-        Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j), 0, 0);
-        float u1 = rv.v[0] + 1e-8f;
-        float mag = sqrtf(-2.0f * logf(u1));
-        float noise = mag * cosf(rv.v[1] * (float)6.283185307179586);
-        float std = expf(log_std);
-        float action = mean + std * noise;
-        actions[(long)i * A + j] = action;
-        float an = (action - mean) / (std + EPS);
-        float lg = -0.5f * (LOG_2PI + 2.0f * log_std + an * an);
-        total = total + lg;
-    }
-    log_probs[i] = total;
+    const float *o = actor_out + (long)i * 2 * A;
+    log_probs[i] = sample_gaussian(o, o + A, A, seed, i, actions + (long)i * A);
 }
 
 // ---------------------------------------------------------------- GAE

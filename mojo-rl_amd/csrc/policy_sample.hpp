@@ -13,17 +13,17 @@ MRL_DEV void sample_categorical(const float *l, int A, uint32_t seed, int i, int
     float max_logit = l[0];
     for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
     float sum_exp = 0.0f;
-    for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
+    for (int a = 0; a < A; ++a) sum_exp = sum_exp + exp32(l[a] - max_logit);
     const float u = random_uniform(rng);
     float cumsum = 0.0f;
     sel = 0;
     for (int a = 0; a < A; ++a) {
-        float prob = expf(l[a] - max_logit) / sum_exp;
+        float prob = exp32(l[a] - max_logit) / sum_exp;
         cumsum = cumsum + prob;
         if (u < cumsum) { sel = a; break; }
     }
-    const float pr = expf(l[sel] - max_logit) / sum_exp;
-    logp = logf(pr + 1e-8f);
+    const float pr = exp32(l[sel] - max_logit) / sum_exp;
+    logp = log32(pr + 1e-8f);
 }
 
 // Gaussian sampling (deep_agents/ppo/kernels.mojo:12-98) of components j0 .. j0 + m of an action
@@ -40,9 +40,9 @@ MRL_DEV float sample_gaussian_part(const float *mean, const float *log_std_p, in
         else if (log_std > 2.0f) log_std = 2.0f;
         Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j0 + j), 0, 0);
         const float u1 = rv.v[0] + 1e-8f;
-        const float mag = sqrtf(-2.0f * logf(u1));
-        const float noise = mag * cosf(rv.v[1] * (float)6.283185307179586);
-        const float std = expf(log_std);
+        const float mag = sqrtf(-2.0f * log32(u1));
+        const float noise = mag * cos32(rv.v[1] * (float)6.283185307179586);
+        const float std = exp32(log_std);
         const float action = mu + std * noise;
         act[j] = action;
         const float an = (action - mu) / (std + EPS);

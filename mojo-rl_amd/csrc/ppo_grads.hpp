@@ -12,21 +12,21 @@ MRL_DEV float actor_grad_discrete_row(const float *l, int action, float advantag
     float max_logit = l[0];
     for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
     float sum_exp = 0.0f;
-    for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
+    for (int a = 0; a < A; ++a) sum_exp = sum_exp + exp32(l[a] - max_logit);
     float p_action = 0.0f;
     for (int a = 0; a < A; ++a) {
-        float p = expf(l[a] - max_logit) / sum_exp;
+        float p = exp32(l[a] - max_logit) / sum_exp;
         if (a == action) p_action = p;
     }
-    float new_logp = logf(p_action + 1e-8f);
-    float ratio = expf(new_logp - old);
+    float new_logp = log32(p_action + 1e-8f);
+    float ratio = exp32(new_logp - old);
     bool clipped = (ratio < 1.0f - clip_eps) || (ratio > 1.0f + clip_eps);
     for (int a = 0; a < A; ++a) {
         float g = 0.0f;
         if (!clipped) {
-            float p = expf(l[a] - max_logit) / sum_exp;
+            float p = exp32(l[a] - max_logit) / sum_exp;
             float d_log_prob = (a == action) ? 1.0f - p : -p;
-            float log_prob_ent = logf(p + 1e-8f);
+            float log_prob_ent = log32(p + 1e-8f);
             float d_entropy = -p * (1.0f + log_prob_ent);
             g = (-advantage * ratio * d_log_prob - ent_coef * d_entropy) / (float)mb;
         }
@@ -52,7 +52,7 @@ MRL_DEV float actor_grad_gaussian_row(const float *o, const float *act, float ad
         float log_std = o[A + j];
         if (log_std < -5.0f) log_std = -5.0f;
         else if (log_std > 2.0f) log_std = 2.0f;
-        float std = expf(log_std);
+        float std = exp32(log_std);
         float an = (act[j] - o[j]) / (std + eps);
         float lg = -0.5f * (log_2pi + 2.0f * log_std + an * an);
         new_log_prob = new_log_prob + lg;
@@ -60,7 +60,7 @@ MRL_DEV float actor_grad_gaussian_row(const float *o, const float *act, float ad
     float diff = new_log_prob - old_log_prob;
     if (diff > 20.0f) diff = 20.0f;
     else if (diff < -20.0f) diff = -20.0f;
-    float ratio = expf(diff);
+    float ratio = exp32(diff);
     float kl = (ratio - 1.0f) - diff;
     if (kl < 0.0f) kl = 0.0f;
     else if (kl > 100.0f) kl = 100.0f;
@@ -74,7 +74,7 @@ MRL_DEV float actor_grad_gaussian_row(const float *o, const float *act, float ad
             float log_std = o[A + j];
             if (log_std < -5.0f) log_std = -5.0f;
             else if (log_std > 2.0f) log_std = 2.0f;
-            float std = expf(log_std);
+            float std = exp32(log_std);
             float an = (act[j] - o[j]) / (std + eps);
             float d_mean = an / (std + eps);
             float d_log_std = an * an - 1.0f;

@@ -23,6 +23,13 @@
 #include <math.h>
 #include "orc.h"
 
+/* fp32 exp / log / cos as the correctly rounded value (through the Float64 routine, rounded once):
+ * the sampled action index, the PPO ratio and its clip test depend on the last bit, and the
+ * correctly rounded value is the one result that two independent math libraries agree on */
+static inline float f32_exp(float x) { return (float)exp((double)x); }
+static inline float f32_log(float x) { return (float)log((double)x); }
+static inline float f32_cos(float x) { return (float)cos((double)x); }
+
 void orc_sample_categorical(const float *logits, int n, int A, uint32_t seed, float *actions,
                             float *log_probs) {
     for (int i = 0; i < n; ++i) {
@@ -32,18 +39,18 @@ void orc_sample_categorical(const float *logits, int n, int A, uint32_t seed, fl
         float max_logit = l[0];
         for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
         float sum_exp = 0.0f;
-        for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
+        for (int a = 0; a < A; ++a) sum_exp = sum_exp + f32_exp(l[a] - max_logit);
         float u = orc_random_uniform(&rng);
         float cumsum = 0.0f;
         int sel = 0;
         for (int a = 0; a < A; ++a) {
-            float prob = expf(l[a] - max_logit) / sum_exp;
+            float prob = f32_exp(l[a] - max_logit) / sum_exp;
             cumsum = cumsum + prob;
             if (u < cumsum) { sel = a; break; }
         }
         actions[i] = (float)sel;
-        float p = expf(l[sel] - max_logit) / sum_exp;
-        log_probs[i] = logf(p + 1e-8f);
+        float p = f32_exp(l[sel] - max_logit) / sum_exp;
+        log_probs[i] = f32_log(p + 1e-8f);
     }
 }
 
@@ -60,9 +67,9 @@ void orc_sample_gaussian(const float *actor_out, int n, int A, uint64_t seed, fl
             float rv[4];
             orc_philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j), 0, 0, rv);
             float u1 = rv[0] + 1e-8f;
-            float mag = sqrtf(-2.0f * logf(u1));
-            float noise = mag * cosf(rv[1] * (float)6.283185307179586);
-            float std = expf(log_std);
+            float mag = sqrtf(-2.0f * f32_log(u1));
+            float noise = mag * f32_cos(rv[1] * (float)6.283185307179586);
+            float std = f32_exp(log_std);
             float action = mean + std * noise;
             actions[(long)i * A + j] = action;
             float an = (action - mean) / (std + EPS);
@@ -131,17 +138,17 @@ void orc_ppo_actor_grad_discrete(const float *logits, const float *old_logp, con
         float max_logit = l[0];
         for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
         float sum_exp = 0.0f;
-        for (int a = 0; a < A; ++a) sum_exp = sum_exp + expf(l[a] - max_logit);
+        for (int a = 0; a < A; ++a) sum_exp = sum_exp + f32_exp(l[a] - max_logit);
         float probs[64];
-        for (int a = 0; a < A; ++a) probs[a] = expf(l[a] - max_logit) / sum_exp;
-        float new_logp = logf(probs[action] + 1e-8f);
+        for (int a = 0; a < A; ++a) probs[a] = f32_exp(l[a] - max_logit) / sum_exp;
+        float new_logp = f32_log(probs[action] + 1e-8f);
         kl[b] = old_logp[b] - new_logp;
-        float ratio = expf(new_logp - old_logp[b]);
+        float ratio = f32_exp(new_logp - old_logp[b]);
         int clipped = (ratio < 1.0f - clip_eps) || (ratio > 1.0f + clip_eps);
         for (int a = 0; a < A; ++a) {
             if (clipped) { grad_logits[(long)b * A + a] = 0.0f; continue; }
             float d_log_prob = (a == action) ? 1.0f - probs[a] : -probs[a];
-            float log_prob_ent = logf(probs[a] + 1e-8f);
+            float log_prob_ent = f32_log(probs[a] + 1e-8f);
             float d_entropy = -probs[a] * (1.0f + log_prob_ent);
             grad_logits[(long)b * A + a] =
                 (-advantage * ratio * d_log_prob - ent_coef * d_entropy) / (float)mb;
@@ -163,7 +170,7 @@ void orc_ppo_actor_grad_gaussian(const float *actor_out, const float *old_logp, 
             float action = actions[(long)b * A + j];
             if (log_std < -5.0f) log_std = -5.0f;
             else if (log_std > 2.0f) log_std = 2.0f;
-            float std = expf(log_std);
+            float std = f32_exp(log_std);
             float an = (action - mean) / (std + eps);
             av[j] = action; mv[j] = mean; sv[j] = std;
             float lg = -0.5f * (log_2pi + 2.0f * log_std + an * an);
@@ -172,7 +179,7 @@ void orc_ppo_actor_grad_gaussian(const float *actor_out, const float *old_logp, 
         float diff = new_log_prob - old_log_prob;
         if (diff > 20.0f) diff = 20.0f;
         else if (diff < -20.0f) diff = -20.0f;
-        float ratio = expf(diff);
+        float ratio = f32_exp(diff);
         float kl = (ratio - 1.0f) - diff;
         if (kl < 0.0f) kl = 0.0f;
         else if (kl > 100.0f) kl = 100.0f;

@@ -38,11 +38,11 @@ def test_sample_categorical(mrl, orc, ctx):
     a, lp = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
     mrl.ppo.sample_actions(ctx, d(logits.reshape(-1)), a, lp, 987654321)
     ctx.synchronize()
-    # the inverse-CDF comparison u < cumsum can flip when u is within an ulp of a boundary
-    same = h(a) == a_h
-    assert same.mean() > 0.9995, same.mean()
-    np.testing.assert_allclose(h(lp)[same], lp_h[same], rtol=1e-5, atol=1e-6)
-    assert set(np.unique(h(a))) <= {0.0, 1.0, 2.0, 3.0}
+    # same fp32 operations in the same order, exp and log correctly rounded on both sides:
+    # every action and every log-probability is the oracle's, bit for bit
+    np.testing.assert_array_equal(h(a), a_h)
+    np.testing.assert_array_equal(h(lp), lp_h)
+    assert set(np.unique(h(a))) == {0.0, 1.0, 2.0, 3.0}
 
 
 def test_sample_gaussian(mrl, orc, ctx):
@@ -54,8 +54,8 @@ def test_sample_gaussian(mrl, orc, ctx):
     a, lp = torch.zeros(n * A, device="cuda"), torch.zeros(n, device="cuda")
     mrl.ppo.sample_continuous_actions(ctx, d(out.reshape(-1)), a, lp, 4242)
     ctx.synchronize()
-    np.testing.assert_allclose(h(a).reshape(n, A), a_h, rtol=2e-5, atol=2e-5)
-    np.testing.assert_allclose(h(lp), lp_h, rtol=1e-4, atol=1e-3)
+    np.testing.assert_array_equal(h(a).reshape(n, A), a_h)
+    np.testing.assert_array_equal(h(lp), lp_h)
 
 
 @pytest.mark.parametrize("T,N", [(1, 1), (7, 65), (512, 4096)])
@@ -114,10 +114,8 @@ def test_actor_grad_discrete(mrl, orc, ctx):
     mrl.ppo.ppo_actor_grad_with_kl(ctx, g, kl, d(logits.reshape(-1)), d(old), d(adv), d(acts), 0.2, 0.01)
     ctx.synchronize()
     gg = h(g).reshape(mb, A)
-    flip = ((gg == 0).all(1) != (g_h == 0).all(1))     # ratio within an ulp of the clip boundary
-    assert flip.mean() < 1e-3
-    np.testing.assert_allclose(gg[~flip], g_h[~flip], rtol=2e-5, atol=1e-9)
-    np.testing.assert_allclose(h(kl), kl_h, rtol=1e-5, atol=1e-6)
+    np.testing.assert_array_equal(gg, g_h)             # incl. which rows the clip test zeroes
+    np.testing.assert_array_equal(h(kl), kl_h)
     assert 0.05 < (g_h == 0).all(1).mean() < 0.95      # both branches exercised
 
 
@@ -135,10 +133,8 @@ def test_actor_grad_gaussian(mrl, orc, ctx):
     mrl.ppo.ppo_continuous_actor_grad(ctx, g, kl, d(out.reshape(-1)), d(old), d(adv), d(acts.reshape(-1)), 0.2, 0.01)
     ctx.synchronize()
     gg = h(g).reshape(mb, 2 * A)
-    flip = ((gg == 0).all(1) != (g_h == 0).all(1))
-    assert flip.mean() < 1e-3
-    np.testing.assert_allclose(gg[~flip], g_h[~flip], rtol=1e-4, atol=1e-9)
-    np.testing.assert_allclose(h(kl), kl_h, rtol=1e-3, atol=1e-6)
+    np.testing.assert_array_equal(gg, g_h)
+    np.testing.assert_array_equal(h(kl), kl_h)
     assert 0.05 < (g_h == 0).all(1).mean() < 0.95
 
 
@@ -275,9 +271,21 @@ def test_fused_policy_kernel_against_layerwise_path_and_oracle(mrl, orc, orcmod,
     np.testing.assert_array_equal(r_obs.reshape(n, obs_dim), obs)
     np.testing.assert_array_equal(actions, r_actions)
     np.testing.assert_allclose(r_values, values_h[:, 0], rtol=1e-4, atol=1e-5)
+    # the kernel's logits differ from the oracle's serial sums at the MLP tolerance, so a draw may
+    # land on the other side of a CDF boundary -- but only where u is that close to one
     same = r_actions == a_h
     assert same.mean() > 0.995, same.mean()
     np.testing.assert_allclose(r_logp[same], lp_h[same], rtol=1e-4, atol=1e-5)
+    if not same.all():
+        rows = np.nonzero(~same)[0]
+        p64 = np.exp(logits_h[rows].astype(np.float64) - logits_h[rows].max(1, keepdims=True))
+        cdf = np.cumsum(p64 / p64.sum(1, keepdims=True), 1)
+        x = (np.uint32(77) ^ (rows.astype(np.uint64) * 2654435761 & 0xFFFFFFFF).astype(np.uint32)).astype(np.uint64)
+        for _ in range(2):               # seeding step, then the draw (deep_rl/gpu/random.mojo:11-29)
+            x ^= (x << np.uint64(13)) & np.uint64(0xFFFFFFFF); x ^= x >> np.uint64(17); x ^= (x << np.uint64(5)) & np.uint64(0xFFFFFFFF)
+        u = x.astype(np.float64) / 4294967295.0
+        assert np.abs(cdf - u[:, None]).min(1).max() < 2e-5
+        assert np.abs(r_actions[rows] - a_h[rows]).max() == 1.0      # the neighbouring action, nothing else
 
 
 @pytest.mark.parametrize("hidden,kind,obs_dim,A,n", [(256, "tanh", 17, 6, 4096), (256, "relu", 24, 4, 333),
