@@ -288,3 +288,66 @@ def test_continuous_batch_matches_single(orc):
         r, d = step_c(orc, singles[i], float(acts[i, 0]), float(acts[i, 1]), env=i)
         assert r == rew[i] and d == don[i]
     assert np.array_equal(states, singles) and np.array_equal(obs, states[:, :8])
+
+
+def _engine_delta(angle, u0, u1, m_power, s_power, direction):
+    """Velocity change of the lander from the engines, lunar_lander_v2.mojo:1025-1095, in float64
+    vector form: the nozzle offset o is built in the lander's frame from the (tip, side) basis, the
+    impulse is -power * o, and it acts at o (main engine) or at o + (-17/30 tip_x, 14/30 tip_y) (side)."""
+    tip = np.array([math.sin(angle), math.cos(angle)])
+    side = np.array([-tip[1], tip[0]])
+    d = np.array([(u0 * 2.0 - 1.0) / 30.0, (u1 * 2.0 - 1.0) / 30.0])
+    flip = np.array([1.0, -1.0])                 # the reference negates the y component of o
+    cross = lambda a, b: a[0] * b[1] - a[1] * b[0]
+    dv, dw = np.zeros(2), 0.0
+    if m_power > 0:
+        o = flip * (tip * (4.0 / 30.0 + 2.0 * d[0]) + side * d[1])
+        imp = -o * 13.0 * m_power
+        dv += imp / 5.0
+        dw += cross(o, imp) / 2.0
+    if s_power > 0:
+        o = flip * (tip * d[0] + side * (3.0 * d[1] + direction * 12.0 / 30.0))
+        imp = -o * 0.6 * s_power
+        dv += imp / 5.0
+        r = o + np.array([-tip[0] * 17.0 / 30.0, tip[1] * 14.0 / 30.0])
+        dw += cross(r, imp) / 2.0
+    return dv, dw
+
+
+def test_engine_impulses_to_1e6_on_a_free_tilted_lander(orc):
+    """Engines pinned tightly: with the leg joints removed the lander is a free body, so one step
+    leaves it at v0 + dv_engine + g dt exactly.  The uniforms are read back from the oracle's own
+    stream (Philox(env + 12345, offset = step_count), elements 0 and 1)."""
+    env, step_count, angle = 2, 7, 0.37
+    u = np.zeros(4, np.float32)
+    orc.orc_philox_uniform4(env + 12345, step_count, 0, u)
+    assert 0.05 < abs(2 * u[0] - 1) and 0.05 < abs(2 * u[1] - 1) and abs(u[0] - u[1]) > 0.05   # a swap would show
+    def free_lander():
+        row = fresh(orc, 9)
+        row[90] = 0                                    # joint count: no legs attached
+        b = row[BOD:BOD + 39].reshape(3, 13)
+        b[0, 2], b[0, 5] = angle, 0.11
+        row[META] = step_count
+        return row
+    base = free_lander()
+    v0 = base[BOD + 3:BOD + 6].astype(np.float64).copy()
+    x0 = base[BOD:BOD + 3].astype(np.float64).copy()
+    cases = [("discrete", 2, (1.0, 0.0, 0.0)), ("discrete", 1, (0.0, 1.0, -1.0)), ("discrete", 3, (0.0, 1.0, 1.0)),
+             ("continuous", (0.5, -0.8), (0.75, 0.6, -1.0)), ("continuous", (-0.2, 0.9), (0.4, 0.8, 1.0))]
+    for kind, action, (mp, sp, direction) in cases:
+        row = free_lander()
+        r, d = np.zeros(1, np.float32), np.zeros(1, np.float32)
+        if kind == "discrete":
+            orc.orc_ll_step(row, env, action, r, d, None, None)
+        else:
+            orc.orc_ll_step_continuous(row, env, action[0], action[1], r, d, None, None)
+        dv, dw = _engine_delta(angle, float(u[0]), float(u[1]), mp, sp, direction)
+        want_v = v0[:2] + dv + np.array([0.0, -10.0 * 0.02])
+        want_w = v0[2] + dw
+        got = row[BOD + 3:BOD + 6].astype(np.float64)
+        np.testing.assert_allclose(got[:2], want_v, rtol=0, atol=1e-6, err_msg=str((kind, action)))
+        np.testing.assert_allclose(got[2], want_w, rtol=0, atol=1e-6, err_msg=str((kind, action)))
+        # semi-implicit Euler: the position moves with the NEW velocity
+        np.testing.assert_allclose(row[BOD:BOD + 2], x0[:2] + want_v * 0.02, rtol=0, atol=2e-6)
+        np.testing.assert_allclose(row[BOD + 2], x0[2] + want_w * 0.02, rtol=0, atol=1e-6)
+        assert np.abs(dv).max() > 0.03                 # the effect is 4 orders above the tolerance

@@ -213,3 +213,56 @@ def test_batch_wrappers(orc):
     dn = np.zeros(n, np.float32); dn[1] = 1
     h2 = h.copy(); orc.orc_hc_reset_batch(h2, dn.ctypes.data, n, 6)
     assert not np.array_equal(h2[1], h[1]) and np.array_equal(h2[0], h[0])
+
+
+def test_bw_terrain_recurrence_over_all_edges(orc):
+    """bipedal_walker_v2.mojo:395-466: y_i from the damped random walk, one Philox draw per point past
+    the start pad (stream seed + 1000, successive step_uniform calls, element 0), all 128 edges kept."""
+    for seed, env in ((3, 0), (11, 7)):
+        cseed = (seed * 2654435761 + (env + 1) * 12345) & (2**64 - 1)
+        row = np.zeros(950, np.float32)
+        orc.orc_bw_reset(row, cseed)
+        e = row[BW_EDG:BW_EDG + 768].reshape(128, 6)
+        f = np.float32
+        y, v, ys, u = f(TH), f(0.0), [], np.zeros(4, np.float32)
+        for i in range(129):
+            v = f(0.8) * v + f(0.01) * (f(1.0) if f(TH) > y else f(-1.0))
+            if i > 20:
+                orc.orc_philox_uniform4((cseed + 1000) & (2**64 - 1), 0, i - 21, u)
+                v = v + (f(u[0]) * f(2.0) - f(1.0)) / f(30.0)
+            y = f(y + v)
+            ys.append(y)
+        ys = np.array(ys, np.float32)
+        np.testing.assert_array_equal(e[:, 1], ys[:128])
+        np.testing.assert_array_equal(e[:, 3], ys[1:129])
+        x = np.arange(129, dtype=np.float32) * np.float32(14.0 / 30.0)
+        np.testing.assert_array_equal(e[:, 0], x[:128])
+        np.testing.assert_array_equal(e[:, 2], x[1:])
+        # unit normals, turned upwards, perpendicular to the edge
+        dx, dy = e[:, 2] - e[:, 0], e[:, 3] - e[:, 1]
+        ln = np.sqrt(dx * dx + dy * dy)
+        np.testing.assert_array_equal(e[:, 4], -dy / ln)
+        np.testing.assert_array_equal(e[:, 5], dx / ln)
+        assert np.ptp(ys[21:]) > 0.05            # the random term is there
+
+
+def test_hc_joint_limits_and_motor_constants(orc):
+    """half_cheetah/constants.mojo:103-120 (limits), :83-89 (topology): back thigh / shin / foot,
+    front thigh / shin / foot."""
+    row = hc_fresh(orc)
+    j = row[HC_JNT:HC_JNT + 102].reshape(6, 17)
+    limits = [(-0.52, 1.05), (-0.785, 0.785), (-0.4, 0.785), (-1.0, 0.7), (-1.2, 0.87), (-0.5, 0.5)]
+    np.testing.assert_array_equal(j[:, 8], np.array([l for l, _ in limits], np.float32))
+    np.testing.assert_array_equal(j[:, 9], np.array([h for _, h in limits], np.float32))
+    assert (j[:, 7] == 0).all()                                   # reference angle: rest pose
+    # a joint pushed past its upper limit is brought back by the position solve, one inside is left alone
+    b = row[HC_BOD:HC_BOD + 91].reshape(7, 13)
+    for k, (lo, hi) in enumerate(limits):
+        r2 = row.copy()
+        b2 = r2[HC_BOD:HC_BOD + 91].reshape(7, 13)
+        child = int(j[k, 2])
+        b2[child, 2] = hi + 0.3
+        rel0 = b2[child, 2] - b2[int(j[k, 1]), 2]
+        hc_step(orc, r2, [0.0] * 6)
+        rel1 = b2[child, 2] - b2[int(j[k, 1]), 2]
+        assert rel1 < rel0 - 0.05, (k, rel0, rel1)
