@@ -26,7 +26,8 @@ enum {
     MRL_OK = 0,
     MRL_E_ARG = -1,      /* bad argument (null pointer, size, unknown id) */
     MRL_E_HIP = -2,      /* a HIP runtime call failed */
-    MRL_E_UNSUPPORTED = -3
+    MRL_E_UNSUPPORTED = -3,
+    MRL_E_SYNC = -4      /* a kernel gave up waiting at one of its internal barriers */
 };
 
 enum mrl_env_id {
@@ -74,6 +75,14 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out);
 int mrl_ctx_destroy(mrl_ctx *ctx);
 /* blocks until the context's stream has drained; DeviceContext.synchronize() */
 int mrl_ctx_synchronize(mrl_ctx *ctx);
+
+/* The fused collection kernel lets groups of wavefronts of a workgroup meet at barriers of their own
+ * (counters in LDS).  Every such wait is bounded: after `polls` polls (MRL_DEFAULT_SPIN_LIMIT unless
+ * set here; 0 restores the default) the waiting wavefront gives up, the workgroup stops stepping, the
+ * kernel ends normally and the next mrl_ctx_synchronize returns MRL_E_SYNC (once).  No counterpart
+ * in the reference; a tiny limit is how a test exercises the error path without hanging anything. */
+#define MRL_DEFAULT_SPIN_LIMIT (1u << 22)
+int mrl_ctx_set_spin_limit(mrl_ctx *ctx, unsigned polls);
 
 /* Device-time accounting per phase, the counterpart of the perf_counter_ns phase timers that
  * train_gpu prints (deep_agents/ppo/ppo.mojo:2062-2067, :2777-2838) measured with HIP events on

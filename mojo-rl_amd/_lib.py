@@ -69,6 +69,7 @@ SIGNATURES = {
     "mrl_ctx_create": [P, C.POINTER(P)],
     "mrl_ctx_destroy": [P],
     "mrl_ctx_synchronize": [P],
+    "mrl_ctx_set_spin_limit": [P, C.c_uint],
     "mrl_profile_begin": [P, I],
     "mrl_profile_sample_every": [P, I],
     "mrl_profile_end": [P, I, C.POINTER(D), C.POINTER(I)],

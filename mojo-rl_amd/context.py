@@ -41,6 +41,11 @@ class DeviceContext:
     def synchronize(self):
         _lib.call("mrl_ctx_synchronize", self.handle)
 
+    def set_spin_limit(self, polls):
+        """Bound on the polls of a wait at a kernel-internal wavefront barrier (0: the default).  A
+        wait that gives up makes the next synchronize() raise; a tiny value exercises that path."""
+        _lib.call("mrl_ctx_set_spin_limit", self.handle, int(polls))
+
     PHASES = ("policy_fwd", "sample_store", "env_step", "post_store", "collect")
 
     def profile_begin(self, max_marks=8192, sample_every=1):

@@ -100,18 +100,32 @@ struct BlockSync {
 // in LDS that only grows; every arrival adds one, and everyone waits until all arrivals of the
 // current round are in.  Every wavefront of the group must call it the same number of times,
 // outside divergent code.  The counter must be zero before the first use.
+//
+// The wait is bounded: after `spin_limit` polls without the round completing, the waiting
+// wavefront raises the workgroup's `failed` word (LDS) and goes on, and so does every later wait of
+// the workgroup as soon as it sees the word raised -- a wavefront that missed a round therefore costs
+// the launch its results, never its end.  The kernel reports the word to the host when it exits.
 struct WaveGroupSync {
     unsigned *counter;
     unsigned target;   // arrivals expected by the end of the round in progress
     unsigned nwaves;
+    unsigned *failed;      // LDS word shared by the workgroup, zero before the first use
+    unsigned spin_limit;   // polls of the counter before a wait gives up
     MRL_DEV void arrive() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // this wavefront's LDS writes are out
         if ((threadIdx.x & 63) == 0)
             __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     MRL_DEV void wait_for(unsigned arrivals) const {
-        while ((int)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - arrivals) < 0)
+        unsigned polls = 0;
+        while ((int)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - arrivals) < 0) {
+            if (++polls > spin_limit ||
+                ((polls & 255u) == 0u && __hip_atomic_load(failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0u)) {
+                __hip_atomic_store(failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                break;
+            }
             __builtin_amdgcn_s_sleep(1);
+        }
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     }
     MRL_DEV void operator()() {

@@ -38,6 +38,8 @@ struct CollectArgs {
     uint64_t reset_seed, reset_stride;
     float *r_obs, *r_actions, *r_logp, *r_values, *r_rewards, *r_dones;   // time-major, row 0
     Accounting acc;                       // r_rewards / r_dones unused here (set per step)
+    unsigned spin_limit;                  // polls before a wait at a wavefront-group barrier gives up
+    int *sync_error;                      // raised (host-visible) by a workgroup whose wait gave up
 };
 
 template <int A, int B>
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     __shared__ float act[PR * PA_MAX];
     __shared__ float shapes[E::NSHAPE];
     __shared__ unsigned long long was_reset;
-    __shared__ unsigned sync_critic, sync_detect;
+    __shared__ unsigned sync_critic, sync_detect, sync_failed;
     __shared__ float hTc[H * HT_LD];   // the critic's activation tile (live during the env step)
     // the actor's activation tile and the env step's contact scratch are never live together
     constexpr int LIST_F = detect_list_floats<E>() + 1;
@@ -90,14 +92,15 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
         was_reset = 0;
         sync_critic = 0;
         sync_detect = 0;
+        sync_failed = 0;
     }
     __syncthreads();
     // wavefront 0, lane = env slot: the env's running episode return and length stay in registers
     const bool owner = t < nenv;
     float ep_return = owner ? a.acc.ep_return[env0 + t] : 0.0f;
     float ep_length = owner ? a.acc.ep_length[env0 + t] : 0.0f;
-    WaveGroupSync critic_sync{&sync_critic, 0u, (unsigned)CRITIC_WAVES};
-    WaveGroupSync detect_sync{&sync_detect, 0u, (unsigned)(NW - 1)};
+    WaveGroupSync critic_sync{&sync_critic, 0u, (unsigned)CRITIC_WAVES, &sync_failed, a.spin_limit};
+    WaveGroupSync detect_sync{&sync_detect, 0u, (unsigned)(NW - 1), &sync_failed, a.spin_limit};
     static_assert((E::DETECT_TASKS + 1) / 2 <= NW - 1, "two detection tasks per wavefront besides wavefront 0");
 
     // Per step: every wavefront runs the actor (the action is what the env step waits for); then
@@ -199,7 +202,11 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
         }
         __syncthreads();   // env step done, values complete
         if (tid < ne) a.r_values[row + tid] = vals[tid];
+        // a wait that gave up: the block's results are void from here on; leave the loop (every
+        // thread reads the same word after the barrier), store what there is and end normally
+        if (sync_failed != 0u) break;
     }
+    if (t == 0 && sync_failed != 0u) *a.sync_error = 1;
 
     if (owner) {
         a.acc.ep_return[env0 + t] = ep_return;
@@ -428,6 +435,8 @@ int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, u
     a.r_rewards = r->r_rewards; a.r_dones = r->r_dones;
     a.acc = Accounting{r->r_rewards, r->r_dones, r->ep_return, r->ep_length, r->done_returns, r->done_lengths,
                        r->done_count, r->done_cap};
+    a.spin_limit = ctx->spin_limit;
+    a.sync_error = ctx->sync_error;
     const dim3 grid(grid_for(r->n_envs, PR));
     int32_t *side = nullptr;
     if (r->env_id == MRL_ENV_CARTPOLE) {

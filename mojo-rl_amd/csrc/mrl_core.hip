@@ -44,6 +44,7 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     c->reduce_scratch_floats = 4096;
     c->prof_every = 1;
     c->prof_active = true;
+    c->spin_limit = MRL_DEFAULT_SPIN_LIMIT;
     CTX_TRY(hipGetDevice(&c->device));
     mrl::ll::Shapes sh = mrl::ll::make_shapes();
     CTX_TRY(hipMalloc(&c->ll_shapes, sizeof(sh)));
@@ -57,6 +58,8 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     CTX_TRY(hipMalloc(&c->reduce_scratch, sizeof(float) * c->reduce_scratch_floats));
     CTX_TRY(hipMalloc(&c->upd_scratch, sizeof(float) * 8192));
     CTX_TRY(hipMemset(c->upd_scratch, 0, sizeof(float) * 8192));
+    CTX_TRY(hipHostMalloc((void **)&c->sync_error, 64, hipHostMallocDefault));
+    *c->sync_error = 0;
     {
         int rc = mrl::clip_static_setup(c->device);
         if (rc != MRL_OK) { mrl_ctx_destroy(c); return rc; }
@@ -75,6 +78,7 @@ int mrl_ctx_destroy(mrl_ctx *ctx) {
     if (ctx->hc_shapes) hipFree(ctx->hc_shapes);
     if (ctx->reduce_scratch) hipFree(ctx->reduce_scratch);
     if (ctx->upd_scratch) hipFree(ctx->upd_scratch);
+    if (ctx->sync_error) hipHostFree(ctx->sync_error);
     if (ctx->mlp_ws) hipFree(ctx->mlp_ws);
     if (ctx->rollout_ws) hipFree(ctx->rollout_ws);
     for (hipEvent_t e : ctx->prof_events) hipEventDestroy(e);
@@ -85,6 +89,18 @@ int mrl_ctx_destroy(mrl_ctx *ctx) {
 int mrl_ctx_synchronize(mrl_ctx *ctx) {
     MRL_CHECK_ARG(ctx != nullptr, "mrl_ctx_synchronize: ctx is NULL");
     MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    if (*(volatile int *)ctx->sync_error != 0) {
+        *ctx->sync_error = 0;
+        return mrl::set_error(MRL_E_SYNC, "mrl_ctx_synchronize: a kernel gave up waiting at one of its internal "
+                              "barriers (limit %u polls); the results of the calls since the last synchronize are void",
+                              ctx->spin_limit);
+    }
+    return MRL_OK;
+}
+
+int mrl_ctx_set_spin_limit(mrl_ctx *ctx, unsigned polls) {
+    MRL_CHECK_ARG(ctx != nullptr, "mrl_ctx_set_spin_limit: ctx is NULL");
+    ctx->spin_limit = polls == 0 ? MRL_DEFAULT_SPIN_LIMIT : polls;
     return MRL_OK;
 }
 

@@ -33,6 +33,11 @@ struct mrl_ctx {
     // (int, at float index 1024; zero between launches), sum-of-squares partials [2048, 4096),
     // advantage {mean, std} of up to 2048 minibatches [4096, 8192)
     float *upd_scratch;
+    // Kernels whose wavefronts meet at barriers of their own (counters in LDS) bound every wait by
+    // spin_limit polls; a wait that gives up raises *sync_error (pinned host memory that the device
+    // writes directly) and the kernel ends normally.  mrl_ctx_synchronize reports and clears it.
+    unsigned spin_limit;
+    int *sync_error;
     // phase timing: events recorded on `stream` at phase boundaries while armed
     bool profiling;
     std::vector<hipEvent_t> prof_events;

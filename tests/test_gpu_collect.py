@@ -168,3 +168,27 @@ def test_fused_collection_through_contacts(mrl, ctx, orc, env, kind, N):
         assert torch.equal(a, c), "%s: one-step launches differ from single steps in %d places" % (name, int((a != c).sum()))
     cnt = int(single.done_count.item())
     assert cnt == int(fused.done_count.item()) == resets
+
+
+def test_barrier_wait_gives_up_and_reports(mrl):
+    """The wavefront-group barriers inside the fused collection kernel are bounded: with a limit of
+    one poll some wait gives up, the kernel still ends normally, and the next synchronize reports it
+    once.  With the default limit the same launch then runs clean."""
+    ctx = mrl.DeviceContext("cuda:0")
+    N, T = 2048, 4
+    one, many = _pair(mrl, ctx, N, T, 256, "relu", "lunar")
+    s0, ss = 99, 7919
+    ctx.set_spin_limit(1)
+    mrl.ppo.rollout_steps(ctx, many.descriptor(), 0, T, s0, ss, 0, 0, 5, 1)
+    with pytest.raises(mrl.MrlError, match="internal barriers"):
+        ctx.synchronize()
+    ctx.synchronize()                       # reported once, then cleared
+    ctx.set_spin_limit(0)
+    one, many = _pair(mrl, ctx, N, T, 256, "relu", "lunar")
+    d1, d2 = one.descriptor(), many.descriptor()
+    for t in range(T):
+        mrl.ppo.rollout_step(ctx, d1, t, s0 + t * ss, 0, 5 + t)
+    mrl.ppo.rollout_steps(ctx, d2, 0, T, s0, ss, 0, 0, 5, 1)
+    ctx.synchronize()
+    assert torch.equal(one.states, many.states) and torch.equal(one.r_rewards, many.r_rewards)
+    ctx.close()
