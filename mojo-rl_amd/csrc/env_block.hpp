@@ -280,32 +280,33 @@ MRL_DEV void reset_rows_block(float *rows, unsigned long long mask, uint64_t see
     }
 }
 
-// Per-(body, vertex) contact lists of phys_step_block: DCAP records per list (a vertex that fills
+// Per-(body, vertex) contact lists of phys_step_block: CAP records per list (a vertex that fills
 // its list sends the env back to detection inside step_finish), list stride in floats.
 constexpr int DETECT_CAP = 4;
-constexpr int DETECT_STRIDE = (DETECT_CAP * CONTACT_SIZE) | 1;
+constexpr int detect_stride(int cap) { return (cap * CONTACT_SIZE) | 1; }
+constexpr int DETECT_STRIDE = detect_stride(DETECT_CAP);
 
 // task `task` of env slot e: detects into its list and records the count
-template <class E>
+template <class E, int CAP = DETECT_CAP>
 MRL_DEV void detect_vertex_task(const float *rows, const float *shapes, float *dlist, int *dcount, int task, int e) {
     int body, vertex, max_verts;
     E::detect_task(task, body, vertex, max_verts);
     dcount[task * E::EPB + e] = edge_detect_vertex<typename E::L>(
-        rows + e * Stage<E>::STRIDE, shapes, body, vertex, max_verts, dlist + (task * E::EPB + e) * DETECT_STRIDE,
-        DETECT_CAP);
+        rows + e * Stage<E>::STRIDE, shapes, body, vertex, max_verts, dlist + (task * E::EPB + e) * detect_stride(CAP),
+        CAP);
 }
 
 // concatenates env slot e's lists in (body, vertex) order into `mine`, cut at MAX_CONTACTS;
 // returns the contact count, or -1 when some list asks for detection to be redone
-template <class E>
+template <class E, int CAP = DETECT_CAP>
 MRL_DEV int merge_vertex_lists(const float *dlist, const int *dcount, int e, float *mine) {
     int n = 0;
     bool redo = false;
     for (int k = 0; k < E::DETECT_TASKS; ++k) {
-        const float *src = dlist + (k * E::EPB + e) * DETECT_STRIDE;
+        const float *src = dlist + (k * E::EPB + e) * detect_stride(CAP);
         const int m = dcount[k * E::EPB + e];
         redo |= m < 0;
-        for (int c = 0; c < m && n < E::L::MAX_CONTACTS; ++c, ++n)
+        for (int c = 0; c < m && c < CAP && n < E::L::MAX_CONTACTS; ++c, ++n)
             for (int f = 0; f < CONTACT_SIZE; ++f) mine[n * CONTACT_SIZE + f] = src[c * CONTACT_SIZE + f];
     }
     return redo ? -1 : n;
@@ -417,7 +418,14 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
 }
 
 // LDS floats of the per-task contact lists that phys_step_block needs (0: the env detects inline)
-template <class E>
-constexpr int detect_list_floats() { return E::DETECT_TASKS * E::EPB * DETECT_STRIDE; }
+template <class E, int CAP = DETECT_CAP>
+constexpr int detect_list_floats() { return E::DETECT_TASKS * E::EPB * detect_stride(CAP); }
+
+// An env's traits with 16 rows per workgroup of four wavefronts (the fused collection kernel runs
+// two such workgroups per CU, so that one's env step overlaps the other's policy forward)
+template <class Base>
+struct Rows16 : Base {
+    static constexpr int EPB = 16, THREADS = 256;
+};
 
 }  // namespace mrl

@@ -24,6 +24,7 @@
 #include "mrl_host.hpp"
 #include "mrl_device.hpp"
 #include "mlp_tile.hpp"
+#include "mlp_tile16.hpp"
 #include "policy_sample.hpp"
 #include "env_block.hpp"
 #include "env_classic.hpp"
@@ -213,6 +214,195 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
         a.acc.ep_length[env0 + t] = ep_length;
     }
     for (int i = t; i < nenv * E::OBS; i += E::THREADS) {
+        const int r = i / E::OBS, c = i - r * E::OBS;
+        a.obs[(size_t)env0 * E::OBS + i] = rows[r * S::STRIDE + c];
+    }
+    S::out(rows, gbase, nenv, t, 0, E::STATE);
+}
+
+// ---------------------------------------------------------------- 16 rows per workgroup
+// The same step for a workgroup of four wavefronts and 16 envs, for launches with at most 16 envs
+// per CU.  A step is a chain -- actor on the matrix cores, then sampling and the env step on ONE
+// wavefront's vector unit -- and the env step costs the same whether 16 or 32 lanes carry an env,
+// while the actor of 16 rows takes half the matrix time of 32 (v_mfma_f32_16x16x4_f32, same bits as
+// the 32-row tiles): few envs are stepped faster spread 16 to a CU than packed 32 to half the CUs.
+//   all four wavefronts     actor  OBS -> H -> H -> A, 64 columns each;
+//   the solver wavefront    sampling, env step (one env per lane 0 .. 15), accounting, resets;
+//   the other three         contact detection, then the critic (80 / 96 / 80 columns) at a barrier
+//                           of their own.
+// Two such workgroups fit a CU (LDS, registers), but running them side by side does not pay: on this
+// hardware a SIMD issues either a matrix or a vector instruction, never both at once (a wavefront of
+// dependent v_fma_f32 that shares its SIMD with a wavefront issuing v_mfma back to back takes the sum
+// of both times), so one workgroup's env step does not hide behind the other's forward passes, and
+// two solver wavefronts of 16 envs cost twice the vector time of one with 32.  With more than 16 envs
+// per CU the 32-row kernel above is the faster one (8192 envs: 38.6 against 39.8 us per step).
+// The solver wavefront is 0 in the lower half of the grid and 2 in the upper half: workgroups i and
+// i + grid / 2 share a CU when the grid is twice the CU count, and their solvers then sit on
+// different SIMDs.
+template <class EB, int ACT, bool GAUSS>
+__global__ __launch_bounds__(256, 2) void collect16_kernel(CollectArgs a) {
+    using E = Rows16<EB>;
+    using S = Stage<E>;
+    constexpr int H = 256, IN = E::OBS, AW = E::ACT_W, R = PR16, T = E::THREADS;
+    constexpr int CAP = 3;      // records per (body, vertex) list: two contacts, the third signals overflow
+    constexpr int KBA = 8;      // k-steps of layer-1 weights fetched ahead
+    static_assert(IN <= PIN_MAX && AW <= PA_MAX && E::DETECT_TASKS > 0 && E::DETECT_TASKS <= 24, "tile limits; split-off detection");
+    __shared__ float rows[R * S::STRIDE];
+    __shared__ float xs[R * XS_LD];
+    __shared__ __align__(16) float w2a[HEAD_LDS(H)];
+    __shared__ float w2c[H + 1];                    // the critic's head: column of H weights, then the bias
+    __shared__ float logits[R * (PA_MAX + 1)];
+    __shared__ float vals[R];
+    __shared__ float act[R * PA_MAX];
+    __shared__ float shapes[E::NSHAPE];
+    __shared__ unsigned long long was_reset;
+    __shared__ unsigned sync_critic, sync_detect, sync_failed;
+    __shared__ float hTc[H * HT16_LD];              // the critic's activation tile (live during the env step)
+    // the actor's activation tile and the env step's contact scratch are never live together
+    constexpr int LIST_F = detect_list_floats<E, CAP>() + 1;
+    constexpr int ENV_F = R * S::CSTRIDE + LIST_F + E::DETECT_TASKS * R + 1;
+    __shared__ float overlay[cmax<H * HT16_LD, ENV_F>()];
+    float *cts = overlay, *dlist = cts + R * S::CSTRIDE;
+    int *dcount = reinterpret_cast<int *>(dlist + LIST_F);
+
+    const int t = threadIdx.x;
+    const int env0 = blockIdx.x * R;
+    const int nenv = min(R, a.n_envs - env0);
+    const int N = a.n_envs;
+    const int sw = (2 * blockIdx.x >= gridDim.x && gridDim.x > 1) ? 2 : 0;   // the solver wavefront
+    float *gbase = a.states + (size_t)env0 * E::STATE;
+
+    S::in(rows, gbase, nenv, t);
+    for (int i = t; i < E::NSHAPE; i += T) shapes[i] = a.shapes[i];
+    stage_head(a.actor_p + IN * H + H + H * H + H, H, a.A, GAUSS, w2a, t, T);
+    for (int i = t; i < H + 1; i += T) w2c[i] = a.critic_p[IN * H + H + H * H + H + i];
+    if (t == 0) {
+        was_reset = 0;
+        sync_critic = 0;
+        sync_detect = 0;
+        sync_failed = 0;
+    }
+    __syncthreads();
+    // solver wavefront, lane = env slot: the env's running episode return and length stay in registers
+    const bool owner = (t >> 6) == sw && (t & 63) < nenv;
+    float ep_return = owner ? a.acc.ep_return[env0 + (t & 63)] : 0.0f;
+    float ep_length = owner ? a.acc.ep_length[env0 + (t & 63)] : 0.0f;
+    WaveGroupSync critic_sync{&sync_critic, 0u, 3u, &sync_failed, a.spin_limit};
+    WaveGroupSync detect_sync{&sync_detect, 0u, 3u, &sync_failed, a.spin_limit};
+
+    for (int k = 0; k < a.n_steps; ++k) {
+        // Nothing but the rows is carried from one step to the next: the thread index, the block's
+        // env count and the parameter pointers pass through empty asm statements at the top of each
+        // step, so the optimiser cannot keep what it derives from them live through the env step,
+        // whose solver needs the registers.
+        int tid = t, ne = __builtin_amdgcn_readfirstlane(nenv), A = __builtin_amdgcn_readfirstlane(a.A), zero = 0;
+        asm volatile("" : "+v"(tid), "+s"(zero), "+s"(ne), "+s"(A) : : "memory");
+        const float *pa = a.actor_p + zero, *pc = a.critic_p + zero;
+        const size_t row = (size_t)(a.t0 + k) * N + env0;   // this block's slice of rollout row t
+        const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
+        const int wave = tid / WAVE, lane = tid % WAVE;
+        const int vw = (wave - sw) & 3;                     // 0: solver, 1 .. 3: helpers
+        // ---- actor, all wavefronts
+        {
+            Hidden16Operands<H, IN, 4, KBA> ops;
+            ops.load(pa, 64 * wave, lane);
+            for (int i = tid; i < R * IN; i += T) {
+                const int r = i / IN, c = i - r * IN;
+                float v = 0.0f;
+                if (r < ne) {
+                    v = rows[r * S::STRIDE + c];
+                    a.r_obs[row * IN + i] = v;
+                }
+                xs[r * XS_LD + c] = v;
+            }
+            __syncthreads();
+            BlockSync bs;
+            hidden_stack16<H, IN, ACT, 4, KBA, true>(pa, xs, overlay, overlay, ops, 64 * wave, lane, bs);
+            head16<H>(w2a, A, overlay, logits, PA_MAX + 1, tid, T);
+            __syncthreads();   // logits complete; the actor's tile is dead from here on
+        }
+        if (vw == 0) {
+            // ---- sample, then the env step of env_block.hpp with the contacts the helpers detect
+            typename E::Carry carry{};
+            if (lane < ne) {
+                const int i = env0 + lane;
+                float logp;
+                if (GAUSS) {
+                    float av[PA_MAX];
+                    logp = sample_gaussian(logits + lane * (PA_MAX + 1), w2a + HEAD_LOG_STD(H), A, sseed, i, av);
+                    for (int j = 0; j < A; ++j) {
+                        act[lane * AW + j] = av[j];
+                        a.r_actions[(row + lane) * AW + j] = av[j];
+                    }
+                } else {
+                    int sel;
+                    sample_categorical(logits + lane * (PA_MAX + 1), A, sseed, i, sel, logp);
+                    act[lane] = (float)sel;
+                    a.r_actions[row + lane] = (float)sel;
+                }
+                a.r_logp[row + lane] = logp;
+                carry = E::step_begin(rows + lane * S::STRIDE, i, act + lane * AW);
+            }
+            detect_sync.target += detect_sync.nwaves;
+            detect_sync.wait_for(detect_sync.target);
+            bool finished = false;
+            if (lane < ne) {
+                float *mine = cts + lane * S::CSTRIDE;
+                const int n = merge_vertex_lists<E, CAP>(dlist, dcount, lane, mine);
+                float r, d;
+                E::step_finish(rows + lane * S::STRIDE, mine, n, shapes, carry, r, d);
+                a.r_rewards[row + lane] = r;
+                a.r_dones[row + lane] = d;
+                ep_return = ep_return + r;
+                ep_length = ep_length + 1.0f;
+                finished = d > 0.5f;
+                if (finished) {
+                    const int slot = atomicAdd(a.acc.done_count, 1);
+                    if (slot < a.acc.done_cap) {
+                        a.acc.done_returns[slot] = ep_return;
+                        a.acc.done_lengths[slot] = ep_length;
+                    }
+                    ep_return = 0.0f;
+                    ep_length = 0.0f;
+                }
+            }
+            reset_rows<E>(rows, &was_reset, __ballot(finished), a.reset_seed + (uint64_t)k * a.reset_stride, env0, lane);
+        } else {
+            // ---- contact detection: (body, vertex) task m * 4 + lane / 16 of env slot lane % 16, a
+            // second pass on helper 0 for the tasks beyond twelve
+            const int m = vw - 1, e = lane % R;
+            if (e < ne)
+                for (int task = m * 4 + lane / R; task < E::DETECT_TASKS; task += 12)
+                    detect_vertex_task<E, CAP>(rows, shapes, dlist, dcount, task, e);
+            detect_sync.arrive();
+            // ---- critic on the three helpers, at their own barrier: helper 1 takes six column
+            // tiles, helpers 0 (which had the second detection pass) and 2 five each
+            const int tl = m * WAVE + lane;
+            if (m == 1) {
+                Hidden16Operands<H, IN, 6, KBA> ops;
+                ops.load(pc, 80, lane);
+                hidden_stack16<H, IN, ACT, 6, KBA, true>(pc, xs, hTc, hTc, ops, 80, lane, critic_sync);
+            } else {
+                const int c0 = m == 0 ? 0 : 176;
+                Hidden16Operands<H, IN, 5, KBA> ops;
+                ops.load(pc, c0, lane);
+                hidden_stack16<H, IN, ACT, 5, KBA, true>(pc, xs, hTc, hTc, ops, c0, lane, critic_sync);
+            }
+            head_rows16<H, 1, 1>(w2c, 1, hTc, vals, 1, tl, 3 * WAVE);
+        }
+        __syncthreads();   // env step done, values complete
+        if (tid < ne) a.r_values[row + tid] = vals[tid];
+        // a wait that gave up: the block's results are void from here on; leave the loop (every
+        // thread reads the same word after the barrier), store what there is and end normally
+        if (sync_failed != 0u) break;
+    }
+    if (t == 0 && sync_failed != 0u) *a.sync_error = 1;
+
+    if (owner) {
+        a.acc.ep_return[env0 + (t & 63)] = ep_return;
+        a.acc.ep_length[env0 + (t & 63)] = ep_length;
+    }
+    for (int i = t; i < nenv * E::OBS; i += T) {
         const int r = i / E::OBS, c = i - r * E::OBS;
         a.obs[(size_t)env0 * E::OBS + i] = rows[r * S::STRIDE + c];
     }
@@ -437,7 +627,11 @@ int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, u
                        r->done_count, r->done_cap};
     a.spin_limit = ctx->spin_limit;
     a.sync_error = ctx->sync_error;
-    const dim3 grid(grid_for(r->n_envs, PR));
+    // LunarLander: with at most 16 envs per CU the 16-row kernel (a shorter chain per step); beyond that
+    // the 32-row kernel, whose single solver wavefront per CU steps twice the envs in the same time
+    const bool lander = r->env_id == MRL_ENV_LUNARLANDER || r->env_id == MRL_ENV_LUNARLANDER_CONTINUOUS;
+    const bool rows16 = lander && r->n_envs <= ctx->n_cus * PR16;
+    const dim3 grid(grid_for(r->n_envs, rows16 ? PR16 : PR));
     int32_t *side = nullptr;
     if (r->env_id == MRL_ENV_CARTPOLE) {
         rc = cartpole_side(ctx, r->states, r->n_envs, &side);
@@ -445,7 +639,15 @@ int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, u
     }
     profile_step_begin(ctx);
     profile_mark(ctx, -1);
-    if (r->env_id == MRL_ENV_LUNARLANDER) {
+    if (r->env_id == MRL_ENV_LUNARLANDER && rows16) {
+        const dim3 block(Rows16<LunarLander>::THREADS);
+        if (act == 1) hipLaunchKernelGGL((collect16_kernel<LunarLander, 1, false>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((collect16_kernel<LunarLander, 2, false>), grid, block, 0, ctx->stream, a);
+    } else if (r->env_id == MRL_ENV_LUNARLANDER_CONTINUOUS && rows16) {
+        const dim3 block(Rows16<LunarLander>::THREADS);
+        if (act == 1) hipLaunchKernelGGL((collect16_kernel<LunarLanderContinuous, 1, true>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((collect16_kernel<LunarLanderContinuous, 2, true>), grid, block, 0, ctx->stream, a);
+    } else if (r->env_id == MRL_ENV_LUNARLANDER) {
         const dim3 block(LunarLander::THREADS);
         if (act == 1) hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 1, false>), grid, block, 0, ctx->stream, a);
         else hipLaunchKernelGGL((collect_kernel<LunarLander, 256, 2, false>), grid, block, 0, ctx->stream, a);

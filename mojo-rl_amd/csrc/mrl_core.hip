@@ -46,6 +46,7 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
     c->prof_active = true;
     c->spin_limit = MRL_DEFAULT_SPIN_LIMIT;
     CTX_TRY(hipGetDevice(&c->device));
+    CTX_TRY(hipDeviceGetAttribute(&c->n_cus, hipDeviceAttributeMultiprocessorCount, c->device));
     mrl::ll::Shapes sh = mrl::ll::make_shapes();
     CTX_TRY(hipMalloc(&c->ll_shapes, sizeof(sh)));
     CTX_TRY(hipMemcpy(c->ll_shapes, &sh, sizeof(sh), hipMemcpyHostToDevice));

@@ -13,6 +13,7 @@
 struct mrl_ctx {
     hipStream_t stream;
     int device;
+    int n_cus;   // compute units of the device
     // CartPole keeps its per-env step counter (truncation at 500) outside the [B,4] state rows;
     // one int32[batch] array per states pointer, created on first use, freed with the context.
     struct Side { int32_t *steps; int batch; };

@@ -92,7 +92,9 @@ def _low_start(E, N, seed, orc):
     return s_h
 
 
-@pytest.mark.parametrize("env,kind,N", [("lunar", "relu", 2048), ("lunarc", "tanh", 2048), ("lunar", "tanh", 77)])
+# up to 4096 envs (16 per CU) run the 16-row kernel, more the 32-row kernel
+@pytest.mark.parametrize("env,kind,N", [("lunar", "relu", 2048), ("lunarc", "tanh", 2048), ("lunar", "tanh", 77),
+                                        ("lunar", "relu", 4128), ("lunarc", "relu", 4128)])
 def test_fused_collection_through_contacts(mrl, ctx, orc, env, kind, N):
     """The fused collection kernel with the envs on the ground: contact detection on the other
     wavefronts, list merge, solver with contacts, crash / landing terminations and resets inside the
@@ -137,7 +139,7 @@ def test_fused_collection_through_contacts(mrl, ctx, orc, env, kind, N):
         if cont:
             orc.orc_ll_step_continuous_batch(s_h, np.ascontiguousarray(acts.reshape(N, 2)), r_h, d_h, o_h, N)
         else:
-            orc.orc_ll_step_batch(s_h, acts, r_h, d_h, o_h, N, 1)
+            orc.orc_ll_step_batch(s_h, acts, r_h, d_h, o_h, N, 8)
         np.testing.assert_array_equal(fused1.r_rewards[t * N:(t + 1) * N].cpu().numpy(), r_h, err_msg="reward, step %d" % t)
         np.testing.assert_array_equal(fused1.r_dones[t * N:(t + 1) * N].cpu().numpy(), d_h, err_msg="done, step %d" % t)
         crashes += int((r_h == -100).sum())
