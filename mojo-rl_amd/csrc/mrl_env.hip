@@ -10,6 +10,7 @@
 #include "mrl_host.hpp"
 #include "env_classic.hpp"
 #include "env_block.hpp"
+#include "env_cheetah_lanes.hpp"
 
 namespace mrl {
 
@@ -129,6 +130,64 @@ __global__ __launch_bounds__(E::THREADS) void phys_step_kernel(float *states, co
     S::out(rows, gbase, nenv, tid, 0, E::DYN_END);
     S::out(rows, gbase, nenv, tid, E::L::META_OFF, E::STATE);
     if (AUTORESET) S::out_rows(rows, gbase, nenv, was_reset, tid, E::DYN_END, E::L::META_OFF);
+}
+
+// HalfCheetah with one lane per body (env_cheetah_lanes.hpp): a workgroup is one wavefront with
+// eight envs, so 4096 envs are 512 wavefronts spread over the chip instead of 64 long ones.  Rows
+// are staged through LDS as in phys_step_kernel; a row whose wiring is not HalfCheetah's own is
+// stepped by lane 0 of its group with the one-lane form.
+struct HalfCheetahLanes : HalfCheetah {
+    static constexpr int EPB = 8, THREADS = 64;
+};
+
+template <bool AUTORESET>
+__global__ __launch_bounds__(64) void hc_lanes_step_kernel(float *states, const float *actions, float *rewards,
+                                                          float *dones, float *obs, const float *shapes_g,
+                                                          int batch, uint64_t reset_seed, Accounting acc) {
+    using E = HalfCheetahLanes;
+    using S = Stage<E>;
+    __shared__ float rows[E::EPB * S::STRIDE];
+    __shared__ float cts[E::EPB * S::CSTRIDE];   // contact scratch of the one-lane form
+    __shared__ float shapes[E::NSHAPE];
+    const int lane = threadIdx.x;
+    const int env0 = blockIdx.x * E::EPB;
+    const int nenv = min(E::EPB, batch - env0);
+    float *gbase = states + (size_t)env0 * E::STATE;
+    S::in(rows, gbase, nenv, lane);
+    for (int i = lane; i < E::NSHAPE; i += E::THREADS) shapes[i] = shapes_g[i];
+    __syncthreads();
+
+    const int slot = lane >> 3, b = lane & 7;
+    const bool live = slot < nenv;
+    // groups beyond the batch work on LDS rows of their own that are never copied out
+    float *row = rows + slot * S::STRIDE;
+    const int env = env0 + (live ? slot : 0);
+    const float *act = actions + (size_t)env * E::ACT_W;
+    const bool ok = live && hc::lanes_row_ok(row, shapes);
+    float r = 0.0f, d = 0.0f;
+    if (ok) hc::step_lanes(row, shapes, act, lane, r, d);
+    else if (live && b == 0) hc::step_row(row, cts + slot * S::CSTRIDE, shapes, env, act, r, d);
+    bool finished = false;
+    if (live && b == 0) {
+        rewards[env] = r;
+        dones[env] = d;
+        account(acc.at(env0), slot, r, d);
+        finished = d > 0.5f;
+        if (AUTORESET && finished) E::reset(row, reset_seed, env);
+    }
+    const unsigned long long fin = __ballot(finished);
+    unsigned long long was_reset = 0;
+#pragma unroll
+    for (int k = 0; k < E::EPB; ++k) was_reset |= ((fin >> (8 * k)) & 1ull) << k;
+    __syncthreads();
+
+    for (int i = lane; i < nenv * E::OBS; i += E::THREADS) {
+        int rr = i / E::OBS, c = i - rr * E::OBS;
+        obs[(size_t)env0 * E::OBS + i] = rows[rr * S::STRIDE + c];
+    }
+    S::out(rows, gbase, nenv, lane, 0, E::DYN_END);
+    S::out(rows, gbase, nenv, lane, E::L::META_OFF, E::STATE);
+    if (AUTORESET) S::out_rows(rows, gbase, nenv, was_reset, lane, E::DYN_END, E::L::META_OFF);
 }
 
 template <class E>
@@ -295,10 +354,16 @@ static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, con
             launch_phys_step<BipedalWalker>(ctx, batch, states, actions, rewards, dones, obs, ctx->bw_shapes,
                                             autoreset, reset_seed, acc);
             break;
-        case MRL_ENV_HALFCHEETAH:
-            launch_phys_step<HalfCheetah>(ctx, batch, states, actions, rewards, dones, obs, ctx->hc_shapes,
-                                          autoreset, reset_seed, acc);
+        case MRL_ENV_HALFCHEETAH: {
+            const dim3 grid(grid_for(batch, HalfCheetahLanes::EPB)), block(HalfCheetahLanes::THREADS);
+            if (autoreset)
+                hipLaunchKernelGGL((hc_lanes_step_kernel<true>), grid, block, 0, ctx->stream, states, actions, rewards,
+                                   dones, obs, ctx->hc_shapes, batch, reset_seed, acc);
+            else
+                hipLaunchKernelGGL((hc_lanes_step_kernel<false>), grid, block, 0, ctx->stream, states, actions, rewards,
+                                   dones, obs, ctx->hc_shapes, batch, reset_seed, acc);
             break;
+        }
         default:
             return set_error(MRL_E_UNSUPPORTED, "mrl_env_step: env_id %d is not built", env_id);
     }

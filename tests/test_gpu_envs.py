@@ -389,6 +389,36 @@ def test_half_cheetah_rollout_parity(mrl, orc, ctx, batch, seed):
     assert n_done == batch and pen > batch      # every row hits the 1000-step limit once; bodies reach the ground
 
 
+def test_half_cheetah_rows_with_other_wiring_take_the_one_lane_form(mrl, orc, ctx):
+    """The body-per-lane step assumes HalfCheetah's own joint table; a row that differs (here: the
+    front foot's joint removed in every other env, so that foot comes off) is stepped by the generic
+    one-lane form.  Both kinds of rows sit side by side in one wavefront and must match the oracle."""
+    batch = 100
+    E = mrl.HalfCheetahPlanarV2
+    s_h = np.zeros((batch, 253), np.float32)
+    orc.orc_hc_reset_batch(s_h, None, batch, 9)
+    s_h[::2, 17 + 91 + 21 + 102] = 5.0          # joint count
+    s = dev(s_h.reshape(-1))
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch * 6, batch, batch, batch * 17))
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 17), np.float32)
+    rng = np.random.default_rng(9)
+    for t in range(40):
+        act = rng.uniform(-1.2, 1.2, (batch, 6)).astype(np.float32)
+        a.copy_(dev(act.reshape(-1)))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_hc_step_batch(s_h, act, r_h, d_h, o_h, batch, 4)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 253)
+        same_bits(sg, s_h, "state, step %d" % t)
+        np.testing.assert_array_equal(r.cpu().numpy(), r_h)
+        s_h[:] = sg
+    # the loose foot has fallen away from its shin in the rows without the joint
+    foot, shin = s_h[:, 17 + 13 * 6: 17 + 13 * 6 + 3], s_h[:, 17 + 13 * 5: 17 + 13 * 5 + 3]
+    rot = lambda body, ly: np.stack([body[:, 0] - ly * np.sin(body[:, 2]), body[:, 1] + ly * np.cos(body[:, 2])], 1)
+    gap = np.hypot(*(rot(shin, -0.106 / 2) - rot(foot, 0.07 / 2)).T)      # distance between the two anchors
+    assert np.median(gap[::2]) > 0.09 and gap[1::2].max() < 0.08
+
+
 @pytest.mark.parametrize("name", ["CartPoleEnv", "PendulumV2", "BipedalWalkerV2", "HalfCheetahPlanarV2",
                                   "LunarLanderV2Continuous"])
 def test_autoreset_equals_step_then_selective_reset(mrl, ctx, name):
