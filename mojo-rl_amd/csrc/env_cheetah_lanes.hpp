@@ -38,6 +38,36 @@ MRL_DEV void wave_sync_lds() {
 template <class V>
 MRL_DEV V group_get(V v, int base, int src) { return __shfl(v, base + src, 64); }
 
+// The two exchanges of a joint slot as DPP row shifts (register to register, no trip through the LDS
+// crossbar).  Rows are 16 lanes, so the two groups of a row shift side by side; a lane at a group's
+// edge picks up a neighbour group's value that it never uses.
+//   from_parent: every child's parent is the body before it, except the front thigh (4), whose
+//                parent is the torso four lanes down;
+//   from_kid<S>: the parent's lane takes the result of its child in slot S -- the next lane, except
+//                the torso in slot 1, whose child is the front thigh four lanes up.
+MRL_DEV float dpp_row_shr1(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xF, 0xF, false)); }
+MRL_DEV float dpp_row_shr4(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xF, 0xF, false)); }
+MRL_DEV float dpp_row_shl1(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x101, 0xF, 0xF, false)); }
+MRL_DEV float dpp_row_shl4(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x104, 0xF, 0xF, false)); }
+MRL_DEV float from_parent(float v, int b) {
+    const float one = dpp_row_shr1(v), four = dpp_row_shr4(v);
+    return b == 4 ? four : one;
+}
+template <int S>
+MRL_DEV float from_kid(float v, int b) {
+    const float one = dpp_row_shl1(v);
+    if (S == 1) {
+        const float four = dpp_row_shl4(v);
+        return b == 0 ? four : one;
+    }
+    return one;
+}
+
+MRL_DEV float from_kid_slot(int s, float v, int b) {
+    const float one = dpp_row_shl1(v), four = dpp_row_shl4(v);
+    return (s == 1 && b == 0) ? four : one;
+}
+
 // true when the row has the wiring and shapes this form assumes
 MRL_DEV bool lanes_row_ok(const float *row, const float *shapes) {
     if ((int)row[L::JOINT_COUNT_OFF] != 6) return false;
@@ -96,8 +126,9 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
     const int j = child ? b - 1 : 0;
     const int par = (b == 1 || b == 4) ? 0 : (child ? b - 1 : 0);
     const int myslot = b == 1 ? 0 : (b == 2 || b == 4) ? 1 : (b == 3 || b == 5) ? 2 : b == 6 ? 3 : -1;
-    // ... and as the parent of the joint that runs in slot s (lane of that child, or my own lane)
-    const int kid[4] = {b == 0 ? 1 : b, b == 0 ? 4 : b == 1 ? 2 : b, b == 2 ? 3 : b == 4 ? 5 : b, b == 5 ? 6 : b};
+    // ... and as the parent of the joint that runs in slot s: bit s of kidmask (the torso has a child in
+    // slots 0 and 1, the front thigh in slot 1 being the one that sits four lanes up)
+    const int kidmask = b == 0 ? 3 : b == 1 ? 2 : (b == 2 || b == 4) ? 4 : b == 5 ? 8 : 0;
 
     const float gx = (float)0.0, gy = (float)-9.81, dt = (float)0.01, friction = (float)0.9, restitution = (float)0.0;
     const float baumgarte = (float)0.2, slop = (float)0.005;
@@ -130,9 +161,13 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
     float lvx[4], lvy[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) { lvx[v] = S[2 + v * 2]; lvy[v] = S[3 + v * 2]; }
-    const float p_im = group_get(im, base, par), p_ii = group_get(ii, base, par);
+    const float p_im = from_parent(im, b), p_ii = from_parent(ii, b);
     const double x_before = (double)x;   // meaningful on lane 0 (the torso)
 
+    // sine and cosine of my body's angle, kept in step with it (recomputed whenever the angle may have
+    // changed): the same values that the one-lane form recomputes at every use
+    float sin_a, cos_a;
+    sincos32(ang, sin_a, cos_a);
     int kept = 0;   // my body's contacts of the current sub-step that made the list
     for (int sub = 0; sub < 5; ++sub) {
         // ---- integrate velocities (integrators/euler.mojo:82-130)
@@ -144,8 +179,6 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
         fx = fy = tau = 0.0f;   // the forces are cleared at the end of every sub-step
         // ---- ground contacts of my body, vertex order (collision/flat_terrain.mojo:69-204); the list
         // of an env is cut at MAX_CONTACTS in (body, vertex) order: contacts before mine are counted
-        float sin_a, cos_a;
-        sincos32(ang, sin_a, cos_a);
         float cpx[4] = {0.0f, 0.0f, 0.0f, 0.0f}, cpy[4] = {0.0f, 0.0f, 0.0f, 0.0f}, cdepth[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         int found = 0;
 #pragma unroll
@@ -199,8 +232,8 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
             cf[q] = f;
         }
         // ... and the joint's lever arms, K^-1 and limit angle (joints/revolute.mojo:90-200), by the child
-        const float p_sin = group_get(sin_a, base, par), p_cos = group_get(cos_a, base, par);
-        const float p_ang = group_get(ang, base, par);
+        const float p_sin = from_parent(sin_a, b), p_cos = from_parent(cos_a, b);
+        const float p_ang = from_parent(ang, b);
         const float rax = lax * p_cos - lay * p_sin, ray = lax * p_sin + lay * p_cos;
         const float rbx = lbx * cos_a - lby * sin_a, rby = lbx * sin_a + lby * cos_a;
         float inv_k11, inv_k12, inv_k22;
@@ -264,7 +297,7 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 // joints/revolute.mojo:100-320 for the joint whose child I am, when its slot is s
-                const float vxa = group_get(vx, base, par), vya = group_get(vy, base, par), wa = group_get(w, base, par);
+                const float vxa = from_parent(vx, b), vya = from_parent(vy, b), wa = from_parent(w, b);
                 const float inv_ma = p_im, inv_ia = p_ii, inv_mb = im, inv_ib = ii;
                 const float vxb = vx, vyb = vy, wb = w;
                 const float va_anchor_x = vxa - wa * ray, va_anchor_y = vya + wa * rax;
@@ -314,9 +347,9 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
                     }
                 }
                 // the parent takes its new velocity from the child of this slot, the child keeps its own
-                const float g_vx = group_get(n_vxa, base, kid[s]), g_vy = group_get(n_vya, base, kid[s]);
-                const float g_w = group_get(cur_wa, base, kid[s]);
-                if (kid[s] != b) { vx = g_vx; vy = g_vy; w = g_w; }
+                const float g_vx = from_kid_slot(s, n_vxa, b), g_vy = from_kid_slot(s, n_vya, b);
+                const float g_w = from_kid_slot(s, cur_wa, b);
+                if ((kidmask >> s) & 1) { vx = g_vx; vy = g_vy; w = g_w; }
                 if (myslot == s) { vx = n_vxb; vy = n_vyb; w = cur_wb; }
             }
         }
@@ -338,6 +371,7 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
             }
             ang = angle;
         }
+        sincos32(ang, sin_a, cos_a);
         // ---- position iterations: my contacts (solvers/impulse.mojo:333-402), then the joints
         // (joints/revolute.mojo:323-495) slot by slot
         for (int it = 0; it < 2; ++it) {
@@ -356,12 +390,11 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
             }
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                const float xa = group_get(x, base, par), ya = group_get(y, base, par), angle_a = group_get(ang, base, par);
+                const float xa = from_parent(x, b), ya = from_parent(y, b), angle_a = from_parent(ang, b);
                 const float inv_ma = p_im, inv_ia = p_ii, inv_mb = im, inv_ib = ii;
                 const float xb = x, yb = y, angle_b = ang;
-                float s_a, c_a, s_b, c_b;
-                sincos32(angle_a, s_a, c_a);
-                sincos32(angle_b, s_b, c_b);
+                const float s_a = from_parent(sin_a, b), c_a = from_parent(cos_a, b);
+                const float s_b = sin_a, c_b = cos_a;
                 const float r_ax = lax * c_a - lay * s_a, r_ay = lax * s_a + lay * c_a;
                 const float r_bx = lbx * c_b - lby * s_b, r_by = lbx * s_b + lby * c_b;
                 const float anchor_ax = xa + r_ax, anchor_ay = ya + r_ay;
@@ -401,10 +434,11 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
                     n_aa = cur_a;
                     n_ab = cur_b;
                 }
-                const float g_x = group_get(n_xa, base, kid[s]), g_y = group_get(n_ya, base, kid[s]);
-                const float g_a = group_get(n_aa, base, kid[s]);
-                if (kid[s] != b) { x = g_x; y = g_y; ang = g_a; }
+                const float g_x = from_kid_slot(s, n_xa, b), g_y = from_kid_slot(s, n_ya, b);
+                const float g_a = from_kid_slot(s, n_aa, b);
+                if ((kidmask >> s) & 1) { x = g_x; y = g_y; ang = g_a; }
                 if (myslot == s) { x = n_xb; y = n_yb; ang = n_ab; }
+                sincos32(ang, sin_a, cos_a);
             }
         }
     }
