@@ -52,24 +52,21 @@ def fwd_flops(E, hidden):
     return 2 * ((E.OBS_DIM * hidden + hidden * hidden + hidden * a) + (E.OBS_DIM * hidden + hidden * hidden + hidden))
 
 
-def cpu_baseline(np, n_envs=2048, steps=60):
-    """Oracle (C restatement of the reference CPU path): LunarLander env step + policy/value forward
-    + sampling, single thread, on a bounded sample of the default workload."""
-    from oracle import orc
-    o = orc.load()
+def _cpu_rollout(np, orc, o, n_envs, steps, seed):
+    """`steps` collection steps of `n_envs` LunarLander envs on the calling thread (the oracle's C
+    restatement of the reference CPU path: actor / critic forward, sampling, env step, reset)."""
     OBS, HIDDEN, NA = 8, 256, 4
     la = orc.layers([(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, NA)])
     lc = orc.layers([(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, 1)])
-    rng = np.random.default_rng(0)
+    rng = np.random.default_rng(seed)
     pa = rng.uniform(-0.1, 0.1, o.orc_mlp_param_size(la, 3)).astype(np.float32)
     pc = rng.uniform(-0.1, 0.1, o.orc_mlp_param_size(lc, 3)).astype(np.float32)
     s = np.zeros((n_envs, 192), np.float32)
-    o.orc_ll_reset_batch(s, n_envs, 1)
+    o.orc_ll_reset_batch(s, n_envs, 1 + seed)
     obs = np.ascontiguousarray(s[:, :8])
     logits, values = np.zeros((n_envs, NA), np.float32), np.zeros((n_envs, 1), np.float32)
     a, lp = np.zeros(n_envs, np.float32), np.zeros(n_envs, np.float32)
     r, d = np.zeros(n_envs, np.float32), np.zeros(n_envs, np.float32)
-    t0 = time.perf_counter()
     for t in range(steps):
         o.orc_mlp_forward(la, 3, n_envs, obs, pa, logits, None)
         o.orc_mlp_forward(lc, 3, n_envs, obs, pc, values, None)
@@ -77,10 +74,31 @@ def cpu_baseline(np, n_envs=2048, steps=60):
         o.orc_ll_step_batch(s, a, r, d, obs, n_envs, 1)
         o.orc_ll_selective_reset_batch(s, d, n_envs, 500 + t)
         obs[:] = s[:, :8]
-    dt = time.perf_counter() - t0
-    return {"value": n_envs * steps / dt, "unit": "env-steps/s", "cores": 1, "kind": "port",
-            "sample": "LunarLander, %d envs x %d collection steps (env step + actor/critic forward + sampling), "
-                      "single thread, %.1f s" % (n_envs, steps, dt)}
+
+
+def cpu_baseline(np, n_envs=2048, steps=120):
+    """The CPU figure beside the GPU one: the oracle timed on this box's host cores on a bounded
+    sample of the default workload -- once on every core of this job's CPU share (the envs split
+    evenly over the threads, each thread its own rollout loop; the C calls release the GIL), and
+    once on a single thread, which is how the reference's own CPU loop runs."""
+    from concurrent.futures import ThreadPoolExecutor
+    from oracle import orc
+    o = orc.load()
+    cores = max(1, min(int(os.environ.get("OMP_NUM_THREADS", "16")), os.cpu_count() or 1, 16))
+    t0 = time.perf_counter()
+    _cpu_rollout(np, orc, o, n_envs // 4, steps, 0)
+    dt1 = time.perf_counter() - t0
+    single = (n_envs // 4) * steps / dt1
+    per = 4 * n_envs // cores
+    t0 = time.perf_counter()
+    with ThreadPoolExecutor(cores) as pool:
+        list(pool.map(lambda k: _cpu_rollout(np, orc, o, per, steps, k), range(cores)))
+    dtc = time.perf_counter() - t0
+    return {"value": per * cores * steps / dtc, "unit": "env-steps/s", "cores": cores, "kind": "port",
+            "single_thread_value": single,
+            "sample": "LunarLander collection steps (env step + actor / critic forward + sampling + reset): "
+                      "%d envs x %d steps on %d threads in %.1f s; %d envs x %d steps on one thread in %.1f s"
+                      % (per * cores, steps, cores, dtc, n_envs // 4, steps, dt1)}
 
 
 def measured_traffic():
@@ -113,6 +131,12 @@ def main():
                     help="collection steps per fused launch (where the workload has a fused collection kernel)")
     ap.add_argument("--update-minibatches", type=int, default=200,
                     help="minibatches of 4096 timed for the PPO-update figure")
+    ap.add_argument("--preroll", type=int, default=400,
+                    help="untimed collection steps before the warm-up, so that the timed steps see the steady-state "
+                         "mix of flight, contacts, finished episodes and resets instead of a fresh reset's free fall")
+    ap.add_argument("--min-timed-ms", type=float, default=150.0,
+                    help="the timed region of `steps` steps is repeated until this much time has been measured; "
+                         "the median repeat is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 64 MiB read + 64 MiB write elementwise kernel 10 times, the "
@@ -148,25 +172,43 @@ def main():
 
     fused = mrl.ppo.rollout_fused(desc)
     SPL = max(1, min(args.steps_per_launch, T)) if fused else 1   # collection steps per launch
+    # untimed: the envs are taken from the reset into the steady-state episode mix, then the warm-up
+    done = 0
+    while done < args.preroll:
+        n = min(T, args.preroll - done)
+        mrl.ppo.rollout_steps(ctx, desc, 0, n, 7 + done, 1, 0, 0, 9000 + done, 1)
+        done += n
     mrl.ppo.rollout_steps(ctx, desc, 0, min(args.warmup, T), 7, 1, 0, 0, 9000, 1)
     ctx.synchronize()
     rb.done_count.zero_()
     ctx.synchronize()
 
-    # ---- timed region: exactly `steps` collection steps through mrl_rollout_steps.  Where that is
-    # one fused launch per call, every launch is bracketed by HIP events; where it issues two
-    # kernels per step, the events go around the kernels of every 8th step (an event between two
-    # launches costs device time, about 3 us each here, so timing every step would slow the region
-    # it measures).
-    ctx.profile_begin(4 * T + 16, sample_every=1 if fused else EVENT_STRIDE)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for c in range(0, T, SPL if fused else T):
-        n = min(SPL, T - c) if fused else T
-        mrl.ppo.rollout_steps(ctx, desc, c, n, 1000 + c, 1, 0, 0, 50000 + c, 1)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    phases = ctx.profile_end()
+    # ---- timed region: exactly `steps` collection steps through mrl_rollout_steps, bracketed by
+    # synchronisations.  Where that is one fused launch per call, every launch is bracketed by HIP
+    # events; where it issues two kernels per step, the events go around the kernels of every 8th step
+    # (an event between two launches costs device time, about 3 us each here, so timing every step
+    # would slow the region it measures).  A short region (the default of a driver that asks for a few
+    # steps) is repeated, the envs carrying on from where they are, until min-timed-ms has been
+    # measured; the line reports the median repeat.
+    def timed_region(rep):
+        ctx.profile_begin(4 * T + 16, sample_every=1 if fused else EVENT_STRIDE)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for c in range(0, T, SPL if fused else T):
+            n = min(SPL, T - c) if fused else T
+            mrl.ppo.rollout_steps(ctx, desc, c, n, 1000 + c + rep * T, 1, 0, 0, 50000 + c + rep * T, 1)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, ctx.profile_end()
+
+    runs, spent = [], 0.0
+    while True:
+        dt_r, ph_r = timed_region(len(runs))
+        runs.append((dt_r, ph_r))
+        spent += dt_r
+        if spent * 1e3 >= args.min_timed_ms or len(runs) >= 400:
+            break
+    runs.sort(key=lambda x: x[0])
+    dt, phases = runs[len(runs) // 2]
     env_steps_per_s = N_ENVS * T / dt
     episodes = int(rb.done_count.item())
 
@@ -185,7 +227,9 @@ def main():
                 "pendulum": "mrl::collect_classic_kernel<mrl::PendulumSlot, %d, true>" % act_id}[args.workload]
         roofline = {"kernel": name + " (policy forward + sampling + env step + auto-reset + rollout stores, %d steps per launch)" % steps_per_launch,
                     "bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": traffic.get(name),
+                    "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
+                    # measured with 250 steps per launch: it describes no other launch shape
+                    "traffic": traffic.get(name) if steps_per_launch == 250 else None,
                     "avg_launch_us": launch_us, "steps_per_launch": steps_per_launch,
                     "us_per_step": launch_us / steps_per_launch}
         kernels["collect_TFLOPs"] = tflops
@@ -218,7 +262,7 @@ def main():
         else:
             name = {"lunarlander": "mrl::phys_step_kernel<mrl::LunarLander, true>",
                     "bipedal": "mrl::phys_step_kernel<mrl::BipedalWalker, true>",
-                    "halfcheetah": "mrl::phys_step_kernel<mrl::HalfCheetah, true>",
+                    "halfcheetah": "mrl::hc_lanes_step_kernel<true>",
                     "cartpole": "mrl::cartpole_step_kernel", "pendulum": "mrl::pendulum_step_kernel"}[args.workload]
             roofline = {"kernel": name + " (env step + auto-reset + post-step stores)", "bound": "hbm",
                         "achieved": env_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": env_gbs / HBM_PEAK_GBS,
@@ -256,6 +300,7 @@ def main():
         "ppo_update_samples_per_s": update_sps,
         "ppo_update": {"minibatches_timed": n_mb, "ms_per_minibatch": 1e3 * dtu / n_mb,
                        "gae_plus_normalise_ms": gae_ms},
+        "timed_repeats": len(runs), "timed_ms_total": 1e3 * spent, "preroll_steps": args.preroll,
         "episodes_finished": episodes,
         "phase_us": ph_us,
         "phase_events": ({"launches_timed": phases["collect"][1], "steps_per_launch": SPL} if fused else
