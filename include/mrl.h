@@ -150,6 +150,10 @@ int mrl_sample_categorical(mrl_ctx *ctx, const float *logits, int n, int num_act
 /* _sample_continuous_actions_kernel, deep_agents/ppo/kernels.mojo:12-98 */
 int mrl_sample_gaussian(mrl_ctx *ctx, const float *actor_out, int n, int action_dim, uint32_t seed,
                         float *actions, float *log_probs);
+/* add_obs_noise_kernel, deep_agents/ppo/kernels.mojo:882-925 (called at ppo_continuous.mojo:2557 and
+ * :2705): obs[i, d] += noise_std * z with z standard normal from Philox(seed + i * obs_dim + d) by
+ * Box-Muller, in place; nothing happens for noise_std <= 0. */
+int mrl_add_obs_noise(mrl_ctx *ctx, float *obs, int n, int obs_dim, float noise_std, uint32_t seed);
 /* The action of the evaluation policies without sampling.  continuous != 0: the mean of the
  * Gaussian head, actions[i, j] = actor_out[i, j] with actor_out rows [mean (A) | log_std (A)]
  * (extract_deterministic_actions in evaluate_gpu, deep_agents/ppo/ppo_continuous.mojo:807-822).

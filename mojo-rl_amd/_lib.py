@@ -86,6 +86,7 @@ SIGNATURES = {
     "mrl_sample_categorical": [P, P, I, I, U32, P, P],
     "mrl_sample_gaussian": [P, P, I, I, U32, P, P],
     "mrl_greedy_actions": [P, P, I, I, I, P],
+    "mrl_add_obs_noise": [P, P, I, I, F, U32],
     "mrl_gae": [P, I, I, P, P, P, P, D, D, P, P],
     "mrl_normalize_advantages": [P, P, I],
     "mrl_gather_minibatch": [P, P, I, I, I] + [P] * 12,

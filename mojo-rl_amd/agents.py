@@ -54,6 +54,9 @@ class _PPOAgentBase:
         env.reset_kernel_gpu(ctx, rb.states, seed)
         rb.obs.copy_(rb.states.view(N, env.STATE_SIZE)[:, :env.OBS_DIM].reshape(-1))
         rb.ep_return.zero_(); rb.ep_length.zero_()
+        noise_std = float(getattr(self, "obs_noise_std", 0.0)) if self.continuous else 0.0
+        if noise_std > 0.0:
+            ppo.add_obs_noise(ctx, rb.obs, N, noise_std, 42)      # ppo_continuous.mojo:2557-2564
         desc = rb.descriptor()
         total_steps, completed = 0, 0
         target_steps = self.target_total_steps or num_episodes * 200
@@ -64,10 +67,19 @@ class _PPOAgentBase:
             rb.done_count.zero_()
             # step t of this rollout draws its seeds from the running step count, which grows by N
             # per step: affine in t, so the whole rollout is one call (one launch where fusable)
-            ppo.rollout_steps(ctx, desc, 0, T,
-                              total_steps * 2654435761, N * 2654435761 + 7919,
-                              total_steps * 1103515245, N * 1103515245 + 12345,
-                              total_steps * 1013904223, N * 1013904223 + 2654435761)
+            if noise_std > 0.0:
+                # observation noise sits between the env step and the next policy forward
+                # (ppo_continuous.mojo:2705-2713): the steps are issued one by one
+                for t in range(T):
+                    ts = total_steps + t * N
+                    ppo.rollout_step(ctx, desc, t, ts * 2654435761 + t * 7919, ts * 1103515245 + t * 12345,
+                                     ts * 1013904223 + t * 2654435761)
+                    ppo.add_obs_noise(ctx, rb.obs, N, noise_std, ts * 2654435761 + t * 7919)
+            else:
+                ppo.rollout_steps(ctx, desc, 0, T,
+                                  total_steps * 2654435761, N * 2654435761 + 7919,
+                                  total_steps * 1103515245, N * 1103515245 + 12345,
+                                  total_steps * 1013904223, N * 1013904223 + 2654435761)
             total_steps += N * T
             # annealing (ppo.mojo:2385-2406)
             progress = min(1.0, total_steps / float(target_steps))
@@ -250,10 +262,16 @@ class DeepPPOContinuousAgent(DeepPPOAgent):
     continuous = True
 
     def __init__(self, obs_dim, action_dim, hidden_dim=64, rollout_len=128, n_envs=1024,
-                 gpu_minibatch_size=256, normalize_rewards=True, entropy_coef=0.0, **kw):
+                 gpu_minibatch_size=256, normalize_rewards=True, entropy_coef=0.01, num_epochs=10,
+                 target_kl=0.02, action_scale=1.0, action_bias=0.0, obs_noise_std=0.0, **kw):
+        # defaults of ppo_continuous.mojo:236-266 where they differ from the discrete agent's
         super().__init__(obs_dim, action_dim, hidden_dim, rollout_len, n_envs, gpu_minibatch_size,
-                         entropy_coef=entropy_coef, **kw)
+                         entropy_coef=entropy_coef, num_epochs=num_epochs, target_kl=target_kl, **kw)
         self.action_dim, self.normalize_rewards = action_dim, normalize_rewards
+        # action_scale / action_bias only enter the reference's host-side evaluation (:661, :1514);
+        # they are carried for callers that do the same
+        self.action_scale, self.action_bias = action_scale, action_bias
+        self.obs_noise_std = obs_noise_std
 
     def _nets(self):
         H = self.hidden_dim

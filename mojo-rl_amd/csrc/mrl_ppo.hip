@@ -58,6 +58,19 @@ __global__ __launch_bounds__(TPB) void sample_gaussian_kernel(const float *__res
     log_probs[i] = sample_gaussian(o, o + A, A, seed, i, actions + (long)i * A);
 }
 
+// add_obs_noise_kernel, deep_agents/ppo/kernels.mojo:882-925: Gaussian noise on every observation
+// entry, one Philox stream per (env, entry), Box-Muller as in the Gaussian sampler
+__global__ __launch_bounds__(TPB) void obs_noise_kernel(float *__restrict__ obs, int n, int obs_dim,
+                                                        float noise_std, uint32_t seed) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (env, entry)
+    if (e >= (long)n * obs_dim) return;
+    Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + e), 0, 0);
+    const float u1 = rv.v[0] + 1e-8f;
+    const float mag = sqrtf(-2.0f * log32(u1));
+    const float noise = mag * cos32(rv.v[1] * (float)6.283185307179586);
+    obs[e] = obs[e] + noise * noise_std;
+}
+
 // ---------------------------------------------------------------- GAE
 // One lane per env scans t = T-1 .. 0; index t*N + env makes every step of the scan a
 // coalesced row access.  deep_agents/ppo/ppo.mojo:2317-2353
@@ -631,6 +644,17 @@ int mrl_ppo_critic_grad(mrl_ctx *ctx, const float *values, const float *old_valu
                   "mrl_ppo_critic_grad: NULL buffer");
     hipLaunchKernelGGL(critic_grad_kernel, dim3(grid_for(mb, TPB)), dim3(TPB), 0, ctx->stream, values,
                        old_values, returns, mb, convention, clipped, value_coef, clip_eps, grad_values);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+int mrl_add_obs_noise(mrl_ctx *ctx, float *obs, int n, int obs_dim, float noise_std, uint32_t seed) {
+    MRL_CHECK_ARG(ctx, "mrl_add_obs_noise: ctx is NULL");
+    MRL_CHECK_ARG(n >= 0 && obs_dim > 0, "mrl_add_obs_noise: bad sizes");
+    if (n == 0 || !(noise_std > 0.0f)) return MRL_OK;   // the reference's kernel returns at once for std <= 0
+    MRL_CHECK_ARG(obs, "mrl_add_obs_noise: NULL buffer");
+    hipLaunchKernelGGL(obs_noise_kernel, dim3(grid_for((long)n * obs_dim, TPB)), dim3(TPB), 0, ctx->stream, obs, n,
+                       obs_dim, noise_std, seed);
     MRL_CHECK_LAUNCH();
     return MRL_OK;
 }

@@ -22,6 +22,13 @@ def sample_continuous_actions(ctx, actor_output, actions, log_probs, seed):
               int(seed) & 0xFFFFFFFF, _ptr(actions), _ptr(log_probs))
 
 
+def add_obs_noise(ctx, obs, n_envs, noise_std, seed):
+    """add_obs_noise_kernel, deep_agents/ppo/kernels.mojo:882-925: Gaussian noise of standard deviation
+    noise_std on every entry of obs [n_envs, OBS_DIM], in place."""
+    _lib.call("mrl_add_obs_noise", ctx.handle, _ptr(obs), n_envs, obs.numel() // max(n_envs, 1), float(noise_std),
+              int(seed) & 0xFFFFFFFF)
+
+
 def greedy_actions(ctx, actor_output, actions, n, continuous):
     """The actions of `n` rows without sampling: the Gaussian head's mean
     (extract_deterministic_actions, deep_agents/ppo/ppo_continuous.mojo:807-822; rows of

@@ -164,6 +164,7 @@ void orc_sample_categorical(const float *logits, int n, int num_actions, uint32_
                             float *actions, float *log_probs);
 void orc_sample_gaussian(const float *actor_out, int n, int action_dim, uint64_t seed,
                          float *actions, float *log_probs);
+void orc_add_obs_noise(float *obs, int n, int obs_dim, float noise_std, uint32_t seed);
 void orc_gae(int T, int N, const float *rewards, const float *values, const float *dones,
              const float *bootstrap, double gamma, double lam, float *adv, float *ret);
 void orc_normalize_advantages(float *adv, int n);               /* ppo.mojo:2356-2371 */

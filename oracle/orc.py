@@ -98,6 +98,7 @@ def load():
         "orc_mlp_backward": (None, [YP, C.c_int, C.c_int, f32p, f32p, f32p, f32p, C.c_void_p]),
         "orc_sample_categorical": (None, [f32p, C.c_int, C.c_int, C.c_uint32, f32p, f32p]),
         "orc_sample_gaussian": (None, [f32p, C.c_int, C.c_int, C.c_uint64, f32p, f32p]),
+        "orc_add_obs_noise": (None, [f32p, C.c_int, C.c_int, C.c_float, C.c_uint32]),
         "orc_gae": (None, [C.c_int, C.c_int, f32p, f32p, f32p, f32p, C.c_double, C.c_double,
                            f32p, f32p]),
         "orc_normalize_advantages": (None, [f32p, C.c_int]),

@@ -80,6 +80,21 @@ void orc_sample_gaussian(const float *actor_out, int n, int A, uint64_t seed, fl
     }
 }
 
+/* add_obs_noise_kernel, deep_agents/ppo/kernels.mojo:882-925 */
+void orc_add_obs_noise(float *obs, int n, int obs_dim, float noise_std, uint32_t seed) {
+    if (!(noise_std > 0.0f)) return;
+    for (int i = 0; i < n; ++i) {
+        for (int d = 0; d < obs_dim; ++d) {
+            float rv[4];
+            orc_philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * obs_dim + d), 0, 0, rv);
+            float u1_safe = rv[0] + 1e-8f;
+            float mag = sqrtf(-2.0f * f32_log(u1_safe));
+            float noise = mag * f32_cos(rv[1] * (float)6.283185307179586);
+            obs[(long)i * obs_dim + d] = obs[(long)i * obs_dim + d] + noise * noise_std;
+        }
+    }
+}
+
 void orc_gae(int T, int N, const float *rewards, const float *values, const float *dones,
              const float *bootstrap, double gamma, double lam, float *adv, float *ret) {
     const float g = (float)gamma;

@@ -58,6 +58,23 @@ def test_sample_gaussian(mrl, orc, ctx):
     np.testing.assert_array_equal(h(lp), lp_h)
 
 
+def test_add_obs_noise(mrl, orc, ctx):
+    rng = np.random.default_rng(12)
+    for n, D, std, seed in ((4096, 24, 0.05, 123456789), (33, 3, 1.5, 4000000000), (1, 8, 0.1, 7)):
+        obs = rng.normal(size=(n, D)).astype(np.float32)
+        want = obs.copy()
+        orc.orc_add_obs_noise(want, n, D, std, seed)
+        x = d(obs.reshape(-1))
+        mrl.ppo.add_obs_noise(ctx, x, n, std, seed)
+        ctx.synchronize()
+        np.testing.assert_array_equal(h(x).reshape(n, D), want)
+        assert np.abs(want - obs).max() > 0
+    x0 = x.clone()
+    mrl.ppo.add_obs_noise(ctx, x, 1, 0.0, 7)             # std <= 0: nothing happens
+    ctx.synchronize()
+    assert torch.equal(x, x0)
+
+
 @pytest.mark.parametrize("T,N", [(1, 1), (7, 65), (512, 4096)])
 def test_gae(mrl, orc, ctx, T, N):
     say("gae", T, N)

@@ -57,3 +57,29 @@ def test_continuous_agent_runs_on_the_continuous_lunar_lander(mrl):
     assert torch.isfinite(agent.rb.states).all()
     got = agent.evaluate_gpu(ctx, mrl.LunarLanderV2Continuous, num_episodes=64, max_steps=400)
     assert np.isfinite(got) and got < 0.0     # three rollouts do not make a pilot
+
+
+def test_observation_noise_enters_the_rollout(mrl, orc):
+    """obs_noise_std > 0 (ppo_continuous.mojo:2557-2564, :2705-2713): the policy sees noisy
+    observations from the first step on, the env rows stay clean, and the stored observation of step
+    0 is the reset observation plus the oracle's noise for the initial seed 42."""
+    ctx = mrl.DeviceContext("cuda:0")
+    N, T, std = 256, 8, 0.05
+    agent = mrl.DeepPPOContinuousAgent(obs_dim=3, action_dim=1, hidden_dim=64, rollout_len=T, n_envs=N,
+                                       gpu_minibatch_size=512, num_epochs=1, target_kl=0.0, obs_noise_std=std, init_seed=4)
+    assert (agent.num_epochs, agent.entropy_coef, agent.action_scale, agent.action_bias) == (1, 0.01, 1.0, 0.0)
+    assert mrl.DeepPPOContinuousAgent(3, 1).target_kl == 0.02 and mrl.DeepPPOContinuousAgent(3, 1).num_epochs == 10
+    m = agent.train_gpu(ctx, mrl.PendulumV2, num_episodes=10**9, max_rollouts=1, seed=6)
+    assert m.rollouts == 1
+    s0 = torch.zeros(N * 8, device="cuda")
+    mrl.PendulumV2.reset_kernel_gpu(ctx, s0, 6)
+    ctx.synchronize()
+    want = s0.view(N, 8)[:, :3].cpu().numpy().copy()
+    orc.orc_add_obs_noise(want, N, 3, std, 42)
+    np.testing.assert_array_equal(agent.rb.r_obs[:N * 3].cpu().numpy().reshape(N, 3), want)
+    # later steps: stored observation = clean observation of the row + noise of that scale
+    rows = agent.rb.states.view(N, 8).cpu().numpy()
+    last = agent.rb.obs.cpu().numpy().reshape(N, 3)
+    z = (last - rows[:, :3]) / std
+    assert 0.7 < z.std() < 1.3 and abs(z.mean()) < 0.2
+    assert np.abs(np.hypot(rows[:, 0], rows[:, 1]) - 1.0).max() < 1e-5      # the rows themselves carry no noise

@@ -212,6 +212,36 @@ def test_sample_gaussian(orc):
     np.testing.assert_allclose(lp, want, rtol=1e-4, atol=1e-4)
 
 
+def test_add_obs_noise(orc):
+    """kernels.mojo:882-925: obs += std * z, z from Philox(seed + i * OBS + d) by Box-Muller -- the
+    standard normal that the Gaussian sampler draws for (mean 0, log_std 0) on the same stream."""
+    n, D = 5000, 8
+    obs0 = np.random.default_rng(1).normal(size=(n, D)).astype(np.float32)
+    obs = obs0.copy()
+    orc.orc_add_obs_noise(obs, n, D, 0.25, 77)
+    z = (obs.astype(np.float64) - obs0) / 0.25
+    assert abs(z.mean()) < 0.02 and abs(z.std() - 1.0) < 0.02
+    assert abs(np.mean(z ** 3)) < 0.05 and abs(np.mean(z ** 4) - 3.0) < 0.15        # Gaussian, not just unit variance
+    assert abs(np.corrcoef(z[:, 0], z[:, 1])[0, 1]) < 0.05                           # entries are independent
+    # the very numbers of the sampler's noise for the same streams
+    out = np.zeros((n, 2 * D), np.float32)
+    a, lp = np.zeros((n, D), np.float32), np.zeros(n, np.float32)
+    orc.orc_sample_gaussian(out, n, D, 77, a, lp)
+    zero = np.zeros((n, D), np.float32)
+    orc.orc_add_obs_noise(zero, n, D, 1.0, 77)
+    np.testing.assert_array_equal(zero, a)
+    # Box-Muller from the oracle's own uniforms, in float64
+    u = np.zeros(4, np.float32)
+    orc.orc_philox_uniform4(77 + 3 * D + 5, 0, 0, u)
+    want = math.sqrt(-2.0 * math.log(float(u[0]) + 1e-8)) * math.cos(2 * math.pi * float(u[1]))
+    assert abs(zero[3, 5] - want) < 1e-5
+    # std <= 0 leaves the observations alone; the same seed gives the same noise
+    same = obs0.copy(); orc.orc_add_obs_noise(same, n, D, 0.0, 77)
+    np.testing.assert_array_equal(same, obs0)
+    again = obs0.copy(); orc.orc_add_obs_noise(again, n, D, 0.25, 77)
+    np.testing.assert_array_equal(again, obs)
+
+
 def test_actor_grad_gaussian_finite_difference(orc):
     rng = np.random.default_rng(10)
     mb, A = 5, 3
