@@ -120,6 +120,14 @@ int mrl_env_selective_reset(mrl_ctx *ctx, int env_id, int batch, float *states, 
                             uint64_t seed);
 int mrl_env_step(mrl_ctx *ctx, int env_id, int batch, float *states, const float *actions,
                  float *rewards, float *dones, float *obs, uint64_t seed);
+/* CartPole's state row has no slot for the step counter behind the 500-step truncation of the
+ * reference's CPU step (envs/cartpole.mojo:454-457), so the counters live beside the rows: by
+ * default in an int32[batch] array that the context creates, zeroed, on the first call that sees a
+ * `states` pointer, and keeps until the context is destroyed.  This call puts them in the caller's
+ * hands instead: `steps` (device, int32[batch], initialised by the caller) becomes the counter array
+ * of `states` -- a caller that copies or moves its rows copies the counters along and binds them to
+ * the new pointer.  steps = NULL forgets the pointer (and frees a library-made array). */
+int mrl_cartpole_bind_steps(mrl_ctx *ctx, const float *states, int batch, int32_t *steps);
 /* step, then re-initialise rows that finished with the selective-reset protocol, then write
  * obs from the (possibly fresh) row: the sequence step_kernel_gpu -> selective_reset_kernel_gpu
  * -> _extract_obs_from_state_kernel of deep_agents/ppo/ppo.mojo:2148-2285 in one launch.

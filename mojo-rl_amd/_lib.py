@@ -78,6 +78,7 @@ SIGNATURES = {
     "mrl_env_selective_reset": [P, I, I, P, P, U64],
     "mrl_env_step": [P, I, I, P, P, P, P, P, U64],
     "mrl_env_step_autoreset": [P, I, I, P, P, P, P, P, U64, U64],
+    "mrl_cartpole_bind_steps": [P, P, I, P],
     "mrl_mlp_param_size": [DP],
     "mrl_mlp_cache_size": [DP],
     "mrl_mlp_out_dim": [DP],

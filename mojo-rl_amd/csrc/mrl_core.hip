@@ -73,7 +73,8 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out) {
 int mrl_ctx_destroy(mrl_ctx *ctx) {
     if (!ctx) return MRL_OK;
     hipStreamSynchronize(ctx->stream);
-    for (auto &kv : ctx->cartpole_steps) hipFree(kv.second.steps);
+    for (auto &kv : ctx->cartpole_steps)
+        if (kv.second.owned) hipFree(kv.second.steps);
     if (ctx->ll_shapes) hipFree(ctx->ll_shapes);
     if (ctx->bw_shapes) hipFree(ctx->bw_shapes);
     if (ctx->hc_shapes) hipFree(ctx->hc_shapes);

@@ -238,6 +238,9 @@ int cartpole_side(mrl_ctx *ctx, const float *states, int batch, int32_t **out) {
         return MRL_OK;
     }
     if (it != ctx->cartpole_steps.end()) {
+        if (!it->second.owned)
+            return set_error(MRL_E_ARG, "CartPole: the step counters bound to these states hold %d envs, the call has %d",
+                             it->second.batch, batch);
         MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
         MRL_CHECK_HIP(hipFree(it->second.steps));
         ctx->cartpole_steps.erase(it);
@@ -245,7 +248,7 @@ int cartpole_side(mrl_ctx *ctx, const float *states, int batch, int32_t **out) {
     int32_t *p = nullptr;
     MRL_CHECK_HIP(hipMalloc(&p, sizeof(int32_t) * (size_t)batch));
     MRL_CHECK_HIP(hipMemsetAsync(p, 0, sizeof(int32_t) * (size_t)batch, ctx->stream));
-    ctx->cartpole_steps[states] = {p, batch};
+    ctx->cartpole_steps[states] = {p, batch, true};
     *out = p;
     return MRL_OK;
 }
@@ -271,6 +274,21 @@ int mrl_env_dims(int env_id, int *state_size, int *obs_dim, int *num_actions, in
     if (obs_dim) *obs_dim = o;
     if (num_actions) *num_actions = na;
     if (action_dim) *action_dim = ad;
+    return MRL_OK;
+}
+
+int mrl_cartpole_bind_steps(mrl_ctx *ctx, const float *states, int batch, int32_t *steps) {
+    MRL_CHECK_ARG(ctx && states, "mrl_cartpole_bind_steps: NULL argument");
+    MRL_CHECK_ARG(batch >= 0, "mrl_cartpole_bind_steps: negative batch");
+    auto it = ctx->cartpole_steps.find(states);
+    if (it != ctx->cartpole_steps.end()) {
+        if (it->second.owned) {
+            MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+            MRL_CHECK_HIP(hipFree(it->second.steps));
+        }
+        ctx->cartpole_steps.erase(it);
+    }
+    if (steps != nullptr) ctx->cartpole_steps[states] = {steps, batch, false};
     return MRL_OK;
 }
 

@@ -16,7 +16,7 @@ struct mrl_ctx {
     int n_cus;   // compute units of the device
     // CartPole keeps its per-env step counter (truncation at 500) outside the [B,4] state rows;
     // one int32[batch] array per states pointer, created on first use, freed with the context.
-    struct Side { int32_t *steps; int batch; };
+    struct Side { int32_t *steps; int batch; bool owned; };   // owned: allocated by the library
     std::unordered_map<const void *, Side> cartpole_steps;
     // device copy of the shape tables (filled at context creation)
     float *ll_shapes, *bw_shapes, *hc_shapes;

@@ -8,6 +8,8 @@ STATE_SIZE / OBS_DIM / NUM_ACTIONS / ACTION_DIM and three static methods
 over flat fp32 device buffers.  The classes below keep those names and argument meanings; the
 compile-time BATCH becomes the leading size of the buffers.  All calls only enqueue.
 """
+import torch
+
 from . import _lib
 from .context import _ptr
 
@@ -67,6 +69,16 @@ class _GPUEnv:
 
 class CartPoleEnv(_GPUEnv):           # envs/cartpole.mojo:120
     ENV_ID, STATE_SIZE, OBS_DIM, NUM_ACTIONS = _lib.ENV_CARTPOLE, 4, 4, 2
+
+    @classmethod
+    def bind_step_counters(cls, ctx, states, steps):
+        """Makes the int32 device tensor `steps` (one entry per env, or None to forget the binding) the
+        per-env step counters behind the 500-step truncation for the rows at `states`; without it the
+        context keeps counters of its own per states pointer."""
+        from .context import _ptr
+        if steps is not None and (steps.dtype != torch.int32 or steps.numel() * cls.STATE_SIZE != states.numel()):
+            raise _lib.MrlError("step counters: one int32 per env")
+        _lib.call("mrl_cartpole_bind_steps", ctx.handle, _ptr(states), states.numel() // cls.STATE_SIZE, _ptr(steps))
 
 
 class PendulumV2(_GPUEnv):            # envs/pendulum/pendulum_v2.mojo:57

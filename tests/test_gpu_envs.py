@@ -71,6 +71,37 @@ def test_cartpole_rollout_parity(mrl, orc, ctx, batch):
         np.testing.assert_array_equal(d.cpu().numpy(), d_h)
 
 
+def test_cartpole_caller_owned_step_counters(mrl, ctx):
+    """Step counters bound by the caller travel with the rows: a copy of the rows, bound to a copy of
+    the counters, carries on exactly like the original -- including the 500-step truncation."""
+    batch = 64
+    E = mrl.CartPoleEnv
+    s1 = torch.zeros(batch * 4, device="cuda")
+    steps1 = torch.full((batch,), 495, dtype=torch.int32, device="cuda")
+    E.bind_step_counters(ctx, s1, steps1)
+    bufs = lambda: tuple(torch.zeros(n, device="cuda") for n in (batch, batch, batch * 4))
+    r1, d1, o1 = bufs(); r2, d2, o2 = bufs()
+    act = lambda t: ((torch.arange(batch, device="cuda") + t) % 2).float()       # push left and right in turn
+    for t in range(3):
+        E.step_kernel_gpu(ctx, s1, act(t), r1, d1, o1, t)
+    ctx.synchronize()
+    assert steps1.tolist() == [498] * batch and d1.sum().item() == 0
+    s2, steps2 = s1.clone(), steps1.clone()          # the rows move: the counters move with them
+    E.bind_step_counters(ctx, s2, steps2)
+    for t in range(3, 6):
+        E.step_kernel_gpu(ctx, s1, act(t), r1, d1, o1, t)
+        E.step_kernel_gpu(ctx, s2, act(t), r2, d2, o2, t)
+        ctx.synchronize()
+        assert torch.equal(s1, s2) and torch.equal(d1, d2) and torch.equal(steps1, steps2)
+        assert d1.sum().item() == (batch if t == 4 else 0)   # step 500 truncates every env
+        E.selective_reset_kernel_gpu(ctx, s1, d1, 9)
+        E.selective_reset_kernel_gpu(ctx, s2, d2, 9)
+    with pytest.raises(mrl.MrlError):
+        E.bind_step_counters(ctx, s1, torch.zeros(3, dtype=torch.int32, device="cuda"))     # one counter per env
+    E.bind_step_counters(ctx, s1, None)
+    E.bind_step_counters(ctx, s2, None)
+
+
 def test_cartpole_truncation_counter(mrl, orc, ctx):
     # always push towards the centre: the pole survives past 500 steps only by truncation
     batch = 8
