@@ -35,6 +35,9 @@ WORKLOADS = {
                 "BipedalWalker continuous, 4096 envs, Gaussian 24-256-256-4 + value"),
     "halfcheetah": ("HalfCheetahPlanarV2", 4096, 256, "tanh", 1112,
                     "HalfCheetah planar continuous, 4096 envs, Gaussian 17-256-256-6 + value"),
+    # per env-step: the 300 x 9 tile table read once (10800 B) + 40 floats of car state read and written
+    "carracing": ("CarRacingV2", 4096, 256, "tanh", 11120,
+                  "CarRacing (state-based) continuous, 4096 envs, Gaussian 13-256-256-3 + value"),
 }
 
 
@@ -262,7 +265,7 @@ def main():
         else:
             name = {"lunarlander": "mrl::phys_step_kernel<mrl::LunarLander, true>",
                     "bipedal": "mrl::phys_step_kernel<mrl::BipedalWalker, true>",
-                    "halfcheetah": "mrl::hc_lanes_step_kernel<true>",
+                    "halfcheetah": "mrl::hc_lanes_step_kernel<true>", "carracing": "mrl::car_step_kernel<true>",
                     "cartpole": "mrl::cartpole_step_kernel", "pendulum": "mrl::pendulum_step_kernel"}[args.workload]
             roofline = {"kernel": name + " (env step + auto-reset + post-step stores)", "bound": "hbm",
                         "achieved": env_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": env_gbs / HBM_PEAK_GBS,

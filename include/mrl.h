@@ -39,7 +39,8 @@ enum mrl_env_id {
     /* LunarLanderV2 as a GPUContinuousEnv: the step_kernel_gpu overload with ACTION_DIM = 2
      * (lunar_lander_v2.mojo:1520-1588); rows, reset and selective reset are those of
      * MRL_ENV_LUNARLANDER */
-    MRL_ENV_LUNARLANDER_CONTINUOUS = 5
+    MRL_ENV_LUNARLANDER_CONTINUOUS = 5,
+    MRL_ENV_CARRACING = 6    /* envs/car_racing/car_racing_v2.mojo:90 CarRacingV2 (GPUContinuousEnv, :947-1150) */
 };
 
 /* layer kinds of an MLP description; deep_rl/model/{linear,linear_relu,linear_tanh,stochastic_actor}.mojo */

@@ -18,6 +18,7 @@ MAX_LAYERS = 8
 LINEAR, LINEAR_RELU, LINEAR_TANH, STOCHASTIC_ACTOR = 0, 1, 2, 3
 ENV_CARTPOLE, ENV_PENDULUM, ENV_LUNARLANDER, ENV_BIPEDAL, ENV_HALFCHEETAH = 0, 1, 2, 3, 4
 ENV_LUNARLANDER_CONTINUOUS = 5
+ENV_CARRACING = 6
 
 
 class Layer(C.Structure):

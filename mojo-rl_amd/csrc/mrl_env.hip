@@ -11,6 +11,7 @@
 #include "env_classic.hpp"
 #include "env_block.hpp"
 #include "env_cheetah_lanes.hpp"
+#include "env_car.hpp"
 
 namespace mrl {
 
@@ -190,6 +191,45 @@ __global__ __launch_bounds__(64) void hc_lanes_step_kernel(float *states, const 
     if (AUTORESET) S::out_rows(rows, gbase, nenv, was_reset, lane, E::DYN_END, E::L::META_OFF);
 }
 
+// CarRacingV2 (env_car.hpp): sixteen lanes per env, rows in global memory
+constexpr int CAR_THREADS = 256, CAR_EPB = CAR_THREADS / cr::GROUP;
+
+template <bool AUTORESET>
+__global__ __launch_bounds__(CAR_THREADS) void car_step_kernel(float *states, const float *actions, float *rewards,
+                                                               float *dones, float *obs, int batch,
+                                                               uint64_t reset_seed, Accounting acc) {
+    const int lane = threadIdx.x & 63, sub = lane & (cr::GROUP - 1);
+    const int env = blockIdx.x * CAR_EPB + threadIdx.x / cr::GROUP;
+    if (env >= batch) return;   // whole groups leave together
+    float *row = states + (size_t)env * cr::STATE;
+    float r, d;
+    cr::step_group(row, actions + (size_t)env * cr::ACT, lane, r, d);
+    if (sub == 0) {
+        rewards[env] = r;
+        dones[env] = d;
+        account(acc, env, r, d);
+    }
+    if (AUTORESET && d > 0.5f) cr::reset_group(row, cr::combined_seed(reset_seed, env), lane);
+    // the observation out of the row: lane 0 wrote it (step) or the group did (reset); a wavefront's
+    // own stores are visible to its later loads once they have been waited for
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (sub < cr::OBS) obs[(size_t)env * cr::OBS + sub] = row[sub];
+}
+
+__global__ __launch_bounds__(CAR_THREADS) void car_reset_kernel(float *states, float *dones, int batch, uint64_t seed,
+                                                                int selective) {
+    const int lane = threadIdx.x & 63, sub = lane & (cr::GROUP - 1);
+    const int env = blockIdx.x * CAR_EPB + threadIdx.x / cr::GROUP;
+    if (env >= batch) return;
+    if (selective) {
+        if (!(dones[env] > 0.5f)) return;
+    }
+    cr::reset_group(states + (size_t)env * cr::STATE, cr::combined_seed(seed, env), lane);
+    if (selective && sub == 0) dones[env] = 0.0f;
+}
+
 template <class E>
 __global__ __launch_bounds__(E::THREADS) void phys_reset_kernel(float *states, const float *dones, int batch,
                                                            uint64_t seed, int selective) {
@@ -268,6 +308,7 @@ int mrl_env_dims(int env_id, int *state_size, int *obs_dim, int *num_actions, in
         case MRL_ENV_LUNARLANDER_CONTINUOUS: s = ll::STATE; o = ll::OBS; na = 0; ad = 2; break;
         case MRL_ENV_BIPEDAL: s = bw::STATE; o = bw::OBS; na = 0; ad = bw::ACT; break;
         case MRL_ENV_HALFCHEETAH: s = hc::STATE; o = hc::OBS; na = 0; ad = hc::ACT; break;
+        case MRL_ENV_CARRACING: s = cr::STATE; o = cr::OBS; na = 0; ad = cr::ACT; break;
         default: return set_error(MRL_E_UNSUPPORTED, "mrl_env_dims: env_id %d is not built", env_id);
     }
     if (state_size) *state_size = s;
@@ -321,6 +362,10 @@ static int env_reset_impl(mrl_ctx *ctx, int env_id, int batch, float *states, fl
             break;
         case MRL_ENV_BIPEDAL: launch_phys_reset<BipedalWalker>(ctx, batch, states, dones, seed, selective); break;
         case MRL_ENV_HALFCHEETAH: launch_phys_reset<HalfCheetah>(ctx, batch, states, dones, seed, selective); break;
+        case MRL_ENV_CARRACING:
+            hipLaunchKernelGGL(car_reset_kernel, dim3(grid_for(batch, CAR_EPB)), dim3(CAR_THREADS), 0, ctx->stream, states,
+                               dones, batch, seed, selective);
+            break;
         default:
             return set_error(MRL_E_UNSUPPORTED, "mrl_env_reset: env_id %d is not built", env_id);
     }
@@ -380,6 +425,16 @@ static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, con
             else
                 hipLaunchKernelGGL((hc_lanes_step_kernel<false>), grid, block, 0, ctx->stream, states, actions, rewards,
                                    dones, obs, ctx->hc_shapes, batch, reset_seed, acc);
+            break;
+        }
+        case MRL_ENV_CARRACING: {
+            const dim3 grid(grid_for(batch, CAR_EPB)), block(CAR_THREADS);
+            if (autoreset)
+                hipLaunchKernelGGL((car_step_kernel<true>), grid, block, 0, ctx->stream, states, actions, rewards, dones,
+                                   obs, batch, reset_seed, acc);
+            else
+                hipLaunchKernelGGL((car_step_kernel<false>), grid, block, 0, ctx->stream, states, actions, rewards, dones,
+                                   obs, batch, reset_seed, acc);
             break;
         }
         default:

@@ -102,3 +102,9 @@ class BipedalWalkerV2(_GPUEnv):       # envs/bipedal_walker/bipedal_walker_v2.mo
 
 class HalfCheetahPlanarV2(_GPUEnv):   # envs/half_cheetah/cheetah_planar_v2.mojo:91
     ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_HALFCHEETAH, 253, 17, 6
+
+
+class CarRacingV2(_GPUEnv):           # envs/car_racing/car_racing_v2.mojo:90
+    """State-based CarRacing: 13-float observation (hull pose and velocity, front wheel angles, wheel
+    spins, speed), action [steering, gas, brake] in [-1, 1]; every row carries its own random track."""
+    ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_CARRACING, 3040, 13, 3

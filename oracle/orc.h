@@ -164,6 +164,17 @@ void orc_sample_categorical(const float *logits, int n, int num_actions, uint32_
                             float *actions, float *log_probs);
 void orc_sample_gaussian(const float *actor_out, int n, int action_dim, uint64_t seed,
                          float *actions, float *log_probs);
+/* ---------------------------------------------------------- CarRacingV2 --- */
+#define ORC_CR_STATE 3040
+int orc_cr_tile_at(const float *row, float x, float y, int num_tiles);
+uint64_t orc_cr_combined_seed(uint64_t seed, int env);
+void orc_cr_reset(float *row, uint64_t combined_seed);
+void orc_cr_step(float *row, const float *action, float *reward, float *done);
+/* dones == NULL: every row; otherwise rows with dones > 0.5 (their flag is cleared) */
+void orc_cr_reset_batch(float *states, float *dones, int batch, uint64_t seed);
+void orc_cr_step_batch(float *states, const float *actions, float *rewards, float *dones, float *obs, int batch,
+                       int n_threads);
+
 void orc_add_obs_noise(float *obs, int n, int obs_dim, float noise_std, uint32_t seed);
 void orc_gae(int T, int N, const float *rewards, const float *values, const float *dones,
              const float *bootstrap, double gamma, double lam, float *adv, float *ret);
