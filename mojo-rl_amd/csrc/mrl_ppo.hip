@@ -73,27 +73,65 @@ __global__ __launch_bounds__(TPB) void obs_noise_kernel(float *__restrict__ obs,
 
 // ---------------------------------------------------------------- GAE
 // One lane per env scans t = T-1 .. 0; index t*N + env makes every step of the scan a
-// coalesced row access.  deep_agents/ppo/ppo.mojo:2317-2353
-__global__ __launch_bounds__(TPB) void gae_kernel(int T, int N, const float *__restrict__ rewards,
-                                                  const float *__restrict__ values,
-                                                  const float *__restrict__ dones,
-                                                  const float *__restrict__ bootstrap, float gamma,
-                                                  float decay, float *__restrict__ adv,
-                                                  float *__restrict__ ret) {
-    int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= N) return;
-    float gae = 0.0f;
-    float next_val = bootstrap[e];
-    for (int t = T - 1; t >= 0; --t) {
-        long idx = (long)t * N + e;
-        float v = values[idx];
+// coalesced row access.  The scan itself is serial, its loads are not: the rows of the next
+// GAE_U steps are requested while the current ones are scanned, so a wavefront waits for memory
+// once per GAE_U steps instead of once per step.  deep_agents/ppo/ppo.mojo:2317-2353
+constexpr int GAE_U = 16;
+
+struct GaeScan {
+    float gae, next_val, gamma, decay;
+    MRL_DEV void step(float r, float v, float d, float *adv, float *ret) {
         float nv = next_val;
-        if (dones[idx] > 0.5f) { nv = 0.0f; gae = 0.0f; }
-        float delta = rewards[idx] + gamma * nv - v;
+        if (d > 0.5f) { nv = 0.0f; gae = 0.0f; }
+        const float delta = r + gamma * nv - v;
         gae = delta + decay * gae;
-        adv[idx] = gae;
-        ret[idx] = gae + v;
+        *adv = gae;
+        *ret = gae + v;
         next_val = v;
+    }
+};
+
+__global__ __launch_bounds__(64) void gae_kernel(int T, int N, const float *__restrict__ rewards,
+                                                 const float *__restrict__ values,
+                                                 const float *__restrict__ dones,
+                                                 const float *__restrict__ bootstrap, float gamma,
+                                                 float decay, float *__restrict__ adv,
+                                                 float *__restrict__ ret) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= N) return;
+    GaeScan s{0.0f, bootstrap[e], gamma, decay};
+    int t = T - 1;
+    for (; (t + 1) % GAE_U != 0; --t) {   // the steps above the last whole group
+        const long idx = (long)t * N + e;
+        s.step(rewards[idx], values[idx], dones[idx], adv + idx, ret + idx);
+    }
+    // t + 1 is a multiple of GAE_U: groups t, t - 1, .. t - GAE_U + 1
+    float r[GAE_U], v[GAE_U], d[GAE_U], nr[GAE_U], nv[GAE_U], nd[GAE_U];
+    if (t >= 0) {
+#pragma unroll
+        for (int j = 0; j < GAE_U; ++j) {
+            const long idx = (long)(t - j) * N + e;
+            r[j] = rewards[idx]; v[j] = values[idx]; d[j] = dones[idx];
+        }
+    }
+    for (; t >= 0; t -= GAE_U) {
+        const bool more = t - GAE_U >= 0;
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < GAE_U; ++j) {
+                const long idx = (long)(t - GAE_U - j) * N + e;
+                nr[j] = rewards[idx]; nv[j] = values[idx]; nd[j] = dones[idx];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < GAE_U; ++j) {
+            const long idx = (long)(t - j) * N + e;
+            s.step(r[j], v[j], d[j], adv + idx, ret + idx);
+        }
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < GAE_U; ++j) { r[j] = nr[j]; v[j] = nv[j]; d[j] = nd[j]; }
+        }
     }
 }
 

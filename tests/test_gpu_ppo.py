@@ -75,7 +75,7 @@ def test_add_obs_noise(mrl, orc, ctx):
     assert torch.equal(x, x0)
 
 
-@pytest.mark.parametrize("T,N", [(1, 1), (7, 65), (512, 4096)])
+@pytest.mark.parametrize("T,N", [(1, 1), (7, 65), (16, 3), (37, 130), (1000, 300), (512, 4096)])
 def test_gae(mrl, orc, ctx, T, N):
     say("gae", T, N)
     rng = np.random.default_rng(2)
