@@ -7,7 +7,10 @@
  *     layouts (row-major, obs at offset 0 of each env row, rollout buffers time-major);
  *   - the caller owns every buffer; the library owns only its mrl_ctx;
  *   - every call only enqueues work on the context's stream (no synchronisation),
- *     like DeviceContext.enqueue_function in the reference;
+ *     like DeviceContext.enqueue_function in the reference.  One exception: the context holds two
+ *     workspaces (layer-by-layer MLP intermediates; policy temporaries of a rollout step) that grow
+ *     on the first call that needs more than they hold, and growing drains the stream, frees and
+ *     allocates.  mrl_ctx_reserve sizes them ahead so that no later call does;
  *   - return value 0 = success; non-zero = failure, text in mrl_last_error()
  *     (thread-local).  A Mojo shim turns non-zero into `raise Error(...)`.
  */
@@ -76,6 +79,14 @@ int mrl_ctx_create(void *hip_stream, mrl_ctx **out);
 int mrl_ctx_destroy(mrl_ctx *ctx);
 /* blocks until the context's stream has drained; DeviceContext.synchronize() */
 int mrl_ctx_synchronize(mrl_ctx *ctx);
+
+/* Workspaces of the context, in floats: what they hold now (either pointer may be NULL), and a
+ * request to hold at least that much (0 = leave as is; never shrinks).  mrl_ctx_reserve drains the
+ * stream when it has to grow one; after a run of the caller's largest shapes mrl_ctx_workspace
+ * tells what to reserve in the next process.  No counterpart in the reference, whose DeviceContext
+ * allocates inside its layers' forward calls. */
+int mrl_ctx_workspace(mrl_ctx *ctx, uint64_t *mlp_floats, uint64_t *rollout_floats);
+int mrl_ctx_reserve(mrl_ctx *ctx, uint64_t mlp_floats, uint64_t rollout_floats);
 
 /* The fused collection kernel lets groups of wavefronts of a workgroup meet at barriers of their own
  * (counters in LDS).  Every such wait is bounded: after `polls` polls (MRL_DEFAULT_SPIN_LIMIT unless

@@ -71,6 +71,8 @@ SIGNATURES = {
     "mrl_ctx_destroy": [P],
     "mrl_ctx_synchronize": [P],
     "mrl_ctx_set_spin_limit": [P, C.c_uint],
+    "mrl_ctx_workspace": [P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
+    "mrl_ctx_reserve": [P, C.c_uint64, C.c_uint64],
     "mrl_profile_begin": [P, I],
     "mrl_profile_sample_every": [P, I],
     "mrl_profile_end": [P, I, C.POINTER(D), C.POINTER(I)],

@@ -41,6 +41,17 @@ class DeviceContext:
     def synchronize(self):
         _lib.call("mrl_ctx_synchronize", self.handle)
 
+    def workspace(self):
+        """(mlp_floats, rollout_floats) that the context's two workspaces hold now."""
+        import ctypes
+        a, b = ctypes.c_uint64(0), ctypes.c_uint64(0)
+        _lib.call("mrl_ctx_workspace", self.handle, ctypes.byref(a), ctypes.byref(b))
+        return a.value, b.value
+
+    def reserve(self, mlp_floats=0, rollout_floats=0):
+        """Size the workspaces ahead, so that no later call has to drain the stream and allocate."""
+        _lib.call("mrl_ctx_reserve", self.handle, int(mlp_floats), int(rollout_floats))
+
     def set_spin_limit(self, polls):
         """Bound on the polls of a wait at a kernel-internal wavefront barrier (0: the default).  A
         wait that gives up makes the next synchronize() raise; a tiny value exercises that path."""

@@ -15,6 +15,17 @@ int set_error(int code, const char *fmt, ...) {
     return code;
 }
 
+int grow_workspace(mrl_ctx *ctx, float **buf, size_t *have, size_t need) {
+    if (*have >= need) return MRL_OK;
+    MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    if (*buf) MRL_CHECK_HIP(hipFree(*buf));
+    *buf = nullptr;
+    *have = 0;
+    MRL_CHECK_HIP(hipMalloc(buf, sizeof(float) * need));
+    *have = need;
+    return MRL_OK;
+}
+
 }  // namespace mrl
 
 extern "C" {
@@ -98,6 +109,20 @@ int mrl_ctx_synchronize(mrl_ctx *ctx) {
                               ctx->spin_limit);
     }
     return MRL_OK;
+}
+
+int mrl_ctx_workspace(mrl_ctx *ctx, uint64_t *mlp_floats, uint64_t *rollout_floats) {
+    MRL_CHECK_ARG(ctx != nullptr, "mrl_ctx_workspace: ctx is NULL");
+    if (mlp_floats) *mlp_floats = ctx->mlp_ws_floats;
+    if (rollout_floats) *rollout_floats = ctx->rollout_ws_floats;
+    return MRL_OK;
+}
+
+int mrl_ctx_reserve(mrl_ctx *ctx, uint64_t mlp_floats, uint64_t rollout_floats) {
+    MRL_CHECK_ARG(ctx != nullptr, "mrl_ctx_reserve: ctx is NULL");
+    int rc = mrl::grow_workspace(ctx, &ctx->mlp_ws, &ctx->mlp_ws_floats, (size_t)mlp_floats);
+    if (rc != MRL_OK) return rc;
+    return mrl::grow_workspace(ctx, &ctx->rollout_ws, &ctx->rollout_ws_floats, (size_t)rollout_floats);
 }
 
 int mrl_ctx_set_spin_limit(mrl_ctx *ctx, unsigned polls) {

@@ -55,6 +55,9 @@ namespace mrl {
 
 int set_error(int code, const char *fmt, ...);
 
+// makes *buf hold at least `need` floats (never shrinks); growing drains the stream first
+int grow_workspace(mrl_ctx *ctx, float **buf, size_t *have, size_t need);
+
 // Post-step bookkeeping of a collection step, done by the env-step kernel itself when the rollout
 // step asks for it (all pointers null otherwise): rollout rows of reward / done, per-env episode
 // return and length, and the device-side list of finished episodes.

@@ -272,16 +272,9 @@ static int check_desc(const mrl_mlp_desc *d, const char *who) {
 
 // grows the context's MLP workspace (activations between layers, split-K partials)
 static int ensure_ws(mrl_ctx *ctx, size_t floats, float **out) {
-    if (ctx->mlp_ws_floats < floats) {
-        MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
-        if (ctx->mlp_ws) MRL_CHECK_HIP(hipFree(ctx->mlp_ws));
-        ctx->mlp_ws = nullptr;
-        ctx->mlp_ws_floats = 0;
-        MRL_CHECK_HIP(hipMalloc(&ctx->mlp_ws, sizeof(float) * floats));
-        ctx->mlp_ws_floats = floats;
-    }
+    int rc = grow_workspace(ctx, &ctx->mlp_ws, &ctx->mlp_ws_floats, floats);
     *out = ctx->mlp_ws;
-    return MRL_OK;
+    return rc;
 }
 
 template <int ACT>

@@ -65,15 +65,7 @@ extern "C" {
 
 // layer-by-layer fallback needs logits/values temporaries
 static int ensure_rollout_ws(mrl_ctx *ctx, size_t need) {
-    if (ctx->rollout_ws_floats < need) {
-        MRL_CHECK_HIP(hipStreamSynchronize(ctx->stream));
-        if (ctx->rollout_ws) MRL_CHECK_HIP(hipFree(ctx->rollout_ws));
-        ctx->rollout_ws = nullptr;
-        ctx->rollout_ws_floats = 0;
-        MRL_CHECK_HIP(hipMalloc(&ctx->rollout_ws, sizeof(float) * need));
-        ctx->rollout_ws_floats = need;
-    }
-    return MRL_OK;
+    return mrl::grow_workspace(ctx, &ctx->rollout_ws, &ctx->rollout_ws_floats, need);
 }
 
 static int policy_step(mrl_ctx *ctx, const char *who, bool gauss, const mrl_mlp_desc *actor,

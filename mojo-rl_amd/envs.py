@@ -8,10 +8,17 @@ STATE_SIZE / OBS_DIM / NUM_ACTIONS / ACTION_DIM and three static methods
 over flat fp32 device buffers.  The classes below keep those names and argument meanings; the
 compile-time BATCH becomes the leading size of the buffers.  All calls only enqueue.
 """
+import collections
+
 import torch
 
 from . import _lib
 from .context import _ptr
+
+# core/vec_env.mojo:25-58: the batched result of one step (observations per env, rewards, done flags).
+# The reference fills it from SIMD vectors on the host; here the three members are the device tensors
+# the step wrote ([batch, OBS_DIM], [batch], [batch]; done flags are 0.0 / 1.0 floats as in the traits).
+VecStepResult = collections.namedtuple("VecStepResult", ["observations", "rewards", "dones"])
 
 
 class _GPUEnv:
@@ -65,6 +72,16 @@ class _GPUEnv:
         _lib.call("mrl_env_step_autoreset", ctx.handle, cls.ENV_ID, b, _ptr(states), _ptr(actions),
                   _ptr(rewards), _ptr(dones), _ptr(obs), int(step_seed) & (2**64 - 1),
                   int(reset_seed) & (2**64 - 1))
+
+
+    @classmethod
+    def step_result(cls, ctx, states, actions, rng_seed=0):
+        """step_kernel_gpu into fresh buffers, returned as a VecStepResult."""
+        b = cls._batch(states)
+        rewards, dones = ctx.enqueue_create_buffer(b), ctx.enqueue_create_buffer(b)
+        obs = ctx.enqueue_create_buffer(b * cls.OBS_DIM)
+        cls.step_kernel_gpu(ctx, states, actions, rewards, dones, obs, rng_seed)
+        return VecStepResult(obs.view(b, cls.OBS_DIM), rewards, dones)
 
 
 class CartPoleEnv(_GPUEnv):           # envs/cartpole.mojo:120

@@ -560,3 +560,19 @@ def test_lander_vertex_over_many_edges_takes_the_serial_detector(mrl, orc, ctx):
         s_h[:] = sg
     say("  leg contacts on the crowded pad:", legs)
     assert legs > 20
+
+
+def test_step_result_is_the_step_in_fresh_buffers(mrl, ctx):
+    """VecStepResult (core/vec_env.mojo:25) from step_result equals what step_kernel_gpu writes."""
+    E, batch = mrl.PendulumV2, 33
+    s1 = torch.zeros(batch * E.STATE_SIZE, device="cuda")
+    E.reset_kernel_gpu(ctx, s1, 4)
+    s2 = s1.clone()
+    act = torch.linspace(-2, 2, batch, device="cuda")
+    r, d_, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch * E.OBS_DIM))
+    E.step_kernel_gpu(ctx, s1, act, r, d_, o, 1)
+    res = E.step_result(ctx, s2, act, 1)
+    ctx.synchronize()
+    assert isinstance(res, mrl.VecStepResult) and res.observations.shape == (batch, E.OBS_DIM)
+    assert torch.equal(res.observations.reshape(-1), o) and torch.equal(res.rewards, r) and torch.equal(res.dones, d_)
+    assert torch.equal(s1, s2)

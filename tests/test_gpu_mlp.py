@@ -124,3 +124,31 @@ def test_mlp_argument_errors(mrl, ctx):
     with pytest.raises(mrl.MrlError):
         mrl.seq(mrl.LinearReLU(8, 16), mrl.Linear(15, 2))       # dims do not chain
     model.forward_gpu_no_cache_ws(ctx, torch.zeros(0, device="cuda"), torch.zeros(0, device="cuda"), p)
+
+
+def test_reserved_workspace_is_not_grown_again(mrl):
+    """A context whose workspace was reserved ahead runs the layer-by-layer path without allocating:
+    the size it reports stays what was reserved, and the result equals the one of a context that
+    grew its workspace on demand."""
+    spec = [(RELU, 5, 33), (TANH, 33, 70), (LIN, 70, 3)]       # not the fused three-layer shape
+    model = mk(mrl, spec)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    p = torch.randn(model.PARAM_SIZE, device="cuda", generator=g) * 0.3
+    x = torch.randn(300 * 5, device="cuda", generator=g)
+    grown, reserved = mrl.DeviceContext("cuda:0"), mrl.DeviceContext("cuda:0")
+    assert grown.workspace() == (0, 0)
+    out_a = torch.zeros(300 * 3, device="cuda")
+    model.forward_gpu_no_cache_ws(grown, out_a, x, p)
+    grown.synchronize()
+    need = grown.workspace()[0]
+    assert need >= 2 * 300 * 70
+    reserved.reserve(mlp_floats=need, rollout_floats=1000)
+    assert reserved.workspace() == (need, 1000)
+    reserved.reserve(mlp_floats=1, rollout_floats=0)              # never shrinks, 0 leaves as is
+    assert reserved.workspace() == (need, 1000)
+    out_b = torch.zeros(300 * 3, device="cuda")
+    before = torch.cuda.memory_allocated()
+    model.forward_gpu_no_cache_ws(reserved, out_b, x, p)
+    reserved.synchronize()
+    assert reserved.workspace() == (need, 1000) and torch.cuda.memory_allocated() == before
+    assert torch.equal(out_a, out_b)
