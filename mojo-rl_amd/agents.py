@@ -109,6 +109,96 @@ class _PPOAgentBase:
             self.train_step_count += total_steps   # ppo_continuous.mojo:3328
         return metrics
 
+    def train_gpu_cpu_env(self, ctx, envs, num_episodes, verbose=False, print_every=10, max_rollouts=None,
+                          seed=0):
+        """Networks on the device, environments on the host (deep_agents/ppo/ppo.mojo:2846-3960,
+        ppo_continuous.mojo:977-2170).  `envs` is a list of exactly n_envs objects of the caller with the
+        reference's CPU env interface: reset_obs_list() -> observation, and step_obs(action: int) (discrete
+        agent, core/env_traits.mojo:163-184) or step_continuous_vec(action: list) (continuous agent,
+        :186-222) -> (observation, reward, done).  Per step: one policy launch, the actions to the host,
+        the envs stepped one by one in index order, finished envs reset at once, the observations back to
+        the device.  The continuous agent hands the envs  clip(action * action_scale + action_bias, -1, 1)
+        and stores the raw action, as the reference does.  The rollout is dropped without an update when
+        the episode target is reached inside it (the reference's early `break`).  GAE, normalisation and
+        the epochs are those of train_gpu, on the device."""
+        if len(envs) != self.n_envs:
+            raise ValueError("expected %d environments, got %d" % (self.n_envs, len(envs)))
+        N, T = self.n_envs, self.rollout_len
+        aw = self.action_dim if self.continuous else 1
+        shape = type("HostEnv", (), dict(ENV_ID=-1, STATE_SIZE=self.obs_dim, OBS_DIM=self.obs_dim,
+                                         NUM_ACTIONS=0 if self.continuous else self.num_actions,
+                                         ACTION_DIM=aw if self.continuous else 0))
+        self._build(ctx, shape)
+        rb, upd = self.rb, self.upd
+        metrics = TrainingMetrics("Deep PPO (GPU+CPU)" + (" continuous" if self.continuous else ""), "CPU Environment")
+        obs_host = torch.zeros(N, self.obs_dim, pin_memory=True)
+        act_host = torch.zeros(N * aw, pin_memory=True)
+        rew_host, done_host = torch.zeros(T * N, pin_memory=True), torch.zeros(T * N, pin_memory=True)
+        actions = torch.zeros(N * aw, device=ctx.device)
+        for i, e in enumerate(envs):
+            obs_host[i] = torch.as_tensor(e.reset_obs_list(), dtype=torch.float32)
+        stream = torch.cuda.stream(ctx.stream)       # the copies go where the library enqueues
+        with stream:
+            rb.obs.copy_(obs_host.reshape(-1))
+        ep_return, ep_steps = [0.0] * N, [0] * N
+        total_steps, completed = 0, 0
+        target_steps = self.target_total_steps or num_episodes * 200
+        a_lr0, c_lr0, ent0 = self.actor_lr, self.critic_lr, self.entropy_coef
+        scale, bias = getattr(self, "action_scale", 1.0), getattr(self, "action_bias", 0.0)
+        while completed < num_episodes:
+            if max_rollouts is not None and metrics.rollouts >= max_rollouts:
+                break
+            for t in range(T):
+                ppo.policy_step(ctx, rb, t, total_steps * 2654435761 + t * 7919, actions)
+                with stream:
+                    act_host.copy_(actions)
+                ctx.synchronize()
+                a_list = act_host.tolist()
+                for i, e in enumerate(envs):
+                    if self.continuous:
+                        a = [min(1.0, max(-1.0, a_list[i * aw + k] * scale + bias)) for k in range(aw)]
+                        nxt, reward, done = e.step_continuous_vec(a)
+                    else:
+                        nxt, reward, done = e.step_obs(int(a_list[i]))
+                    rew_host[t * N + i] = float(reward)
+                    done_host[t * N + i] = 1.0 if done else 0.0
+                    ep_return[i] += float(reward)
+                    ep_steps[i] += 1
+                    if done:
+                        metrics.log_episodes([ep_return[i]], [ep_steps[i]])
+                        completed += 1
+                        if (self.checkpoint_every > 0 and self.checkpoint_path != ""
+                                and completed % self.checkpoint_every == 0):
+                            self.save_checkpoint(self.checkpoint_path)
+                        ep_return[i], ep_steps[i] = 0.0, 0
+                        nxt = e.reset_obs_list()
+                    obs_host[i] = torch.as_tensor(nxt, dtype=torch.float32)
+                total_steps += N
+                with stream:
+                    rb.obs.copy_(obs_host.reshape(-1))
+                ctx.synchronize()       # obs_host is rewritten while the envs of the next step run
+            if completed >= num_episodes:
+                break
+            with stream:
+                rb.r_rewards.copy_(rew_host)
+                rb.r_dones.copy_(done_host)
+            progress = min(1.0, total_steps / float(target_steps))
+            if self.anneal_lr:
+                self.actor.optimizer.lr = a_lr0 * (1.0 - progress)
+                self.critic.optimizer.lr = c_lr0 * (1.0 - progress)
+            upd.entropy_coef = ent0 * (1.0 - progress) if self.anneal_entropy else ent0
+            upd.update(self.num_epochs, seed=seed * 7919 + metrics.rollouts)
+            ctx.synchronize()           # the pinned reward / done arrays are rewritten by the next rollout
+            metrics.rollouts += 1
+            metrics.total_steps = total_steps
+            if verbose and metrics.rollouts % print_every == 0:
+                print("rollout %d  steps %d  episodes %d  mean return (last 100) %.2f" % (
+                    metrics.rollouts, total_steps, completed, metrics.mean_reward()), flush=True)
+        metrics.total_steps = total_steps
+        if self.continuous:
+            self.train_step_count += total_steps
+        return metrics
+
     def evaluate_gpu(self, ctx, env, num_episodes=100, max_steps=1000, verbose=False, stochastic=True,
                      steps_per_readback=32):
         """DeepPPOContinuousAgent.evaluate_gpu (deep_agents/ppo/ppo_continuous.mojo:703-975): run the

@@ -179,6 +179,17 @@ class RolloutBuffers:
         return r
 
 
+def policy_step(ctx, rb, t, sample_seed, actions):
+    """Policy half of collection step t on rb.obs (actor + critic forward, sampling, pre-step store into
+    rollout row t); `actions` [N * act_width] receives what the envs are to be stepped with.  Enqueue only."""
+    N, od, aw = rb.n_envs, rb.env.OBS_DIM, rb.act_width
+    name = "mrl_policy_step_gaussian" if rb.continuous else "mrl_policy_step_discrete"
+    _lib.call(name, ctx.handle, C.byref(rb.actor.desc), C.byref(rb.critic.desc), N, _ptr(rb.obs),
+              _ptr(rb.actor_params), _ptr(rb.critic_params), int(sample_seed) & 0xFFFFFFFF, _ptr(actions),
+              _ptr(rb.r_obs[t * N * od:]), _ptr(rb.r_actions[t * N * aw:]), _ptr(rb.r_log_probs[t * N:]),
+              _ptr(rb.r_values[t * N:]))
+
+
 def rollout_step(ctx, desc, t, sample_seed, step_seed=0, reset_seed=0):
     """One pass of train_gpu's inner loop body (ppo.mojo:2069-2285, ppo_continuous.mojo:2619-2850),
     enqueue only."""

@@ -83,3 +83,79 @@ def test_observation_noise_enters_the_rollout(mrl, orc):
     z = (last - rows[:, :3]) / std
     assert 0.7 < z.std() < 1.3 and abs(z.mean()) < 0.2
     assert np.abs(np.hypot(rows[:, 0], rows[:, 1]) - 1.0).max() < 1e-5      # the rows themselves carry no noise
+
+
+class _SignEnv:
+    """A host env with the reference's CPU interface: the observation is a random point, the reward is
+    1 when the action names the sign of its first entry, an episode lasts `length` steps."""
+
+    def __init__(self, seed, length=8, continuous=False):
+        self.rng, self.length, self.continuous = np.random.default_rng(seed), length, continuous
+        self.t, self.obs, self.log = 0, None, []          # log: (action, reward, done) of every step
+
+    def _draw(self):
+        self.obs = self.rng.uniform(-1, 1, 3).astype(np.float32)
+        return self.obs.tolist()
+
+    def reset_obs_list(self):
+        self.t = 0
+        return self._draw()
+
+    def _step(self, good, action):
+        self.t += 1
+        done = self.t >= self.length
+        self.log.append((action, 1.0 if good else 0.0, done))
+        return self._draw(), 1.0 if good else 0.0, done
+
+    def step_obs(self, action):
+        assert isinstance(action, int) and not self.continuous
+        return self._step((action == 1) == (self.obs[0] > 0), action)
+
+    def step_continuous_vec(self, action):
+        assert self.continuous and len(action) == 2 and all(-1.0 <= a <= 1.0 for a in action)
+        return self._step((action[0] > 0) == (self.obs[0] > 0), list(action))
+
+
+@pytest.mark.parametrize("continuous", [False, True])
+def test_train_gpu_cpu_env_steps_host_envs_and_learns(mrl, continuous):
+    """train_gpu_cpu_env: the envs are the caller's host objects; the rollout buffers hold what they
+    reported, the metrics list their episodes in completion order, and the policy learns the task."""
+    ctx = mrl.DeviceContext("cuda:0")
+    N, T, L = 16, 32, 8
+    if continuous:
+        agent = mrl.DeepPPOContinuousAgent(3, 2, hidden_dim=64, rollout_len=T, n_envs=N, gpu_minibatch_size=128,
+                                           num_epochs=4, actor_lr=3e-3, critic_lr=3e-3, entropy_coef=0.0,
+                                           anneal_lr=False, target_kl=0.0, normalize_rewards=False)
+    else:
+        agent = mrl.DeepPPOAgent(3, 2, hidden_dim=64, rollout_len=T, n_envs=N, gpu_minibatch_size=128,
+                                 num_epochs=4, actor_lr=3e-3, critic_lr=3e-3, entropy_coef=0.0,
+                                 anneal_lr=False, target_kl=0.0)
+    envs = [_SignEnv(100 + i, L, continuous) for i in range(N)]
+    with pytest.raises(ValueError):
+        agent.train_gpu_cpu_env(ctx, envs[:-1], 10)
+    m = agent.train_gpu_cpu_env(ctx, envs, num_episodes=10 ** 9, max_rollouts=1)
+    # one rollout: T steps of every env, in the buffers exactly as the envs saw them
+    assert m.rollouts == 1 and m.total_steps == N * T and all(len(e.log) == T for e in envs)
+    rb = agent.rb
+    want_r = np.array([[e.log[t][1] for e in envs] for t in range(T)], np.float32)
+    want_d = np.array([[float(e.log[t][2]) for e in envs] for t in range(T)], np.float32)
+    np.testing.assert_array_equal(rb.r_rewards.cpu().numpy().reshape(T, N), want_r)
+    np.testing.assert_array_equal(rb.r_dones.cpu().numpy().reshape(T, N), want_d)
+    acts = rb.r_actions.cpu().numpy().reshape(T, N, -1)
+    for t in range(T):
+        for i, e in enumerate(envs):
+            if continuous:   # the envs get the clipped action, the buffer keeps the raw one
+                np.testing.assert_allclose(np.clip(acts[t, i], -1, 1), e.log[t][0], rtol=0, atol=0)
+            else:
+                assert int(acts[t, i, 0]) == e.log[t][0]
+    assert len(m.episode_rewards) == N * T // L and m.episode_steps == [L] * (N * T // L)
+    first = float(np.mean(m.episode_rewards))
+    # keep training: the returns go up from about L / 2 towards L
+    m2 = agent.train_gpu_cpu_env(ctx, envs, num_episodes=10 ** 9, max_rollouts=25)
+    last = float(np.mean(m2.episode_rewards[-64:]))
+    print("sign env, continuous=%s: mean return %.2f -> %.2f of %d" % (continuous, first, last, L), flush=True)
+    assert first < 0.7 * L and last > 0.85 * L
+    # the episode target inside a rollout ends the call without an update for that rollout
+    t_before = agent.actor.optimizer.t
+    m3 = agent.train_gpu_cpu_env(ctx, envs, num_episodes=5)
+    assert m3.rollouts == 0 and len(m3.episode_rewards) >= 5 and agent.actor.optimizer.t == t_before
