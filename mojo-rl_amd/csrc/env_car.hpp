@@ -3,13 +3,16 @@
 // (physics2d/car/layout.mojo:42-110).
 //
 // A row is 12 KB, almost all of it the track, and a step looks five points up in the tile list (the
-// four wheels before the physics, the hull after it): the tile scan is the step's memory traffic.
-// Sixteen lanes share an env: each scans every sixteenth tile for all points of a lookup at once
-// (neighbouring lanes read neighbouring tiles), and the first tile in list order that holds a point
-// is the minimum over the group -- what the reference's scan-until-hit returns.  The four wheels'
-// forces are computed on four lanes and summed in wheel order; the rest of the (small) state update
-// is done by every lane of the group alike, and lane 0 writes the row.  Rows stay in global memory:
-// apart from the tiles a step touches forty floats.
+// four wheels before the physics, the hull after it): the tile table is the step's memory traffic.
+// A wavefront takes an env: it copies the table (tiles and visited flags, 12 KB, one contiguous range)
+// into LDS with 16-byte loads -- every cache line is fetched once; tile by tile, the 36-byte records
+// would make each line cross the vector cache nine times -- in one batch of independent loads at the
+// start of the step, and lane l keeps the vertices of tiles l, l + 64, .. l + 256 in registers for both
+// lookups, so a step waits for memory once.  The first tile in list order that holds a point is the
+// minimum over the wavefront of each lane's first hit -- what the reference's scan-until-hit returns;
+// friction and visited flag of that tile are read from the LDS copy.  The four
+// wheels' forces are computed on four lanes and summed in wheel order; the rest of the (small)
+// state update is done by every lane alike, and lane 0 writes the row.
 //
 // Arithmetic: the reference's CPU step (CarDynamics.step_with_obs in fp32, action decoding, reward and
 // termination in Float64, car_racing_v2.mojo:258-287, :781-846) with the GPU trait's row protocol
@@ -23,7 +26,8 @@ namespace cr {
 
 constexpr int STATE = 3040, OBS = 13, ACT = 3;
 constexpr int HULL = 13, WHEELS = 19, CTRL = 31, META = 34, TRACK = 40, VISITED = 2740;
-constexpr int MAX_TILES = 300, TILE = 9, GROUP = 16;
+constexpr int MAX_TILES = 300, TILE = 9;
+constexpr int STEP_LANES = 64, SLOTS = 5;   // a wavefront per env; SLOTS * 64 >= MAX_TILES tiles in its registers
 enum { H_X, H_Y, H_ANGLE, H_VX, H_VY, H_OMEGA };
 enum { W_OMEGA, W_JOINT, W_PHASE, W_SIZE };
 enum { M_STEP, M_TOTAL, M_DONE, M_TRUNC, M_VISITED, M_NUM_TILES };
@@ -41,32 +45,69 @@ MRL_DEV bool point_in_quad(float px, float py, float v0x, float v0y, float v1x, 
     return all_positive || all_negative;
 }
 
-// index of the first tile (list order) that holds point p, -1 if none, for NP points at once; called
-// by the 16 lanes of a group together (sub = lane in the group)
-template <int NP>
-MRL_DEV void tiles_at(const float *row, const float (&px)[NP], const float (&py)[NP], int num_tiles, int sub,
-                      int (&idx)[NP]) {
-    constexpr int NONE = 1 << 30;
+// The tile table of one env: a copy in LDS (`lds`, TABLE floats: tiles, then visited flags, as in the
+// row) made by the wavefront, and the vertices of tiles sub + 64 * i in the registers of lane `sub`.
+constexpr int TABLE = STATE - TRACK;   // 3000 floats, a multiple of 4; row + TRACK is 16-byte aligned
+struct Tiles {
+    float v[SLOTS][8];     // four vertices
+    const float *lds;
+
+    MRL_DEV void load(const float *row, float *table, int sub) {
+        constexpr int N4 = TABLE / 4, ROUNDS = (N4 + STEP_LANES - 1) / STEP_LANES;
+        const float4 *src = reinterpret_cast<const float4 *>(row + TRACK);
+        float4 *dst = reinterpret_cast<float4 *>(table);
+        static_assert(N4 > STEP_LANES * (ROUNDS - 1) && N4 <= STEP_LANES * ROUNDS, "only the last round is partial");
+        float4 tmp[ROUNDS];
 #pragma unroll
-    for (int p = 0; p < NP; ++p) idx[p] = NONE;
-    for (int t = sub; t < num_tiles; t += GROUP) {
-        const float *T = row + TRACK + t * TILE;
-        const float v0x = T[0], v0y = T[1], v1x = T[2], v1y = T[3], v2x = T[4], v2y = T[5], v3x = T[6], v3y = T[7];
+        for (int i = 0; i < ROUNDS - 1; ++i) tmp[i] = src[sub + STEP_LANES * i];
+        const int last = sub + STEP_LANES * (ROUNDS - 1);
+        tmp[ROUNDS - 1] = src[last < N4 ? last : N4 - 1];
 #pragma unroll
-        for (int p = 0; p < NP; ++p)
-            if (idx[p] == NONE && point_in_quad(px[p], py[p], v0x, v0y, v1x, v1y, v2x, v2y, v3x, v3y)) idx[p] = t;
-    }
+        for (int i = 0; i < ROUNDS - 1; ++i) dst[sub + STEP_LANES * i] = tmp[i];
+        if (last < N4) dst[last] = tmp[ROUNDS - 1];
+        // the wavefront's own LDS writes, read back by other lanes of the same wavefront
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        lds = table;
+        // slots past the table (tiles 300 .. 319) read the visited flags behind it; never used
 #pragma unroll
-    for (int p = 0; p < NP; ++p) {
-        int v = idx[p];
+        for (int i = 0; i < SLOTS; ++i) {
+            const float *T = table + (sub + STEP_LANES * i) * TILE;
 #pragma unroll
-        for (int off = GROUP / 2; off > 0; off >>= 1) {
-            const int o = __shfl_xor(v, off, 64);
-            v = o < v ? o : v;
+            for (int k = 0; k < 8; ++k) v[i][k] = T[k];
         }
-        idx[p] = v == NONE ? -1 : v;
     }
-}
+    MRL_DEV float friction(int t) const { return lds[t * TILE + 8]; }
+    MRL_DEV float visited(int t) const { return lds[MAX_TILES * TILE + t]; }
+
+    // index of the first tile (list order) that holds point p, -1 if none, for NP points at once
+    template <int NP>
+    MRL_DEV void at(const float (&px)[NP], const float (&py)[NP], int num_tiles, int sub, int (&idx)[NP]) const {
+        constexpr int NONE = 1 << 30;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) idx[p] = NONE;
+#pragma unroll
+        for (int i = 0; i < SLOTS; ++i) {
+            const int t = sub + STEP_LANES * i;
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+                if (t < num_tiles && idx[p] == NONE &&
+                    point_in_quad(px[p], py[p], v[i][0], v[i][1], v[i][2], v[i][3], v[i][4], v[i][5], v[i][6], v[i][7]))
+                    idx[p] = t;
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            int m = idx[p];
+#pragma unroll
+            for (int off = STEP_LANES / 2; off > 0; off >>= 1) {
+                const int o = __shfl_xor(m, off, 64);
+                m = o < m ? o : m;
+            }
+            idx[p] = m == NONE ? -1 : m;
+        }
+    }
+};
 
 // CarDynamics._update_steering_angle, physics2d/car/car_dynamics.mojo:118-150
 MRL_DEV float update_steering_angle(float current, float target, float dt) {
@@ -142,12 +183,19 @@ MRL_DEV void wheel_forces(float wheel_omega, float joint_angle, float hull_angle
     omega_o = omega;
 }
 
-// One env step by the 16 lanes of a group (lane = lane in the wavefront).  Every lane returns the
-// same reward / done; lane 0 of the group has written the row.
-MRL_DEV void step_group(float *row, const float *action, int lane, float &reward, float &done) {
-    const int sub = lane & (GROUP - 1), base = lane & ~(GROUP - 1);
+// One env step by the 64 lanes of a wavefront (sub = lane; table = TABLE floats of LDS of its own).  Every
+// lane returns the same reward / done and the observation the row now starts with; lane 0 has written the row.
+MRL_DEV void step_wave(float *row, float *table, const float *action, int sub, float &reward, float &done,
+                       float (&ob)[OBS]) {
     float *M = row + META;
-    if (M[M_DONE] > 0.5f) { reward = 0.0f; done = 1.0f; return; }   // car_racing_v2.mojo:1564-1572
+    if (M[M_DONE] > 0.5f) {   // car_racing_v2.mojo:1564-1572
+#pragma unroll
+        for (int k = 0; k < OBS; ++k) ob[k] = row[k];
+        reward = 0.0f; done = 1.0f;
+        return;
+    }
+    Tiles tiles;
+    tiles.load(row, table, sub);
     int num_tiles = (int)M[M_NUM_TILES];
     if (num_tiles <= 0) num_tiles = 100;
     // ---- controls, car_racing_v2.mojo:262-268 (Float64)
@@ -182,7 +230,7 @@ MRL_DEV void step_group(float *row, const float *action, int lane, float &reward
         wpy[w] = y + lxs[w] * sin_a + lys[w] * cos_a;
     }
     int under[4];
-    tiles_at<4>(row, wpx, wpy, num_tiles, sub, under);
+    tiles.at<4>(wpx, wpy, num_tiles, sub, under);
     // ---- my wheel (sub & 3): compute_wheel_forces
     const int mw = sub & 3;
     float my_limit, my_omega, my_lx, my_ly;
@@ -190,7 +238,7 @@ MRL_DEV void step_group(float *row, const float *action, int lane, float &reward
         float lim[4];
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            const float surface = under[w] >= 0 ? row[TRACK + under[w] * TILE + 8] : (float)0.6;
+            const float surface = under[w] >= 0 ? tiles.friction(under[w] >= 0 ? under[w] : 0) : (float)0.6;
             lim[w] = (float)(1000000.0 * SIZE_ * SIZE_) * surface;
         }
         my_limit = mw == 0 ? lim[0] : mw == 1 ? lim[1] : mw == 2 ? lim[2] : lim[3];
@@ -206,10 +254,10 @@ MRL_DEV void step_group(float *row, const float *action, int lane, float &reward
     float total_fx = 0.0f, total_fy = 0.0f, total_torque = 0.0f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-        total_fx = total_fx + __shfl(fx, base + w, 64);
-        total_fy = total_fy + __shfl(fy, base + w, 64);
-        total_torque = total_torque + __shfl(tq, base + w, 64);
-        const float nom = __shfl(om, base + w, 64);
+        total_fx = total_fx + __shfl(fx, w, 64);
+        total_fy = total_fy + __shfl(fy, w, 64);
+        total_torque = total_torque + __shfl(tq, w, 64);
+        const float nom = __shfl(om, w, 64);
         w_omega[w] = nom;
         w_phase[w] = w_phase[w] + nom * dt;
     }
@@ -244,10 +292,10 @@ MRL_DEV void step_group(float *row, const float *action, int lane, float &reward
     // ---- tile under the hull, reward (car_racing_v2.mojo:781-809), termination (:811-846)
     const float hpx[1] = {x}, hpy[1] = {y};
     int tile_idx[1];
-    tiles_at<1>(row, hpx, hpy, num_tiles, sub, tile_idx);
+    tiles.at<1>(hpx, hpy, num_tiles, sub, tile_idx);
     double step_reward = -0.1;
     float tiles_visited = M[M_VISITED];
-    const bool fresh = tile_idx[0] >= 0 && !(row[VISITED + (tile_idx[0] >= 0 ? tile_idx[0] : 0)] > 0.5f);
+    const bool fresh = tile_idx[0] >= 0 && !(tiles.visited(tile_idx[0] >= 0 ? tile_idx[0] : 0) > 0.5f);
     if (fresh) {
         tiles_visited = tiles_visited + 1.0f;
         step_reward += 100.0 / (double)num_tiles;
@@ -265,6 +313,12 @@ MRL_DEV void step_group(float *row, const float *action, int lane, float &reward
     if (truncated) is_done = true;
     reward = (float)step_reward;
     done = is_done ? 1.0f : 0.0f;
+    // observation (update_observation, car_dynamics.mojo:292-350; _update_observation, :848-898)
+    ob[0] = x; ob[1] = y; ob[2] = angle; ob[3] = vx; ob[4] = vy; ob[5] = omega;
+    ob[6] = joint_fl; ob[7] = joint_fr;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) ob[8 + w] = w_omega[w];
+    ob[12] = sqrtf(vx * vx + vy * vy);
     // ---- lane 0 writes the row (the reads above are done: every lane holds its values in registers)
     if (sub == 0) {
         row[CTRL + 0] = steering; row[CTRL + 1] = gas; row[CTRL + 2] = brake;
@@ -277,12 +331,8 @@ MRL_DEV void step_group(float *row, const float *action, int lane, float &reward
             row[WHEELS + w * W_SIZE + W_JOINT] = joints[w];
             row[WHEELS + w * W_SIZE + W_PHASE] = w_phase[w];
         }
-        // observation (update_observation, car_dynamics.mojo:292-350; _update_observation, :848-898)
-        row[0] = x; row[1] = y; row[2] = angle; row[3] = vx; row[4] = vy; row[5] = omega;
-        row[6] = joint_fl; row[7] = joint_fr;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) row[8 + w] = w_omega[w];
-        row[12] = sqrtf(vx * vx + vy * vy);
+        for (int k = 0; k < OBS; ++k) row[k] = ob[k];
         if (fresh) row[VISITED + tile_idx[0]] = 1.0f;
         M[M_VISITED] = tiles_visited;
         M[M_TOTAL] = total;
@@ -386,12 +436,14 @@ MRL_DEV int generate_track(float *row, uint64_t seed) {
     return num_tiles;
 }
 
-// _reset_env_gpu, car_racing_v2.mojo:1155-1300, by the 16 lanes of a group: lane 0 walks the track (it
-// writes the tiles it makes), then all lanes clear what is left of the row and lane 0 places the car
-MRL_DEV void reset_group(float *row, uint64_t cseed, int lane) {
+// _reset_env_gpu, car_racing_v2.mojo:1155-1300, by a group of GROUP lanes of a wavefront: its lane 0
+// walks the track (it writes the tiles it makes), then all lanes clear what is left of the row and
+// place the car; the observation of the fresh row is (start_x, start_y, start_angle, 0, .. 0)
+template <int GROUP>
+MRL_DEV void reset_group(float *row, uint64_t cseed, int lane, float &start_x, float &start_y, float &start_angle) {
     const int sub = lane & (GROUP - 1), base = lane & ~(GROUP - 1);
     int num_tiles = 0;
-    float start_x = 0.0f, start_y = 0.0f, start_angle = 0.0f;
+    start_x = 0.0f; start_y = 0.0f; start_angle = 0.0f;
     if (sub == 0) {
         num_tiles = generate_track(row, cseed);
         const float *t0 = row + TRACK;

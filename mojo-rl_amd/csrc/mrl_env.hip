@@ -191,42 +191,51 @@ __global__ __launch_bounds__(64) void hc_lanes_step_kernel(float *states, const 
     if (AUTORESET) S::out_rows(rows, gbase, nenv, was_reset, lane, E::DYN_END, E::L::META_OFF);
 }
 
-// CarRacingV2 (env_car.hpp): sixteen lanes per env, rows in global memory
-constexpr int CAR_THREADS = 256, CAR_EPB = CAR_THREADS / cr::GROUP;
+// CarRacingV2 (env_car.hpp): a wavefront per env for the step, sixteen lanes per env for a reset of
+// its own (where one lane of the group walks the track); rows in global memory
+constexpr int CAR_THREADS = 256, CAR_EPB = CAR_THREADS / cr::STEP_LANES;
+constexpr int CAR_RESET_GROUP = 16, CAR_RESET_EPB = CAR_THREADS / CAR_RESET_GROUP;
 
 template <bool AUTORESET>
 __global__ __launch_bounds__(CAR_THREADS) void car_step_kernel(float *states, const float *actions, float *rewards,
                                                                float *dones, float *obs, int batch,
                                                                uint64_t reset_seed, Accounting acc) {
-    const int lane = threadIdx.x & 63, sub = lane & (cr::GROUP - 1);
-    const int env = blockIdx.x * CAR_EPB + threadIdx.x / cr::GROUP;
-    if (env >= batch) return;   // whole groups leave together
+    __shared__ __align__(16) float tables[CAR_EPB][cr::TABLE];   // each wavefront's copy of its env's tile table
+    const int sub = threadIdx.x & 63, wave = threadIdx.x / cr::STEP_LANES;
+    const int env = blockIdx.x * CAR_EPB + wave;
+    if (env >= batch) return;   // whole wavefronts leave together
     float *row = states + (size_t)env * cr::STATE;
-    float r, d;
-    cr::step_group(row, actions + (size_t)env * cr::ACT, lane, r, d);
+    float r, d, ob[cr::OBS];
+    cr::step_wave(row, tables[wave], actions + (size_t)env * cr::ACT, sub, r, d, ob);
     if (sub == 0) {
         rewards[env] = r;
         dones[env] = d;
         account(acc, env, r, d);
     }
-    if (AUTORESET && d > 0.5f) cr::reset_group(row, cr::combined_seed(reset_seed, env), lane);
-    // the observation out of the row: lane 0 wrote it (step) or the group did (reset); a wavefront's
-    // own stores are visible to its later loads once they have been waited for
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    if (sub < cr::OBS) obs[(size_t)env * cr::OBS + sub] = row[sub];
+    if (AUTORESET && d > 0.5f) {
+        float sx, sy, sa;
+        cr::reset_group<cr::STEP_LANES>(row, cr::combined_seed(reset_seed, env), sub, sx, sy, sa);
+#pragma unroll
+        for (int k = 3; k < cr::OBS; ++k) ob[k] = 0.0f;
+        ob[0] = sx; ob[1] = sy; ob[2] = sa;
+    }
+    // the observation the row now starts with, straight from the registers (every lane holds all of it)
+    float mine = ob[0];
+#pragma unroll
+    for (int k = 1; k < cr::OBS; ++k) mine = sub == k ? ob[k] : mine;
+    if (sub < cr::OBS) obs[(size_t)env * cr::OBS + sub] = mine;
 }
 
 __global__ __launch_bounds__(CAR_THREADS) void car_reset_kernel(float *states, float *dones, int batch, uint64_t seed,
                                                                 int selective) {
-    const int lane = threadIdx.x & 63, sub = lane & (cr::GROUP - 1);
-    const int env = blockIdx.x * CAR_EPB + threadIdx.x / cr::GROUP;
+    const int lane = threadIdx.x & 63, sub = lane & (CAR_RESET_GROUP - 1);
+    const int env = blockIdx.x * CAR_RESET_EPB + threadIdx.x / CAR_RESET_GROUP;
     if (env >= batch) return;
     if (selective) {
         if (!(dones[env] > 0.5f)) return;
     }
-    cr::reset_group(states + (size_t)env * cr::STATE, cr::combined_seed(seed, env), lane);
+    float sx, sy, sa;
+    cr::reset_group<CAR_RESET_GROUP>(states + (size_t)env * cr::STATE, cr::combined_seed(seed, env), lane, sx, sy, sa);
     if (selective && sub == 0) dones[env] = 0.0f;
 }
 
@@ -363,7 +372,7 @@ static int env_reset_impl(mrl_ctx *ctx, int env_id, int batch, float *states, fl
         case MRL_ENV_BIPEDAL: launch_phys_reset<BipedalWalker>(ctx, batch, states, dones, seed, selective); break;
         case MRL_ENV_HALFCHEETAH: launch_phys_reset<HalfCheetah>(ctx, batch, states, dones, seed, selective); break;
         case MRL_ENV_CARRACING:
-            hipLaunchKernelGGL(car_reset_kernel, dim3(grid_for(batch, CAR_EPB)), dim3(CAR_THREADS), 0, ctx->stream, states,
+            hipLaunchKernelGGL(car_reset_kernel, dim3(grid_for(batch, CAR_RESET_EPB)), dim3(CAR_THREADS), 0, ctx->stream, states,
                                dones, batch, seed, selective);
             break;
         default:
