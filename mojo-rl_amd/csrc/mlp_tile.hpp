@@ -20,7 +20,7 @@ constexpr int HT_LD = PR + 1;
 template <int ACT>
 MRL_DEV float activate(float x) {
     if (ACT == 1) return x > 0.0f ? x : 0.0f;
-    if (ACT == 2) return tanhf(x);
+    if (ACT == 2) return tanh_mlp(x);
     return x;
 }
 

