@@ -175,13 +175,17 @@ def main():
 
     fused = mrl.ppo.rollout_fused(desc)
     SPL = max(1, min(args.steps_per_launch, T)) if fused else 1   # collection steps per launch
-    # untimed: the envs are taken from the reset into the steady-state episode mix, then the warm-up
+    # untimed: the envs are taken from the reset into the steady-state episode mix, then the warm-up;
+    # fused launches have the shape of the timed ones (SPL steps) as far as the counts allow, so that a
+    # kernel trace of the run averages over launches of one kind
     done = 0
-    while done < args.preroll:
-        n = min(T, args.preroll - done)
-        mrl.ppo.rollout_steps(ctx, desc, 0, n, 7 + done, 1, 0, 0, 9000 + done, 1)
-        done += n
-    mrl.ppo.rollout_steps(ctx, desc, 0, min(args.warmup, T), 7, 1, 0, 0, 9000, 1)
+    for phase, count in (("preroll", args.preroll), ("warmup", min(args.warmup, T))):
+        left = count
+        while left > 0:
+            n = min(SPL if fused else T, left)
+            mrl.ppo.rollout_steps(ctx, desc, 0, n, 7 + done, 1, 0, 0, 9000 + done, 1)
+            done += n
+            left -= n
     ctx.synchronize()
     rb.done_count.zero_()
     ctx.synchronize()

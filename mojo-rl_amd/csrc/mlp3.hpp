@@ -27,9 +27,8 @@ struct FwdLoss {
     const float *r_obs, *r_act, *r_adv, *r_ret, *r_logp, *r_val;
     const float *adv_stats;                               // {mean, std} of the minibatch's advantages; null: as they are
     float *g_actor_out, *g_values, *kl;                   // [mb, head], [mb], [mb]
-    float *kl_part;                                       // [row tiles]
-    int *arrived;                                         // zero between launches
-    int32_t *kl_flag;                                     // null: no test
+    float *kl_part;                                       // [row tiles] sums of the tiles' KL estimates, for the test
+    int32_t *kl_flag;                                     // null: no test (nothing is left in kl_part)
     int mb, A, continuous, clip_value;                    // A = actions (discrete) or action width (continuous)
     float clip_eps, ent_coef, value_coef, target_kl;
 };

@@ -125,30 +125,11 @@ __global__ __launch_bounds__(2 * H) void mlp3_fwd_kernel(int B, int IN, Mlp3Nets
         fl.kl[b] = kl;
     }
     if (fl.kl_flag == nullptr) return;
-    // KL test: every actor tile leaves the sum of its rows' estimates; the last one to arrive adds
-    // the tiles up in order, compares the mean with target_kl and re-arms the counter
+    // KL test: every actor tile leaves the sum of its rows' estimates; the kernel that applies the
+    // update adds the tiles up and compares the mean with target_kl
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) kl += __shfl_xor(kl, off, 64);
-    int last = 0;
-    if (t == 0) {
-        __hip_atomic_store(&fl.kl_part[blockIdx.x], kl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __threadfence();
-        last = atomicAdd(fl.arrived, 1) == (int)gridDim.x - 1;
-    }
-    last = __shfl(last, 0, 64);
-    if (!last) return;
-    __threadfence();
-    float sum = 0.0f;
-    for (int i = t; i < (int)gridDim.x; i += 64)
-        sum += __hip_atomic_load(&fl.kl_part[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    if (t == 0) {
-        const float mean = sum / (float)fl.mb;
-        fl.kl_flag[1] = __float_as_int(mean);
-        if (mean > fl.target_kl) fl.kl_flag[0] = 1;
-        *fl.arrived = 0;
-    }
+    if (t == 0) fl.kl_part[blockIdx.x] = kl;
 }
 
 template <int ACT>
@@ -481,31 +462,12 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
         }
     }
     if (fl.kl_flag != nullptr && blockIdx.y == 0 && t < 64) {
-        // KL test: every actor tile leaves the sum of its rows' estimates; the last one to arrive
-        // adds the tiles up in order, compares the mean with target_kl and re-arms the counter
+        // KL test: every actor tile leaves the sum of its rows' estimates; the kernel that applies the
+        // update (clip + Adam) adds the tiles up and compares the mean with target_kl, so that nothing
+        // here waits for other workgroups
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) kl += __shfl_xor(kl, off, 64);
-        int last = 0;
-        if (t == 0) {
-            __hip_atomic_store(&fl.kl_part[blockIdx.x], kl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __threadfence();
-            last = atomicAdd(fl.arrived, 1) == (int)gridDim.x - 1;
-        }
-        last = __shfl(last, 0, 64);
-        if (last) {
-            __threadfence();
-            float sum = 0.0f;
-            for (int i = t; i < (int)gridDim.x; i += 64)
-                sum += __hip_atomic_load(&fl.kl_part[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-            if (t == 0) {
-                const float mean = sum / (float)fl.mb;
-                fl.kl_flag[1] = __float_as_int(mean);
-                if (mean > fl.target_kl) fl.kl_flag[0] = 1;
-                *fl.arrived = 0;
-            }
-        }
+        if (t == 0) fl.kl_part[blockIdx.x] = kl;
     }
     __syncthreads();   // g2s complete
 

@@ -13,8 +13,9 @@
 //
 // KL early stop: the reference copies the per-sample KL to the host after the actor's loss
 // gradient and breaks out of the minibatch and epoch loops when its mean exceeds target_kl.
-// Here the mean is tested on the device (kl_flag[0] is raised and stays raised) and the kernel
-// that applies the update does nothing once the flag is up: the parameters end exactly where
+// Here the mean is tested on the device, by the kernel that applies the update (from the per-tile
+// sums that the loss gradients leave; kl_flag[0] is raised and stays raised), and that kernel
+// does nothing once the flag is up: the parameters end exactly where
 // the reference's break leaves them, without a host round trip.  kl_flag[2] counts the updates
 // that were applied, for the host's optimiser step counters.
 #include "mrl_host.hpp"
@@ -240,14 +241,39 @@ __global__ __launch_bounds__(UTPB) void sq_partial2_kernel(AdamNets nets, float 
 
 // global-norm clip (ppo.mojo:382-534; actor and critic separately) + Adam (adam.mojo:52-105)
 // + log_std clamp (kernels.mojo:842-873); grid = (blocks, nets).  Does nothing once stop[0] != 0.
+// kl_part != nullptr: the KL early-stop test of this minibatch has not been made yet: kl_part[0 .. kl_n)
+// hold the row tiles' sums of the per-sample estimates.  Every workgroup adds them up in the same order,
+// so all of them come to the same verdict; workgroup (0, 0) records it (stop[0] raised and sticky,
+// stop[1] = the mean's bits).
 __global__ __launch_bounds__(UTPB) void clip_adam2_kernel(AdamNets nets, const float *__restrict__ partial,
                                                           int nb, int part_stride, float max_norm, float beta1,
                                                           float beta2,
                                                           float omb1, float omb2, float eps,
-                                                          int32_t *__restrict__ stop) {
+                                                          int32_t *__restrict__ stop,
+                                                          const float *__restrict__ kl_part, int kl_n, int kl_mb,
+                                                          float target_kl) {
     __shared__ float smem[4];
     __shared__ float scale_s;
+    __shared__ int stop_s;
     if (stop != nullptr && stop[0] != 0) return;
+    if (stop != nullptr && kl_part != nullptr) {
+        if (threadIdx.x < 64) {
+            float sum = 0.0f;
+            for (int i = threadIdx.x; i < kl_n; i += 64) sum += kl_part[i];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+            if (threadIdx.x == 0) {
+                const float mean = sum / (float)kl_mb;
+                stop_s = mean > target_kl;
+                if (blockIdx.x == 0 && blockIdx.y == 0) {
+                    stop[1] = __float_as_int(mean);
+                    if (mean > target_kl) stop[0] = 1;
+                }
+            }
+        }
+        __syncthreads();
+        if (stop_s) return;
+    }
     const AdamNet &a = nets.n[blockIdx.y];
     float scale = 1.0f;
     if (max_norm > 0.0f) {
@@ -357,7 +383,6 @@ static int update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *in
         fl.adv_stats = u->norm_adv_per_minibatch ? stats : nullptr;
         fl.g_actor_out = u->g_actor_out; fl.g_values = u->g_values; fl.kl = u->kl;
         fl.kl_part = ctx->upd_scratch + SCR_KL;
-        fl.arrived = reinterpret_cast<int *>(ctx->upd_scratch + SCR_ARRIVED);
         fl.kl_flag = u->target_kl > 0.0f ? u->kl_flag : nullptr;
         fl.mb = mb; fl.A = cont ? u->act_width : head; fl.continuous = cont ? 1 : 0;
         fl.clip_value = u->clip_value ? 1 : 0;
@@ -429,7 +454,9 @@ static int update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *in
     }
     hipLaunchKernelGGL(clip_adam2_kernel, dim3(grid_for(nmax, UTPB), 2), dim3(UTPB), 0, ctx->stream, an, part, nb,
                        stride, u->max_grad_norm, (float)u->beta1, (float)u->beta2, (float)(1.0 - u->beta1),
-                       (float)(1.0 - u->beta2), (float)u->eps, u->target_kl > 0.0f ? u->kl_flag : nullptr);
+                       (float)(1.0 - u->beta2), (float)u->eps, u->target_kl > 0.0f ? u->kl_flag : nullptr,
+                       paired && u->target_kl > 0.0f ? ctx->upd_scratch + SCR_KL : nullptr, grid_for(mb, 32), mb,
+                       u->target_kl);
     MRL_CHECK_LAUNCH();
     return MRL_OK;
 }
