@@ -26,7 +26,7 @@ HBM_PEAK_GBS, MFMA_FP32_PEAK_TFLOPS = 8000.0, 157.3
 # name -> env class, envs, hidden width, hidden activation, algorithmic bytes per env-step (live
 # fields of the reference row layout, each read once and written once), description
 WORKLOADS = {
-    "cartpole": ("CartPoleEnv", 4096, 64, "relu", 60, "CartPole-v1 discrete, 4096 envs, nets 4-64-64-2 / 4-64-64-1"),
+    "cartpole": ("CartPoleEnv", 4096, 64, "tanh", 60, "CartPole-v1 discrete, 4096 envs, nets 4-64-64-2 / 4-64-64-1 (tanh)"),
     "pendulum": ("PendulumV2", 16384, 64, "tanh", 72, "Pendulum continuous, 16384 envs, Gaussian 3-64-64-1 + value"),
     "lunarlander": ("LunarLanderV2", 8192, 256, "relu", 672,
                     "LunarLander-v2 discrete, 8192 envs, policy 8-256-256-4 + value 8-256-256-1 "
