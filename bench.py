@@ -231,7 +231,9 @@ def main():
         act_id = 1 if ACT == "relu" else 2
         name = {"lunarlander": "mrl::collect_kernel<mrl::LunarLander, %d, %d, false>" % (HIDDEN, act_id),
                 "cartpole": "mrl::collect_classic_kernel<mrl::CartPoleSlot, %d, false>" % act_id,
-                "pendulum": "mrl::collect_classic_kernel<mrl::PendulumSlot, %d, true>" % act_id}[args.workload]
+                "pendulum": "mrl::collect_classic_kernel<mrl::PendulumSlot, %d, true>" % act_id,
+                "bipedal": "mrl::collect_walker_kernel<mrl::BipedalWalker, %d, false>" % act_id,
+                "halfcheetah": "mrl::collect_walker_kernel<mrl::HalfCheetah16, %d, true>" % act_id}[args.workload]
         roofline = {"kernel": name + " (policy forward + sampling + env step + auto-reset + rollout stores, %d steps per launch)" % steps_per_launch,
                     "bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": tflops / MFMA_FP32_PEAK_TFLOPS,

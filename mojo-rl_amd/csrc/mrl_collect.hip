@@ -28,20 +28,10 @@
 #include "policy_sample.hpp"
 #include "env_block.hpp"
 #include "env_classic.hpp"
+#include "collect_args.hpp"
 
 namespace mrl {
 
-struct CollectArgs {
-    float *states, *obs;                  // [N][STATE], [N][OBS]
-    const float *actor_p, *critic_p, *shapes;
-    int n_envs, A, t0, n_steps;
-    uint32_t sample_seed, sample_stride;
-    uint64_t reset_seed, reset_stride;
-    float *r_obs, *r_actions, *r_logp, *r_values, *r_rewards, *r_dones;   // time-major, row 0
-    Accounting acc;                       // r_rewards / r_dones unused here (set per step)
-    unsigned spin_limit;                  // polls before a wait at a wavefront-group barrier gives up
-    int *sync_error;                      // raised (host-visible) by a workgroup whose wait gave up
-};
 
 template <int A, int B>
 constexpr int cmax() { return A > B ? A : B; }
@@ -584,7 +574,7 @@ extern "C" {
 
 int mrl_rollout_fused(const mrl_rollout *r) {
     int act = 0;
-    return r != nullptr && collect_fusable(r, r->num_actions == 0, &act) ? 1 : 0;
+    return r != nullptr && (collect_fusable(r, r->num_actions == 0, &act) || collect_walker_fusable(r, &act)) ? 1 : 0;
 }
 
 int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, uint32_t sample_seed,
@@ -595,7 +585,8 @@ int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, u
     if (n_steps == 0) return MRL_OK;
     const bool gauss = r->num_actions == 0;
     int act = 0;
-    if (!collect_fusable(r, gauss, &act)) {
+    const bool walker = collect_walker_fusable(r, &act);
+    if (!walker && !collect_fusable(r, gauss, &act)) {
         for (int k = 0; k < n_steps; ++k) {
             int rc = mrl_rollout_step(ctx, r, t0 + k, sample_seed + (uint32_t)k * sample_stride,
                                       step_seed + (uint64_t)k * step_stride, reset_seed + (uint64_t)k * reset_stride);
@@ -639,7 +630,10 @@ int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, u
     }
     profile_step_begin(ctx);
     profile_mark(ctx, -1);
-    if (r->env_id == MRL_ENV_LUNARLANDER && rows16) {
+    if (walker) {
+        rc = launch_collect_walker(ctx, r, a, act);
+        if (rc) return rc;
+    } else if (r->env_id == MRL_ENV_LUNARLANDER && rows16) {
         const dim3 block(Rows16<LunarLander>::THREADS);
         if (act == 1) hipLaunchKernelGGL((collect16_kernel<LunarLander, 1, false>), grid, block, 0, ctx->stream, a);
         else hipLaunchKernelGGL((collect16_kernel<LunarLander, 2, false>), grid, block, 0, ctx->stream, a);

@@ -1,0 +1,198 @@
+// Fused collection kernel of the two walkers (BipedalWalker, HalfCheetah planar) with the agents'
+// 256-wide Gaussian nets: many rollout steps of a block's 16 envs in ONE launch, like the kernels of
+// mrl_collect.hip.  The env rows stay in LDS from the first step to the last; per step and block
+//   policy   wavefronts 0 .. 3 the actor  OBS -> 256 -> 256 -> A, wavefronts 4 .. 7 the critic
+//            OBS -> 256 -> 256 -> 1, side by side on the fp32 matrix cores (the 16-row tiles of
+//            mlp_tile16.hpp, 64 columns per wavefront, weights streamed from L2), heads out of LDS;
+//   sample   one lane per (env, action component): every component has a Philox stream of its own;
+//   env step BipedalWalker: the workgroup-level step of env_block.hpp (contact detection on every
+//            wavefront, solver on wavefront 0, lidar rays on every wavefront, wave-cooperative
+//            resets); HalfCheetah: one lane per body on wavefronts 0 and 1 (env_cheetah_lanes.hpp);
+//   rollout row t of obs, action, log-prob, value, reward, done written on the way.
+// With these envs the step is 70 - 80 % env step, which is one wavefront's instruction stream, so the
+// critic is not moved beside it: what the fusion buys is the launch gaps, the observation / action
+// round trip through HBM, the staging of the rows in and out of LDS every step, and a policy forward
+// with both nets of a 16-row tile on one CU.
+//
+// It gives what n_steps calls of mrl_rollout_step give (same per-env streams: seeds are affine in
+// the step number), except that the finished-episode list is appended in the order in which blocks
+// get there rather than step by step.
+#include "mrl_host.hpp"
+#include "mrl_device.hpp"
+#include "mlp_tile.hpp"
+#include "mlp_tile16.hpp"
+#include "policy_sample.hpp"
+#include "env_block.hpp"
+#include "env_cheetah_lanes.hpp"
+#include "collect_args.hpp"
+
+namespace mrl {
+
+// HalfCheetah's traits with the block shape of this kernel
+struct HalfCheetah16 : HalfCheetah {
+    static constexpr int EPB = 16, THREADS = 512;
+};
+
+template <int A, int B>
+constexpr int wmax() { return A > B ? A : B; }
+
+template <class E, int ACT, bool LANES>
+__global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
+    using S = Stage<E>;
+    constexpr int H = 256, IN = E::OBS, AW = E::ACT_W, R = PR16, T = 512, KBA = 8;
+    static_assert(E::EPB == R && E::THREADS == T && IN <= PIN_MAX && AW <= PA_MAX, "16 envs per workgroup of eight wavefronts");
+    __shared__ float rows[R * S::STRIDE];
+    __shared__ float xs[R * XS_LD];
+    __shared__ __align__(16) float w2a[HEAD_LDS(H)];
+    __shared__ float w2c[H + 1];                    // the critic's head: column of H weights, then the bias
+    __shared__ float logits[R * (PA_MAX + 1)];
+    __shared__ float vals[R];
+    __shared__ float act[R * PA_MAX];               // [env][AW]
+    __shared__ float part[R * PA_MAX];              // log-probability per (env, component)
+    __shared__ float shapes[E::NSHAPE];
+    __shared__ unsigned long long was_reset;
+    // the two activation tiles and the env step's scratch (contact lists) are never live together
+    constexpr int LIST_F = detect_list_floats<E>() + 1;
+    constexpr int ENV_F = R * S::CSTRIDE + LIST_F + E::DETECT_TASKS * R + 1;
+    __shared__ float overlay[wmax<2 * H * HT16_LD, ENV_F>()];
+    float *cts = overlay, *dlist = cts + R * S::CSTRIDE;
+    int *dcount = reinterpret_cast<int *>(dlist + LIST_F);
+
+    const int t = threadIdx.x;
+    const int env0 = blockIdx.x * R;
+    const int nenv = min(R, a.n_envs - env0);
+    const int N = a.n_envs;
+    float *gbase = a.states + (size_t)env0 * E::STATE;
+
+    S::in(rows, gbase, nenv, t);
+    for (int i = t; i < E::NSHAPE; i += T) shapes[i] = a.shapes[i];
+    stage_head(a.actor_p + IN * H + H + H * H + H, H, a.A, true, w2a, t, T);
+    for (int i = t; i < H + 1; i += T) w2c[i] = a.critic_p[IN * H + H + H * H + H + i];
+    if (t == 0) was_reset = 0;
+    __syncthreads();
+
+    for (int k = 0; k < a.n_steps; ++k) {
+        // nothing but the rows is carried from one step to the next (see collect16_kernel)
+        int tid = t, ne = __builtin_amdgcn_readfirstlane(nenv), A = __builtin_amdgcn_readfirstlane(a.A), zero = 0;
+        asm volatile("" : "+v"(tid), "+s"(zero), "+s"(ne), "+s"(A) : : "memory");
+        const size_t row = (size_t)(a.t0 + k) * N + env0;   // this block's slice of rollout row t
+        const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
+        const uint64_t rseed = a.reset_seed + (uint64_t)k * a.reset_stride;
+        const int wave = tid / WAVE, lane = tid % WAVE;
+        const int net = wave >> 2;                           // 0: actor, 1: critic
+        // ---- policy: both nets side by side
+        {
+            const float *p = (net ? a.critic_p : a.actor_p) + zero;
+            float *tile = overlay + net * (H * HT16_LD);
+            Hidden16Operands<H, IN, 4, KBA> ops;
+            ops.load(p, 64 * (wave & 3), lane);
+            for (int i = tid; i < R * IN; i += T) {
+                const int r = i / IN, c = i - r * IN;
+                float v = 0.0f;
+                if (r < ne) {
+                    v = rows[r * S::STRIDE + c];
+                    a.r_obs[row * IN + i] = v;
+                }
+                xs[r * XS_LD + c] = v;
+            }
+            __syncthreads();
+            BlockSync bs;
+            hidden_stack16<H, IN, ACT, 4, KBA, true>(p, xs, tile, tile, ops, 64 * (wave & 3), lane, bs);
+            if (net == 0) head16<H>(w2a, A, tile, logits, PA_MAX + 1, tid, T / 2);
+            else head_rows16<H, 1, 1>(w2c, 1, tile, vals, 1, tid - T / 2, T / 2);
+            __syncthreads();   // means and values complete; the tiles are dead from here on
+        }
+        // ---- Gaussian sampling, one lane per (env, component); the log-probability is the sum of the
+        // components' terms in component order
+        for (int e = tid; e < ne * A; e += T) {
+            const int r = e / A, j = e - r * A;
+            float av;
+            part[r * PA_MAX + j] = sample_gaussian_part(logits + r * (PA_MAX + 1) + j, w2a + HEAD_LOG_STD(H) + j, 1, A, j,
+                                                        sseed, env0 + r, &av);
+            act[r * AW + j] = av;
+            a.r_actions[row * AW + e] = av;
+        }
+        if (tid < ne) a.r_values[row + tid] = vals[tid];
+        __syncthreads();
+        if (tid < ne) {
+            float logp = 0.0f;
+            for (int j = 0; j < A; ++j) logp = logp + part[tid * PA_MAX + j];
+            a.r_logp[row + tid] = logp;
+        }
+        // ---- env step with auto-reset, reward / done into rollout row t, episode accounting
+        Accounting acc = a.acc;
+        acc.r_rewards = a.r_rewards + (size_t)(a.t0 + k) * N;
+        acc.r_dones = a.r_dones + (size_t)(a.t0 + k) * N;
+        acc = acc.at(env0);
+        if constexpr (!LANES) {
+            phys_step_block<E, true>(rows, cts, shapes, dlist, dcount, &was_reset, act, nullptr, nullptr, env0, ne,
+                                     rseed, acc, tid);
+        } else {
+            // HalfCheetah: eight lanes per env, eight envs per wavefront, on wavefronts 0 and 1; a row
+            // whose wiring is not HalfCheetah's own is stepped by lane 0 of its group in the one-lane form
+            if (wave < 2) {
+                const int slot = wave * 8 + (lane >> 3), b = lane & 7;
+                const bool live = slot < ne;
+                float *rowp = rows + slot * S::STRIDE;
+                const int env = env0 + (live ? slot : 0);
+                const float *ap = act + (live ? slot : 0) * AW;
+                const bool ok = live && hc::lanes_row_ok(rowp, shapes);
+                float r = 0.0f, d = 0.0f;
+                if (ok) hc::step_lanes(rowp, shapes, ap, lane, r, d);
+                else if (live && b == 0) hc::step_row(rowp, cts + slot * S::CSTRIDE, shapes, env, ap, r, d);
+                if (live && b == 0) {
+                    account(acc, slot, r, d);
+                    if (d > 0.5f) E::reset(rowp, rseed, env);
+                }
+            }
+        }
+        __syncthreads();   // env step done: the rows hold the next observation
+    }
+
+    for (int i = t; i < nenv * E::OBS; i += T) {
+        const int r = i / E::OBS, c = i - r * E::OBS;
+        a.obs[(size_t)env0 * E::OBS + i] = rows[r * S::STRIDE + c];
+    }
+    S::out(rows, gbase, nenv, t, 0, E::STATE);
+}
+
+bool collect_walker_fusable(const mrl_rollout *r, int *act) {
+    if (r->num_actions != 0) return false;
+    int obs, aw;
+    if (r->env_id == MRL_ENV_BIPEDAL) { obs = BipedalWalker::OBS; aw = BipedalWalker::ACT_W; }
+    else if (r->env_id == MRL_ENV_HALFCHEETAH) { obs = HalfCheetah::OBS; aw = HalfCheetah::ACT_W; }
+    else return false;
+    const mrl_mlp_desc &a = r->actor, &c = r->critic;
+    if (a.n_layers != 3 || c.n_layers != 3) return false;
+    const int k0 = a.layers[0].kind;
+    if (k0 != MRL_LINEAR_RELU && k0 != MRL_LINEAR_TANH) return false;
+    for (const mrl_mlp_desc *d : {&a, &c}) {
+        if (d->layers[0].kind != k0 || d->layers[1].kind != k0) return false;
+        if (d->layers[0].in_dim != obs || d->layers[0].out_dim != 256 || d->layers[1].out_dim != 256) return false;
+    }
+    if (a.layers[2].kind != MRL_STOCHASTIC_ACTOR || a.layers[2].out_dim != aw) return false;
+    if (c.layers[2].kind != MRL_LINEAR || c.layers[2].out_dim != 1) return false;
+    // 16-byte loads of the weight rows
+    if (reinterpret_cast<uintptr_t>(r->actor_params) % 16 != 0 || reinterpret_cast<uintptr_t>(r->critic_params) % 16 != 0)
+        return false;
+    *act = (k0 == MRL_LINEAR_RELU) ? 1 : 2;
+    return true;
+}
+
+int launch_collect_walker(mrl_ctx *ctx, const mrl_rollout *r, const CollectArgs &args, int act) {
+    CollectArgs a = args;
+    const dim3 grid(grid_for(r->n_envs, PR16)), block(512);
+    if (r->env_id == MRL_ENV_BIPEDAL) {
+        a.shapes = ctx->bw_shapes;
+        if (act == 1) hipLaunchKernelGGL((collect_walker_kernel<BipedalWalker, 1, false>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((collect_walker_kernel<BipedalWalker, 2, false>), grid, block, 0, ctx->stream, a);
+    } else {
+        a.shapes = ctx->hc_shapes;
+        if (act == 1) hipLaunchKernelGGL((collect_walker_kernel<HalfCheetah16, 1, true>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((collect_walker_kernel<HalfCheetah16, 2, true>), grid, block, 0, ctx->stream, a);
+    }
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
+}  // namespace mrl

@@ -20,7 +20,7 @@ def ctx(mrl):
 
 def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
     E = {"lunar": mrl.LunarLanderV2, "lunarc": mrl.LunarLanderV2Continuous, "cartpole": mrl.CartPoleEnv,
-         "pendulum": mrl.PendulumV2}[env]
+         "pendulum": mrl.PendulumV2, "bipedal": mrl.BipedalWalkerV2, "cheetah": mrl.HalfCheetahPlanarV2}[env]
     lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
     head = mrl.StochasticActor(hidden, E.ACTION_DIM) if E.ACTION_DIM else mrl.Linear(hidden, E.NUM_ACTIONS)
     actor = mrl.seq(lin(E.OBS_DIM, hidden), lin(hidden, hidden), head)
@@ -40,6 +40,10 @@ def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
         elif env == "cartpole":
             rows[::3, 0] = 2.39       # cart next to the edge of the track, moving outwards
             rows[::3, 1] = 2.0
+        elif env == "bipedal":
+            rows[::3, 942] = 1995.0   # step counter (first metadata float) close to its limit of 2000
+        elif env == "cheetah":
+            rows[::3, 245] = 995.0    # step counter (first metadata float) close to its limit of 1000
         else:
             rows[::3, 4] = 197.0      # step counter close to the limit
         rb.obs.copy_(rows[:, :E.OBS_DIM].reshape(-1))
@@ -54,6 +58,11 @@ def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
     ("pendulum", 8192, 12, 64, "tanh"), ("pendulum", 1000, 9, 64, "relu"),
     ("cartpole", 300, 6, 256, "relu"),        # not fusable
     ("lunarc", 8192, 12, 256, "tanh"), ("lunarc", 77, 6, 256, "relu"), ("lunarc", 300, 6, 64, "tanh"),
+    # the walkers: legs on the ground from the first step (contacts, joint limits, lidar), falls and
+    # step-limit endings with in-place resets inside the launch
+    ("bipedal", 4096, 12, 256, "tanh"), ("bipedal", 77, 7, 256, "relu"), ("bipedal", 500, 64, 256, "tanh"),
+    ("cheetah", 4096, 12, 256, "tanh"), ("cheetah", 77, 7, 256, "relu"), ("cheetah", 500, 64, 256, "tanh"),
+    ("cheetah", 300, 5, 64, "tanh"),          # not fusable
 ])
 def test_rollout_steps_equals_single_steps(mrl, ctx, env, N, T, hidden, kind):
     print("case", env, N, T, hidden, kind, flush=True)
