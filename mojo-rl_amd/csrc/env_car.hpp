@@ -52,6 +52,9 @@ struct Tiles {
     float v[SLOTS][8];     // four vertices
     const float *lds;
 
+    // FLAGS_COHERENT: the visited flags are read past the vector cache, for a kernel that steps the same
+    // env again and again and so reads flags that an earlier step of its own launch has written
+    template <bool FLAGS_COHERENT = false>
     MRL_DEV void load(const float *row, float *table, int sub) {
         constexpr int N4 = TABLE / 4, ROUNDS = (N4 + STEP_LANES - 1) / STEP_LANES;
         const float4 *src = reinterpret_cast<const float4 *>(row + TRACK);
@@ -65,6 +68,21 @@ struct Tiles {
 #pragma unroll
         for (int i = 0; i < ROUNDS - 1; ++i) dst[sub + STEP_LANES * i] = tmp[i];
         if (last < N4) dst[last] = tmp[ROUNDS - 1];
+        if (FLAGS_COHERENT) {
+            constexpr int F0 = MAX_TILES * TILE;
+            float f[(MAX_TILES + STEP_LANES - 1) / STEP_LANES];
+#pragma unroll
+            for (int i = 0; i < (MAX_TILES + STEP_LANES - 1) / STEP_LANES; ++i) {
+                const int k = sub + STEP_LANES * i;
+                f[i] = __hip_atomic_load(row + VISITED + (k < MAX_TILES ? k : MAX_TILES - 1), __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int i = 0; i < (MAX_TILES + STEP_LANES - 1) / STEP_LANES; ++i) {
+                const int k = sub + STEP_LANES * i;
+                if (k < MAX_TILES) table[F0 + k] = f[i];
+            }
+        }
         // the wavefront's own LDS writes, read back by other lanes of the same wavefront
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -183,19 +201,23 @@ MRL_DEV void wheel_forces(float wheel_omega, float joint_angle, float hull_angle
     omega_o = omega;
 }
 
-// One env step by the 64 lanes of a wavefront (sub = lane; table = TABLE floats of LDS of its own).  Every
-// lane returns the same reward / done and the observation the row now starts with; lane 0 has written the row.
-MRL_DEV void step_wave(float *row, float *table, const float *action, int sub, float &reward, float &done,
-                       float (&ob)[OBS]) {
-    float *M = row + META;
+// One env step by the 64 lanes of a wavefront (sub = lane; table = TABLE floats of LDS of its own).  `head`
+// = the row's first TRACK floats (observation, hull, wheels, controls, metadata) wherever the caller keeps
+// them: the row itself, or a copy that a kernel holds on chip over many steps; `row` is read for the tile
+// table and takes the visited flags.  Every lane returns the same reward / done and the observation the row
+// now starts with; lane 0 has written `head`.
+template <bool FLAGS_COHERENT = false>
+MRL_DEV void step_wave(float *head, float *row, float *table, const float *action, int sub, float &reward,
+                       float &done, float (&ob)[OBS]) {
+    float *M = head + META;
     if (M[M_DONE] > 0.5f) {   // car_racing_v2.mojo:1564-1572
 #pragma unroll
-        for (int k = 0; k < OBS; ++k) ob[k] = row[k];
+        for (int k = 0; k < OBS; ++k) ob[k] = head[k];
         reward = 0.0f; done = 1.0f;
         return;
     }
     Tiles tiles;
-    tiles.load(row, table, sub);
+    tiles.template load<FLAGS_COHERENT>(row, table, sub);
     int num_tiles = (int)M[M_NUM_TILES];
     if (num_tiles <= 0) num_tiles = 100;
     // ---- controls, car_racing_v2.mojo:262-268 (Float64)
@@ -208,16 +230,16 @@ MRL_DEV void step_wave(float *row, float *table, const float *action, int sub, f
     const float steering = (float)steering_d, gas = (float)gas_d, brake = (float)brake_d;
     const float dt = (float)0.02;
     // ---- state
-    float x = row[HULL + H_X], y = row[HULL + H_Y], angle = row[HULL + H_ANGLE];
-    float vx = row[HULL + H_VX], vy = row[HULL + H_VY], omega = row[HULL + H_OMEGA];
+    float x = head[HULL + H_X], y = head[HULL + H_Y], angle = head[HULL + H_ANGLE];
+    float vx = head[HULL + H_VX], vy = head[HULL + H_VY], omega = head[HULL + H_OMEGA];
     float w_omega[4], w_phase[4];
 #pragma unroll
-    for (int w = 0; w < 4; ++w) { w_omega[w] = row[WHEELS + w * W_SIZE + W_OMEGA]; w_phase[w] = row[WHEELS + w * W_SIZE + W_PHASE]; }
+    for (int w = 0; w < 4; ++w) { w_omega[w] = head[WHEELS + w * W_SIZE + W_OMEGA]; w_phase[w] = head[WHEELS + w * W_SIZE + W_PHASE]; }
     // ---- steering joints (update_steering, car_dynamics.mojo:68-116)
     const float target_angle = steering * (float)0.4;
-    const float joint_fl = update_steering_angle(row[WHEELS + 0 * W_SIZE + W_JOINT], target_angle, dt);
-    const float joint_fr = update_steering_angle(row[WHEELS + 1 * W_SIZE + W_JOINT], target_angle, dt);
-    const float joint_rl = row[WHEELS + 2 * W_SIZE + W_JOINT], joint_rr = row[WHEELS + 3 * W_SIZE + W_JOINT];
+    const float joint_fl = update_steering_angle(head[WHEELS + 0 * W_SIZE + W_JOINT], target_angle, dt);
+    const float joint_fr = update_steering_angle(head[WHEELS + 1 * W_SIZE + W_JOINT], target_angle, dt);
+    const float joint_rl = head[WHEELS + 2 * W_SIZE + W_JOINT], joint_rr = head[WHEELS + 3 * W_SIZE + W_JOINT];
     // ---- friction limit under each wheel (get_wheel_friction_limits, tile_collision.mojo:160-230)
     float sin_a, cos_a;
     sincos32(angle, sin_a, cos_a);
@@ -321,18 +343,18 @@ MRL_DEV void step_wave(float *row, float *table, const float *action, int sub, f
     ob[12] = sqrtf(vx * vx + vy * vy);
     // ---- lane 0 writes the row (the reads above are done: every lane holds its values in registers)
     if (sub == 0) {
-        row[CTRL + 0] = steering; row[CTRL + 1] = gas; row[CTRL + 2] = brake;
-        row[HULL + H_X] = x; row[HULL + H_Y] = y; row[HULL + H_ANGLE] = angle;
-        row[HULL + H_VX] = vx; row[HULL + H_VY] = vy; row[HULL + H_OMEGA] = omega;
+        head[CTRL + 0] = steering; head[CTRL + 1] = gas; head[CTRL + 2] = brake;
+        head[HULL + H_X] = x; head[HULL + H_Y] = y; head[HULL + H_ANGLE] = angle;
+        head[HULL + H_VX] = vx; head[HULL + H_VY] = vy; head[HULL + H_OMEGA] = omega;
         const float joints[4] = {joint_fl, joint_fr, joint_rl, joint_rr};
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            row[WHEELS + w * W_SIZE + W_OMEGA] = w_omega[w];
-            row[WHEELS + w * W_SIZE + W_JOINT] = joints[w];
-            row[WHEELS + w * W_SIZE + W_PHASE] = w_phase[w];
+            head[WHEELS + w * W_SIZE + W_OMEGA] = w_omega[w];
+            head[WHEELS + w * W_SIZE + W_JOINT] = joints[w];
+            head[WHEELS + w * W_SIZE + W_PHASE] = w_phase[w];
         }
 #pragma unroll
-        for (int k = 0; k < OBS; ++k) row[k] = ob[k];
+        for (int k = 0; k < OBS; ++k) head[k] = ob[k];
         if (fresh) row[VISITED + tile_idx[0]] = 1.0f;
         M[M_VISITED] = tiles_visited;
         M[M_TOTAL] = total;
@@ -438,9 +460,10 @@ MRL_DEV int generate_track(float *row, uint64_t seed) {
 
 // _reset_env_gpu, car_racing_v2.mojo:1155-1300, by a group of GROUP lanes of a wavefront: its lane 0
 // walks the track (it writes the tiles it makes), then all lanes clear what is left of the row and
-// place the car; the observation of the fresh row is (start_x, start_y, start_angle, 0, .. 0)
+// place the car; the observation of the fresh row is (start_x, start_y, start_angle, 0, .. 0); returns the
+// number of tiles of the new track
 template <int GROUP>
-MRL_DEV void reset_group(float *row, uint64_t cseed, int lane, float &start_x, float &start_y, float &start_angle) {
+MRL_DEV int reset_group(float *row, uint64_t cseed, int lane, float &start_x, float &start_y, float &start_angle) {
     const int sub = lane & (GROUP - 1), base = lane & ~(GROUP - 1);
     int num_tiles = 0;
     start_x = 0.0f; start_y = 0.0f; start_angle = 0.0f;
@@ -471,6 +494,7 @@ MRL_DEV void reset_group(float *row, uint64_t cseed, int lane, float &start_x, f
         else if (i == META + M_NUM_TILES) v = (float)num_tiles;
         row[i] = v;
     }
+    return num_tiles;
 }
 
 }  // namespace cr

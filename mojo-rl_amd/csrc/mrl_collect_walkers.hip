@@ -1,6 +1,7 @@
-// Fused collection kernel of the two walkers (BipedalWalker, HalfCheetah planar) with the agents'
-// 256-wide Gaussian nets: many rollout steps of a block's 16 envs in ONE launch, like the kernels of
-// mrl_collect.hip.  The env rows stay in LDS from the first step to the last; per step and block
+// Fused collection kernels of the continuous-control envs beyond the classic ones (BipedalWalker,
+// HalfCheetah planar, CarRacingV2) with the agents' 256-wide Gaussian nets: many rollout steps of a
+// block's 16 envs in ONE launch, like the kernels of mrl_collect.hip.  The env rows (CarRacing: the 40
+// floats in front of the track) stay in LDS from the first step to the last; per step and block
 //   policy   wavefronts 0 .. 3 the actor  OBS -> 256 -> 256 -> A, wavefronts 4 .. 7 the critic
 //            OBS -> 256 -> 256 -> 1, side by side on the fp32 matrix cores (the 16-row tiles of
 //            mlp_tile16.hpp, 64 columns per wavefront, weights streamed from L2), heads out of LDS;
@@ -8,6 +9,8 @@
 //   env step BipedalWalker: the workgroup-level step of env_block.hpp (contact detection on every
 //            wavefront, solver on wavefront 0, lidar rays on every wavefront, wave-cooperative
 //            resets); HalfCheetah: one lane per body on wavefronts 0 and 1 (env_cheetah_lanes.hpp);
+//            CarRacing: a wavefront per env, two rounds of eight (env_car.hpp); the tile tables stay in
+//            global memory and are staged through LDS every step (16 x 12 KB do not fit beside the rest);
 //   rollout row t of obs, action, log-prob, value, reward, done written on the way.
 // With these envs the step is 70 - 80 % env step, which is one wavefront's instruction stream, so the
 // critic is not moved beside it: what the fusion buys is the launch gaps, the observation / action
@@ -24,6 +27,7 @@
 #include "policy_sample.hpp"
 #include "env_block.hpp"
 #include "env_cheetah_lanes.hpp"
+#include "env_car.hpp"
 #include "collect_args.hpp"
 
 namespace mrl {
@@ -35,6 +39,56 @@ struct HalfCheetah16 : HalfCheetah {
 
 template <int A, int B>
 constexpr int wmax() { return A > B ? A : B; }
+
+// The policy half of a step, by all 512 threads: observation tile from `obs_at(row, column)` (also out to
+// rollout row t), actor on wavefronts 0 .. 3 and critic on 4 .. 7 (tiles = 2 * H * HT16_LD floats of LDS),
+// Gaussian sampling on one lane per (env, action component) -- the log-probability is the sum of the
+// components' terms in component order --, rollout row t of action, log-prob and value.  Leaves the
+// actions in act[env][AW]; ends with the block in step (everything above complete).
+template <int IN, int AW, int ACT, class ObsAt>
+MRL_DEV void policy16_gauss(const CollectArgs &a, ObsAt obs_at, int tid, int ne, int A, int zero, size_t row,
+                            uint32_t sseed, int env0, float *xs, float *tiles, const float *w2a, const float *w2c,
+                            float *logits, float *vals, float *act, float *part) {
+    constexpr int H = 256, R = PR16, T = 512, KBA = 8;
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    const int net = wave >> 2;                           // 0: actor, 1: critic
+    {
+        const float *p = (net ? a.critic_p : a.actor_p) + zero;
+        float *tile = tiles + net * (H * HT16_LD);
+        Hidden16Operands<H, IN, 4, KBA> ops;
+        ops.load(p, 64 * (wave & 3), lane);
+        for (int i = tid; i < R * IN; i += T) {
+            const int r = i / IN, c = i - r * IN;
+            float v = 0.0f;
+            if (r < ne) {
+                v = obs_at(r, c);
+                a.r_obs[row * IN + i] = v;
+            }
+            xs[r * XS_LD + c] = v;
+        }
+        __syncthreads();
+        BlockSync bs;
+        hidden_stack16<H, IN, ACT, 4, KBA, true>(p, xs, tile, tile, ops, 64 * (wave & 3), lane, bs);
+        if (net == 0) head16<H>(w2a, A, tile, logits, PA_MAX + 1, tid, T / 2);
+        else head_rows16<H, 1, 1>(w2c, 1, tile, vals, 1, tid - T / 2, T / 2);
+        __syncthreads();   // means and values complete; the tiles are dead from here on
+    }
+    for (int e = tid; e < ne * A; e += T) {
+        const int r = e / A, j = e - r * A;
+        float av;
+        part[r * PA_MAX + j] = sample_gaussian_part(logits + r * (PA_MAX + 1) + j, w2a + HEAD_LOG_STD(H) + j, 1, A, j,
+                                                    sseed, env0 + r, &av);
+        act[r * AW + j] = av;
+        a.r_actions[row * AW + e] = av;
+    }
+    if (tid < ne) a.r_values[row + tid] = vals[tid];
+    __syncthreads();
+    if (tid < ne) {
+        float logp = 0.0f;
+        for (int j = 0; j < A; ++j) logp = logp + part[tid * PA_MAX + j];
+        a.r_logp[row + tid] = logp;
+    }
+}
 
 template <class E, int ACT, bool LANES>
 __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
@@ -79,46 +133,8 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
         const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
         const uint64_t rseed = a.reset_seed + (uint64_t)k * a.reset_stride;
         const int wave = tid / WAVE, lane = tid % WAVE;
-        const int net = wave >> 2;                           // 0: actor, 1: critic
-        // ---- policy: both nets side by side
-        {
-            const float *p = (net ? a.critic_p : a.actor_p) + zero;
-            float *tile = overlay + net * (H * HT16_LD);
-            Hidden16Operands<H, IN, 4, KBA> ops;
-            ops.load(p, 64 * (wave & 3), lane);
-            for (int i = tid; i < R * IN; i += T) {
-                const int r = i / IN, c = i - r * IN;
-                float v = 0.0f;
-                if (r < ne) {
-                    v = rows[r * S::STRIDE + c];
-                    a.r_obs[row * IN + i] = v;
-                }
-                xs[r * XS_LD + c] = v;
-            }
-            __syncthreads();
-            BlockSync bs;
-            hidden_stack16<H, IN, ACT, 4, KBA, true>(p, xs, tile, tile, ops, 64 * (wave & 3), lane, bs);
-            if (net == 0) head16<H>(w2a, A, tile, logits, PA_MAX + 1, tid, T / 2);
-            else head_rows16<H, 1, 1>(w2c, 1, tile, vals, 1, tid - T / 2, T / 2);
-            __syncthreads();   // means and values complete; the tiles are dead from here on
-        }
-        // ---- Gaussian sampling, one lane per (env, component); the log-probability is the sum of the
-        // components' terms in component order
-        for (int e = tid; e < ne * A; e += T) {
-            const int r = e / A, j = e - r * A;
-            float av;
-            part[r * PA_MAX + j] = sample_gaussian_part(logits + r * (PA_MAX + 1) + j, w2a + HEAD_LOG_STD(H) + j, 1, A, j,
-                                                        sseed, env0 + r, &av);
-            act[r * AW + j] = av;
-            a.r_actions[row * AW + e] = av;
-        }
-        if (tid < ne) a.r_values[row + tid] = vals[tid];
-        __syncthreads();
-        if (tid < ne) {
-            float logp = 0.0f;
-            for (int j = 0; j < A; ++j) logp = logp + part[tid * PA_MAX + j];
-            a.r_logp[row + tid] = logp;
-        }
+        policy16_gauss<IN, AW, ACT>(a, [&](int r, int c) { return rows[r * S::STRIDE + c]; }, tid, ne, A, zero, row, sseed, env0,
+                                    xs, overlay, w2a, w2c, logits, vals, act, part);
         // ---- env step with auto-reset, reward / done into rollout row t, episode accounting
         Accounting acc = a.acc;
         acc.r_rewards = a.r_rewards + (size_t)(a.t0 + k) * N;
@@ -156,11 +172,97 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
     S::out(rows, gbase, nenv, t, 0, E::STATE);
 }
 
+// CarRacingV2: the rows stay in global memory (12 KB each, nearly all of it the track); the block keeps the
+// 40 floats in front of the track -- observation, hull, wheels, controls, metadata -- of its 16 envs in LDS
+// over the whole launch.  Env step: a wavefront per env in two rounds of eight; each wavefront stages its
+// env's tile table through LDS (over the activation tiles, which are dead by then), steps, accounts, and
+// rebuilds the env when it finished (one lane walks the new track: only this block waits for it).
+template <int ACT>
+__global__ __launch_bounds__(512) void collect_car_kernel(CollectArgs a) {
+    constexpr int H = 256, IN = cr::OBS, AW = cr::ACT, R = PR16, T = 512, HEAD = cr::TRACK;
+    static_assert(IN <= PIN_MAX && AW <= PA_MAX && cr::TABLE % 4 == 0, "tile limits");
+    __shared__ float heads[R * (HEAD + 1)];
+    __shared__ float xs[R * XS_LD];
+    __shared__ __align__(16) float w2a[HEAD_LDS(H)];
+    __shared__ float w2c[H + 1];
+    __shared__ float logits[R * (PA_MAX + 1)];
+    __shared__ float vals[R];
+    __shared__ float act[R * PA_MAX];
+    __shared__ float part[R * PA_MAX];
+    __shared__ __align__(16) float overlay[wmax<2 * H * HT16_LD, 8 * cr::TABLE>()];
+
+    const int t = threadIdx.x;
+    const int env0 = blockIdx.x * R;
+    const int nenv = min(R, a.n_envs - env0);
+    const int N = a.n_envs;
+    for (int i = t; i < nenv * HEAD; i += T) {
+        const int r = i / HEAD, c = i - r * HEAD;
+        heads[r * (HEAD + 1) + c] = a.states[(size_t)(env0 + r) * cr::STATE + c];
+    }
+    stage_head(a.actor_p + IN * H + H + H * H + H, H, a.A, true, w2a, t, T);
+    for (int i = t; i < H + 1; i += T) w2c[i] = a.critic_p[IN * H + H + H * H + H + i];
+    __syncthreads();
+
+    for (int k = 0; k < a.n_steps; ++k) {
+        int tid = t, ne = __builtin_amdgcn_readfirstlane(nenv), A = __builtin_amdgcn_readfirstlane(a.A), zero = 0;
+        asm volatile("" : "+v"(tid), "+s"(zero), "+s"(ne), "+s"(A) : : "memory");
+        const size_t row = (size_t)(a.t0 + k) * N + env0;
+        const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
+        const uint64_t rseed = a.reset_seed + (uint64_t)k * a.reset_stride;
+        const int wave = tid / WAVE, sub = tid % WAVE;
+        policy16_gauss<IN, AW, ACT>(a, [&](int r, int c) { return heads[r * (HEAD + 1) + c]; }, tid, ne, A, zero, row, sseed,
+                                    env0, xs, overlay, w2a, w2c, logits, vals, act, part);
+        Accounting acc = a.acc;
+        acc.r_rewards = a.r_rewards + (size_t)(a.t0 + k) * N;
+        acc.r_dones = a.r_dones + (size_t)(a.t0 + k) * N;
+        acc = acc.at(env0);
+        __syncthreads();   // the sampling's reads of the means are done before the tables go over the tiles
+#pragma unroll 1
+        for (int round = 0; round < 2; ++round) {
+            const int slot = round * 8 + wave;
+            if (slot < ne) {
+                const int env = env0 + slot;
+                float *head = heads + slot * (HEAD + 1);
+                float *grow = a.states + (size_t)env * cr::STATE;
+                float r, d, ob[cr::OBS];
+                cr::step_wave<true>(head, grow, overlay + wave * cr::TABLE, act + slot * AW, sub, r, d, ob);
+                if (sub == 0) account(acc, slot, r, d);
+                if (d > 0.5f) {
+                    float sx, sy, sa;
+                    const int nt = cr::reset_group<cr::STEP_LANES>(grow, cr::combined_seed(rseed, env), sub, sx, sy, sa);
+                    if (sub < HEAD) {
+                        float v = 0.0f;
+                        if (sub == 0 || sub == cr::HULL + cr::H_X) v = sx;
+                        else if (sub == 1 || sub == cr::HULL + cr::H_Y) v = sy;
+                        else if (sub == 2 || sub == cr::HULL + cr::H_ANGLE) v = sa;
+                        else if (sub == cr::META + cr::M_NUM_TILES) v = (float)nt;
+                        head[sub] = v;
+                    }
+                    // the new track is read back by this wavefront at its next step: nothing older may
+                    // linger in the vector cache
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                }
+            }
+        }
+        __syncthreads();   // env step done: the heads hold the next observation
+    }
+
+    for (int i = t; i < nenv * HEAD; i += T) {
+        const int r = i / HEAD, c = i - r * HEAD;
+        a.states[(size_t)(env0 + r) * cr::STATE + c] = heads[r * (HEAD + 1) + c];
+    }
+    for (int i = t; i < nenv * IN; i += T) {
+        const int r = i / IN, c = i - r * IN;
+        a.obs[(size_t)env0 * IN + i] = heads[r * (HEAD + 1) + c];
+    }
+}
+
 bool collect_walker_fusable(const mrl_rollout *r, int *act) {
     if (r->num_actions != 0) return false;
     int obs, aw;
     if (r->env_id == MRL_ENV_BIPEDAL) { obs = BipedalWalker::OBS; aw = BipedalWalker::ACT_W; }
     else if (r->env_id == MRL_ENV_HALFCHEETAH) { obs = HalfCheetah::OBS; aw = HalfCheetah::ACT_W; }
+    else if (r->env_id == MRL_ENV_CARRACING) { obs = cr::OBS; aw = cr::ACT; }
     else return false;
     const mrl_mlp_desc &a = r->actor, &c = r->critic;
     if (a.n_layers != 3 || c.n_layers != 3) return false;
@@ -186,6 +288,9 @@ int launch_collect_walker(mrl_ctx *ctx, const mrl_rollout *r, const CollectArgs 
         a.shapes = ctx->bw_shapes;
         if (act == 1) hipLaunchKernelGGL((collect_walker_kernel<BipedalWalker, 1, false>), grid, block, 0, ctx->stream, a);
         else hipLaunchKernelGGL((collect_walker_kernel<BipedalWalker, 2, false>), grid, block, 0, ctx->stream, a);
+    } else if (r->env_id == MRL_ENV_CARRACING) {
+        if (act == 1) hipLaunchKernelGGL((collect_car_kernel<1>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((collect_car_kernel<2>), grid, block, 0, ctx->stream, a);
     } else {
         a.shapes = ctx->hc_shapes;
         if (act == 1) hipLaunchKernelGGL((collect_walker_kernel<HalfCheetah16, 1, true>), grid, block, 0, ctx->stream, a);

@@ -206,7 +206,7 @@ __global__ __launch_bounds__(CAR_THREADS) void car_step_kernel(float *states, co
     if (env >= batch) return;   // whole wavefronts leave together
     float *row = states + (size_t)env * cr::STATE;
     float r, d, ob[cr::OBS];
-    cr::step_wave(row, tables[wave], actions + (size_t)env * cr::ACT, sub, r, d, ob);
+    cr::step_wave(row, row, tables[wave], actions + (size_t)env * cr::ACT, sub, r, d, ob);
     if (sub == 0) {
         rewards[env] = r;
         dones[env] = d;

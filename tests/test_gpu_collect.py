@@ -20,7 +20,8 @@ def ctx(mrl):
 
 def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
     E = {"lunar": mrl.LunarLanderV2, "lunarc": mrl.LunarLanderV2Continuous, "cartpole": mrl.CartPoleEnv,
-         "pendulum": mrl.PendulumV2, "bipedal": mrl.BipedalWalkerV2, "cheetah": mrl.HalfCheetahPlanarV2}[env]
+         "pendulum": mrl.PendulumV2, "bipedal": mrl.BipedalWalkerV2, "cheetah": mrl.HalfCheetahPlanarV2,
+         "car": mrl.CarRacingV2}[env]
     lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
     head = mrl.StochasticActor(hidden, E.ACTION_DIM) if E.ACTION_DIM else mrl.Linear(hidden, E.NUM_ACTIONS)
     actor = mrl.seq(lin(E.OBS_DIM, hidden), lin(hidden, hidden), head)
@@ -42,6 +43,8 @@ def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
             rows[::3, 1] = 2.0
         elif env == "bipedal":
             rows[::3, 942] = 1995.0   # step counter (first metadata float) close to its limit of 2000
+        elif env == "car":
+            rows[::3, 34] = 495.0     # step counter (first metadata float) close to its limit of 500
         elif env == "cheetah":
             rows[::3, 245] = 995.0    # step counter (first metadata float) close to its limit of 1000
         else:
@@ -63,6 +66,10 @@ def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
     ("bipedal", 4096, 12, 256, "tanh"), ("bipedal", 77, 7, 256, "relu"), ("bipedal", 500, 64, 256, "tanh"),
     ("cheetah", 4096, 12, 256, "tanh"), ("cheetah", 77, 7, 256, "relu"), ("cheetah", 500, 64, 256, "tanh"),
     ("cheetah", 300, 5, 64, "tanh"),          # not fusable
+    # CarRacing: tiles are visited from the first step on (the flags an env wrote are read back by later
+    # steps of the same launch), truncations rebuild the track inside the launch
+    ("car", 4096, 12, 256, "tanh"), ("car", 77, 7, 256, "relu"), ("car", 300, 48, 256, "tanh"),
+    ("car", 100, 5, 64, "tanh"),              # not fusable
 ])
 def test_rollout_steps_equals_single_steps(mrl, ctx, env, N, T, hidden, kind):
     print("case", env, N, T, hidden, kind, flush=True)
