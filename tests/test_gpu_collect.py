@@ -188,6 +188,74 @@ def test_fused_collection_through_contacts(mrl, ctx, orc, env, kind, N):
     assert cnt == int(fused.done_count.item()) == resets
 
 
+@pytest.mark.parametrize("env,kind,N", [("bipedal", "tanh", 512), ("cheetah", "tanh", 512), ("car", "relu", 300),
+                                        ("bipedal", "relu", 45)])
+def test_fused_walker_collection_against_the_oracle(mrl, ctx, orc, env, kind, N):
+    """The fused collection kernels of BipedalWalker, HalfCheetah and CarRacingV2 in launches of one step,
+    against the oracle fed the kernel's own actions: rewards and done flags exact, the rows (state after
+    the in-launch reset of finished envs) and the observation bit for bit; then the same 64 steps in two
+    launches give the same buffers."""
+    import numpy as np
+    print("case walker oracle", env, kind, N, flush=True)
+    T = 64
+    E, step, reset = {"bipedal": (mrl.BipedalWalkerV2, orc.orc_bw_step_batch, orc.orc_bw_reset_batch),
+                      "cheetah": (mrl.HalfCheetahPlanarV2, orc.orc_hc_step_batch, orc.orc_hc_reset_batch),
+                      "car": (mrl.CarRacingV2, orc.orc_cr_step_batch, orc.orc_cr_reset_batch)}[env]
+    S, OBS, AW = E.STATE_SIZE, E.OBS_DIM, E.ACTION_DIM
+    lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
+    actor = mrl.seq(lin(OBS, 256), lin(256, 256), mrl.StochasticActor(256, AW))
+    critic = mrl.seq(lin(OBS, 256), lin(256, 256), mrl.Linear(256, 1))
+    g = torch.Generator(device="cuda").manual_seed(11)
+    ap = (torch.rand(actor.PARAM_SIZE, device="cuda", generator=g) - 0.5) * 0.3
+    ap[-AW:] = 0.3                                   # log_std: lively actions, so that walkers fall
+    cp = (torch.rand(critic.PARAM_SIZE, device="cuda", generator=g) - 0.5) * 0.3
+    s0_h = np.zeros((N, S), np.float32)
+    reset(s0_h, None, N, 17)
+    meta0 = {"bipedal": 942, "cheetah": 245, "car": 34}[env]
+    s0_h[::5, meta0] = {"bipedal": 1990.0, "cheetah": 990.0, "car": 490.0}[env]   # some rows near the step limit
+    rbs = []
+    for _ in range(2):
+        rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N, T)
+        rb.actor_params, rb.critic_params = ap, cp
+        rb.states.copy_(torch.from_numpy(s0_h.reshape(-1)).cuda())
+        rb.obs.copy_(rb.states.view(N, S)[:, :OBS].reshape(-1))
+        rbs.append(rb)
+    fused1, fused = rbs
+    assert mrl.ppo.rollout_fused(fused.descriptor()) == 1
+    s0, ss, r0, rs = 31337, 2654435761 * N + 7919, 5, 0x9E3779B97F
+    s_h = s0_h.copy()
+    r_h, d_h, o_h = np.zeros(N, np.float32), np.zeros(N, np.float32), np.zeros((N, OBS), np.float32)
+    d1 = fused1.descriptor()
+    finished = 0
+    for t in range(T):
+        mrl.ppo.rollout_steps(ctx, d1, t, 1, (s0 + t * ss) & 0xFFFFFFFF, 0, 0, 0, (r0 + t * rs) & (2**64 - 1), 0)
+        ctx.synchronize()
+        acts = np.ascontiguousarray(fused1.r_actions[t * N * AW:(t + 1) * N * AW].cpu().numpy().reshape(N, AW))
+        step(s_h, acts, r_h, d_h, o_h, N, 8)
+        np.testing.assert_array_equal(fused1.r_rewards[t * N:(t + 1) * N].cpu().numpy(), r_h, err_msg="reward, step %d" % t)
+        np.testing.assert_array_equal(fused1.r_dones[t * N:(t + 1) * N].cpu().numpy(), d_h, err_msg="done, step %d" % t)
+        finished += int(d_h.sum())
+        flags = d_h.copy()                      # kept alive over the call that reads it through a raw pointer
+        reset(s_h, flags.ctypes.data, N, (r0 + t * rs) & (2**64 - 1))
+        sg = fused1.states.cpu().numpy().reshape(N, S)
+        assert np.array_equal(sg.view(np.uint32), s_h.view(np.uint32)), "state, step %d: %d floats differ" % (
+            t, int((sg.view(np.uint32) != s_h.view(np.uint32)).sum()))
+        assert np.array_equal(fused1.obs.cpu().numpy().reshape(N, OBS).view(np.uint32), s_h[:, :OBS].view(np.uint32))
+    print("  finished episodes", finished, flush=True)
+    assert finished >= N // 5
+    dfused = fused.descriptor()
+    k = 29
+    mrl.ppo.rollout_steps(ctx, dfused, 0, k, s0, ss & 0xFFFFFFFF, 0, 0, r0, rs)
+    mrl.ppo.rollout_steps(ctx, dfused, k, T - k, (s0 + k * ss) & 0xFFFFFFFF, ss & 0xFFFFFFFF, 0, 0,
+                          (r0 + k * rs) & (2**64 - 1), rs)
+    ctx.synchronize()
+    for name in ("r_obs", "r_actions", "r_log_probs", "r_values", "r_rewards", "r_dones", "states", "obs",
+                 "ep_return", "ep_length"):
+        a, b = getattr(fused1, name), getattr(fused, name)
+        assert torch.equal(a, b), "%s: the 64-step range differs from one-step launches in %d places" % (name, int((a != b).sum()))
+    assert int(fused.done_count.item()) == finished
+
+
 def test_barrier_wait_gives_up_and_reports(mrl):
     """The wavefront-group barriers inside the fused collection kernel are bounded: with a limit of
     one poll some wait gives up, the kernel still ends normally, and the next synchronize reports it
