@@ -59,6 +59,26 @@ def test_continuous_agent_runs_on_the_continuous_lunar_lander(mrl):
     assert np.isfinite(got) and got < 0.0     # three rollouts do not make a pilot
 
 
+@pytest.mark.parametrize("env_name,obs_dim,action_dim", [("BipedalWalkerV2", 24, 4), ("HalfCheetahPlanarV2", 17, 6)])
+def test_continuous_agent_runs_on_the_walkers(mrl, env_name, obs_dim, action_dim):
+    """The walkers behind the continuous agent with the reference's 256-wide nets: the fused collection
+    kernel, GAE and the update run over several rollouts and keep every buffer finite; the default KL
+    early stop is on."""
+    ctx = mrl.DeviceContext("cuda:0")
+    E = getattr(mrl, env_name)
+    agent = mrl.DeepPPOContinuousAgent(obs_dim=obs_dim, action_dim=action_dim, hidden_dim=256, rollout_len=96,
+                                       n_envs=400, gpu_minibatch_size=4096, num_epochs=3, init_seed=5)
+    m = agent.train_gpu(ctx, E, num_episodes=10**9, max_rollouts=4, seed=1)
+    assert mrl.ppo.rollout_fused(agent.rb.descriptor())
+    assert m.rollouts == 4 and m.total_steps == 4 * 96 * 400
+    assert all(np.isfinite(m.episode_rewards)) and all(1 <= n <= 2000 for n in m.episode_steps)
+    if env_name == "BipedalWalkerV2":
+        assert len(m.episode_rewards) > 100        # an untrained walker falls within a few dozen steps
+    assert torch.isfinite(agent.actor.params).all() and torch.isfinite(agent.critic.params).all()
+    assert torch.isfinite(agent.rb.states).all() and torch.isfinite(agent.rb.r_log_probs).all()
+    assert agent.actor.optimizer.t > 0
+
+
 def test_observation_noise_enters_the_rollout(mrl, orc):
     """obs_noise_std > 0 (ppo_continuous.mojo:2557-2564, :2705-2713): the policy sees noisy
     observations from the first step on, the env rows stay clean, and the stored observation of step
