@@ -79,11 +79,49 @@ def _cpu_rollout(np, orc, o, n_envs, steps, seed):
         obs[:] = s[:, :8]
 
 
+def _cpu_update(np, orc, o, mb, seed):
+    """One PPO minibatch update of `mb` samples on the calling thread with the oracle's pieces in the
+    reference's order: per-minibatch advantage normalisation, actor and critic forward with caches,
+    loss gradients, backward, global-norm clip, Adam (north-star nets 8-256-256-4 and 8-256-256-1)."""
+    OBS, HIDDEN, NA = 8, 256, 4
+    la = orc.layers([(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, NA)])
+    lc = orc.layers([(1, OBS, HIDDEN), (1, HIDDEN, HIDDEN), (0, HIDDEN, 1)])
+    rng = np.random.default_rng(seed)
+    pa = rng.uniform(-0.1, 0.1, o.orc_mlp_param_size(la, 3)).astype(np.float32)
+    pc = rng.uniform(-0.1, 0.1, o.orc_mlp_param_size(lc, 3)).astype(np.float32)
+    obs = rng.normal(size=(mb, OBS)).astype(np.float32)
+    act = rng.integers(0, NA, mb).astype(np.float32)
+    adv, ret = rng.normal(size=mb).astype(np.float32), rng.normal(size=mb).astype(np.float32)
+    old_lp, old_v = np.full(mb, -1.3, np.float32), rng.normal(size=mb).astype(np.float32)
+    o.orc_normalize_minibatch_host(adv, mb)
+    for layers, params, lr in ((la, pa, 3e-4), (lc, pc, 1e-3)):
+        actor = layers is la
+        width = NA if actor else 1
+        cache = np.zeros(mb * o.orc_mlp_cache_size(layers, 3), np.float32)
+        out = np.zeros((mb, width), np.float32)
+        o.orc_mlp_forward(layers, 3, mb, obs, params, out, cache.ctypes.data)
+        g_out = np.zeros((mb, width), np.float32)
+        if actor:
+            kl = np.zeros(mb, np.float32)
+            o.orc_ppo_actor_grad_discrete(out, old_lp, adv, act, mb, NA, 0.2, 0.01, g_out, kl)
+        else:
+            gv = np.zeros(mb, np.float32)
+            o.orc_ppo_critic_grad(out.reshape(-1), old_v, ret, mb, 0, 1, 0.5, 0.2, gv)
+            g_out[:, 0] = gv
+        g = np.zeros(params.size, np.float32)
+        o.orc_mlp_backward(layers, 3, mb, g_out, params, cache, g, None)
+        o.orc_clip_grad_norm(g, g.size, 0.5)
+        state = np.zeros(2 * g.size, np.float32)
+        o.orc_adam_step(params, g, state, g.size, 1, lr, 0.9, 0.999, 1e-8)
+
+
 def cpu_baseline(np, n_envs=2048, steps=120):
-    """The CPU figure beside the GPU one: the oracle timed on this box's host cores on a bounded
-    sample of the default workload -- once on every core of this job's CPU share (the envs split
-    evenly over the threads, each thread its own rollout loop; the C calls release the GIL), and
-    once on a single thread, which is how the reference's own CPU loop runs."""
+    """The CPU figures beside the GPU ones: the oracle timed on this box's host cores on a bounded
+    sample of the default workload.  Rollout: once on every core of this job's CPU share (the envs
+    split evenly over the threads, each thread its own rollout loop; the C calls release the GIL), and
+    once on a single thread, which is how the reference's own CPU loop runs.  Update: minibatches of
+    4096 on one thread (the reference's CPU trainer is a serial loop over samples and layers) and one
+    minibatch per thread on all cores."""
     from concurrent.futures import ThreadPoolExecutor
     from oracle import orc
     o = orc.load()
@@ -97,11 +135,21 @@ def cpu_baseline(np, n_envs=2048, steps=120):
     with ThreadPoolExecutor(cores) as pool:
         list(pool.map(lambda k: _cpu_rollout(np, orc, o, per, steps, k), range(cores)))
     dtc = time.perf_counter() - t0
+    mb = 4096
+    t0 = time.perf_counter()
+    _cpu_update(np, orc, o, mb, 0)
+    du1 = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    with ThreadPoolExecutor(cores) as pool:
+        list(pool.map(lambda k: _cpu_update(np, orc, o, mb, k), range(cores)))
+    duc = time.perf_counter() - t0
     return {"value": per * cores * steps / dtc, "unit": "env-steps/s", "cores": cores, "kind": "port",
             "single_thread_value": single,
+            "update_samples_per_s": mb * cores / duc, "update_single_thread_samples_per_s": mb / du1,
             "sample": "LunarLander collection steps (env step + actor / critic forward + sampling + reset): "
-                      "%d envs x %d steps on %d threads in %.1f s; %d envs x %d steps on one thread in %.1f s"
-                      % (per * cores, steps, cores, dtc, n_envs // 4, steps, dt1)}
+                      "%d envs x %d steps on %d threads in %.1f s; %d envs x %d steps on one thread in %.1f s; "
+                      "PPO update: %d minibatches of %d samples, one per thread, in %.1f s; one minibatch on one "
+                      "thread in %.1f s" % (per * cores, steps, cores, dtc, n_envs // 4, steps, dt1, cores, mb, duc, du1)}
 
 
 def measured_traffic():
