@@ -90,8 +90,6 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     const bool owner = t < nenv;
     float ep_return = owner ? a.acc.ep_return[env0 + t] : 0.0f;
     float ep_length = owner ? a.acc.ep_length[env0 + t] : 0.0f;
-    WaveGroupSync critic_sync{&sync_critic, 0u, (unsigned)CRITIC_WAVES, &sync_failed, a.spin_limit};
-    WaveGroupSync detect_sync{&sync_detect, 0u, (unsigned)(NW - 1), &sync_failed, a.spin_limit};
     static_assert((E::DETECT_TASKS + 1) / 2 <= NW - 1, "two detection tasks per wavefront besides wavefront 0");
 
     // Per step: every wavefront runs the actor (the action is what the env step waits for); then
@@ -108,6 +106,11 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
         const size_t row = (size_t)(a.t0 + k) * N + env0;   // this block's slice of rollout row t
         const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
         const int wave = tid / WAVE, lane = tid % WAVE;
+        // the barriers of the wavefront groups, rebuilt every step from the step number (the critic's
+        // hidden stack meets three times per step, the detection once), so that nothing of them is
+        // carried through the env step in registers
+        WaveGroupSync critic_sync{&sync_critic, (unsigned)k * 3u * CRITIC_WAVES, (unsigned)CRITIC_WAVES, &sync_failed, a.spin_limit};
+        WaveGroupSync detect_sync{&sync_detect, (unsigned)k * (NW - 1), (unsigned)(NW - 1), &sync_failed, a.spin_limit};
         // ---- actor, all wavefronts
         {
             HiddenOperands<H, 1, 32> ops;
@@ -277,8 +280,6 @@ __global__ __launch_bounds__(256, 2) void collect16_kernel(CollectArgs a) {
     const bool owner = (t >> 6) == sw && (t & 63) < nenv;
     float ep_return = owner ? a.acc.ep_return[env0 + (t & 63)] : 0.0f;
     float ep_length = owner ? a.acc.ep_length[env0 + (t & 63)] : 0.0f;
-    WaveGroupSync critic_sync{&sync_critic, 0u, 3u, &sync_failed, a.spin_limit};
-    WaveGroupSync detect_sync{&sync_detect, 0u, 3u, &sync_failed, a.spin_limit};
 
     for (int k = 0; k < a.n_steps; ++k) {
         // Nothing but the rows is carried from one step to the next: the thread index, the block's
@@ -292,6 +293,10 @@ __global__ __launch_bounds__(256, 2) void collect16_kernel(CollectArgs a) {
         const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
         const int wave = tid / WAVE, lane = tid % WAVE;
         const int vw = (wave - sw) & 3;                     // 0: solver, 1 .. 3: helpers
+        // the helpers' barriers, rebuilt every step from the step number (the critic's hidden stack meets
+        // three times per step, the detection once): nothing of them stays in registers through the env step
+        WaveGroupSync critic_sync{&sync_critic, (unsigned)k * 9u, 3u, &sync_failed, a.spin_limit};
+        WaveGroupSync detect_sync{&sync_detect, (unsigned)k * 3u, 3u, &sync_failed, a.spin_limit};
         // ---- actor, all wavefronts
         {
             Hidden16Operands<H, IN, 4, KBA> ops;
