@@ -140,6 +140,13 @@ int mrl_env_step(mrl_ctx *ctx, int env_id, int batch, float *states, const float
  * of `states` -- a caller that copies or moves its rows copies the counters along and binds them to
  * the new pointer.  steps = NULL forgets the pointer (and frees a library-made array). */
 int mrl_cartpole_bind_steps(mrl_ctx *ctx, const float *states, int batch, int32_t *steps);
+/* LunarLanderV2's struct parameters ENABLE_WIND / WIND_POWER / TURBULENCE_POWER
+ * (envs/lunar_lander/lunar_lander_v2.mojo:123-127; defaults off, 15.0, 1.5) as a setting of the
+ * context, for both action forms: while no leg touches the ground every step first adds
+ * tanh(sin(0.02 t) + sin(pi 0.01 t)) * power as an impulse to the lander's vx (wind) and omega
+ * (turbulence), computed in Float64 as _apply_wind does (:983-1023), with t = the row's step
+ * count as in the GPU trait (:2041-2105).  Takes effect for steps enqueued after the call. */
+int mrl_lunar_set_wind(mrl_ctx *ctx, int enable, double wind_power, double turbulence_power);
 /* step, then re-initialise rows that finished with the selective-reset protocol, then write
  * obs from the (possibly fresh) row: the sequence step_kernel_gpu -> selective_reset_kernel_gpu
  * -> _extract_obs_from_state_kernel of deep_agents/ppo/ppo.mojo:2148-2285 in one launch.

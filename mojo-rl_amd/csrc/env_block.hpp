@@ -45,7 +45,7 @@ MRL_DEV void account(const Accounting &acc, int i, float r, float d) { account(a
 struct LunarLander {
     using L = ll::L;
     static constexpr int STATE = ll::STATE, OBS = ll::OBS, ACT_W = 1, EPB = 32, THREADS = 512;
-    static constexpr int DYN_END = L::JOINTS_OFF, NSHAPE = 3 * SHAPE_SIZE;
+    static constexpr int DYN_END = L::JOINTS_OFF, NSHAPE = ll::NSHAPE_FLOATS;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
         ll::step_row(row, cts, shapes, env, (int)a[0], r, d);
@@ -68,7 +68,9 @@ struct LunarLander {
         else { body = 2; vertex = k - 10; max_verts = 4; }
     }
     using Carry = ll::StepCarry;
-    static MRL_DEV Carry step_begin(float *row, int env, const float *a) { return ll::step_begin(row, env, (int)a[0]); }
+    static MRL_DEV Carry step_begin(float *row, int env, const float *a, const float *shapes) {
+        return ll::step_begin(row, env, (int)a[0], shapes);
+    }
     static MRL_DEV void step_finish(float *row, float *cts, int n, const float *shapes, const Carry &c, float &r,
                                     float &d) {
         ll::step_finish(row, cts, n, shapes, c, r, d);
@@ -82,11 +84,11 @@ struct LunarLanderContinuous : LunarLander {
     static constexpr int ACT_W = 2;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
-        const Carry c = ll::step_begin_continuous(row, env, a);
+        const Carry c = ll::step_begin_continuous(row, env, a, shapes);
         ll::step_finish(row, cts, -1, shapes, c, r, d);
     }
-    static MRL_DEV Carry step_begin(float *row, int env, const float *a) {
-        return ll::step_begin_continuous(row, env, a);
+    static MRL_DEV Carry step_begin(float *row, int env, const float *a, const float *shapes) {
+        return ll::step_begin_continuous(row, env, a, shapes);
     }
 };
 
@@ -122,7 +124,7 @@ struct BipedalWalker {
         else { body = 1 + (k - 5) / 4; vertex = (k - 5) % 4; max_verts = 4; }
     }
     struct Carry { float act[bw::ACT]; };
-    static MRL_DEV Carry step_begin(float *row, int, const float *a) {
+    static MRL_DEV Carry step_begin(float *row, int, const float *a, const float *) {
         Carry c;
         bw::step_motors(row, a, c.act);
         return c;
@@ -149,7 +151,7 @@ struct HalfCheetah {
     static constexpr int DETECT_TASKS = 0;
     static MRL_DEV void detect_task(int, int &, int &, int &) {}
     struct Carry {};
-    static MRL_DEV Carry step_begin(float *, int, const float *) { return Carry{}; }
+    static MRL_DEV Carry step_begin(float *, int, const float *, const float *) { return Carry{}; }
     static MRL_DEV void step_finish(float *, float *, int, const float *, const Carry &, float &, float &) {}
 };
 
@@ -337,7 +339,7 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
         if (wave == 0) {
             if (lane < nenv) sums = account_before(acc, lane);
             if (lane < nenv)
-                carry = E::step_begin(rows + lane * S::STRIDE, env0 + lane, actions + (size_t)lane * E::ACT_W);
+                carry = E::step_begin(rows + lane * S::STRIDE, env0 + lane, actions + (size_t)lane * E::ACT_W, shapes);
         } else {
             const int task = (wave - 1) * 2 + lane / HALF, e = lane % HALF;
             if (task < NT && e < nenv) detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
@@ -369,7 +371,7 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
             static_assert(WAVE % E::EPB == 0 && E::EPB <= WAVE, "lane groups of EPB inside a wavefront");
             constexpr int SLOTS = E::THREADS / E::EPB;
             const int e = tid % E::EPB;
-            if (tid < nenv) carry = E::step_begin(rows + tid * S::STRIDE, env0 + tid, actions + (size_t)tid * E::ACT_W);
+            if (tid < nenv) carry = E::step_begin(rows + tid * S::STRIDE, env0 + tid, actions + (size_t)tid * E::ACT_W, shapes);
             if (e < nenv)
                 for (int task = tid / E::EPB; task < E::DETECT_TASKS; task += SLOTS)
                     detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);

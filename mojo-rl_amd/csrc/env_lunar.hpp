@@ -47,8 +47,10 @@ constexpr double FPS = 50.0;
 constexpr double DT = 0.02;
 constexpr int TERRAIN_CHUNKS = 11;
 
-// polygon table shared by all envs: hull (6 vertices) and two identical legs (4 vertices)
-struct Shapes { float v[3 * SHAPE_SIZE]; };
+// polygon table shared by all envs: hull (6 vertices) and two identical legs (4 vertices); behind it
+// the wind setting of the context [on (0 / 1), wind power, turbulence power, unused], off by default
+constexpr int WIND_OFF = 3 * SHAPE_SIZE, NSHAPE_FLOATS = WIND_OFF + 4;
+struct Shapes { float v[NSHAPE_FLOATS]; };
 inline Shapes make_shapes() {
     Shapes s{};
     const double lv[6][2] = {{-14.0, 17.0}, {-17.0, 0.0}, {-17.0, -10.0},
@@ -298,7 +300,26 @@ struct StepCarry {
     bool skip;   // the row was already finished: reward 0, done 1, nothing moves
 };
 
-MRL_DEV StepCarry step_begin(float *row, int env, int action) {
+// Wind and turbulence (struct parameters ENABLE_WIND / WIND_POWER / TURBULENCE_POWER of the reference,
+// lunar_lander_v2.mojo:123-127; _apply_wind, :983-1023): skipped while a leg touches the ground;
+// otherwise tanh(sin(0.02 t) + sin(pi 0.01 t)) times the power as an impulse on the lander's vx and
+// omega, in Float64, before the engines.  t is the row's step count, as in the GPU trait (:2041-2105):
+// the row has no slot for the CPU env's two running indices.
+MRL_DEV void apply_wind(float *row, int step_count, const float *shapes) {
+    if (!(shapes[WIND_OFF] > 0.5f)) return;
+    if (row[6] > 0.5f || row[7] > 0.5f) return;
+    const double k = 0.01, t = (double)step_count, pi = 3.14159265358979323846;
+    const double wind_mag = ::tanh(::sin(0.02 * t) + ::sin(pi * k * t)) * (double)shapes[WIND_OFF + 1];
+    const double torque_mag = ::tanh(::sin(0.02 * t) + ::sin(pi * k * t)) * (double)shapes[WIND_OFF + 2];
+    float *B = row + L::BODIES_OFF;
+    const double vx = (double)B[IDX_VX], omega = (double)B[IDX_OMEGA];
+    const double dvx = wind_mag * DT / LANDER_MASS;
+    const double domega = torque_mag * DT / LANDER_INERTIA;
+    B[IDX_VX] = (float)(vx + dvx);
+    B[IDX_OMEGA] = (float)(omega + domega);
+}
+
+MRL_DEV StepCarry step_begin(float *row, int env, int action, const float *shapes) {
     StepCarry c;
     c.skip = row[L::META_OFF + META_DONE] > 0.5f;
     c.step_count = (int)row[L::META_OFF + META_STEP];
@@ -307,7 +328,10 @@ MRL_DEV StepCarry step_begin(float *row, int env, int action) {
     if (action == 2) c.m_power = 1.0;
     else if (action == 1) { c.s_power = 1.0; direction = -1.0; }
     else if (action == 3) { c.s_power = 1.0; direction = 1.0; }
-    if (!c.skip) apply_engines(row, env, c.step_count, c.m_power, c.s_power, direction);
+    if (!c.skip) {
+        apply_wind(row, c.step_count, shapes);
+        apply_engines(row, env, c.step_count, c.m_power, c.s_power, direction);
+    }
     return c;
 }
 
@@ -315,7 +339,7 @@ MRL_DEV StepCarry step_begin(float *row, int env, int action) {
 // fp64 like the rest of the engine arithmetic): a[0] in [-1, 1] is the main throttle, remapped to
 // (a0 + 1) / 2 and clipped to [0, 1]; a[1] clipped to [-1, 1] fires the left (< -0.5) or right
 // (> 0.5) engine with power (|a1| - 0.5) * 2.  Both engines can fire in one step.
-MRL_DEV StepCarry step_begin_continuous(float *row, int env, const float *a) {
+MRL_DEV StepCarry step_begin_continuous(float *row, int env, const float *a, const float *shapes) {
     StepCarry c;
     c.skip = row[L::META_OFF + META_DONE] > 0.5f;
     c.step_count = (int)row[L::META_OFF + META_STEP];
@@ -328,7 +352,10 @@ MRL_DEV StepCarry step_begin_continuous(float *row, int env, const float *a) {
     if (side_action < -0.5) { direction = -1.0; s_power = (-side_action - 0.5) * 2.0; }
     else if (side_action > 0.5) { direction = 1.0; s_power = (side_action - 0.5) * 2.0; }
     c.m_power = m_power; c.s_power = s_power;
-    if (!c.skip) apply_engines(row, env, c.step_count, m_power, s_power, direction);
+    if (!c.skip) {
+        apply_wind(row, c.step_count, shapes);
+        apply_engines(row, env, c.step_count, m_power, s_power, direction);
+    }
     return c;
 }
 
@@ -379,7 +406,7 @@ MRL_DEV void step_finish(float *row, float *contacts, int n_given, const float *
 // one env step on an LDS-resident row by one lane; `contacts` = this lane's contact scratch
 MRL_DEV void step_row(float *row, float *contacts, const float *shapes, int env, int action,
                       float &reward, float &done) {
-    const StepCarry c = step_begin(row, env, action);
+    const StepCarry c = step_begin(row, env, action, shapes);
     step_finish(row, contacts, -1, shapes, c, reward, done);
 }
 

@@ -149,7 +149,7 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
                     a.r_actions[row + lane] = (float)sel;
                 }
                 a.r_logp[row + lane] = logp;
-                carry = E::step_begin(rows + lane * S::STRIDE, i, act + lane * AW);
+                carry = E::step_begin(rows + lane * S::STRIDE, i, act + lane * AW, shapes);
             }
             detect_sync.target += detect_sync.nwaves;
             detect_sync.wait_for(detect_sync.target);
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(256, 2) void collect16_kernel(CollectArgs a) {
                     a.r_actions[row + lane] = (float)sel;
                 }
                 a.r_logp[row + lane] = logp;
-                carry = E::step_begin(rows + lane * S::STRIDE, i, act + lane * AW);
+                carry = E::step_begin(rows + lane * S::STRIDE, i, act + lane * AW, shapes);
             }
             detect_sync.target += detect_sync.nwaves;
             detect_sync.wait_for(detect_sync.target);

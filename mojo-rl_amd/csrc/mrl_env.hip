@@ -7,6 +7,7 @@
 // detect its contacts where the env splits that off, and the fields that a step can change are
 // copied back with coalesced stores.  HBM sees each row once in and the changed part once out;
 // nothing is re-read.
+#include <cmath>
 #include "mrl_host.hpp"
 #include "env_classic.hpp"
 #include "env_block.hpp"
@@ -339,6 +340,25 @@ int mrl_cartpole_bind_steps(mrl_ctx *ctx, const float *states, int batch, int32_
         ctx->cartpole_steps.erase(it);
     }
     if (steps != nullptr) ctx->cartpole_steps[states] = {steps, batch, false};
+    return MRL_OK;
+}
+
+__global__ void lunar_wind_kernel(float *shapes, float on, float wind_power, float turbulence_power) {
+    if (threadIdx.x == 0) {
+        shapes[mrl::ll::WIND_OFF] = on;
+        shapes[mrl::ll::WIND_OFF + 1] = wind_power;
+        shapes[mrl::ll::WIND_OFF + 2] = turbulence_power;
+    }
+}
+
+int mrl_lunar_set_wind(mrl_ctx *ctx, int enable, double wind_power, double turbulence_power) {
+    MRL_CHECK_ARG(ctx, "mrl_lunar_set_wind: NULL ctx");
+    MRL_CHECK_ARG(std::isfinite(wind_power) && std::isfinite(turbulence_power),
+                  "mrl_lunar_set_wind: powers must be finite");
+    // on the context's stream: steps enqueued before the call keep the old setting, steps after it see the new one
+    hipLaunchKernelGGL(lunar_wind_kernel, dim3(1), dim3(64), 0, ctx->stream, ctx->ll_shapes, enable ? 1.0f : 0.0f,
+                       (float)wind_power, (float)turbulence_power);
+    MRL_CHECK_LAUNCH();
     return MRL_OK;
 }
 

@@ -105,12 +105,19 @@ class PendulumV2(_GPUEnv):            # envs/pendulum/pendulum_v2.mojo:57
 class LunarLanderV2(_GPUEnv):         # envs/lunar_lander/lunar_lander_v2.mojo:123
     ENV_ID, STATE_SIZE, OBS_DIM, NUM_ACTIONS = _lib.ENV_LUNARLANDER, 192, 8, 4
 
+    @staticmethod
+    def set_wind(ctx, enable, wind_power=15.0, turbulence_power=1.5):
+        """The struct parameters ENABLE_WIND / WIND_POWER / TURBULENCE_POWER (lunar_lander_v2.mojo:123-127)
+        as a setting of the context, shared by both action forms, for steps enqueued from now on."""
+        _lib.call("mrl_lunar_set_wind", ctx.handle, int(bool(enable)), float(wind_power), float(turbulence_power))
+
 
 class LunarLanderV2Continuous(_GPUEnv):
     """LunarLanderV2 as a GPUContinuousEnv (the reference overloads step_kernel_gpu on the one
     struct by ACTION_DIM, lunar_lander_v2.mojo:1520-1588; here the overload is a class of its
     own): action[0] main throttle in [-1, 1], action[1] side control in [-1, 1]."""
     ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_LUNARLANDER_CONTINUOUS, 192, 8, 2
+    set_wind = LunarLanderV2.set_wind
 
 
 class BipedalWalkerV2(_GPUEnv):       # envs/bipedal_walker/bipedal_walker_v2.mojo:103

@@ -112,6 +112,8 @@ void orc_ll_shapes(float shapes[3 * 20]);
 uint64_t orc_ll_combined_seed(uint64_t seed, int env);
 void orc_ll_reset(float *row, uint64_t combined_seed);
 /* contacts_out (8*9 floats) and n_contacts_out may be NULL */
+/* wind / turbulence setting of all LunarLander rows stepped from now on (off by default) */
+void orc_ll_set_wind(int enable, double wind_power, double turbulence_power);
 void orc_ll_step(float *row, int env, int action, float *reward, float *done,
                  float *contacts_out, int *n_contacts_out);
 /* the continuous-action overload: a0 = main throttle in [-1, 1], a1 = side control in [-1, 1] */

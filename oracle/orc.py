@@ -74,6 +74,7 @@ def load():
         "orc_ll_shapes": (None, [f32p]),
         "orc_ll_combined_seed": (C.c_uint64, [C.c_uint64, C.c_int]),
         "orc_ll_reset": (None, [f32p, C.c_uint64]),
+        "orc_ll_set_wind": (None, [C.c_int, C.c_double, C.c_double]),
         "orc_ll_step": (None, [f32p, C.c_int, C.c_int, f32p, f32p, C.c_void_p, C.c_void_p]),
         "orc_ll_step_continuous": (None, [f32p, C.c_int, C.c_float, C.c_float, f32p, f32p, C.c_void_p, C.c_void_p]),
         "orc_ll_step_continuous_batch": (None, [f32p, f32p, f32p, f32p, f32p, C.c_int]),

@@ -228,6 +228,34 @@ static void apply_engines(const orc_layout *L, float *row, int env, int step_cou
 static void step_powers(float *row, int env, double m_power, double s_power, double direction, float *reward,
                         float *done, float *contacts_out, int *n_contacts_out);
 
+/* Wind and turbulence, the struct parameters ENABLE_WIND / WIND_POWER / TURBULENCE_POWER of the
+ * reference (lunar_lander_v2.mojo:123-127), off by default: one setting for all rows stepped after
+ * the call.  _apply_wind (CPU, :983-1023): skipped while a leg touches the ground; otherwise
+ * tanh(sin(0.02 t) + sin(pi 0.01 t)) times the power, as an impulse on the lander's vx and omega, in
+ * Float64, before the engines.  The CPU env keeps two running indices that start at random values of
+ * its own generator; the GPU row has no slot for them and the GPU trait uses the step count of the row
+ * for both (:2041-2105): that protocol is followed here, with the CPU's Float64 arithmetic. */
+static int g_wind_on = 0;
+static double g_wind_power = 15.0, g_turbulence_power = 1.5;
+void orc_ll_set_wind(int enable, double wind_power, double turbulence_power) {
+    g_wind_on = enable;
+    g_wind_power = wind_power;
+    g_turbulence_power = turbulence_power;
+}
+static void apply_wind(const orc_layout *L, float *row, int step_count) {
+    if (!g_wind_on) return;
+    if (row[6] > 0.5f || row[7] > 0.5f) return;
+    const double k = 0.01, t = (double)step_count, pi = 3.14159265358979323846;
+    const double wind_mag = tanh(sin(0.02 * t) + sin(pi * k * t)) * g_wind_power;
+    const double torque_mag = tanh(sin(0.02 * t) + sin(pi * k * t)) * g_turbulence_power;
+    float *B = row + L->bodies_off;
+    const double vx = (double)B[ORC_IDX_VX], omega = (double)B[ORC_IDX_OMEGA];
+    const double dvx = wind_mag * DT / LANDER_MASS;
+    const double domega = torque_mag * DT / LANDER_INERTIA;
+    B[ORC_IDX_VX] = (float)(vx + dvx);
+    B[ORC_IDX_OMEGA] = (float)(omega + domega);
+}
+
 void orc_ll_step(float *row, int env, int action, float *reward, float *done, float *contacts_out,
                  int *n_contacts_out) {
     double m_power = 0.0, s_power = 0.0, direction = 0.0;
@@ -268,6 +296,7 @@ static void step_powers(float *row, int env, double m_power, double s_power, dou
 
     int step_count = (int)row[L.meta_off + META_STEP];
 
+    apply_wind(&L, row, step_count);
     apply_engines(&L, row, env, step_count, m_power, s_power, direction);
 
     const float gx = (float)0.0, gy = (float)-10.0, dt = (float)DT;

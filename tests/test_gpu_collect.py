@@ -188,6 +188,72 @@ def test_fused_collection_through_contacts(mrl, ctx, orc, env, kind, N):
     assert cnt == int(fused.done_count.item()) == resets
 
 
+@pytest.mark.parametrize("env,N", [("lunar", 600), ("lunarc", 600), ("lunar", 4128), ("lunarc", 4128)])
+def test_fused_collection_with_wind(mrl, orc, env, N):
+    """Wind and turbulence switched on for the context: the fused kernels (16-row form up to 4096 envs,
+    32-row form above) against the oracle with the same setting, step by step on the kernel's own
+    actions, and the same range as one launch against the single steps, bit for bit.  The rows start
+    at different step counts, which is the time the gusts are a function of."""
+    import numpy as np
+    print("case wind", env, N, flush=True)
+    T = 24
+    ctx = mrl.DeviceContext("cuda:0")           # a context of its own: the setting belongs to the context
+    E = mrl.LunarLanderV2 if env == "lunar" else mrl.LunarLanderV2Continuous
+    cont = env == "lunarc"
+    head = mrl.StochasticActor(256, 2) if cont else mrl.Linear(256, 4)
+    actor = mrl.seq(mrl.LinearTanh(8, 256), mrl.LinearTanh(256, 256), head)
+    critic = mrl.seq(mrl.LinearTanh(8, 256), mrl.LinearTanh(256, 256), mrl.Linear(256, 1))
+    g = torch.Generator(device="cuda").manual_seed(11)
+    ap = (torch.rand(actor.PARAM_SIZE, device="cuda", generator=g) - 0.5) * 0.3
+    cp = (torch.rand(critic.PARAM_SIZE, device="cuda", generator=g) - 0.5) * 0.3
+    s0_h = np.zeros((N, 192), np.float32)
+    orc.orc_ll_reset_batch(s0_h, N, 17)
+    s0_h[:, 188] = (np.arange(N) * 7) % 900
+    rbs = []
+    for _ in range(3):
+        rb = mrl.ppo.RolloutBuffers(ctx, E, actor, critic, N, T)
+        rb.actor_params, rb.critic_params = ap, cp
+        rb.states.copy_(torch.from_numpy(s0_h.reshape(-1)).cuda())
+        rb.obs.copy_(rb.states.view(N, 192)[:, :8].reshape(-1))
+        rbs.append(rb)
+    calm, single, fused = rbs
+    s0, ss, r0, rs = 31337, 2654435761 * N + 7919, 5, 0x9E3779B97F
+    aw = 2 if cont else 1
+    d0 = calm.descriptor()
+    mrl.ppo.rollout_steps(ctx, d0, 0, T, s0, ss & 0xFFFFFFFF, 0, 0, r0, rs)      # before the switch: no wind
+    E.set_wind(ctx, True, 15.0, 1.5)
+    orc.orc_ll_set_wind(1, 15.0, 1.5)
+    try:
+        s_h = s0_h.copy()
+        r_h, d_h, o_h = np.zeros(N, np.float32), np.zeros(N, np.float32), np.zeros((N, 8), np.float32)
+        d1 = single.descriptor()
+        for t in range(T):
+            mrl.ppo.rollout_steps(ctx, d1, t, 1, (s0 + t * ss) & 0xFFFFFFFF, 0, 0, 0, (r0 + t * rs) & (2**64 - 1), 0)
+            ctx.synchronize()
+            acts = single.r_actions[t * N * aw:(t + 1) * N * aw].cpu().numpy()
+            if cont:
+                orc.orc_ll_step_continuous_batch(s_h, np.ascontiguousarray(acts.reshape(N, 2)), r_h, d_h, o_h, N)
+            else:
+                orc.orc_ll_step_batch(s_h, acts, r_h, d_h, o_h, N, 8)
+            np.testing.assert_array_equal(single.r_rewards[t * N:(t + 1) * N].cpu().numpy(), r_h, err_msg="reward, step %d" % t)
+            np.testing.assert_array_equal(single.r_dones[t * N:(t + 1) * N].cpu().numpy(), d_h, err_msg="done, step %d" % t)
+            orc.orc_ll_selective_reset_batch(s_h, d_h, N, (r0 + t * rs) & (2**64 - 1))
+            sg = single.states.cpu().numpy().reshape(N, 192)
+            np.testing.assert_allclose(sg, s_h, rtol=1e-5, atol=1e-6, err_msg="state, step %d" % t)
+            s_h[:] = sg
+        mrl.ppo.rollout_steps(ctx, fused.descriptor(), 0, T, s0, ss & 0xFFFFFFFF, 0, 0, r0, rs)
+        ctx.synchronize()
+    finally:
+        orc.orc_ll_set_wind(0, 15.0, 1.5)
+    for name in ("r_obs", "r_actions", "r_log_probs", "r_values", "r_rewards", "r_dones", "states", "obs"):
+        a, b = getattr(single, name), getattr(fused, name)
+        assert torch.equal(a, b), "%s: fused range differs from single steps in %d places" % (name, int((a != b).sum()))
+    # the gusts moved the landers: against the calm run the horizontal velocities differ on most rows
+    dv = (fused.states.view(N, 192)[:, 11] - calm.states.view(N, 192)[:, 11]).abs()
+    print("  rows whose vx differs from the calm run: %d of %d, largest %.3f" % (int((dv > 1e-3).sum()), N, float(dv.max())), flush=True)
+    assert int((dv > 1e-3).sum()) > N // 2
+
+
 @pytest.mark.parametrize("env,kind,N", [("bipedal", "tanh", 512), ("cheetah", "tanh", 512), ("car", "relu", 300),
                                         ("bipedal", "relu", 45)])
 def test_fused_walker_collection_against_the_oracle(mrl, ctx, orc, env, kind, N):

@@ -286,6 +286,66 @@ def test_lunar_lander_continuous_rollout_parity(mrl, orc, ctx, batch, seed, low)
     assert not low or n_done > 100
 
 
+@pytest.mark.parametrize("cont", [False, True])
+def test_lunar_lander_wind_parity(mrl, orc, cont):
+    """ENABLE_WIND (lunar_lander_v2.mojo:123-127, :983-1023) as a setting of the context: 64 steps of both
+    action forms against the oracle with the same setting, bit for bit; the rows start at different step
+    counts (the gusts are a function of the step count), a quarter of them low enough to touch down,
+    where the wind stops."""
+    batch, seed = 2048, 12
+    say("lunar wind, continuous", cont)
+    own = mrl.DeviceContext("cuda:0")           # the setting belongs to the context: not the shared one
+    E = mrl.LunarLanderV2Continuous if cont else mrl.LunarLanderV2
+    s_h = np.zeros((batch, 192), np.float32)
+    orc.orc_ll_reset_batch(s_h, batch, seed)
+    rng = np.random.default_rng(seed)
+    s_h[:, 188] = rng.integers(0, 900, batch)
+    b = s_h[:, 8:47].reshape(batch, 3, 13)
+    b[::4, :, 1] -= rng.uniform(7.5, 9.4, batch // 4).astype(np.float32)[:, None]
+    s = dev(s_h.reshape(-1))
+    aw = 2 if cont else 1
+    a = torch.zeros(batch * aw, device="cuda")
+    r, d, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch * 8))
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 8), np.float32)
+    E.set_wind(own, True, 15.0, 1.5)
+    orc.orc_ll_set_wind(1, 15.0, 1.5)
+    legs = 0
+    try:
+        for t in range(64):
+            if t == 40:       # other powers from here on
+                E.set_wind(own, True, 7.0, 3.0)
+                orc.orc_ll_set_wind(1, 7.0, 3.0)
+            act = llc_policy(rng, s_h[:, :8]) if cont else ll_policy(rng, s_h[:, :8], t)
+            a.copy_(dev(act.reshape(-1)))
+            E.step_kernel_gpu(own, s, a, r, d, o, t)
+            if cont:
+                orc.orc_ll_step_continuous_batch(s_h, act, r_h, d_h, o_h, batch)
+            else:
+                orc.orc_ll_step_batch(s_h, act, r_h, d_h, o_h, batch, 8)
+            own.synchronize()
+            sg = s.cpu().numpy().reshape(batch, 192)
+            same_bits(sg, s_h, "state, step %d" % t)
+            np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+            np.testing.assert_array_equal(r.cpu().numpy(), r_h)
+            legs += int((o_h[:, 6] + o_h[:, 7] > 0).sum())
+            s_h[:] = sg
+    finally:
+        orc.orc_ll_set_wind(0, 15.0, 1.5)
+    say("  leg-contact observations:", legs)
+    assert legs > 100
+    # switched off again, a step is the calm step
+    E.set_wind(own, False)
+    act = llc_policy(rng, s_h[:, :8]) if cont else ll_policy(rng, s_h[:, :8], 0)
+    a.copy_(dev(act.reshape(-1)))
+    E.step_kernel_gpu(own, s, a, r, d, o, 0)
+    if cont:
+        orc.orc_ll_step_continuous_batch(s_h, act, r_h, d_h, o_h, batch)
+    else:
+        orc.orc_ll_step_batch(s_h, act, r_h, d_h, o_h, batch, 8)
+    own.synchronize()
+    same_bits(s.cpu().numpy().reshape(batch, 192), s_h, "state, calm step")
+
+
 def test_lunar_lander_continuous_corners_equal_discrete_actions(mrl, ctx):
     batch = 512
     D, Cn = mrl.LunarLanderV2, mrl.LunarLanderV2Continuous

@@ -351,3 +351,80 @@ def test_engine_impulses_to_1e6_on_a_free_tilted_lander(orc):
         np.testing.assert_allclose(row[BOD:BOD + 2], x0[:2] + want_v * 0.02, rtol=0, atol=2e-6)
         np.testing.assert_allclose(row[BOD + 2], x0[2] + want_w * 0.02, rtol=0, atol=1e-6)
         assert np.abs(dv).max() > 0.03                 # the effect is 4 orders above the tolerance
+
+
+def _twin_step(orc, row, wind, power=15.0, turbulence=1.5, cont=False):
+    """One no-op step of a copy of `row` with the wind setting on or off."""
+    twin = row.copy()
+    orc.orc_ll_set_wind(1 if wind else 0, power, turbulence)
+    try:
+        if cont:
+            step_c(orc, twin, -1.0, 0.0)
+        else:
+            step(orc, twin, 0)
+    finally:
+        orc.orc_ll_set_wind(0, 15.0, 1.5)
+    return twin
+
+
+def _momenta(row, about):
+    """Linear momentum in x of lander + legs, and their angular momentum about the point `about`."""
+    b = row[BOD:BOD + 39].reshape(3, 13).astype(np.float64)
+    m, inertia = 1.0 / b[:, 10], 1.0 / b[:, 11]
+    x, y = b[:, 0] - about[0], b[:, 1] - about[1]
+    return (m * b[:, 3]).sum(), (inertia * b[:, 5] + m * (x * b[:, 4] - y * b[:, 3])).sum()
+
+
+def _gust(t, power):
+    return math.tanh(math.sin(0.02 * t) + math.sin(math.pi * 0.01 * t)) * power
+
+
+def test_wind_is_an_impulse_on_the_lander_in_free_flight(orc):
+    """_apply_wind (lunar_lander_v2.mojo:983-1023): force tanh(sin(0.02 t) + sin(pi 0.01 t)) * WIND_POWER on
+    the lander for one DT, torque with TURBULENCE_POWER likewise, t = the row's step count.  The joints
+    pass momentum between lander and legs but create none, so the system's momenta show the impulses:
+    p_x gains F DT, the angular momentum about a fixed point P gains tau DT - (y_lander - y_P) F DT
+    (P = where the centre of mass was before the step, which keeps the terms small in fp32)."""
+    for cont in (False, True):
+        for t0 in (0, 40, 130, 333):
+            row = fresh(orc, 9)
+            for _ in range(20):     # the legs are reset a third of a unit below their joints: let them swing in
+                step(orc, row, 0)
+            row[META] = t0
+            b = row[BOD:BOD + 39].reshape(3, 13).astype(np.float64)
+            m = 1.0 / b[:, 10]
+            P = ((m * b[:, 0]).sum() / m.sum(), (m * b[:, 1]).sum() / m.sum())
+            y = float(row[BOD + 1]) - P[1]
+            assert 0.01 < y < 0.1       # the legs hang below the lander
+            calm, windy = _twin_step(orc, row, False, cont=cont), _twin_step(orc, row, True, cont=cont)
+            (p0, l0), (p1, l1) = _momenta(calm, P), _momenta(windy, P)
+            f, tau = _gust(t0, 15.0), _gust(t0, 1.5)
+            if t0 == 0:     # sin(0) + sin(0): no gust at the first step of an episode
+                np.testing.assert_array_equal(calm, windy)
+                continue
+            assert abs(f) > 4.0
+            np.testing.assert_allclose(p1 - p0, f * 0.02, rtol=2e-3)
+            np.testing.assert_allclose(l1 - l0, tau * 0.02 - y * f * 0.02, rtol=1e-2)
+            # turbulence alone: only the spin changes; wind alone: the spin of the system about its own
+            # centre of mass stays (the force acts at the lander's centre, the legs hang symmetrically)
+            spin = _twin_step(orc, row, True, power=0.0, turbulence=1.5, cont=cont)
+            ps, ls = _momenta(spin, P)
+            np.testing.assert_allclose(ps, p0, atol=1e-5)
+            np.testing.assert_allclose(ls - l0, tau * 0.02, rtol=1e-2)
+            # a stronger wind, same time: the impulse scales with the power
+            strong = _twin_step(orc, row, True, power=30.0, turbulence=0.0, cont=cont)
+            np.testing.assert_allclose(_momenta(strong, P)[0] - p0, 2 * f * 0.02, rtol=2e-3)
+
+
+def test_wind_stops_with_a_leg_on_the_ground_and_is_off_by_default(orc):
+    row = fresh(orc, 9)
+    row[META] = 40
+    calm = _twin_step(orc, row, False)
+    never_set = row.copy()
+    step(orc, never_set, 0)
+    np.testing.assert_array_equal(calm, never_set)
+    for leg in (6, 7):      # the contact flags of the previous observation gate the wind
+        grounded = row.copy()
+        grounded[leg] = 1.0
+        np.testing.assert_array_equal(_twin_step(orc, grounded, True), _twin_step(orc, grounded, False))
+    assert not np.array_equal(_twin_step(orc, row, True), calm)
