@@ -12,8 +12,9 @@
 //                        env per lane), reward / done of rollout row t, episode accounting,
 //                        in-place reset;
 //     wavefronts 1 .. 7  contact detection for that env step;
-//     wavefronts 5 .. 7  then the critic  OBS -> H -> H -> 1  (its value is only stored, so it does
-//                        not hold up the env step; these wavefronts meet at a barrier of their own);
+//     all of these but   then the critic  OBS -> H -> H -> 1  (its value is only stored, so it does
+//     wavefront 4        not hold up the env step; the six wavefronts meet at a barrier of their own,
+//                        and wavefront 4, which shares wavefront 0's SIMD, stays out of its way);
 //   rollout row t of obs, action, log-prob and value written on the way.
 // No workgroup waits for another, so there is nothing between two steps but the block's own
 // barriers; the launch ends when every block has done its n_steps.
@@ -40,12 +41,9 @@ template <class E, int H, int ACT, bool GAUSS>
 __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     using S = Stage<E>;
     constexpr int IN = E::OBS, AW = E::ACT_W, NW = E::THREADS / WAVE;
-    // the critic's wavefronts: the last three, so that none of them shares a SIMD with wavefront 0
-    // (wavefronts of a workgroup go round the four SIMDs) and its solver keeps that SIMD's issue
-    // slots to itself
     // the critic runs on the six wavefronts that do not share a SIMD with wavefront 0 (1, 2, 3, 5, 6,
-    // 7: two per SIMD, so that one's MFMAs cover the other's loads and epilogues); its eight column
-    // tiles are dealt out 3 / 3 / 2 per SIMD
+    // 7: two per SIMD, so that one's MFMAs cover the other's loads and epilogues; wavefront 0's solver
+    // keeps its SIMD's issue slots to itself); its eight column tiles are dealt out 3 / 3 / 2 per SIMD
     constexpr int CRITIC_TPW = 2, CRITIC_WAVES = 6, CRITIC_T = CRITIC_WAVES * WAVE;
     static_assert(E::EPB == PR && E::THREADS == 2 * H && NW == 8 && H == 256, "one 32-row policy tile per block");
     static_assert(IN <= PIN_MAX && AW <= PA_MAX && E::DETECT_TASKS > 0, "policy tile limits; split-off detection");
