@@ -15,6 +15,13 @@ SOURCES = ["mrl_core.hip", "mrl_env.hip", "mrl_mlp.hip", "mrl_mlp3.hip", "mrl_pp
 # code generation off.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value"]
+# The collection kernels run a long env step inside a loop over the rollout steps.  The machine-level
+# loop-invariant code motion lifts the double-precision constants of that step (the polynomial
+# coefficients of exp / log / sincos, two registers each) out of the loop into registers of their own,
+# the register allocator then spills them, and every use becomes a dependent load from private memory in
+# the middle of the solver wavefront's chain.  Without that pass these kernels need no private memory.
+EXTRA_FLAGS = {"mrl_collect.hip": ["-mllvm", "-disable-machine-licm"],
+               "mrl_collect_walkers.hip": ["-mllvm", "-disable-machine-licm"]}
 
 
 def _run(cmd, verbose):
@@ -41,7 +48,7 @@ def build(verbose=False, incremental=False, jobs=8):
         objs.append(obj)
         fresh = os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), newest_header)
         if not (incremental and fresh):
-            todo.append(["hipcc"] + FLAGS + ["-c", src, "-o", obj])
+            todo.append(["hipcc"] + FLAGS + EXTRA_FLAGS.get(s, []) + ["-c", src, "-o", obj])
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(lambda c: _run(c, verbose), todo))
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs, verbose)

@@ -142,7 +142,7 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
                     }
                 } else {
                     int sel;
-                    sample_categorical(logits + lane * (PA_MAX + 1), A, sseed, i, sel, logp);
+                    sample_categorical_few(logits + lane * (PA_MAX + 1), A, sseed, i, sel, logp);
                     act[lane] = (float)sel;
                     a.r_actions[row + lane] = (float)sel;
                 }
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(256, 2) void collect16_kernel(CollectArgs a) {
                     }
                 } else {
                     int sel;
-                    sample_categorical(logits + lane * (PA_MAX + 1), A, sseed, i, sel, logp);
+                    sample_categorical_few(logits + lane * (PA_MAX + 1), A, sseed, i, sel, logp);
                     act[lane] = (float)sel;
                     a.r_actions[row + lane] = (float)sel;
                 }
@@ -512,7 +512,7 @@ __global__ __launch_bounds__(CLASSIC_THREADS) void collect_classic_kernel(Collec
                 for (int j = 0; j < A; ++j) a.r_actions[(row + tid) * AW + j] = av[j];
             } else {
                 int sel;
-                sample_categorical(logits + tid * (PA_MAX + 1), A, sseed, i, sel, logp);
+                sample_categorical_few(logits + tid * (PA_MAX + 1), A, sseed, i, sel, logp);
                 av[0] = (float)sel;
                 a.r_actions[row + tid] = av[0];
             }

@@ -23,6 +23,8 @@
 
 namespace mrl {
 
+static_assert(SAMPLE_A_MAX == PA_MAX, "the sampler's action limit is the policy tile's");
+
 template <int H, int ACT, bool GAUSS, int TPW>
 __global__ __launch_bounds__(TPW == 1 ? 2 * H : 4 * H / TPW) void policy_kernel(
     const float *__restrict__ obs, int n, int IN, int A, const float *__restrict__ actor_p,
@@ -78,7 +80,7 @@ __global__ __launch_bounds__(TPW == 1 ? 2 * H : 4 * H / TPW) void policy_kernel(
         const int i = row0 + t;
         int sel;
         float logp;
-        sample_categorical(logits + t * (PA_MAX + 1), A, seed, i, sel, logp);
+        sample_categorical_few(logits + t * (PA_MAX + 1), A, seed, i, sel, logp);
         actions[i] = (float)sel;
         r_actions[i] = (float)sel;
         r_logp[i] = logp;

@@ -42,7 +42,8 @@ __global__ __launch_bounds__(TPB) void sample_categorical_kernel(const float *__
     if (i >= n) return;
     int sel;
     float logp;
-    sample_categorical(logits + (long)i * A, A, seed, i, sel, logp);
+    if (A <= SAMPLE_A_MAX) sample_categorical_few(logits + (long)i * A, A, seed, i, sel, logp);
+    else sample_categorical(logits + (long)i * A, A, seed, i, sel, logp);
     actions[i] = (float)sel;
     log_probs[i] = logp;
 }

@@ -26,6 +26,45 @@ MRL_DEV void sample_categorical(const float *l, int A, uint32_t seed, int i, int
     logp = log32(pr + 1e-8f);
 }
 
+// The same draw for at most SAMPLE_A_MAX actions (the fused kernels' policy heads), bit for bit.
+constexpr int SAMPLE_A_MAX = 8;
+MRL_DEV void sample_categorical_few(const float *l, int A, uint32_t seed, int i, int &sel, float &logp) {
+    uint32_t rng = seed ^ ((uint32_t)i * 2654435761u);
+    rng = xorshift32(rng);
+    float max_logit = l[0];
+    for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
+    // every exponential is taken once and kept (the reference recomputes them for the probabilities and for
+    // the drawn action: the same values); all slots are walked so that the array stays in registers
+    float e[SAMPLE_A_MAX];
+    float sum_exp = 0.0f;
+#pragma unroll
+    for (int a = 0; a < SAMPLE_A_MAX; ++a) {
+        e[a] = 0.0f;
+        if (a < A) {
+            e[a] = exp32(l[a] - max_logit);
+            sum_exp = sum_exp + e[a];
+        }
+    }
+    const float u = random_uniform(rng);
+    float cumsum = 0.0f, e_sel = e[0];
+    bool found = false;
+    sel = 0;
+#pragma unroll
+    for (int a = 0; a < SAMPLE_A_MAX; ++a) {
+        if (a < A) {
+            const float prob = e[a] / sum_exp;
+            cumsum = cumsum + prob;
+            if (!found && u < cumsum) {
+                sel = a;
+                e_sel = e[a];
+                found = true;
+            }
+        }
+    }
+    const float pr = e_sel / sum_exp;
+    logp = log32(pr + 1e-8f);
+}
+
 // Gaussian sampling (deep_agents/ppo/kernels.mojo:12-98) of components j0 .. j0 + m of an action
 // with A components: one Philox stream per (env, component), Box-Muller, clamped log_std;
 // returns the summed log-probability of those components and leaves them in act[0 .. m).
