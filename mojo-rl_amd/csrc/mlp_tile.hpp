@@ -137,12 +137,7 @@ struct WaveGroupSync {
 
 // NT = the column tiles this wavefront really has (ops.ntile, known at compile time here): the
 // MFMAs, weight loads and epilogues of the other TPW - NT slots are left out.
-// SEQ: layer 1 walks the wavefront's column tiles one after the other instead of side by side, as one
-// run of NT * H / 2 k-steps whose operands sit in a ring of KB registers each: the operands of k-step
-// s + KB are requested right after the MFMA of k-step s has read its own, so the loads stay KB MFMAs
-// ahead with half the registers of the block form, across the change of tile as well.  Every accumulator
-// still takes its k products in ascending order: the bits are those of the side-by-side form.
-template <int H, int ACT, int TPW, int KB, bool H2_ON_HT, int NT, bool SEQ, class Sync>
+template <int H, int ACT, int TPW, int KB, bool H2_ON_HT, int NT, class Sync>
 MRL_DEV void hidden_stack_tiles(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
                                 const TileCache tc, HiddenOperands<H, TPW, KB> &ops, int tid, Sync &sync) {
     static_assert(PR * (H + 1) <= H * HT_LD, "h2 fits into hT");
@@ -192,27 +187,6 @@ MRL_DEV void hidden_stack_tiles(const float *__restrict__ p, int IN, const float
         floatx16 c[TPW];
 #pragma unroll
         for (int q = 0; q < NT; ++q) c[q] = floatx16{0};
-        if constexpr (SEQ && NT > 0) {
-            constexpr int S = H / 2;   // k-steps per tile
-            static_assert(S % KB == 0, "the ring divides a tile's k-steps");
-            float a[KB], b[KB];
-#pragma unroll
-            for (int j = 0; j < KB; ++j) {
-                a[j] = hT[(2 * j + half) * HT_LD + l31];
-                b[j] = bv[0][j];
-            }
-#pragma unroll
-            for (int st = 0; st < NT * S; ++st) {
-                const int q = st / S, j = st % KB;
-                c[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[j], c[q], 0, 0, 0);
-                if (st + KB < NT * S) {
-                    const int q2 = (st + KB) / S, k = 2 * ((st + KB) % S) + half;
-                    a[j] = hT[k * HT_LD + l31];
-                    b[j] = W1[k * H + col[q2]];
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        } else {
         float a[KB], na[KB], nb[TPW][KB];
 #pragma unroll
         for (int j = 0; j < KB; ++j) a[j] = hT[(2 * j + half) * HT_LD + l31];
@@ -245,7 +219,6 @@ MRL_DEV void hidden_stack_tiles(const float *__restrict__ p, int IN, const float
                 }
             }
         }
-        }
         if (H2_ON_HT) sync();
 #pragma unroll
         for (int q = 0; q < NT; ++q) {
@@ -265,20 +238,20 @@ MRL_DEV void hidden_stack_tiles(const float *__restrict__ p, int IN, const float
     sync();
 }
 
-template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32), bool H2_ON_HT = false, bool SEQ = false, class Sync = BlockSync>
+template <int H, int ACT, int TPW = 2, int KB = (TPW == 2 ? 8 : 32), bool H2_ON_HT = false, class Sync = BlockSync>
 MRL_DEV void hidden_stack(const float *__restrict__ p, int IN, const float *xs, float *hT, float *h2,
                           const TileCache tc, HiddenOperands<H, TPW, KB> &ops, int tid = threadIdx.x,
                           Sync &&sync = Sync()) {
     // ops.ntile is the same for all lanes of a wavefront; a wavefront with fewer tiles than slots
     // runs the variant without the spare slots' work (every variant meets the same barriers)
-    if (ops.ntile >= TPW) return hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, TPW, SEQ>(p, IN, xs, hT, h2, tc, ops, tid, sync);
+    if (ops.ntile >= TPW) return hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, TPW>(p, IN, xs, hT, h2, tc, ops, tid, sync);
     if constexpr (TPW >= 3) {
-        if (ops.ntile == 2) return hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, 2, SEQ>(p, IN, xs, hT, h2, tc, ops, tid, sync);
+        if (ops.ntile == 2) return hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, 2>(p, IN, xs, hT, h2, tc, ops, tid, sync);
     }
     if constexpr (TPW >= 2) {
-        if (ops.ntile == 1) return hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, 1, SEQ>(p, IN, xs, hT, h2, tc, ops, tid, sync);
+        if (ops.ntile == 1) return hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, 1>(p, IN, xs, hT, h2, tc, ops, tid, sync);
     }
-    hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, 0, SEQ>(p, IN, xs, hT, h2, tc, ops, tid, sync);
+    hidden_stack_tiles<H, ACT, TPW, KB, H2_ON_HT, 0>(p, IN, xs, hT, h2, tc, ops, tid, sync);
 }
 
 // floats of LDS that hold one net's head parameters, every row padded to PA_MAX columns with
