@@ -302,14 +302,32 @@ MRL_DEV void detect_vertex_task(const float *rows, const float *shapes, float *d
 // returns the contact count, or -1 when some list asks for detection to be redone
 template <class E, int CAP = DETECT_CAP>
 MRL_DEV int merge_vertex_lists(const float *dlist, const int *dcount, int e, float *mine) {
-    int n = 0;
-    bool redo = false;
+    // all counts first (independent loads, one round trip), then only the lists that hold something:
+    // most steps of most envs have no contact at all
+    int m[E::DETECT_TASKS];
+#pragma unroll
+    for (int k = 0; k < E::DETECT_TASKS; ++k) m[k] = dcount[k * E::EPB + e];
+    bool redo = false, any = false;
+#pragma unroll
     for (int k = 0; k < E::DETECT_TASKS; ++k) {
-        const float *src = dlist + (k * E::EPB + e) * detect_stride(CAP);
-        const int m = dcount[k * E::EPB + e];
-        redo |= m < 0;
-        for (int c = 0; c < m && c < CAP && n < E::L::MAX_CONTACTS; ++c, ++n)
-            for (int f = 0; f < CONTACT_SIZE; ++f) mine[n * CONTACT_SIZE + f] = src[c * CONTACT_SIZE + f];
+        redo |= m[k] < 0;
+        any |= m[k] > 0;
+    }
+    int n = 0;
+    if (any) {
+#pragma unroll
+        for (int k = 0; k < E::DETECT_TASKS; ++k) {
+            const float *src = dlist + (k * E::EPB + e) * detect_stride(CAP);
+            for (int c = 0; c < m[k] && c < CAP && n < E::L::MAX_CONTACTS; ++c, ++n) {
+                // a record is read whole before it is written (the two LDS ranges never overlap, which the
+                // compiler cannot see: it would wait for every float on its own)
+                float rec[CONTACT_SIZE];
+#pragma unroll
+                for (int f = 0; f < CONTACT_SIZE; ++f) rec[f] = src[c * CONTACT_SIZE + f];
+#pragma unroll
+                for (int f = 0; f < CONTACT_SIZE; ++f) mine[n * CONTACT_SIZE + f] = rec[f];
+            }
+        }
     }
     return redo ? -1 : n;
 }

@@ -387,9 +387,13 @@ MRL_DEV void step_finish(float *row, float *contacts, int n_given, const float *
     if (obs[0] >= 1.0f || obs[0] <= -1.0f) { terminated = true; r = -100.0f; }
     bool both_legs = obs[6] > 0.5f && obs[7] > 0.5f;
     double speed = ::sqrt(vx * vx + vy * vy);
+    // every slot is read (one round trip to the lane's scratch for all of them), the count cuts afterwards
     bool lander_contact = false;
-    for (int k = 0; k < n; ++k)
-        if ((int)contacts[k * CONTACT_SIZE + C_BODY_A] == 0) lander_contact = true;
+#pragma unroll
+    for (int k = 0; k < L::MAX_CONTACTS; ++k) {
+        const int body = (int)contacts[k * CONTACT_SIZE + C_BODY_A];
+        lander_contact = lander_contact || (k < n && body == 0);
+    }
     if (lander_contact) { terminated = true; r = -100.0f; }
     if (speed < 0.01 && ::fabs(omega) < 0.01 && both_legs) { terminated = true; r = r + 100.0f; }
     if (step_count >= 1000) terminated = true;

@@ -152,6 +152,8 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
             detect_sync.target += detect_sync.nwaves;
             detect_sync.wait_for(detect_sync.target);
             bool finished = false;
+            int slot = 0;
+            float fin_return = 0.0f, fin_length = 0.0f;
             if (lane < ne) {
                 float *mine = cts + lane * S::CSTRIDE;
                 const int n = merge_vertex_lists<E>(dlist, dcount, lane, mine);
@@ -165,16 +167,19 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
                 ep_length = ep_length + 1.0f;
                 finished = d > 0.5f;
                 if (finished) {
-                    const int slot = atomicAdd(a.acc.done_count, 1);
-                    if (slot < a.acc.done_cap) {
-                        a.acc.done_returns[slot] = ep_return;
-                        a.acc.done_lengths[slot] = ep_length;
-                    }
+                    // the slot in the finished-episode list comes back from L2 while the row is rebuilt
+                    slot = atomicAdd(a.acc.done_count, 1);
+                    fin_return = ep_return;
+                    fin_length = ep_length;
                     ep_return = 0.0f;
                     ep_length = 0.0f;
                 }
             }
             reset_rows<E>(rows, &was_reset, __ballot(finished), a.reset_seed + (uint64_t)k * a.reset_stride, env0, lane);
+            if (finished && slot < a.acc.done_cap) {
+                a.acc.done_returns[slot] = fin_return;
+                a.acc.done_lengths[slot] = fin_length;
+            }
         } else {
             // ---- contact detection: one (body, vertex) task per half of wavefronts 1 .. 7
             const int task = (wave - 1) * 2 + lane / (WAVE / 2), e = lane % (WAVE / 2);
