@@ -11,17 +11,44 @@ MRL_DEV float actor_grad_discrete_row(const float *l, int action, float advantag
                                       float clip_eps, float ent_coef, float *g_row) {
     float max_logit = l[0];
     for (int a = 1; a < A; ++a) if (l[a] > max_logit) max_logit = l[a];
+    // every exponential once (the reference takes exp(l[a] - max) again for the probabilities and for the
+    // gradient: the same values); heads wider than the array fall back to recomputing
+    constexpr int KEEP = 8;
+    float e[KEEP];
     float sum_exp = 0.0f;
-    for (int a = 0; a < A; ++a) sum_exp = sum_exp + exp32(l[a] - max_logit);
-    float p_action = 0.0f;
-    for (int a = 0; a < A; ++a) {
-        float p = exp32(l[a] - max_logit) / sum_exp;
-        if (a == action) p_action = p;
+#pragma unroll
+    for (int a = 0; a < KEEP; ++a) {
+        e[a] = 0.0f;
+        if (a < A) {
+            e[a] = exp32(l[a] - max_logit);
+            sum_exp = sum_exp + e[a];
+        }
     }
+    for (int a = KEEP; a < A; ++a) sum_exp = sum_exp + exp32(l[a] - max_logit);
+    float p_action = 0.0f;
+#pragma unroll
+    for (int a = 0; a < KEEP; ++a)
+        if (a < A && a == action) p_action = e[a] / sum_exp;
+    for (int a = KEEP; a < A; ++a)
+        if (a == action) p_action = exp32(l[a] - max_logit) / sum_exp;
     float new_logp = log32(p_action + 1e-8f);
     float ratio = exp32(new_logp - old);
     bool clipped = (ratio < 1.0f - clip_eps) || (ratio > 1.0f + clip_eps);
-    for (int a = 0; a < A; ++a) {
+#pragma unroll
+    for (int a = 0; a < KEEP; ++a) {
+        if (a < A) {
+            float g = 0.0f;
+            if (!clipped) {
+                float p = e[a] / sum_exp;
+                float d_log_prob = (a == action) ? 1.0f - p : -p;
+                float log_prob_ent = log32(p + 1e-8f);
+                float d_entropy = -p * (1.0f + log_prob_ent);
+                g = (-advantage * ratio * d_log_prob - ent_coef * d_entropy) / (float)mb;
+            }
+            g_row[a] = g;
+        }
+    }
+    for (int a = KEEP; a < A; ++a) {
         float g = 0.0f;
         if (!clipped) {
             float p = exp32(l[a] - max_logit) / sum_exp;
@@ -47,11 +74,25 @@ MRL_DEV float actor_grad_discrete_one(int b, const float *__restrict__ logits, c
 MRL_DEV float actor_grad_gaussian_row(const float *o, const float *act, float advantage, float old_log_prob,
                                       int mb, int A, float clip_eps, float ent_coef, float *g) {
     const float eps = 1e-6f, log_2pi = (float)1.8378770664093453;
+    // exp(log_std) of the first KEEP components is taken once (the reference takes it again for the
+    // gradient: the same value); wider actions recompute the rest
+    constexpr int KEEP = 8;
+    float stdv[KEEP];
     float new_log_prob = 0.0f;
-    for (int j = 0; j < A; ++j) {
-        float log_std = o[A + j];
-        if (log_std < -5.0f) log_std = -5.0f;
-        else if (log_std > 2.0f) log_std = 2.0f;
+    auto clamped = [](float log_std) { return log_std < -5.0f ? -5.0f : (log_std > 2.0f ? 2.0f : log_std); };
+#pragma unroll
+    for (int j = 0; j < KEEP; ++j) {
+        stdv[j] = 1.0f;
+        if (j < A) {
+            const float log_std = clamped(o[A + j]);
+            stdv[j] = exp32(log_std);
+            float an = (act[j] - o[j]) / (stdv[j] + eps);
+            float lg = -0.5f * (log_2pi + 2.0f * log_std + an * an);
+            new_log_prob = new_log_prob + lg;
+        }
+    }
+    for (int j = KEEP; j < A; ++j) {
+        const float log_std = clamped(o[A + j]);
         float std = exp32(log_std);
         float an = (act[j] - o[j]) / (std + eps);
         float lg = -0.5f * (log_2pi + 2.0f * log_std + an * an);
@@ -68,13 +109,9 @@ MRL_DEV float actor_grad_gaussian_row(const float *o, const float *act, float ad
     if (clipped_ratio < 1.0f - clip_eps) clipped_ratio = 1.0f - clip_eps;
     else if (clipped_ratio > 1.0f + clip_eps) clipped_ratio = 1.0f + clip_eps;
     bool is_clipped = clipped_ratio * advantage < ratio * advantage;
-    for (int j = 0; j < A; ++j) {
+    auto grads = [&](int j, float std) {
         float gm = 0.0f, gs = 0.0f;
         if (!is_clipped) {
-            float log_std = o[A + j];
-            if (log_std < -5.0f) log_std = -5.0f;
-            else if (log_std > 2.0f) log_std = 2.0f;
-            float std = exp32(log_std);
             float an = (act[j] - o[j]) / (std + eps);
             float d_mean = an / (std + eps);
             float d_log_std = an * an - 1.0f;
@@ -87,7 +124,11 @@ MRL_DEV float actor_grad_gaussian_row(const float *o, const float *act, float ad
         }
         g[j] = gm;
         g[A + j] = gs;
-    }
+    };
+#pragma unroll
+    for (int j = 0; j < KEEP; ++j)
+        if (j < A) grads(j, stdv[j]);
+    for (int j = KEEP; j < A; ++j) grads(j, is_clipped ? 1.0f : exp32(clamped(o[A + j])));
     return kl;
 }
 MRL_DEV float actor_grad_gaussian_one(int b, const float *__restrict__ actor_out, const float *__restrict__ old_logp,
