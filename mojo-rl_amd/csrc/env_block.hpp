@@ -5,6 +5,7 @@
 #include "mrl_host.hpp"
 #include "env_lunar.hpp"
 #include "env_walkers.hpp"
+#include "env_bipedal_lanes.hpp"
 
 namespace mrl {
 
@@ -67,6 +68,7 @@ struct LunarLander {
         else if (k < 10) { body = 1; vertex = k - 6; max_verts = 4; }
         else { body = 2; vertex = k - 10; max_verts = 4; }
     }
+    static constexpr bool LANES_PHYSICS = false;   // (BipedalWalker: the physics by one lane per body)
     using Carry = ll::StepCarry;
     static MRL_DEV Carry step_begin(float *row, int env, const float *a, const float *shapes) {
         return ll::step_begin(row, env, (int)a[0], shapes);
@@ -133,6 +135,15 @@ struct BipedalWalker {
                                     float &d) {
         bw::step_finish<false>(row, cts, n, shapes, c.act, r, d);
     }
+    // step_finish in two parts: the physics by the eight lanes of an env's group (env_bipedal_lanes.hpp),
+    // then the rest by the env's lane
+    static constexpr bool LANES_PHYSICS = true;
+    static constexpr int LANES_PER_ENV = bw::LANES_PER_ENV;
+    static MRL_DEV bool lanes_ok(const float *row) { return bw::lanes_row_ok(row); }
+    static MRL_DEV void physics_lanes(float *row, float *cts, int n, int lane) { bw::physics_lanes(row, cts, n, lane); }
+    static MRL_DEV void step_tail(float *row, const float *cts, int n, const Carry &c, float &r, float &d) {
+        bw::step_tail<false>(row, cts, n, c.act, r, d);
+    }
 };
 
 struct HalfCheetah {
@@ -143,6 +154,7 @@ struct HalfCheetah {
                              float &r, float &d) {
         hc::step_row(row, cts, shapes, env, a, r, d);
     }
+    static constexpr bool LANES_PHYSICS = false;
     static constexpr int POST_TASKS = 0;
     static MRL_DEV void post_task(float *, int) {}
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { hc::reset_row(row, walker_seed(seed, env)); }
@@ -395,13 +407,36 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
                     detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
             __syncthreads();
         }
+        int lanes_n = 0;          // LANES_PHYSICS: the env's contact count; -1: the one-lane form steps this env
+        if constexpr (E::LANES_PHYSICS) {
+            // the physics of the step by one lane per body: the env's lane merges the contact lists, then
+            // LANES_PER_ENV lanes per env (the first wavefronts of the block) run the solver, then the env's
+            // lane goes on below with what follows the physics
+            static_assert(E::DETECT_TASKS > 0 && E::EPB * E::LANES_PER_ENV <= E::THREADS, "a lane group per env");
+            if (tid < nenv) {
+                const int n = merge_vertex_lists<E>(dlist, dcount, tid, cts + tid * S::CSTRIDE);
+                dcount[tid] = (n >= 0 && E::lanes_ok(rows + tid * S::STRIDE)) ? n : -1;   // (the counts are spent)
+            }
+            __syncthreads();
+            const int slot = tid / E::LANES_PER_ENV;
+            if (slot < nenv) {
+                const int n = dcount[slot];
+                if (n >= 0) E::physics_lanes(rows + slot * S::STRIDE, cts + slot * S::CSTRIDE, n, tid % WAVE);
+            }
+            __syncthreads();
+            if (tid < nenv) lanes_n = dcount[tid];
+        }
         if (tid < WAVE) {
             bool finished = false;
             if (tid < nenv) {
                 const int env = env0 + tid;
                 const EpisodeSums sums = account_before(acc, tid);
                 float r, d;
-                if constexpr (E::DETECT_TASKS > 0) {
+                if constexpr (E::LANES_PHYSICS) {
+                    float *mine = cts + tid * S::CSTRIDE;
+                    if (lanes_n >= 0) E::step_tail(rows + tid * S::STRIDE, mine, lanes_n, carry, r, d);
+                    else E::step_finish(rows + tid * S::STRIDE, mine, -1, shapes, carry, r, d);
+                } else if constexpr (E::DETECT_TASKS > 0) {
                     float *mine = cts + tid * S::CSTRIDE;
                     const int n = merge_vertex_lists<E>(dlist, dcount, tid, mine);
                     E::step_finish(rows + tid * S::STRIDE, mine, n, shapes, carry, r, d);

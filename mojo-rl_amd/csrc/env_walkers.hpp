@@ -317,11 +317,21 @@ MRL_DEV void step_motors(float *row, const float *action, float *act) {
     }
 }
 
+// what follows the physics of a step: contact flags, observation, reward, termination; `n` = the
+// contacts of the step, whose body indices are still in `contacts`
+template <bool LIDAR = true>
+MRL_DEV void step_tail(float *row, const float *contacts, int n, const float *act, float &reward, float &done);
+
 template <bool LIDAR = true>
 MRL_DEV void step_finish(float *row, float *contacts, int n_given, const float *shapes, const float *act,
                          float &reward, float &done) {
     int n = reg_physics_substep<L, Topology, false, false>(row, shapes, contacts, (float)0.0, (float)-10.0, (float)(1.0 / FPS),
                                       (float)2.5, (float)0.0, (float)0.2, (float)0.005, 6, 2, n_given);
+    step_tail<LIDAR>(row, contacts, n, act, reward, done);
+}
+
+template <bool LIDAR>
+MRL_DEV void step_tail(float *row, const float *contacts, int n, const float *act, float &reward, float &done) {
     bool left = false, right = false, hull = false;
     for (int c = 0; c < n; ++c) {
         int b = (int)contacts[c * CONTACT_SIZE + C_BODY_A];

@@ -7,7 +7,7 @@
 //            mlp_tile16.hpp, 64 columns per wavefront, weights streamed from L2), heads out of LDS;
 //   sample   one lane per (env, action component): every component has a Philox stream of its own;
 //   env step BipedalWalker: the workgroup-level step of env_block.hpp (contact detection on every
-//            wavefront, solver on wavefront 0, lidar rays on every wavefront, wave-cooperative
+//            wavefront, solver with one lane per body on wavefronts 0 and 1, lidar rays on every wavefront, wave-cooperative
 //            resets); HalfCheetah: one lane per body on wavefronts 0 and 1 (env_cheetah_lanes.hpp);
 //            CarRacing: a wavefront per env, two rounds of eight (env_car.hpp); the tile tables stay in
 //            global memory and are staged through LDS every step (16 x 12 KB do not fit beside the rest);

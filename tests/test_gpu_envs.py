@@ -510,6 +510,43 @@ def test_half_cheetah_rows_with_other_wiring_take_the_one_lane_form(mrl, orc, ct
     assert np.median(gap[::2]) > 0.09 and gap[1::2].max() < 0.08
 
 
+def test_bipedal_walker_rows_with_other_wiring_take_the_one_lane_form(mrl, orc, ctx):
+    """The walker's solver runs with one lane per body for rows that have the walker's own four joints; a
+    row with another joint table (here: the last joint missing, so that lower leg 2 hangs loose) is stepped
+    by the one-lane form.  Both kinds of rows sit side by side in one workgroup and must match the oracle."""
+    batch = 100
+    E = mrl.BipedalWalkerV2
+    s_h = np.zeros((batch, 950), np.float32)
+    orc.orc_bw_reset_batch(s_h, None, batch, 9)
+    JOINT_COUNT = 24 + 65 + 15 + 68
+    assert (s_h[:, JOINT_COUNT] == 4.0).all()
+    s_h[::2, JOINT_COUNT] = 3.0
+    s = dev(s_h.reshape(-1))
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch * 4, batch, batch, batch * 24))
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 24), np.float32)
+    rng = np.random.default_rng(9)
+    for t in range(40):
+        act = rng.uniform(-1.2, 1.2, (batch, 4)).astype(np.float32)
+        a.copy_(dev(act.reshape(-1)))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_bw_step_batch(s_h, act, r_h, d_h, o_h, batch, 4)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 950)
+        same_bits(sg, s_h, "state, step %d" % t)
+        np.testing.assert_array_equal(r.cpu().numpy(), r_h)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        s_h[:] = sg
+        if t == 20:
+            # the loose lower leg has come away from its upper leg in the rows without the joint
+            up, low = s_h[:, 24 + 13 * 3: 24 + 13 * 3 + 3], s_h[:, 24 + 13 * 4: 24 + 13 * 4 + 3]
+            J = s_h[:, 24 + 65 + 15 + 3 * 17: 24 + 65 + 15 + 4 * 17]       # [type, a, b, ax, ay, bx, by, ...]
+            world = lambda body, lx, ly: np.stack([body[:, 0] + lx * np.cos(body[:, 2]) - ly * np.sin(body[:, 2]),
+                                                   body[:, 1] + lx * np.sin(body[:, 2]) + ly * np.cos(body[:, 2])], 1)
+            gap = np.hypot(*(world(up, J[:, 3], J[:, 4]) - world(low, J[:, 5], J[:, 6])).T)   # between the two anchors
+            say("  anchor gap of joint 3, medians: without the joint %.3f, with it %.3f" % (np.median(gap[::2]), np.median(gap[1::2])))
+            assert np.median(gap[::2]) > 0.3 and np.median(gap[1::2]) < 0.05
+
+
 @pytest.mark.parametrize("name", ["CartPoleEnv", "PendulumV2", "BipedalWalkerV2", "HalfCheetahPlanarV2",
                                   "LunarLanderV2Continuous"])
 def test_autoreset_equals_step_then_selective_reset(mrl, ctx, name):
