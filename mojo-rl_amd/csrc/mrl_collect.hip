@@ -487,6 +487,10 @@ __global__ __launch_bounds__(CLASSIC_THREADS) void collect_classic_kernel(Collec
     HiddenOperands<H, TPW, KB> ops;
     ops.load(t / TN ? a.critic_p : a.actor_p, IN, t);
     __syncthreads();
+    // the policy does not change during the launch: exp(log_std) of the Gaussian head once for all the steps
+    float stdv[PA_MAX];
+#pragma unroll
+    for (int j = 0; j < PA_MAX; ++j) stdv[j] = (GAUSS && owner && j < a.A) ? exp32(gaussian_log_std(w2s[0][HEAD_LOG_STD(H) + j])) : 1.0f;
 
     for (int k = 0; k < a.n_steps; ++k) {
         // (the empty asm keeps what the optimiser derives from these values inside the step)
@@ -513,7 +517,7 @@ __global__ __launch_bounds__(CLASSIC_THREADS) void collect_classic_kernel(Collec
             const int i = env0 + tid;
             float av[PA_MAX], logp;
             if (GAUSS) {
-                logp = sample_gaussian(logits + tid * (PA_MAX + 1), w2s[0] + HEAD_LOG_STD(H), A, sseed, i, av);
+                logp = sample_gaussian(logits + tid * (PA_MAX + 1), w2s[0] + HEAD_LOG_STD(H), A, sseed, i, av, stdv);
                 for (int j = 0; j < A; ++j) a.r_actions[(row + tid) * AW + j] = av[j];
             } else {
                 int sel;

@@ -68,20 +68,21 @@ MRL_DEV void sample_categorical_few(const float *l, int A, uint32_t seed, int i,
 // Gaussian sampling (deep_agents/ppo/kernels.mojo:12-98) of components j0 .. j0 + m of an action
 // with A components: one Philox stream per (env, component), Box-Muller, clamped log_std;
 // returns the summed log-probability of those components and leaves them in act[0 .. m).
+// std_p (optional): exp of the clamped log_std of the same components, taken ahead by a caller whose
+// log_std does not change from call to call.
+MRL_DEV float gaussian_log_std(float log_std) { return log_std < -5.0f ? -5.0f : (log_std > 2.0f ? 2.0f : log_std); }
 MRL_DEV float sample_gaussian_part(const float *mean, const float *log_std_p, int m, int A, int j0,
-                                   uint32_t seed, int i, float *act) {
+                                   uint32_t seed, int i, float *act, const float *std_p = nullptr) {
     const float EPS = 1e-6f, LOG_2PI = (float)1.8378770664093453;
     float total = 0.0f;
     for (int j = 0; j < m; ++j) {
         const float mu = mean[j];
-        float log_std = log_std_p[j];
-        if (log_std < -5.0f) log_std = -5.0f;
-        else if (log_std > 2.0f) log_std = 2.0f;
+        const float log_std = gaussian_log_std(log_std_p[j]);
         Uniform4 rv = philox_uniform4((uint64_t)((int64_t)seed + (int64_t)i * A + j0 + j), 0, 0);
         const float u1 = rv.v[0] + 1e-8f;
         const float mag = sqrtf(-2.0f * log32(u1));
         const float noise = mag * cos32(rv.v[1] * (float)6.283185307179586);
-        const float std = exp32(log_std);
+        const float std = std_p != nullptr ? std_p[j] : exp32(log_std);
         const float action = mu + std * noise;
         act[j] = action;
         const float an = (action - mu) / (std + EPS);
@@ -90,8 +91,8 @@ MRL_DEV float sample_gaussian_part(const float *mean, const float *log_std_p, in
     return total;
 }
 MRL_DEV float sample_gaussian(const float *mean_row, const float *log_std_p, int A, uint32_t seed, int i,
-                              float *act) {
-    return sample_gaussian_part(mean_row, log_std_p, A, A, 0, seed, i, act);
+                              float *act, const float *std_p = nullptr) {
+    return sample_gaussian_part(mean_row, log_std_p, A, A, 0, seed, i, act, std_p);
 }
 
 }  // namespace mrl
