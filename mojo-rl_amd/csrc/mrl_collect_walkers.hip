@@ -105,10 +105,12 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
     __shared__ float part[R * PA_MAX];              // log-probability per (env, component)
     __shared__ float shapes[E::NSHAPE];
     __shared__ unsigned long long was_reset;
+    __shared__ unsigned sync_actor, sync_critic, sync_failed;   // barriers of the wavefront groups (LANES)
     // the two activation tiles and the env step's scratch (contact lists) are never live together
     constexpr int LIST_F = detect_list_floats<E>() + 1;
     constexpr int ENV_F = R * S::CSTRIDE + LIST_F + E::DETECT_TASKS * R + 1;
     __shared__ float overlay[wmax<2 * H * HT16_LD, ENV_F>()];
+    static_assert(!LANES || R * S::CSTRIDE <= H * HT16_LD, "the one-lane fallback's contact scratch stays below the critic's tile");
     float *cts = overlay, *dlist = cts + R * S::CSTRIDE;
     int *dcount = reinterpret_cast<int *>(dlist + LIST_F);
 
@@ -122,7 +124,12 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
     for (int i = t; i < E::NSHAPE; i += T) shapes[i] = a.shapes[i];
     stage_head(a.actor_p + IN * H + H + H * H + H, H, a.A, true, w2a, t, T);
     for (int i = t; i < H + 1; i += T) w2c[i] = a.critic_p[IN * H + H + H * H + H + i];
-    if (t == 0) was_reset = 0;
+    if (t == 0) {
+        was_reset = 0;
+        sync_actor = 0;
+        sync_critic = 0;
+        sync_failed = 0;
+    }
     __syncthreads();
 
     for (int k = 0; k < a.n_steps; ++k) {
@@ -133,8 +140,49 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
         const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
         const uint64_t rseed = a.reset_seed + (uint64_t)k * a.reset_stride;
         const int wave = tid / WAVE, lane = tid % WAVE;
-        policy16_gauss<IN, AW, ACT>(a, [&](int r, int c) { return rows[r * S::STRIDE + c]; }, tid, ne, A, zero, row, sseed, env0,
-                                    xs, overlay, w2a, w2c, logits, vals, act, part);
+        if constexpr (LANES) {
+            // HalfCheetah's env step keeps wavefronts 0 and 1 busy for most of the step and nothing else:
+            // only the actor goes ahead of it (wavefronts 0 .. 3, one per SIMD); the critic, whose value is
+            // only stored, runs beside the env step on wavefronts 2, 3, 6 and 7 -- the two SIMDs that do not
+            // host the env's wavefronts.  Both groups meet at bounded barriers of their own, rebuilt every
+            // step from the step number (five rounds per step for the actor's group, three for the critic's).
+            for (int i = tid; i < R * IN; i += T) {
+                const int r = i / IN, c = i - r * IN;
+                float v = 0.0f;
+                if (r < ne) {
+                    v = rows[r * S::STRIDE + c];
+                    a.r_obs[row * IN + i] = v;
+                }
+                xs[r * XS_LD + c] = v;
+            }
+            __syncthreads();
+            WaveGroupSync actor_sync{&sync_actor, (unsigned)k * 20u, 4u, &sync_failed, a.spin_limit};
+            if (wave < 4) {
+                const float *p = a.actor_p + zero;
+                Hidden16Operands<H, IN, 4, KBA> ops;
+                ops.load(p, 64 * wave, lane);
+                hidden_stack16<H, IN, ACT, 4, KBA, true>(p, xs, overlay, overlay, ops, 64 * wave, lane, actor_sync);
+                head16<H>(w2a, A, overlay, logits, PA_MAX + 1, tid, T / 2);
+                actor_sync();   // means complete
+                for (int e = tid; e < ne * A; e += T / 2) {
+                    const int r = e / A, j = e - r * A;
+                    float av;
+                    part[r * PA_MAX + j] = sample_gaussian_part(logits + r * (PA_MAX + 1) + j, w2a + HEAD_LOG_STD(H) + j, 1, A,
+                                                                j, sseed, env0 + r, &av);
+                    act[r * AW + j] = av;
+                    a.r_actions[row * AW + e] = av;
+                }
+                actor_sync();   // actions and the log-probability terms complete
+                if (tid < ne) {
+                    float logp = 0.0f;
+                    for (int j = 0; j < A; ++j) logp = logp + part[tid * PA_MAX + j];
+                    a.r_logp[row + tid] = logp;
+                }
+            }
+        } else {
+            policy16_gauss<IN, AW, ACT>(a, [&](int r, int c) { return rows[r * S::STRIDE + c]; }, tid, ne, A, zero, row, sseed,
+                                        env0, xs, overlay, w2a, w2c, logits, vals, act, part);
+        }
         // ---- env step with auto-reset, reward / done into rollout row t, episode accounting
         Accounting acc = a.acc;
         acc.r_rewards = a.r_rewards + (size_t)(a.t0 + k) * N;
@@ -160,10 +208,27 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
                     account(acc, slot, r, d);
                     if (d > 0.5f) E::reset(rowp, rseed, env);
                 }
+            } else if (wave & 2) {
+                // ---- critic beside the env step: member g = 0 .. 3 of its group is wavefront 2, 3, 6, 7
+                const int g = (wave & 1) + ((wave >> 2) << 1);
+                const float *p = a.critic_p + zero;
+                float *tile = overlay + H * HT16_LD;   // (the one-lane fallback's contact scratch lies below it)
+                WaveGroupSync critic_sync{&sync_critic, (unsigned)k * 12u, 4u, &sync_failed, a.spin_limit};
+                Hidden16Operands<H, IN, 4, KBA> ops;
+                ops.load(p, 64 * g, lane);
+                hidden_stack16<H, IN, ACT, 4, KBA, true>(p, xs, tile, tile, ops, 64 * g, lane, critic_sync);
+                head_rows16<H, 1, 1>(w2c, 1, tile, vals, 1, g * WAVE + lane, T / 2);
             }
         }
         __syncthreads();   // env step done: the rows hold the next observation
+        if constexpr (LANES) {
+            if (tid < ne) a.r_values[row + tid] = vals[tid];
+            // a wait that gave up: the block's results are void from here on; leave the loop, store what
+            // there is and end normally
+            if (sync_failed != 0u) break;
+        }
     }
+    if (LANES && t == 0 && sync_failed != 0u) *a.sync_error = 1;
 
     for (int i = t; i < nenv * E::OBS; i += T) {
         const int r = i / E::OBS, c = i - r * E::OBS;
