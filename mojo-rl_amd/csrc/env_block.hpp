@@ -350,11 +350,19 @@ MRL_DEV int merge_vertex_lists(const float *dlist, const int *dcount, int e, flo
 // ([nenv][ACT_W], global or LDS), rewards / dones = the block's slice of the per-step outputs
 // (may be null), acc = rollout accounting with its pointers already offset to the block's first
 // env.  AUTORESET: rows that finished are re-initialised in place and recorded in *was_reset.
-template <class E, bool AUTORESET>
+// (what phys_step_block runs beside the one-lane-per-body solver when the caller has nothing for it)
+struct NoSideJob {
+    MRL_DEV void operator()(int) const {}
+};
+
+// `side`: work of the caller's that the wavefronts without a part in the one-lane-per-body solver (LANES_PHYSICS
+// envs: wavefronts 2 and up) do while wavefronts 0 and 1 run it, called as side(tid) between the two block
+// barriers around the solver; it must not touch the rows or the contact scratch `cts`.
+template <class E, bool AUTORESET, class Side = NoSideJob>
 MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float *dlist, int *dcount,
                              unsigned long long *was_reset, const float *actions, float *rewards,
                              float *dones, int env0, int nenv, uint64_t reset_seed, const Accounting &acc,
-                             int tid = threadIdx.x) {
+                             int tid = threadIdx.x, Side side = Side{}) {
     using S = Stage<E>;
     if constexpr (E::DETECT_TASKS > 0 && E::POST_TASKS == 0) {
         // wavefront 0: first half of the step (reads and writes velocities only); the halves of the
@@ -423,6 +431,8 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
                 const int n = dcount[slot];
                 if (n >= 0) E::physics_lanes(rows + slot * S::STRIDE, cts + slot * S::CSTRIDE, n, tid % WAVE);
             }
+            static_assert(E::EPB * E::LANES_PER_ENV <= 2 * WAVE, "the solver's lanes are wavefronts 0 and 1");
+            if (tid >= 2 * WAVE) side(tid);
             __syncthreads();
             if (tid < nenv) lanes_n = dcount[tid];
         }

@@ -2,20 +2,24 @@
 // HalfCheetah planar, CarRacingV2) with the agents' 256-wide Gaussian nets: many rollout steps of a
 // block's 16 envs in ONE launch, like the kernels of mrl_collect.hip.  The env rows (CarRacing: the 40
 // floats in front of the track) stay in LDS from the first step to the last; per step and block
-//   policy   wavefronts 0 .. 3 the actor  OBS -> 256 -> 256 -> A, wavefronts 4 .. 7 the critic
-//            OBS -> 256 -> 256 -> 1, side by side on the fp32 matrix cores (the 16-row tiles of
-//            mlp_tile16.hpp, 64 columns per wavefront, weights streamed from L2), heads out of LDS;
+//   policy   the actor  OBS -> 256 -> 256 -> A  on wavefronts 0 .. 3 and the critic  OBS -> 256 -> 256 -> 1
+//            on four others, on the fp32 matrix cores (the 16-row tiles of mlp_tile16.hpp, 64 columns
+//            per wavefront, weights streamed from L2), heads out of LDS.  The walkers: only the actor runs
+//            ahead of the env step; the critic, whose value is only stored, runs beside the one-lane-per-
+//            body solver on wavefronts 2, 3, 6 and 7 (the two SIMDs that the solver's wavefronts 0 and 1
+//            do not use).  CarRacing, whose env step takes every wavefront: both nets side by side
+//            (critic on wavefronts 4 .. 7) ahead of it;
 //   sample   one lane per (env, action component): every component has a Philox stream of its own;
 //   env step BipedalWalker: the workgroup-level step of env_block.hpp (contact detection on every
-//            wavefront, solver with one lane per body on wavefronts 0 and 1, lidar rays on every wavefront, wave-cooperative
-//            resets); HalfCheetah: one lane per body on wavefronts 0 and 1 (env_cheetah_lanes.hpp);
-//            CarRacing: a wavefront per env, two rounds of eight (env_car.hpp); the tile tables stay in
-//            global memory and are staged through LDS every step (16 x 12 KB do not fit beside the rest);
+//            wavefront, solver with one lane per body on wavefronts 0 and 1, lidar rays on every
+//            wavefront, wave-cooperative resets); HalfCheetah: one lane per body on wavefronts 0 and 1
+//            (env_cheetah_lanes.hpp); CarRacing: a wavefront per env, two rounds of eight (env_car.hpp);
+//            the tile tables stay in global memory and are staged through LDS every step (16 x 12 KB do
+//            not fit beside the rest);
 //   rollout row t of obs, action, log-prob, value, reward, done written on the way.
-// With these envs the step is 70 - 80 % env step, which is one wavefront's instruction stream, so the
-// critic is not moved beside it: what the fusion buys is the launch gaps, the observation / action
-// round trip through HBM, the staging of the rows in and out of LDS every step, and a policy forward
-// with both nets of a 16-row tile on one CU.
+// With these envs the step is 70 - 80 % env step, a chain of one or two wavefronts' instructions: what the
+// fusion buys is the launch gaps, the observation / action round trip through HBM, the staging of the rows
+// in and out of LDS every step, and a policy forward of a 16-row tile on one CU.
 //
 // It gives what n_steps calls of mrl_rollout_step give (same per-env streams: seeds are affine in
 // the step number), except that the finished-episode list is appended in the order in which blocks
@@ -90,6 +94,55 @@ MRL_DEV void policy16_gauss(const CollectArgs &a, ObsAt obs_at, int tid, int ne,
     }
 }
 
+// The actor's half of policy16_gauss by wavefronts 0 .. 3 alone (the observation tile xs is complete, every
+// thread of the four passes its tid): hidden stack on `tile`, Gaussian sampling, rollout row t of action and
+// log-prob; leaves the actions in act[env][AW].  The four wavefronts meet at `sync`, five rounds per call.
+template <int IN, int AW, int ACT>
+MRL_DEV void actor16_gauss(const CollectArgs &a, int tid, int ne, int A, int zero, size_t row, uint32_t sseed, int env0,
+                           const float *xs, float *tile, const float *w2a, float *logits, float *act, float *part,
+                           WaveGroupSync &sync) {
+    constexpr int H = 256, KBA = 8, TA = 4 * WAVE;
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    const float *p = a.actor_p + zero;
+    Hidden16Operands<H, IN, 4, KBA> ops;
+    ops.load(p, 64 * wave, lane);
+    hidden_stack16<H, IN, ACT, 4, KBA, true>(p, xs, tile, tile, ops, 64 * wave, lane, sync);
+    head16<H>(w2a, A, tile, logits, PA_MAX + 1, tid, TA);
+    sync();   // means complete
+    for (int e = tid; e < ne * A; e += TA) {
+        const int r = e / A, j = e - r * A;
+        float av;
+        part[r * PA_MAX + j] = sample_gaussian_part(logits + r * (PA_MAX + 1) + j, w2a + HEAD_LOG_STD(H) + j, 1, A, j,
+                                                    sseed, env0 + r, &av);
+        act[r * AW + j] = av;
+        a.r_actions[row * AW + e] = av;
+    }
+    sync();   // actions and the log-probability terms complete
+    if (tid < ne) {
+        float logp = 0.0f;
+        for (int j = 0; j < A; ++j) logp = logp + part[tid * PA_MAX + j];
+        a.r_logp[row + tid] = logp;
+    }
+}
+constexpr unsigned ACTOR16_ROUNDS = 5, CRITIC16_ROUNDS = 3;
+
+// The critic's half by wavefronts 2, 3, 6 and 7 (the two SIMDs that do not host wavefronts 0 and 1), on a
+// barrier of their own: values of the block's rows into vals.
+template <int IN, int ACT>
+MRL_DEV void critic16_side(const CollectArgs &a, int zero, int k, int tid, const float *xs, float *tile, const float *w2c,
+                           float *vals, unsigned *sync_word, unsigned *failed) {
+    constexpr int H = 256, KBA = 8;
+    const int wave = tid / WAVE, lane = tid % WAVE;
+    if (!(wave & 2)) return;
+    const int g = (wave & 1) + ((wave >> 2) << 1);   // 0 .. 3
+    const float *p = a.critic_p + zero;
+    WaveGroupSync sync{sync_word, (unsigned)k * CRITIC16_ROUNDS * 4u, 4u, failed, a.spin_limit};
+    Hidden16Operands<H, IN, 4, KBA> ops;
+    ops.load(p, 64 * g, lane);
+    hidden_stack16<H, IN, ACT, 4, KBA, true>(p, xs, tile, tile, ops, 64 * g, lane, sync);
+    head_rows16<H, 1, 1>(w2c, 1, tile, vals, 1, g * WAVE + lane, 4 * WAVE);
+}
+
 template <class E, int ACT, bool LANES>
 __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
     using S = Stage<E>;
@@ -105,12 +158,12 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
     __shared__ float part[R * PA_MAX];              // log-probability per (env, component)
     __shared__ float shapes[E::NSHAPE];
     __shared__ unsigned long long was_reset;
-    __shared__ unsigned sync_actor, sync_critic, sync_failed;   // barriers of the wavefront groups (LANES)
+    __shared__ unsigned sync_actor, sync_critic, sync_failed;   // barriers of the actor's and the critic's wavefronts
     // the two activation tiles and the env step's scratch (contact lists) are never live together
     constexpr int LIST_F = detect_list_floats<E>() + 1;
     constexpr int ENV_F = R * S::CSTRIDE + LIST_F + E::DETECT_TASKS * R + 1;
     __shared__ float overlay[wmax<2 * H * HT16_LD, ENV_F>()];
-    static_assert(!LANES || R * S::CSTRIDE <= H * HT16_LD, "the one-lane fallback's contact scratch stays below the critic's tile");
+    static_assert(R * S::CSTRIDE <= H * HT16_LD, "the solver's contact scratch stays below the critic's tile");
     float *cts = overlay, *dlist = cts + R * S::CSTRIDE;
     int *dcount = reinterpret_cast<int *>(dlist + LIST_F);
 
@@ -140,57 +193,38 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
         const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
         const uint64_t rseed = a.reset_seed + (uint64_t)k * a.reset_stride;
         const int wave = tid / WAVE, lane = tid % WAVE;
-        if constexpr (LANES) {
-            // HalfCheetah's env step keeps wavefronts 0 and 1 busy for most of the step and nothing else:
-            // only the actor goes ahead of it (wavefronts 0 .. 3, one per SIMD); the critic, whose value is
-            // only stored, runs beside the env step on wavefronts 2, 3, 6 and 7 -- the two SIMDs that do not
-            // host the env's wavefronts.  Both groups meet at bounded barriers of their own, rebuilt every
-            // step from the step number (five rounds per step for the actor's group, three for the critic's).
-            for (int i = tid; i < R * IN; i += T) {
-                const int r = i / IN, c = i - r * IN;
-                float v = 0.0f;
-                if (r < ne) {
-                    v = rows[r * S::STRIDE + c];
-                    a.r_obs[row * IN + i] = v;
-                }
-                xs[r * XS_LD + c] = v;
+        // The env step keeps wavefronts 0 and 1 busy for most of the step (the solver with one lane per body)
+        // and the others for little or nothing: only the actor goes ahead of it (wavefronts 0 .. 3, one per
+        // SIMD); the critic, whose value is only stored, runs beside the solver on wavefronts 2, 3, 6 and 7 --
+        // the two SIMDs that do not host wavefronts 0 and 1.  Both groups meet at bounded barriers of their
+        // own, rebuilt every step from the step number.
+        for (int i = tid; i < R * IN; i += T) {
+            const int r = i / IN, c = i - r * IN;
+            float v = 0.0f;
+            if (r < ne) {
+                v = rows[r * S::STRIDE + c];
+                a.r_obs[row * IN + i] = v;
             }
-            __syncthreads();
-            WaveGroupSync actor_sync{&sync_actor, (unsigned)k * 20u, 4u, &sync_failed, a.spin_limit};
-            if (wave < 4) {
-                const float *p = a.actor_p + zero;
-                Hidden16Operands<H, IN, 4, KBA> ops;
-                ops.load(p, 64 * wave, lane);
-                hidden_stack16<H, IN, ACT, 4, KBA, true>(p, xs, overlay, overlay, ops, 64 * wave, lane, actor_sync);
-                head16<H>(w2a, A, overlay, logits, PA_MAX + 1, tid, T / 2);
-                actor_sync();   // means complete
-                for (int e = tid; e < ne * A; e += T / 2) {
-                    const int r = e / A, j = e - r * A;
-                    float av;
-                    part[r * PA_MAX + j] = sample_gaussian_part(logits + r * (PA_MAX + 1) + j, w2a + HEAD_LOG_STD(H) + j, 1, A,
-                                                                j, sseed, env0 + r, &av);
-                    act[r * AW + j] = av;
-                    a.r_actions[row * AW + e] = av;
-                }
-                actor_sync();   // actions and the log-probability terms complete
-                if (tid < ne) {
-                    float logp = 0.0f;
-                    for (int j = 0; j < A; ++j) logp = logp + part[tid * PA_MAX + j];
-                    a.r_logp[row + tid] = logp;
-                }
-            }
-        } else {
-            policy16_gauss<IN, AW, ACT>(a, [&](int r, int c) { return rows[r * S::STRIDE + c]; }, tid, ne, A, zero, row, sseed,
-                                        env0, xs, overlay, w2a, w2c, logits, vals, act, part);
+            xs[r * XS_LD + c] = v;
         }
+        __syncthreads();
+        if (wave < 4) {
+            WaveGroupSync actor_sync{&sync_actor, (unsigned)k * ACTOR16_ROUNDS * 4u, 4u, &sync_failed, a.spin_limit};
+            actor16_gauss<IN, AW, ACT>(a, tid, ne, A, zero, row, sseed, env0, xs, overlay, w2a, logits, act, part, actor_sync);
+        }
+        float *critic_tile = overlay + H * HT16_LD;   // (above the env step's contact scratch cts)
         // ---- env step with auto-reset, reward / done into rollout row t, episode accounting
         Accounting acc = a.acc;
         acc.r_rewards = a.r_rewards + (size_t)(a.t0 + k) * N;
         acc.r_dones = a.r_dones + (size_t)(a.t0 + k) * N;
         acc = acc.at(env0);
         if constexpr (!LANES) {
+            // (the critic's tile lies over contact lists that are spent by the time the solver runs)
+            auto side = [&](int th) {
+                critic16_side<IN, ACT>(a, zero, k, th, xs, critic_tile, w2c, vals, &sync_critic, &sync_failed);
+            };
             phys_step_block<E, true>(rows, cts, shapes, dlist, dcount, &was_reset, act, nullptr, nullptr, env0, ne,
-                                     rseed, acc, tid);
+                                     rseed, acc, tid, side);
         } else {
             // HalfCheetah: eight lanes per env, eight envs per wavefront, on wavefronts 0 and 1; a row
             // whose wiring is not HalfCheetah's own is stepped by lane 0 of its group in the one-lane form
@@ -208,27 +242,17 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
                     account(acc, slot, r, d);
                     if (d > 0.5f) E::reset(rowp, rseed, env);
                 }
-            } else if (wave & 2) {
-                // ---- critic beside the env step: member g = 0 .. 3 of its group is wavefront 2, 3, 6, 7
-                const int g = (wave & 1) + ((wave >> 2) << 1);
-                const float *p = a.critic_p + zero;
-                float *tile = overlay + H * HT16_LD;   // (the one-lane fallback's contact scratch lies below it)
-                WaveGroupSync critic_sync{&sync_critic, (unsigned)k * 12u, 4u, &sync_failed, a.spin_limit};
-                Hidden16Operands<H, IN, 4, KBA> ops;
-                ops.load(p, 64 * g, lane);
-                hidden_stack16<H, IN, ACT, 4, KBA, true>(p, xs, tile, tile, ops, 64 * g, lane, critic_sync);
-                head_rows16<H, 1, 1>(w2c, 1, tile, vals, 1, g * WAVE + lane, T / 2);
+            } else {
+                critic16_side<IN, ACT>(a, zero, k, tid, xs, critic_tile, w2c, vals, &sync_critic, &sync_failed);
             }
         }
         __syncthreads();   // env step done: the rows hold the next observation
-        if constexpr (LANES) {
-            if (tid < ne) a.r_values[row + tid] = vals[tid];
-            // a wait that gave up: the block's results are void from here on; leave the loop, store what
-            // there is and end normally
-            if (sync_failed != 0u) break;
-        }
+        if (tid < ne) a.r_values[row + tid] = vals[tid];
+        // a wait that gave up: the block's results are void from here on; leave the loop, store what
+        // there is and end normally
+        if (sync_failed != 0u) break;
     }
-    if (LANES && t == 0 && sync_failed != 0u) *a.sync_error = 1;
+    if (t == 0 && sync_failed != 0u) *a.sync_error = 1;
 
     for (int i = t; i < nenv * E::OBS; i += T) {
         const int r = i / E::OBS, c = i - r * E::OBS;
