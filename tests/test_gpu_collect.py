@@ -322,13 +322,15 @@ def test_fused_walker_collection_against_the_oracle(mrl, ctx, orc, env, kind, N)
     assert int(fused.done_count.item()) == finished
 
 
-def test_barrier_wait_gives_up_and_reports(mrl):
-    """The wavefront-group barriers inside the fused collection kernel are bounded: with a limit of
-    one poll some wait gives up, the kernel still ends normally, and the next synchronize reports it
-    once.  With the default limit the same launch then runs clean."""
+@pytest.mark.parametrize("env", ["lunar", "bipedal", "cheetah"])
+def test_barrier_wait_gives_up_and_reports(mrl, env):
+    """The wavefront-group barriers inside the fused collection kernels (LunarLander: critic and contact
+    detection beside the solver; the walkers: actor ahead of the env step, critic beside it) are bounded:
+    with a limit of one poll some wait gives up, the kernel still ends normally, and the next synchronize
+    reports it once.  With the default limit the same launch then runs clean."""
     ctx = mrl.DeviceContext("cuda:0")
     N, T = 2048, 4
-    one, many = _pair(mrl, ctx, N, T, 256, "relu", "lunar")
+    one, many = _pair(mrl, ctx, N, T, 256, "relu", env)
     s0, ss = 99, 7919
     ctx.set_spin_limit(1)
     mrl.ppo.rollout_steps(ctx, many.descriptor(), 0, T, s0, ss, 0, 0, 5, 1)
@@ -336,7 +338,7 @@ def test_barrier_wait_gives_up_and_reports(mrl):
         ctx.synchronize()
     ctx.synchronize()                       # reported once, then cleared
     ctx.set_spin_limit(0)
-    one, many = _pair(mrl, ctx, N, T, 256, "relu", "lunar")
+    one, many = _pair(mrl, ctx, N, T, 256, "relu", env)
     d1, d2 = one.descriptor(), many.descriptor()
     for t in range(T):
         mrl.ppo.rollout_step(ctx, d1, t, s0 + t * ss, 0, 5 + t)
