@@ -88,7 +88,7 @@ int mrl_ctx_synchronize(mrl_ctx *ctx);
 int mrl_ctx_workspace(mrl_ctx *ctx, uint64_t *mlp_floats, uint64_t *rollout_floats);
 int mrl_ctx_reserve(mrl_ctx *ctx, uint64_t mlp_floats, uint64_t rollout_floats);
 
-/* The fused collection kernel lets groups of wavefronts of a workgroup meet at barriers of their own
+/* The fused collection kernels let groups of wavefronts of a workgroup meet at barriers of their own
  * (counters in LDS).  Every such wait is bounded: after `polls` polls (MRL_DEFAULT_SPIN_LIMIT unless
  * set here; 0 restores the default) the waiting wavefront gives up, the workgroup stops stepping, the
  * kernel ends normally and the next mrl_ctx_synchronize returns MRL_E_SYNC (once).  No counterpart
