@@ -51,8 +51,10 @@ struct LunarLander {
                              float &r, float &d) {
         ll::step_row(row, cts, shapes, env, (int)a[0], r, d);
     }
-    static constexpr int POST_TASKS = 0;
-    static MRL_DEV void post_task(float *, int) {}
+    static constexpr int POST_TASKS = 0, POST_WORDS = 0, POST_PARTS = 1;
+    static MRL_DEV void post_share(const float *, int, unsigned *) {}
+    static MRL_DEV float post_task(const float *, int, const unsigned *) { return 0.0f; }
+    static MRL_DEV void post_join(float *, int, const float *) {}
     static MRL_DEV void reset(float *row, uint64_t seed, int env) {
         ll::reset_row(row, ll::combined_seed(seed, env));
     }
@@ -99,19 +101,30 @@ struct BipedalWalker {
     static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 16, THREADS = 512;
     static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = bw::NSHAPE_FLOATS;
     // the ten lidar rays of the observation are left out of the step and run afterwards, spread
-    // over all wavefronts of the block: task k = half k % 2 of the edges for ray k / 2.  The two
-    // halves of a ray sit EPB lanes apart in one wavefront and exchange their minima there.
-    static constexpr int POST_TASKS = 20;
+    // over all wavefronts of the block: task k = part k % 3 of the edges for ray k / 3; the parts of
+    // a ray meet in LDS (post_join).
+    static constexpr int POST_PARTS = 3, POST_TASKS = 10 * POST_PARTS;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
         bw::step_row<false>(row, cts, shapes, env, a, r, d);
     }
-    static MRL_DEV void post_task(float *row, int task) {
-        static_assert(2 * EPB <= 64 && (THREADS / EPB) % 2 == 0 && POST_TASKS % 2 == 0, "both halves of a ray in one wavefront, in the same pass");
-        float t = bw::lidar_value_part(row, task >> 1, task & 1, 2);
-        const float other = __shfl_xor(t, EPB, 64);
-        t = other < t ? other : t;
-        if ((task & 1) == 0) row[14 + (task >> 1)] = t;
+    // ahead of the rays, once per env and by all its lanes: the mask of the edges within lidar range of the hull
+    static constexpr int POST_WORDS = EdgeMask<L>::WORDS;
+    static MRL_DEV void post_share(const float *row, int slot, unsigned *words) {
+        bw::lidar_near_share<THREADS / EPB, EPB>(row, slot, words);
+    }
+    static MRL_DEV float post_task(const float *row, int task, const unsigned *words) {
+        return bw::lidar_value_part<POST_PARTS>(row, task / POST_PARTS, task % POST_PARTS, words);
+    }
+    // parts = the values of the env's tasks
+    static MRL_DEV void post_join(float *row, int ray, const float *parts) {
+        float t = parts[ray * POST_PARTS];
+#pragma unroll
+        for (int k = 1; k < POST_PARTS; ++k) {
+            const float other = parts[ray * POST_PARTS + k];
+            t = other < t ? other : t;
+        }
+        row[14 + ray] = t;
     }
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { bw::reset_row(row, walker_seed(seed, env)); }
     static constexpr bool WAVE_RESET = true;
@@ -155,8 +168,10 @@ struct HalfCheetah {
         hc::step_row(row, cts, shapes, env, a, r, d);
     }
     static constexpr bool LANES_PHYSICS = false;
-    static constexpr int POST_TASKS = 0;
-    static MRL_DEV void post_task(float *, int) {}
+    static constexpr int POST_TASKS = 0, POST_WORDS = 0, POST_PARTS = 1;
+    static MRL_DEV void post_share(const float *, int, unsigned *) {}
+    static MRL_DEV float post_task(const float *, int, const unsigned *) { return 0.0f; }
+    static MRL_DEV void post_join(float *, int, const float *) {}
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { hc::reset_row(row, walker_seed(seed, env)); }
     static constexpr bool WAVE_RESET = false;
     static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
@@ -475,8 +490,22 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
             const unsigned long long fin = *was_reset;
             constexpr int SLOTS = E::THREADS / E::EPB;   // tasks in flight per env
             const int e = tid % E::EPB;
-            if (e < nenv && !((fin >> e) & 1ull))
-                for (int task = tid / E::EPB; task < E::POST_TASKS; task += SLOTS) E::post_task(rows + e * S::STRIDE, task);
+            // what the tasks of an env share is worked out first, by all its lanes, into the (spent)
+            // contact counts; the tasks leave their values in the (spent) contact lists, where the
+            // first lanes of the env put those of one result together
+            const bool live = e < nenv && !((fin >> e) & 1ull);
+            const int slot = tid / E::EPB;
+            unsigned *words = reinterpret_cast<unsigned *>(dcount) + e * E::POST_WORDS;
+            float *parts = dlist + e * E::POST_TASKS;
+            static_assert(E::POST_WORDS <= E::DETECT_TASKS && E::POST_TASKS <= detect_stride(1) * E::DETECT_TASKS &&
+                          E::POST_TASKS <= SLOTS, "words and task values fit the counts and lists, a task per lane");
+            if constexpr (E::POST_WORDS > 0) {
+                if (live) E::post_share(rows + e * S::STRIDE, slot, words);
+                __syncthreads();
+            }
+            if (live && slot < E::POST_TASKS) parts[slot] = E::post_task(rows + e * S::STRIDE, slot, words);
+            __syncthreads();
+            if (live && slot < E::POST_TASKS / E::POST_PARTS) E::post_join(rows + e * S::STRIDE, slot, parts);
             if (AUTORESET) reset_rows_block<E>(rows, fin, reset_seed, env0, tid);
         }
     }

@@ -119,12 +119,31 @@ MRL_DEV float lidar_value(const float *row, int i, const EdgeMask<L> *near) {
     return lidar_ray_near<L>(row, mine, hull_x, hull_y, cs * lidar_range, sn * lidar_range);
 }
 
-// Lidar ray i against a share of the edges only: part `part` of `nparts` takes the edges of the
-// mask words [part * WORDS / nparts, (part + 1) * WORDS / nparts); the ray's value is the minimum
-// over the parts (every part starts from 1, the value of a ray that hits nothing, and a hit
-// replaces it only by something smaller: the minimum over all edges, however they are grouped).
-// The edge set is picked for the ray's own x extent.
-MRL_DEV float lidar_value_part(const float *row, int i, int part, int nparts) {
+// The lidar rays of an env spread over the lanes of a block.
+//
+// lidar_near_share: ahead of the rays, once per env, the mask of the edges within lidar range of the
+// hull in x (every ray stays inside that range), each of the env's `SLOTS` lanes testing its share of
+// the edges; the four lanes of an env in a wavefront (they sit EPB lanes apart) combine their bits and
+// store sixteen of them.  words = the env's WORDS mask words.
+template <int SLOTS, int EPB>
+MRL_DEV void lidar_near_share(const float *row, int slot, unsigned *words) {
+    constexpr int PER = L::MAX_EDGES / SLOTS;
+    static_assert(PER * SLOTS == L::MAX_EDGES && 4 * EPB == 64 && 4 * PER == 16, "sixteen mask bits per wavefront");
+    const float hull_x = row[L::BODIES_OFF + IDX_X], lidar_range = (float)LIDAR_RANGE;
+    unsigned b = edges_near_bits<L, PER>(row, hull_x - lidar_range, hull_x + lidar_range, 0.02f, slot * PER) << (PER * (slot & 3));
+    b |= __shfl_xor(b, EPB, 64);
+    b |= __shfl_xor(b, 2 * EPB, 64);
+    if ((slot & 3) == 0) reinterpret_cast<unsigned short *>(words)[slot >> 2] = (unsigned short)b;
+}
+
+// Lidar ray i against a share of those edges: part `part` of NPARTS takes the edges whose number is
+// `part` modulo NPARTS (the edges in range are a run of neighbours, so the shares come out even); the
+// ray's value is the minimum over the parts (every part starts from 1, the value of a ray that hits
+// nothing, and a hit replaces it only by something smaller: the minimum over all edges, however they
+// are grouped).  lidar_ray_pick looks at each edge's extent against the ray's own, as lidar_ray_near does.
+template <int NPARTS>
+MRL_DEV float lidar_value_part(const float *row, int i, int part, const unsigned *near) {
+    static_assert(NPARTS == 2 || NPARTS == 3, "share masks for two or three parts");
     const float *B = row + L::BODIES_OFF;
     const float hull_x = B[IDX_X], hull_y = B[IDX_Y], hull_angle_rad = B[IDX_ANGLE];
     const float lidar_range = (float)LIDAR_RANGE;
@@ -135,12 +154,21 @@ MRL_DEV float lidar_value_part(const float *row, int i, int part, int nparts) {
     const float rdx = cs * lidar_range, rdy = sn * lidar_range;
     if (!(hull_x == hull_x)) return part == 0 ? lidar_ray<L>(row, hull_x, hull_y, rdx, rdy) : 1.0f;
     const float end_x = hull_x + rdx;
-    const float lo = hull_x < end_x ? hull_x : end_x, hi = hull_x < end_x ? end_x : hull_x;
-    if (!(lo == lo && hi == hi)) return part == 0 ? lidar_ray<L>(row, hull_x, hull_y, rdx, rdy) : 1.0f;
-    constexpr int W = EdgeMask<L>::WORDS;
+    if (!(end_x == end_x)) return part == 0 ? lidar_ray<L>(row, hull_x, hull_y, rdx, rdy) : 1.0f;
     EdgeMask<L> mine;
-    edges_near<L>(row, lo, hi, 0.02f, mine, part * W / nparts, (part + 1) * W / nparts);
-    return lidar_ray_near<L>(row, mine, hull_x, hull_y, rdx, rdy);
+#pragma unroll
+    for (int q = 0; q < EdgeMask<L>::WORDS; ++q) {
+        // bits k of word q with (32 q + k) % NPARTS == part
+        unsigned share;
+        if (NPARTS == 2) {
+            share = part ? 0xaaaaaaaau : 0x55555555u;
+        } else {
+            const int j = (part + q) % 3;    // 32 q + k = part (mod 3)  <=>  k = part + q (mod 3)
+            share = j == 0 ? 0x49249249u : (j == 1 ? 0x92492492u : 0x24924924u);
+        }
+        mine.w[q] = lidar_ray_pick<L>(row, near[q] & share, q, hull_x, rdx);
+    }
+    return lidar_ray_picked<L>(row, mine, hull_x, hull_y, rdx, rdy);
 }
 
 MRL_DEV void observe(float *row) {

@@ -96,6 +96,27 @@ struct EdgeMask {
 // the edges any such vertex passes, decided with the same fp32 bounds the pre-check uses.
 // widen = 0 gives exactly that; lidar passes its own safety margin on top.  Only the mask words
 // [q0, q1) are worked out (a caller that splits the edges over several lanes); the rest is zero.
+MRL_DEV bool edge_near(const float *E, float xlo, float xhi, float widen) {
+    const float e_x0 = E[0], e_x1 = E[2];
+    const float margin = 0.1f;
+    float x_min = e_x0 - margin, x_max = e_x1 + margin;
+    if (e_x0 > e_x1) { x_min = e_x1 - margin; x_max = e_x0 + margin; }
+    return !(xhi < x_min - widen || xlo > x_max + widen);
+}
+
+// bits 0 .. N - 1: the mask bits of edges e0 .. e0 + N - 1 (a caller that spreads one mask over many lanes)
+template <class L, int N>
+MRL_DEV unsigned edges_near_bits(const float *row, float xlo, float xhi, float widen, int e0) {
+    int n_edges = (int)row[L::EDGE_COUNT_OFF];
+    if (n_edges > L::MAX_EDGES) n_edges = L::MAX_EDGES;
+    const float *edges = row + L::EDGES_OFF;
+    unsigned bits = 0;
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+        bits |= (unsigned)(e0 + k < n_edges && edge_near(edges + (e0 + k) * 6, xlo, xhi, widen)) << k;
+    return bits;
+}
+
 template <class L>
 MRL_DEV void edges_near(const float *row, float xlo, float xhi, float widen, EdgeMask<L> &m, int q0 = 0,
                         int q1 = EdgeMask<L>::WORDS) {
@@ -116,11 +137,7 @@ MRL_DEV void edges_near(const float *row, float xlo, float xhi, float widen, Edg
             for (int j = 0; j < 8; ++j) {
                 const int k = k0 + j, e = e0 + k;
                 if (e >= L::MAX_EDGES) continue;
-                const float e_x0 = edges[e * 6], e_x1 = edges[e * 6 + 2];
-                const float margin = 0.1f;
-                float x_min = e_x0 - margin, x_max = e_x1 + margin;
-                if (e_x0 > e_x1) { x_min = e_x1 - margin; x_max = e_x0 + margin; }
-                bits |= (unsigned)!(xhi < x_min - widen || xlo > x_max + widen) << k;
+                bits |= (unsigned)edge_near(edges + e * 6, xlo, xhi, widen) << k;
             }
         }
         m.w[q] = bits & word_bits(n_edges - e0);
@@ -370,6 +387,41 @@ MRL_DEV float lidar_ray_near(const float *row, const EdgeMask<L> &near, float ox
             const float elo = x0 < x1 ? x0 : x1, ehi = x0 < x1 ? x1 : x0;
             if (ehi < rlo || elo > rhi) continue;
             lidar_edge(E, ox, oy, rdx, rdy, min_t);
+        }
+    }
+    return min_t;
+}
+
+// lidar_ray_near in two passes, for a caller that splits a ray's edges over several lanes: the
+// candidates `cand` of mask word q that pass the x-extent test of lidar_ray_near ...
+template <class L>
+MRL_DEV unsigned lidar_ray_pick(const float *row, unsigned cand, int q, float ox, float rdx) {
+    const float ex_ = ox + rdx;
+    const float rlo = (ox < ex_ ? ox : ex_) - 0.01f, rhi = (ox > ex_ ? ox : ex_) + 0.01f;
+    unsigned keep = 0;
+    while (cand) {
+        const int k = __ffs((int)cand) - 1;
+        cand &= cand - 1;
+        const float *E = row + L::EDGES_OFF + (q * 32 + k) * 6;
+        const float x0 = E[0], x1 = E[2];
+        const float elo = x0 < x1 ? x0 : x1, ehi = x0 < x1 ? x1 : x0;
+        if (!(ehi < rlo || elo > rhi)) keep |= 1u << k;
+    }
+    return keep;
+}
+// ... and the ray against exactly those.  Lanes that walk unequal candidate sets together spend the
+// intersection test only as often as the longest picked set asks, not once per candidate of any lane.
+template <class L>
+MRL_DEV float lidar_ray_picked(const float *row, const EdgeMask<L> &picked, float ox, float oy, float rdx,
+                               float rdy) {
+    float min_t = 1.0f;
+#pragma unroll
+    for (int q = 0; q < EdgeMask<L>::WORDS; ++q) {
+        unsigned mask = picked.w[q];
+        while (mask) {
+            const int e = q * 32 + __ffs((int)mask) - 1;
+            mask &= mask - 1;
+            lidar_edge(row + L::EDGES_OFF + e * 6, ox, oy, rdx, rdy, min_t);
         }
     }
     return min_t;
