@@ -143,7 +143,7 @@ MRL_DEV void lidar_near_share(const float *row, int slot, unsigned *words) {
 // are grouped).  lidar_ray_pick looks at each edge's extent against the ray's own, as lidar_ray_near does.
 template <int NPARTS>
 MRL_DEV float lidar_value_part(const float *row, int i, int part, const unsigned *near) {
-    static_assert(NPARTS == 2 || NPARTS == 3, "share masks for two or three parts");
+    static_assert(NPARTS >= 2 && NPARTS <= 4, "share masks for two to four parts");
     const float *B = row + L::BODIES_OFF;
     const float hull_x = B[IDX_X], hull_y = B[IDX_Y], hull_angle_rad = B[IDX_ANGLE];
     const float lidar_range = (float)LIDAR_RANGE;
@@ -162,6 +162,8 @@ MRL_DEV float lidar_value_part(const float *row, int i, int part, const unsigned
         unsigned share;
         if (NPARTS == 2) {
             share = part ? 0xaaaaaaaau : 0x55555555u;
+        } else if (NPARTS == 4) {
+            share = 0x11111111u << part;
         } else {
             const int j = (part + q) % 3;    // 32 q + k = part (mod 3)  <=>  k = part + q (mod 3)
             share = j == 0 ? 0x49249249u : (j == 1 ? 0x92492492u : 0x24924924u);
@@ -311,10 +313,27 @@ MRL_DEV void reset_row_wave(float *row, uint64_t cseed, int lane) {
                           MOTORS_TORQUE);
     }
     wave_sync();
-    // observation: lanes 0 .. 9 one lidar ray each, lane 10 the rest
-    if (lane < 10) {
-        row[14 + lane] = lidar_value(row, lane, nullptr);
-    } else if (lane == 10) {
+    // observation: the edges within lidar range of the hull, two tested per lane; then lane 4 r + p takes
+    // part p of ray r's edges and the four of a ray exchange their minima; lane 40 the rest
+    unsigned near[EdgeMask<L>::WORDS];
+    {
+        const float hull_x = B[IDX_X], lidar_range = (float)LIDAR_RANGE;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const unsigned long long m = __ballot(edges_near_bits<L, 1>(row, hull_x - lidar_range, hull_x + lidar_range, 0.02f, lane + 64 * h) != 0u);
+            near[2 * h] = (unsigned)m;
+            near[2 * h + 1] = (unsigned)(m >> 32);
+        }
+    }
+    if (lane < 40) {
+        float t = lidar_value_part<4>(row, lane >> 2, lane & 3, near);
+#pragma unroll
+        for (int off = 1; off <= 2; off <<= 1) {
+            const float other = __shfl_xor(t, off, 64);
+            t = other < t ? other : t;
+        }
+        if ((lane & 3) == 0) row[14 + (lane >> 2)] = t;
+    } else if (lane == 40) {
         float o[14];
         observe_state(row, o);
 #pragma unroll
