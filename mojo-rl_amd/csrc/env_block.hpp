@@ -64,7 +64,8 @@ struct LunarLander {
     }
     // contact detection runs beside the engines of wavefront 0: every half of wavefronts 1 .. 7
     // takes one (body, vertex) pair of the block's 32 envs -- hull 6 vertices, legs 4 each
-    static constexpr int DETECT_TASKS = 14;
+    static constexpr int DETECT_TASKS = 14, DETECT_WORDS = 0;
+    static MRL_DEV void detect_share(const float *, const float *, int, unsigned *) {}
     static MRL_DEV void detect_task(int k, int &body, int &vertex, int &max_verts) {
         if (k < 6) { body = 0; vertex = k; max_verts = 6; }
         else if (k < 10) { body = 1; vertex = k - 6; max_verts = 4; }
@@ -134,6 +135,11 @@ struct BipedalWalker {
     // contact detection ahead of the step, spread over all wavefronts: one (body, vertex) pair of
     // one env per lane -- hull 5 vertices, the four leg segments 4 each, against the 128 edges
     static constexpr int DETECT_TASKS = 21;
+    // ahead of the pairs, once per env and by all its lanes: the mask of the edges near any of its bodies
+    static constexpr int DETECT_WORDS = EdgeMask<L>::WORDS;
+    static MRL_DEV void detect_share(const float *row, const float *shapes, int slot, unsigned *words) {
+        bw::detect_near_share<THREADS / EPB, EPB>(row, shapes, slot, words);
+    }
     static MRL_DEV void detect_task(int k, int &body, int &vertex, int &max_verts) {
         if (k < 5) { body = 0; vertex = k; max_verts = 5; }
         else { body = 1 + (k - 5) / 4; vertex = (k - 5) % 4; max_verts = 4; }
@@ -175,7 +181,8 @@ struct HalfCheetah {
     static MRL_DEV void reset(float *row, uint64_t seed, int env) { hc::reset_row(row, walker_seed(seed, env)); }
     static constexpr bool WAVE_RESET = false;
     static MRL_DEV void reset_wave(float *, uint64_t, int, int) {}
-    static constexpr int DETECT_TASKS = 0;
+    static constexpr int DETECT_TASKS = 0, DETECT_WORDS = 0;
+    static MRL_DEV void detect_share(const float *, const float *, int, unsigned *) {}
     static MRL_DEV void detect_task(int, int &, int &, int &) {}
     struct Carry {};
     static MRL_DEV Carry step_begin(float *, int, const float *, const float *) { return Carry{}; }
@@ -317,12 +324,13 @@ constexpr int DETECT_STRIDE = detect_stride(DETECT_CAP);
 
 // task `task` of env slot e: detects into its list and records the count
 template <class E, int CAP = DETECT_CAP>
-MRL_DEV void detect_vertex_task(const float *rows, const float *shapes, float *dlist, int *dcount, int task, int e) {
+MRL_DEV void detect_vertex_task(const float *rows, const float *shapes, float *dlist, int *dcount, int task, int e,
+                                const unsigned *near = nullptr) {
     int body, vertex, max_verts;
     E::detect_task(task, body, vertex, max_verts);
     dcount[task * E::EPB + e] = edge_detect_vertex<typename E::L>(
         rows + e * Stage<E>::STRIDE, shapes, body, vertex, max_verts, dlist + (task * E::EPB + e) * detect_stride(CAP),
-        CAP);
+        CAP, near);
 }
 
 // concatenates env slot e's lists in (body, vertex) order into `mine`, cut at MAX_CONTACTS;
@@ -425,9 +433,17 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
             constexpr int SLOTS = E::THREADS / E::EPB;
             const int e = tid % E::EPB;
             if (tid < nenv) carry = E::step_begin(rows + tid * S::STRIDE, env0 + tid, actions + (size_t)tid * E::ACT_W, shapes);
+            // (what the pairs of an env share goes behind the contact counts: detect_count_ints)
+            const unsigned *near = nullptr;
+            if constexpr (E::DETECT_WORDS > 0) {
+                unsigned *words = reinterpret_cast<unsigned *>(dcount + E::DETECT_TASKS * E::EPB + 1) + e * E::DETECT_WORDS;
+                if (e < nenv) E::detect_share(rows + e * S::STRIDE, shapes, tid / E::EPB, words);
+                __syncthreads();
+                near = words;
+            }
             if (e < nenv)
                 for (int task = tid / E::EPB; task < E::DETECT_TASKS; task += SLOTS)
-                    detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
+                    detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e, near);
             __syncthreads();
         }
         int lanes_n = 0;          // LANES_PHYSICS: the env's contact count; -1: the one-lane form steps this env
@@ -510,6 +526,10 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
         }
     }
 }
+
+// LDS ints of phys_step_block's contact counts: one per list (and one spare), then what an env's tasks share
+template <class E>
+constexpr int detect_count_ints() { return E::DETECT_TASKS * E::EPB + 1 + E::DETECT_WORDS * E::EPB; }
 
 // LDS floats of the per-task contact lists that phys_step_block needs (0: the env detects inline)
 template <class E, int CAP = DETECT_CAP>

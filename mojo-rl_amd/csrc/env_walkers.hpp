@@ -78,6 +78,7 @@ inline Shapes make_shapes() {
     rect_shape(s.v + 40, LOWER_W / 2, LOWER_H / 2, 0);
     rect_shape(s.v + 60, UPPER_W / 2, UPPER_H / 2, 0);
     rect_shape(s.v + 80, LOWER_W / 2, LOWER_H / 2, 0);
+    for (int k = 0; k < 5; ++k) shape_set_bounds(s.v + k * SHAPE_SIZE);
     return s;
 }
 
@@ -117,6 +118,21 @@ MRL_DEV float lidar_value(const float *row, int i, const EdgeMask<L> *near) {
     EdgeMask<L> mine;
     edges_near<L>(row, hull_x - lidar_range, hull_x + lidar_range, 0.02f, mine);
     return lidar_ray_near<L>(row, mine, hull_x, hull_y, cs * lidar_range, sn * lidar_range);
+}
+
+// Ahead of contact detection by one lane per (body, vertex), once per env and by all its `SLOTS` lanes: the
+// mask of the edges near any of its bodies (words = the env's WORDS mask words); lanes and stores as
+// in lidar_near_share.
+template <int SLOTS, int EPB>
+MRL_DEV void detect_near_share(const float *row, const float *shapes, int slot, unsigned *words) {
+    constexpr int PER = L::MAX_EDGES / SLOTS;
+    static_assert(PER * SLOTS == L::MAX_EDGES && 4 * EPB == 64 && 4 * PER == 16, "sixteen mask bits per wavefront");
+    float xlo, xhi;
+    bodies_x_interval<L>(row, shapes, xlo, xhi);
+    unsigned b = edges_near_bits<L, PER>(row, xlo, xhi, 0.0f, slot * PER) << (PER * (slot & 3));
+    b |= __shfl_xor(b, EPB, 64);
+    b |= __shfl_xor(b, 2 * EPB, 64);
+    if ((slot & 3) == 0) reinterpret_cast<unsigned short *>(words)[slot >> 2] = (unsigned short)b;
 }
 
 // The lidar rays of an env spread over the lanes of a block.

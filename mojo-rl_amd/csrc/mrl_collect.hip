@@ -59,7 +59,7 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     __shared__ float hTc[H * HT_LD];   // the critic's activation tile (live during the env step)
     // the actor's activation tile and the env step's contact scratch are never live together
     constexpr int LIST_F = detect_list_floats<E>() + 1;
-    constexpr int ENV_F = PR * S::CSTRIDE + LIST_F + E::DETECT_TASKS * E::EPB + 1;
+    constexpr int ENV_F = PR * S::CSTRIDE + LIST_F + detect_count_ints<E>();
     __shared__ float overlay[cmax<H * HT_LD, ENV_F>()];
     float *cts = overlay, *dlist = cts + PR * S::CSTRIDE;
     int *dcount = reinterpret_cast<int *>(dlist + LIST_F);
@@ -256,7 +256,7 @@ __global__ __launch_bounds__(256, 2) void collect16_kernel(CollectArgs a) {
     __shared__ float hTc[H * HT16_LD];              // the critic's activation tile (live during the env step)
     // the actor's activation tile and the env step's contact scratch are never live together
     constexpr int LIST_F = detect_list_floats<E, CAP>() + 1;
-    constexpr int ENV_F = R * S::CSTRIDE + LIST_F + E::DETECT_TASKS * R + 1;
+    constexpr int ENV_F = R * S::CSTRIDE + LIST_F + detect_count_ints<E>();
     __shared__ float overlay[cmax<H * HT16_LD, ENV_F>()];
     float *cts = overlay, *dlist = cts + R * S::CSTRIDE;
     int *dcount = reinterpret_cast<int *>(dlist + LIST_F);

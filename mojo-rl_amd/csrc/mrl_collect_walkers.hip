@@ -161,7 +161,7 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
     __shared__ unsigned sync_actor, sync_critic, sync_failed;   // barriers of the actor's and the critic's wavefronts
     // the two activation tiles and the env step's scratch (contact lists) are never live together
     constexpr int LIST_F = detect_list_floats<E>() + 1;
-    constexpr int ENV_F = R * S::CSTRIDE + LIST_F + E::DETECT_TASKS * R + 1;
+    constexpr int ENV_F = R * S::CSTRIDE + LIST_F + detect_count_ints<E>();
     __shared__ float overlay[wmax<2 * H * HT16_LD, ENV_F>()];
     static_assert(R * S::CSTRIDE <= H * HT16_LD, "the solver's contact scratch stays below the critic's tile");
     float *cts = overlay, *dlist = cts + R * S::CSTRIDE;

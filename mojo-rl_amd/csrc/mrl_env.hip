@@ -109,7 +109,7 @@ __global__ __launch_bounds__(E::THREADS) void phys_step_kernel(float *states, co
     __shared__ float shapes[E::NSHAPE];
     __shared__ unsigned long long was_reset;   // rows re-initialised by this launch, one bit each
     __shared__ float dlist[detect_list_floats<E>() + 1];
-    __shared__ int dcount[E::DETECT_TASKS * E::EPB + 1];
+    __shared__ int dcount[detect_count_ints<E>()];
     const int tid = threadIdx.x;
     const int env0 = blockIdx.x * E::EPB;
     const int nenv = min(E::EPB, batch - env0);

@@ -117,6 +117,44 @@ MRL_DEV unsigned edges_near_bits(const float *row, float xlo, float xhi, float w
     return bits;
 }
 
+// Slots 18 and 19 of a polygon shape (past its eight vertices) may hold max |x| and max |y| over its
+// local vertices; a table whose shapes all carry them lets bodies_x_interval bound an env's vertices
+// without visiting them.
+constexpr int SHAPE_BOUND_X = 18, SHAPE_BOUND_Y = 19;
+static_assert(2 + 2 * MAX_POLY_VERTS <= SHAPE_BOUND_X && SHAPE_BOUND_Y < SHAPE_SIZE, "free slots of a shape");
+inline void shape_set_bounds(float *S) {
+    float bx = 0.0f, by = 0.0f;
+    for (int v = 0; v < (int)S[1] && v < MAX_POLY_VERTS; ++v) {
+        const float ax = S[2 + 2 * v] < 0.0f ? -S[2 + 2 * v] : S[2 + 2 * v];
+        const float ay = S[3 + 2 * v] < 0.0f ? -S[3 + 2 * v] : S[3 + 2 * v];
+        bx = ax > bx ? ax : bx;
+        by = ay > by ? ay : by;
+    }
+    S[SHAPE_BOUND_X] = bx;
+    S[SHAPE_BOUND_Y] = by;
+}
+
+// An x interval that holds every polygon vertex of the row's bodies.  A vertex sits at
+// fl(fl(x + fl(lx cos)) - fl(ly sin)); |fl(lx cos)| <= max |lx| and |fl(ly sin)| <= max |ly| (sine and
+// cosine are at most 1 and rounding is monotone), so the same two additions with the bounds in
+// place of the products enclose it, again because rounding is monotone.  A NaN centre gives the
+// whole axis (a NaN coordinate passes the pre-check of every edge).
+template <class L>
+MRL_DEV void bodies_x_interval(const float *row, const float *shapes, float &xlo, float &xhi) {
+    xlo = 3.0e38f; xhi = -3.0e38f;
+    bool odd = false;
+#pragma unroll
+    for (int b = 0; b < L::NUM_BODIES; ++b) {
+        const float *B = row + L::BODIES_OFF + b * BODY_SIZE;
+        const float *S = shapes + (int)B[IDX_SHAPE] * SHAPE_SIZE;
+        const float x = B[IDX_X], lo = (x - S[SHAPE_BOUND_X]) - S[SHAPE_BOUND_Y], hi = (x + S[SHAPE_BOUND_X]) + S[SHAPE_BOUND_Y];
+        odd = odd || !(lo == lo) || !(hi == hi);
+        xlo = lo < xlo ? lo : xlo;
+        xhi = hi > xhi ? hi : xhi;
+    }
+    if (odd) { xlo = -3.0e38f; xhi = 3.0e38f; }
+}
+
 template <class L>
 MRL_DEV void edges_near(const float *row, float xlo, float xhi, float widen, EdgeMask<L> &m, int q0 = 0,
                         int q1 = EdgeMask<L>::WORDS) {
@@ -268,9 +306,11 @@ MRL_DEV int edge_detect(const float *row, const float *shapes, float *contacts) 
 // -1 when the caller has to fall back to edge_detect: the body is not a polygon of at most
 // max_verts vertices (the caller planned one lane per vertex for that many), or the vertex
 // touched `cap` edges or more (the list holds cap records; the last one only signals overflow).
+// near != nullptr: the mask words of the edges whose pre-check can pass for some vertex of the env
+// (edges_near_bits over bodies_x_interval), worked out once for all its vertices.
 template <class L>
 MRL_DEV int edge_detect_vertex(const float *row, const float *shapes, int b, int v, int max_verts,
-                               float *contacts, int cap) {
+                               float *contacts, int cap, const unsigned *near = nullptr) {
     const float *B = row + L::BODIES_OFF + b * BODY_SIZE;
     const float *S = shapes + (int)B[IDX_SHAPE] * SHAPE_SIZE;
     int n_verts = (int)S[1];
@@ -291,10 +331,22 @@ MRL_DEV int edge_detect_vertex(const float *row, const float *shapes, int b, int
     for (int q = 0; q < (L::MAX_EDGES + 31) / 32; ++q) {
         // (all slots tested, the word cut to the existing edges afterwards: see edges_near)
         unsigned mask = 0;
+        if (near != nullptr) {
+            // only the edges the caller found near the env's bodies at all; the vertex's own
+            // survivors are picked first, so that lanes with unequal sets share the full tests
+            unsigned cand = near[q];
+            while (cand) {
+                const int k = __ffs((int)cand) - 1;
+                cand &= cand - 1;
+                const int e = q * 32 + k;
+                if (edge_x_pass(edges[e * 6], edges[e * 6 + 2], world_x)) mask |= 1u << k;
+            }
+        } else {
 #pragma unroll
-        for (int k = 0; k < 32; ++k) {
-            const int e = q * 32 + k;
-            if (e < L::MAX_EDGES) mask |= (unsigned)edge_x_pass(edges[e * 6], edges[e * 6 + 2], world_x) << k;
+            for (int k = 0; k < 32; ++k) {
+                const int e = q * 32 + k;
+                if (e < L::MAX_EDGES) mask |= (unsigned)edge_x_pass(edges[e * 6], edges[e * 6 + 2], world_x) << k;
+            }
         }
         mask &= word_bits(n_edges - q * 32);
         while (mask) {
