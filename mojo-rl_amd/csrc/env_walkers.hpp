@@ -273,14 +273,31 @@ MRL_DEV void reset_row_wave(float *row, uint64_t cseed, int lane) {
     }
     wave_sync();
     if (lane == 0) {
+        // the heights are one serial chain; sixteen steps at a time between registers, so that no
+        // step waits for an LDS access
         float y = (float)TERRAIN_HEIGHT, velocity = 0.0f;
-        for (int i = 0; i <= N_EDGES; ++i) {
+        constexpr int CH = 16;
+        static_assert(N_EDGES % CH == 0, "whole chunks, then the last step");
+        auto step = [&](int i, float noise) {
             const float terrain_height = (float)TERRAIN_HEIGHT;
             velocity = 0.8f * velocity + 0.01f * (terrain_height > y ? 1.0f : -1.0f);
-            if (i > TERRAIN_STARTPAD) velocity = velocity + tmp[i];
+            if (i > TERRAIN_STARTPAD) velocity = velocity + noise;
             y = y + velocity;
-            tmp[YS + i] = y;
+        };
+        for (int i0 = 0; i0 < N_EDGES; i0 += CH) {
+            float nz[CH], ys[CH];
+#pragma unroll
+            for (int j = 0; j < CH; ++j) nz[j] = i0 + j > TERRAIN_STARTPAD ? tmp[i0 + j] : 0.0f;
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                step(i0 + j, nz[j]);
+                ys[j] = y;
+            }
+#pragma unroll
+            for (int j = 0; j < CH; ++j) tmp[YS + i0 + j] = ys[j];
         }
+        step(N_EDGES, tmp[N_EDGES]);
+        tmp[YS + N_EDGES] = y;
     }
     wave_sync();
     float ya[2], yb[2];   // this lane's edges lane and lane + 64: heights at both ends
