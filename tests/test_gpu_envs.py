@@ -547,6 +547,59 @@ def test_bipedal_walker_rows_with_other_wiring_take_the_one_lane_form(mrl, orc, 
             assert np.median(gap[::2]) > 0.3 and np.median(gap[1::2]) < 0.05
 
 
+def test_bipedal_walker_bodies_strewn_over_the_terrain(mrl, orc, ctx):
+    """Contact detection picks, once per env, the terrain edges near any of its bodies and each (body, vertex)
+    pair then looks only at those: rows whose bodies lie metres apart (with the joints, which then pull them
+    together violently, and without), rows with a NaN or infinite body position and ordinary rows side by
+    side must all match the oracle bit for bit, contacts of the far bodies included."""
+    def same(a, b, what):
+        # bit for bit, except that a NaN matches any NaN (host and GPU differ in the sign of a generated NaN)
+        a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)
+        bad = (a.view(np.uint32) != b.view(np.uint32)) & ~(np.isnan(a) & np.isnan(b))
+        assert not bad.any(), "%s: %d of %d floats differ, first at %s: %r vs %r" % (
+            what, int(bad.sum()), bad.size, np.argwhere(bad)[0], a[bad][0], b[bad][0])
+
+    batch = 96
+    E = mrl.BipedalWalkerV2
+    s_h = np.zeros((batch, 950), np.float32)
+    orc.orc_bw_reset_batch(s_h, None, batch, 21)
+    BODIES, JOINT_COUNT = 24, 24 + 65 + 15 + 68
+    rng = np.random.default_rng(21)
+    for i in range(batch):
+        kind = i % 4
+        if kind == 3:
+            continue
+        for b in range(5):
+            s_h[i, BODIES + 13 * b] += np.float32((b - 1) * rng.uniform(3.0, 9.0))     # x: up to 27 m to the right, one 9 m to the left
+            s_h[i, BODIES + 13 * b + 1] -= np.float32(rng.uniform(0.0, 0.6))              # y: towards / into the ground
+            s_h[i, BODIES + 13 * b + 2] = np.float32(rng.uniform(-3.0, 3.0))              # angle
+        if kind == 1:
+            s_h[i, JOINT_COUNT] = 0.0
+        if kind == 2 and i % 8 == 2:
+            s_h[i, BODIES + 13 * (i % 5)] = np.float32(np.nan if i % 16 == 2 else np.inf)
+    s = dev(s_h.reshape(-1))
+    a, r, d, o = (torch.zeros(n, device="cuda") for n in (batch * 4, batch, batch, batch * 24))
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 24), np.float32)
+    touched = 0
+    for t in range(12):
+        act = rng.uniform(-1.2, 1.2, (batch, 4)).astype(np.float32)
+        a.copy_(dev(act.reshape(-1)))
+        E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+        orc.orc_bw_step_batch(s_h, act, r_h, d_h, o_h, batch, 4)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 950)
+        same(sg, s_h, "state, step %d" % t)
+        same(r.cpu().numpy(), r_h, "reward, step %d" % t)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        same(o.cpu().numpy().reshape(batch, 24), o_h, "observation, step %d" % t)
+        s_h[:] = sg
+        if t == 0:
+            # the far legs did touch the ground: their contact flags in the observation
+            touched = int((o_h[:, 8] > 0.5).sum() + (o_h[:, 13] > 0.5).sum())
+    say("  leg contact flags set after the first step: %d" % touched)
+    assert touched > 10
+
+
 @pytest.mark.parametrize("name", ["CartPoleEnv", "PendulumV2", "BipedalWalkerV2", "HalfCheetahPlanarV2",
                                   "LunarLanderV2Continuous"])
 def test_autoreset_equals_step_then_selective_reset(mrl, ctx, name):
