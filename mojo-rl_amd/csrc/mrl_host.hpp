@@ -68,7 +68,7 @@ struct Accounting {
     int32_t *done_count;
     int32_t done_cap;
     // the same accounting seen from env i: per-env pointers advanced, the shared list untouched
-    __host__ __device__ Accounting at(int i) const {
+    __host__ __device__ __forceinline__ Accounting at(int i) const {
         Accounting a = *this;
         if (r_rewards != nullptr) {
             a.r_rewards += i; a.r_dones += i; a.ep_return += i; a.ep_length += i;
