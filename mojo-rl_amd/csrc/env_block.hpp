@@ -367,6 +367,35 @@ MRL_DEV int merge_vertex_lists(const float *dlist, const int *dcount, int e, flo
     return redo ? -1 : n;
 }
 
+// merge_vertex_lists by the lanes that made the lists: the lane of (env slot e, task) moves its own list to
+// its place in the env's merged list -- behind the contacts of the tasks before it -- so that all lists move
+// at once.  Returns what merge_vertex_lists returns (every lane of the env gets the same value).
+template <class E, int CAP = DETECT_CAP>
+MRL_DEV int merge_vertex_list_of_task(const float *dlist, const int *dcount, int e, int task, float *mine) {
+    int m[E::DETECT_TASKS];
+#pragma unroll
+    for (int k = 0; k < E::DETECT_TASKS; ++k) m[k] = dcount[k * E::EPB + e];
+    bool redo = false;
+    int before = 0, total = 0, own = 0;
+#pragma unroll
+    for (int k = 0; k < E::DETECT_TASKS; ++k) {
+        redo |= m[k] < 0;
+        const int c = m[k] < 0 ? 0 : (m[k] < CAP ? m[k] : CAP);
+        before += k < task ? c : 0;
+        own = k == task ? c : own;
+        total += c;
+    }
+    const float *src = dlist + (task * E::EPB + e) * detect_stride(CAP);
+    for (int c = 0; c < own && before + c < E::L::MAX_CONTACTS; ++c) {
+        float rec[CONTACT_SIZE];
+#pragma unroll
+        for (int f = 0; f < CONTACT_SIZE; ++f) rec[f] = src[c * CONTACT_SIZE + f];
+#pragma unroll
+        for (int f = 0; f < CONTACT_SIZE; ++f) mine[(before + c) * CONTACT_SIZE + f] = rec[f];
+    }
+    return redo ? -1 : (total < E::L::MAX_CONTACTS ? total : E::L::MAX_CONTACTS);
+}
+
 // One step of the block's LDS-resident rows (all threads of the block call it, between two
 // __syncthreads of the caller): wavefront 0 steps one env per lane, the other wavefronts detect
 // contacts where the env splits that off.  `actions` = the actions of the block's envs
@@ -452,20 +481,26 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
             // LANES_PER_ENV lanes per env (the first wavefronts of the block) run the solver, then the env's
             // lane goes on below with what follows the physics
             static_assert(E::DETECT_TASKS > 0 && E::EPB * E::LANES_PER_ENV <= E::THREADS, "a lane group per env");
-            if (tid < nenv) {
-                const int n = merge_vertex_lists<E>(dlist, dcount, tid, cts + tid * S::CSTRIDE);
-                dcount[tid] = (n >= 0 && E::lanes_ok(rows + tid * S::STRIDE)) ? n : -1;   // (the counts are spent)
+            // (the env's contact count goes where its tasks' shared words were: they are spent, the counts are not yet)
+            static_assert(E::DETECT_WORDS >= 1 && E::DETECT_TASKS <= E::THREADS / E::EPB, "a word per env, a lane per task");
+            int *ncontacts = dcount + E::DETECT_TASKS * E::EPB + 1;
+            {
+                const int e = tid % E::EPB, task = tid / E::EPB;
+                if (e < nenv && task < E::DETECT_TASKS) {
+                    const int n = merge_vertex_list_of_task<E>(dlist, dcount, e, task, cts + e * S::CSTRIDE);
+                    if (task == 0) ncontacts[e] = (n >= 0 && E::lanes_ok(rows + e * S::STRIDE)) ? n : -1;
+                }
             }
             __syncthreads();
             const int slot = tid / E::LANES_PER_ENV;
             if (slot < nenv) {
-                const int n = dcount[slot];
+                const int n = ncontacts[slot];
                 if (n >= 0) E::physics_lanes(rows + slot * S::STRIDE, cts + slot * S::CSTRIDE, n, tid % WAVE);
             }
             static_assert(E::EPB * E::LANES_PER_ENV <= 2 * WAVE, "the solver's lanes are wavefronts 0 and 1");
             if (tid >= 2 * WAVE) side(tid);
             __syncthreads();
-            if (tid < nenv) lanes_n = dcount[tid];
+            if (tid < nenv) lanes_n = ncontacts[tid];
         }
         if (tid < WAVE) {
             bool finished = false;
