@@ -374,26 +374,33 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
     }
     stage_head(params + IN * H + H + H * H + H, H, A, GAUSS, w2s, t, T);
     for (int i = t; i < PR * (2 * PA_MAX + 1); i += T) g2s[i] = 0.0f;
-    // the loss lane of row t (wavefront 0) asks for its row's rollout entries now
+    // The loss lanes ask for their rows' rollout entries now.  Critic: the lane of row t (wavefront 0).
+    // Actor: eight lanes per row, lane lj on logit / action component lj (rows lr, lr + T / 8, ...), so
+    // that a row's exponentials and logarithms are taken side by side instead of one after the other.
+    static_assert(PA_MAX == 8 && T % 8 == 0, "eight lanes per row");
+    constexpr int LR = (PR + T / 8 - 1) / (T / 8);   // rows per actor loss lane (lanes past the tile's rows idle)
     const bool loss_lane = t < nrow;
-    const long src = loss_lane ? fl.idx[row0 + t] : 0;
-    float l_adv = 0.0f, l_logp = 0.0f, l_ret = 0.0f, l_val = 0.0f, l_mean = 0.0f, l_std = 1.0f, l_act[PA_MAX];
-#pragma unroll
-    for (int j = 0; j < PA_MAX; ++j) l_act[j] = 0.0f;
-    if (loss_lane) {
-        if (blockIdx.y == 1) {
+    const int lr = t >> 3, lj = t & 7;
+    float l_ret = 0.0f, l_val = 0.0f, l_mean = 0.0f, l_std = 1.0f;
+    float l_adv[LR], l_logp[LR], l_act[LR];   // l_act: the action (discrete) or its component lj
+    if (blockIdx.y == 1) {
+        if (loss_lane) {
+            const long src = fl.idx[row0 + t];
             l_ret = fl.r_ret[src];
             if (fl.clip_value) l_val = fl.r_val[src];
-        } else {
-            l_adv = fl.r_adv[src];
-            l_logp = fl.r_logp[src];
-            if (fl.adv_stats != nullptr) { l_mean = fl.adv_stats[0]; l_std = fl.adv_stats[1]; }
-            if (fl.continuous) {
+        }
+    } else {
+        if (fl.adv_stats != nullptr) { l_mean = fl.adv_stats[0]; l_std = fl.adv_stats[1]; }
 #pragma unroll
-                for (int j = 0; j < PA_MAX; ++j)
-                    if (j < A) l_act[j] = fl.r_act[src * A + j];
-            } else {
-                l_act[0] = fl.r_act[src];
+        for (int q = 0; q < LR; ++q) {
+            const int r = lr + q * (T / 8);
+            l_adv[q] = 0.0f; l_logp[q] = 0.0f; l_act[q] = 0.0f;
+            if (r < nrow) {
+                const long src = fl.idx[row0 + r];
+                l_adv[q] = fl.r_adv[src];
+                l_logp[q] = fl.r_logp[src];
+                if (!fl.continuous) l_act[q] = fl.r_act[src];
+                else if (lj < A) l_act[q] = fl.r_act[src * A + lj];
             }
         }
     }
@@ -433,43 +440,59 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
     };
     fetch(0);
 
-    // ---- loss gradients of the tile's rows, one lane per row (wavefront 0), into g2s and out
-    float kl = 0.0f;
-    if (loss_lane) {
-        const int b = (int)row0 + t;
-        float *g2row = g2s + t * (2 * PA_MAX + 1);
-        if (blockIdx.y == 1) {   // critic
+    // ---- loss gradients of the tile's rows into g2s and out
+    if (blockIdx.y == 1) {   // critic: one lane per row
+        if (loss_lane) {
             const float g = critic_grad_value(ys[t * (PA_MAX + 1)], l_val, l_ret, fl.mb, fl.continuous, fl.clip_value,
                                               fl.value_coef, fl.clip_eps);
-            g2row[0] = g;
-            fl.g_values[b] = g;
-        } else {
-            float adv = l_adv;
+            g2s[t * (2 * PA_MAX + 1)] = g;
+            fl.g_values[(int)row0 + t] = g;
+        }
+    } else {
+        // (rows past nrow are worked on like the others -- their lanes take part in the exchanges -- and not stored)
+#pragma unroll
+        for (int q = 0; q < LR; ++q) {
+            const int r = lr + q * (T / 8), b = (int)row0 + r;
+            float *g2row = g2s + r * (2 * PA_MAX + 1);
+            float adv = l_adv[q];
             if (fl.adv_stats != nullptr) adv = (adv - l_mean) / (l_std + 1e-8f);
-            float o[2 * PA_MAX], g[2 * PA_MAX];
-            for (int a = 0; a < A; ++a) o[a] = ys[t * (PA_MAX + 1) + a];
+            const float mine = ys[(r < PR ? r : 0) * (PA_MAX + 1) + lj];
+            float kl;
             if (fl.continuous) {
-                for (int j = 0; j < A; ++j) o[A + j] = w2s[HEAD_LOG_STD(H) + j];   // clamped inside the gradient, as in the stored output
-                kl = actor_grad_gaussian_row(o, l_act, adv, l_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
+                float gm, gs;   // (log_std is clamped inside the gradient, as in the stored output)
+                kl = actor_grad_gaussian_lanes(mine, w2s[HEAD_LOG_STD(H) + lj], l_act[q], lj, lane & ~7, adv, l_logp[q], fl.mb,
+                                               A, fl.clip_eps, fl.ent_coef, gm, gs);
+                if (r < nrow && lj < A) {
+                    g2row[lj] = gm;
+                    g2row[A + lj] = gs;
+                    fl.g_actor_out[(size_t)b * ld + lj] = gm;
+                    fl.g_actor_out[(size_t)b * ld + A + lj] = gs;
+                }
             } else {
-                kl = actor_grad_discrete_row(o, (int)l_act[0], adv, l_logp, fl.mb, A, fl.clip_eps, fl.ent_coef, g);
+                float g;
+                kl = actor_grad_discrete_lanes(mine, lj, lane & ~7, (int)l_act[q], adv, l_logp[q], fl.mb, A, fl.clip_eps,
+                                               fl.ent_coef, g);
+                if (r < nrow && lj < A) {
+                    g2row[lj] = g;
+                    fl.g_actor_out[(size_t)b * ld + lj] = g;
+                }
             }
-            for (int j = 0; j < ld; ++j) {
-                g2row[j] = g[j];
-                fl.g_actor_out[(size_t)b * ld + j] = g[j];
+            if (r < nrow && lj == 0) {
+                fl.kl[b] = kl;
+                g2row[2 * PA_MAX] = kl;   // (the spare float of the row, for the tile's sum below)
             }
-            fl.kl[b] = kl;
         }
     }
+    __syncthreads();   // g2s complete
     if (fl.kl_flag != nullptr && blockIdx.y == 0 && t < 64) {
         // KL test: every actor tile leaves the sum of its rows' estimates; the kernel that applies the
         // update (clip + Adam) adds the tiles up and compares the mean with target_kl, so that nothing
         // here waits for other workgroups
+        float kl = t < nrow ? g2s[t * (2 * PA_MAX + 1) + 2 * PA_MAX] : 0.0f;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) kl += __shfl_xor(kl, off, 64);
         if (t == 0) fl.kl_part[blockIdx.x] = kl;
     }
-    __syncthreads();   // g2s complete
 
     // ---- back through the head and layer 1's activation, on the matrix cores; wavefront w owns
     // columns [32w, 32w + 32) of the hidden layers throughout

@@ -61,6 +61,41 @@ MRL_DEV float actor_grad_discrete_row(const float *l, int action, float advantag
     }
     return old - new_logp;
 }
+// actor_grad_discrete_row by eight lanes of a wavefront (lanes base .. base + 7, A <= 8), lane j on logit j:
+// every lane takes one exponential and one entropy logarithm instead of A of each; the sums run over the
+// lanes' values in the order the one-lane form adds them, so the bits are the same.  lj = logit j (anything
+// for j >= A); g_out = gradient slot j (0 for j >= A); every lane returns the sample's KL estimate.
+MRL_DEV float actor_grad_discrete_lanes(float lj, int j, int base, int action, float advantage, float old, int mb,
+                                        int A, float clip_eps, float ent_coef, float &g_out) {
+    float max_logit = __shfl(lj, base, 64);
+#pragma unroll
+    for (int a = 1; a < 8; ++a) {
+        const float la = __shfl(lj, base + a, 64);
+        if (a < A && la > max_logit) max_logit = la;
+    }
+    const float e = j < A ? exp32(lj - max_logit) : 0.0f;
+    float sum_exp = 0.0f, e_action = 0.0f;
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+        const float ea = __shfl(e, base + a, 64);
+        if (a < A) sum_exp = sum_exp + ea;
+        if (a < A && a == action) e_action = ea;
+    }
+    const float p_action = (action >= 0 && action < A) ? e_action / sum_exp : 0.0f;
+    const float new_logp = log32(p_action + 1e-8f);
+    const float ratio = exp32(new_logp - old);
+    const bool clipped = (ratio < 1.0f - clip_eps) || (ratio > 1.0f + clip_eps);
+    float g = 0.0f;
+    if (!clipped && j < A) {
+        float p = e / sum_exp;
+        float d_log_prob = (j == action) ? 1.0f - p : -p;
+        float log_prob_ent = log32(p + 1e-8f);
+        float d_entropy = -p * (1.0f + log_prob_ent);
+        g = (-advantage * ratio * d_log_prob - ent_coef * d_entropy) / (float)mb;
+    }
+    g_out = g;
+    return old - new_logp;
+}
 MRL_DEV float actor_grad_discrete_one(int b, const float *__restrict__ logits, const float *__restrict__ old_logp,
                                       const float *__restrict__ adv, const float *__restrict__ actions, int mb,
                                       int A, float clip_eps, float ent_coef, float *__restrict__ grad_logits) {
@@ -136,6 +171,52 @@ MRL_DEV float actor_grad_gaussian_one(int b, const float *__restrict__ actor_out
                                       int A, float clip_eps, float ent_coef, float *__restrict__ grad_out) {
     return actor_grad_gaussian_row(actor_out + (long)b * 2 * A, actions + (long)b * A, adv[b], old_logp[b], mb, A,
                                    clip_eps, ent_coef, grad_out + (long)b * 2 * A);
+}
+
+// actor_grad_gaussian_row by eight lanes of a wavefront (lanes base .. base + 7, A <= 8), lane j on action
+// component j (its mean, raw log_std and action; anything for j >= A): one exp(log_std) per lane, the
+// log-probability summed over the lanes' terms in component order.  gm / gs = gradient slots j and A + j.
+MRL_DEV float actor_grad_gaussian_lanes(float mean_j, float log_std_j, float act_j, int j, int base, float advantage,
+                                        float old_log_prob, int mb, int A, float clip_eps, float ent_coef, float &gm,
+                                        float &gs) {
+    const float eps = 1e-6f, log_2pi = (float)1.8378770664093453;
+    const float log_std = log_std_j < -5.0f ? -5.0f : (log_std_j > 2.0f ? 2.0f : log_std_j);
+    const float std = j < A ? exp32(log_std) : 1.0f;
+    float lg;
+    {
+        float an = (act_j - mean_j) / (std + eps);
+        lg = -0.5f * (log_2pi + 2.0f * log_std + an * an);
+    }
+    float new_log_prob = 0.0f;
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+        const float v = __shfl(lg, base + a, 64);
+        if (a < A) new_log_prob = new_log_prob + v;
+    }
+    float diff = new_log_prob - old_log_prob;
+    if (diff > 20.0f) diff = 20.0f;
+    else if (diff < -20.0f) diff = -20.0f;
+    float ratio = exp32(diff);
+    float kl = (ratio - 1.0f) - diff;
+    if (kl < 0.0f) kl = 0.0f;
+    else if (kl > 100.0f) kl = 100.0f;
+    float clipped_ratio = ratio;
+    if (clipped_ratio < 1.0f - clip_eps) clipped_ratio = 1.0f - clip_eps;
+    else if (clipped_ratio > 1.0f + clip_eps) clipped_ratio = 1.0f + clip_eps;
+    const bool is_clipped = clipped_ratio * advantage < ratio * advantage;
+    gm = 0.0f; gs = 0.0f;
+    if (!is_clipped && j < A) {
+        float an = (act_j - mean_j) / (std + eps);
+        float d_mean = an / (std + eps);
+        float d_log_std = an * an - 1.0f;
+        gm = (-advantage * ratio * d_mean) / (float)mb;
+        gs = (-advantage * ratio * d_log_std - ent_coef * 1.0f) / (float)mb;
+        if (gm > 10.0f) gm = 10.0f;
+        else if (gm < -10.0f) gm = -10.0f;
+        if (gs > 10.0f) gs = 10.0f;
+        else if (gs < -10.0f) gs = -10.0f;
+    }
+    return kl;
 }
 
 // ppo.mojo:538-633 (convention 0) and kernels.mojo:416-486 (convention 1)
