@@ -56,6 +56,7 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
     __shared__ float shapes[E::NSHAPE];
     __shared__ unsigned long long was_reset;
     __shared__ unsigned sync_critic, sync_detect, sync_failed;
+    __shared__ int ncontacts[PR];   // an env's contact count after the merge of its lists (-1: detect again)
     __shared__ float hTc[H * HT_LD];   // the critic's activation tile (live during the env step)
     // the actor's activation tile and the env step's contact scratch are never live together
     constexpr int LIST_F = detect_list_floats<E>() + 1;
@@ -108,7 +109,7 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
         // hidden stack meets three times per step, the detection once), so that nothing of them is
         // carried through the env step in registers
         WaveGroupSync critic_sync{&sync_critic, (unsigned)k * 3u * CRITIC_WAVES, (unsigned)CRITIC_WAVES, &sync_failed, a.spin_limit};
-        WaveGroupSync detect_sync{&sync_detect, (unsigned)k * (NW - 1), (unsigned)(NW - 1), &sync_failed, a.spin_limit};
+        WaveGroupSync detect_sync{&sync_detect, (unsigned)k * 2u * (NW - 1), (unsigned)(NW - 1), &sync_failed, a.spin_limit};
         // ---- actor, all wavefronts
         {
             HiddenOperands<H, 1, 32> ops;
@@ -149,14 +150,15 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
                 a.r_logp[row + lane] = logp;
                 carry = E::step_begin(rows + lane * S::STRIDE, i, act + lane * AW, shapes);
             }
-            detect_sync.target += detect_sync.nwaves;
+            // (the detecting wavefronts meet twice: lists complete, then every list moved to its place in its env's list)
+            detect_sync.target += 2 * detect_sync.nwaves;
             detect_sync.wait_for(detect_sync.target);
             bool finished = false;
             int slot = 0;
             float fin_return = 0.0f, fin_length = 0.0f;
             if (lane < ne) {
                 float *mine = cts + lane * S::CSTRIDE;
-                const int n = merge_vertex_lists<E>(dlist, dcount, lane, mine);
+                const int n = ncontacts[lane];
                 float r, d;
                 E::step_finish(rows + lane * S::STRIDE, mine, n, shapes, carry, r, d);
                 // rollout row t and the episode accounting of account(), on the running sums that
@@ -184,6 +186,13 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
             // ---- contact detection: one (body, vertex) task per half of wavefronts 1 .. 7
             const int task = (wave - 1) * 2 + lane / (WAVE / 2), e = lane % (WAVE / 2);
             if (task < E::DETECT_TASKS && e < ne) detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
+            // the lists are merged by the lanes that made them, all at once, instead of one after the other by
+            // the solver's wavefront: once every list of the block is in, each lane moves its own
+            detect_sync();
+            if (task < E::DETECT_TASKS && e < ne) {
+                const int n = merge_vertex_list_of_task<E>(dlist, dcount, e, task, cts + e * S::CSTRIDE);
+                if (task == 0) ncontacts[e] = n;
+            }
             detect_sync.arrive();
             if (wave != 4) {
                 // ---- critic, on its own barrier: member g = 0 .. 5 of the group is wavefront g + 1
