@@ -301,6 +301,23 @@ MRL_DEV void physics_lanes(float *row, float *contacts, int n, int lane) {
         Bp[IDX_X] = x; Bp[IDX_Y] = y; Bp[IDX_ANGLE] = ang; Bp[IDX_VX] = vx; Bp[IDX_VY] = vy; Bp[IDX_OMEGA] = w;
         row[L::FORCES_OFF + b * 3] = 0.0f; row[L::FORCES_OFF + b * 3 + 1] = 0.0f; row[L::FORCES_OFF + b * 3 + 2] = 0.0f;
     }
+    // ---- observation entries 0 .. 7 and 9 .. 12 (observe_state: the same expressions on the same values), every
+    // body's lane its own: the hull 0 .. 3, a leg segment its angle and angular velocity against its parent's.
+    // The contact flags (8, 13) and the lidar are left to what follows (step_tail<false, false>).
+    {
+        const double p_ang = (double)from_parent(ang, b), p_w = (double)from_parent(w, b);
+        if (b == 0) {
+            const double hull_angle = ang, hull_omega = w, hull_vx = vx, hull_vy = vy;
+            row[0] = (float)hull_angle;
+            row[1] = (float)(hull_omega / 5.0);
+            row[2] = (float)(hull_vx * (600.0 / SCALE) / FPS);
+            row[3] = (float)(hull_vy * (400.0 / SCALE) / FPS);
+        } else if (b <= 4) {
+            const int leg = (b - 1) >> 1, at = 4 + 5 * leg + (((b - 1) & 1) ? 2 : 0);
+            row[at] = (float)(((double)ang - p_ang) / 1.0);
+            row[at + 1] = (float)(((double)w - p_w) / 10.0);
+        }
+    }
 }
 
 }  // namespace bw

@@ -161,7 +161,7 @@ struct BipedalWalker {
     static MRL_DEV bool lanes_ok(const float *row) { return bw::lanes_row_ok(row); }
     static MRL_DEV void physics_lanes(float *row, float *cts, int n, int lane) { bw::physics_lanes(row, cts, n, lane); }
     static MRL_DEV void step_tail(float *row, const float *cts, int n, const Carry &c, float &r, float &d) {
-        bw::step_tail<false>(row, cts, n, c.act, r, d);
+        bw::step_tail<false, false>(row, cts, n, c.act, r, d);
     }
 };
 

@@ -399,7 +399,8 @@ MRL_DEV void step_motors(float *row, const float *action, float *act) {
 
 // what follows the physics of a step: contact flags, observation, reward, termination; `n` = the
 // contacts of the step, whose body indices are still in `contacts`
-template <bool LIDAR = true>
+// STATE_OBS = false: observation entries 0 .. 7 and 9 .. 12 are in the row already (physics_lanes leaves them)
+template <bool LIDAR = true, bool STATE_OBS = true>
 MRL_DEV void step_tail(float *row, const float *contacts, int n, const float *act, float &reward, float &done);
 
 template <bool LIDAR = true>
@@ -410,7 +411,7 @@ MRL_DEV void step_finish(float *row, float *contacts, int n_given, const float *
     step_tail<LIDAR>(row, contacts, n, act, reward, done);
 }
 
-template <bool LIDAR>
+template <bool LIDAR, bool STATE_OBS>
 MRL_DEV void step_tail(float *row, const float *contacts, int n, const float *act, float &reward, float &done) {
     bool left = false, right = false, hull = false;
     for (int c = 0; c < n; ++c) {
@@ -425,8 +426,12 @@ MRL_DEV void step_tail(float *row, const float *contacts, int n, const float *ac
     if (hull) M[META_GAME_OVER] = 1.0f;
     const float *B = row + L::BODIES_OFF;
     M[META_SCROLL] = B[IDX_X] - (float)(600.0 / SCALE / 5.0);
+    static_assert(STATE_OBS || !LIDAR, "the lidar form writes the whole observation");
     if (LIDAR) {
         observe(row);
+    } else if (!STATE_OBS) {
+        row[8] = left ? 1.0f : 0.0f;
+        row[13] = right ? 1.0f : 0.0f;
     } else {
         float o[14];
         observe_state(row, o);
