@@ -204,6 +204,16 @@ int mrl_rms_normalize(mrl_ctx *ctx, const double *state, float *x, int n);
  * reference runs a host Fisher-Yates shuffle (deep_agents/ppo/ppo.mojo:2425-2434,
  * core/utils/shuffle.mojo:21-82) and copies the indices to the device. */
 int mrl_permutation(mrl_ctx *ctx, int32_t *indices, int n, uint64_t seed);
+/* shuffle_indices, core/utils/shuffle.mojo:21-48 (the same loop inline at deep_agents/ppo/ppo.mojo:
+ * 2425-2434), on draws that the caller supplies: indices[0..n) = the result of
+ *     for i = n-1 .. 1:  j = min(Int(u * Float64(i + 1)), i);  swap(indices[i], indices[j])
+ * started from 0..n-1, where iteration i takes u = uniforms[n - 1 - i] (device, Float64, n - 1 values in
+ * [0, 1], i.e. the draws of random_float64() in the order the loop consumes them).  Index for index the
+ * permutation of the serial loop, computed in parallel; workspace is device scratch of 2n + 1 int32.
+ * A caller that feeds the reference's own random stream gets the reference's minibatches; without one,
+ * mrl_permutation is the cheaper call. */
+int mrl_permutation_from_uniforms(mrl_ctx *ctx, int32_t *indices, int n, const double *uniforms,
+                                  int32_t *workspace);
 /* mean of kl[0..mb) against target_kl on the device: flag[0] is set to 1 when the mean exceeds
  * target_kl (never cleared by the library), flag[1] receives the bits of the mean (flag holds 4
  * int32; [2] and [3] belong to mrl_ppo_update_minibatch).  Replaces
@@ -354,6 +364,15 @@ int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *i
  * runs with step counts actor_t0 + k + 1 / critic_t0 + k + 1 */
 int mrl_ppo_update_epoch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int n_minibatches,
                          int actor_t0, int critic_t0);
+
+/* The statistics that the fused update normalises a minibatch's advantages with
+ * (deep_agents/ppo/ppo.mojo:2478-2511 with the kernel at :637-653 -- mean and variance over the
+ * minibatch's gathered advantages): stats[2k] = mean, stats[2k + 1] = sqrt(variance + 1e-8) of the
+ * rows indices[k * minibatch .. (k + 1) * minibatch) of `advantages`, for k < n_minibatches.  This is
+ * the launch mrl_ppo_update_epoch makes ahead of its minibatches, written to the caller's buffer
+ * (device, 2 * n_minibatches floats); a normalised advantage is (A - mean) / (stats[2k + 1] + 1e-8). */
+int mrl_minibatch_adv_stats(mrl_ctx *ctx, const int32_t *indices, const float *advantages, int minibatch,
+                            int n_minibatches, float *stats);
 
 #ifdef __cplusplus
 }

@@ -105,6 +105,7 @@ SIGNATURES = {
     "mrl_rms_update": [P, P, P, I],
     "mrl_rms_normalize": [P, P, P, I],
     "mrl_permutation": [P, P, I, U64],
+    "mrl_permutation_from_uniforms": [P, P, I, P, P],
     "mrl_kl_check": [P, P, I, F, P],
     "mrl_init_uniform": [P, P, I, F, F, U64],
     "mrl_policy_step_discrete": [P, DP, DP, I, P, P, P, U32, P, P, P, P, P],
@@ -114,6 +115,7 @@ SIGNATURES = {
     "mrl_rollout_fused": [RP],
     "mrl_ppo_update_minibatch": [P, UP, P, I, I],
     "mrl_ppo_update_epoch": [P, UP, P, I, I, I],
+    "mrl_minibatch_adv_stats": [P, P, P, I, I, P],
 }
 _SPECIAL = {"mrl_version": (C.c_int, []), "mrl_last_error": (C.c_char_p, [])}
 # size queries return a count, not a status

@@ -9,7 +9,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmrl_hip.so")
-SOURCES = ["mrl_core.hip", "mrl_env.hip", "mrl_mlp.hip", "mrl_mlp3.hip", "mrl_ppo.hip", "mrl_policy.hip", "mrl_rollout.hip", "mrl_collect.hip", "mrl_collect_walkers.hip", "mrl_update.hip"]
+SOURCES = ["mrl_core.hip", "mrl_env.hip", "mrl_mlp.hip", "mrl_mlp3.hip", "mrl_ppo.hip", "mrl_policy.hip", "mrl_rollout.hip", "mrl_collect.hip", "mrl_collect_walkers.hip", "mrl_update.hip", "mrl_shuffle.hip"]
 # -ffp-contract=off: fp32/fp64 results follow the written order of operations (the GEMM inner
 # loops spell out fmaf / MFMA themselves).  The -target-feature pair switches packed-fp32
 # code generation off.

@@ -471,6 +471,19 @@ int mrl_ppo_update_minibatch(mrl_ctx *ctx, const mrl_update *u, const int32_t *i
     return update_minibatch(ctx, u, indices, actor_t, critic_t, nullptr);
 }
 
+int mrl_minibatch_adv_stats(mrl_ctx *ctx, const int32_t *indices, const float *advantages, int minibatch,
+                            int n_minibatches, float *stats) {
+    MRL_CHECK_ARG(ctx != nullptr, "mrl_minibatch_adv_stats: ctx is NULL");
+    MRL_CHECK_ARG(minibatch > 0 && n_minibatches >= 0, "mrl_minibatch_adv_stats: bad sizes");
+    if (n_minibatches == 0) return MRL_OK;
+    MRL_CHECK_ARG(indices && advantages && stats, "mrl_minibatch_adv_stats: NULL buffer");
+    // the launch mrl_ppo_update_epoch makes ahead of its minibatches, into the caller's buffer
+    hipLaunchKernelGGL(adv_stats_kernel, dim3(n_minibatches), dim3(UTPB), 0, ctx->stream, indices, advantages,
+                       minibatch, stats);
+    MRL_CHECK_LAUNCH();
+    return MRL_OK;
+}
+
 int mrl_ppo_update_epoch(mrl_ctx *ctx, const mrl_update *u, const int32_t *indices, int n_minibatches,
                          int actor_t0, int critic_t0) {
     MRL_CHECK_ARG(ctx != nullptr, "mrl_ppo_update_epoch: ctx is NULL");

@@ -115,6 +115,34 @@ def permutation(ctx, indices, seed):
     _lib.call("mrl_permutation", ctx.handle, _ptr(indices), indices.numel(), int(seed) & (2**64 - 1))
 
 
+def shuffle_indices(ctx, indices, uniforms, workspace=None):
+    """shuffle_indices of core/utils/shuffle.mojo:21-48 on supplied draws: fills the int32 device buffer
+    with the permutation that the reference's Fisher-Yates loop produces when iteration i = n-1 .. 1
+    draws uniforms[n - 1 - i] (float64 device tensor of n - 1 values).  workspace: int32 device
+    scratch of 2n + 1 entries, allocated here when not given."""
+    n = indices.numel()
+    if indices.dtype != torch.int32:
+        raise _lib.MrlError("permutation indices must be int32")
+    if n > 1 and (uniforms.dtype != torch.float64 or uniforms.numel() < n - 1):
+        raise _lib.MrlError("shuffle_indices needs n - 1 float64 uniforms")
+    if workspace is None:
+        workspace = torch.empty(2 * n + 1, dtype=torch.int32, device=indices.device)
+    elif workspace.dtype != torch.int32 or workspace.numel() < 2 * n + 1:
+        raise _lib.MrlError("shuffle_indices needs an int32 workspace of 2n + 1 entries")
+    _lib.call("mrl_permutation_from_uniforms", ctx.handle, _ptr(indices), n, _ptr(uniforms) if n > 1 else None,
+              _ptr(workspace))
+    return workspace
+
+
+def minibatch_adv_stats(ctx, indices, advantages, minibatch, stats):
+    """stats[2k], stats[2k + 1] = mean and sqrt(variance + 1e-8) of the advantages of minibatch k of
+    `indices` (ppo.mojo:2478-2511): what the fused update normalises with."""
+    n_mb = indices.numel() // minibatch
+    if indices.dtype != torch.int32 or stats.numel() < 2 * n_mb:
+        raise _lib.MrlError("minibatch_adv_stats needs int32 indices and 2 floats per minibatch")
+    _lib.call("mrl_minibatch_adv_stats", ctx.handle, _ptr(indices), _ptr(advantages), minibatch, n_mb, _ptr(stats))
+
+
 def kl_check(ctx, kl, target_kl, flag):
     """Device-side early-stop test: flag[0] (int32) becomes 1 when mean(kl) > target_kl and stays
     1; flag[1] holds the bits of the mean (ppo.mojo:2557-2573 without the host copy)."""

@@ -199,6 +199,8 @@ void orc_clamp_log_std(float *params, int offset, int action_dim);
 typedef struct { double count, mean, var_sum; } orc_rms;
 void orc_rms_update(orc_rms *r, const float *x, int n);
 void orc_rms_normalize(const orc_rms *r, float *x, int n);
+/* shuffle_indices, core/utils/shuffle.mojo:21-48, on the draws u[0 .. n-2] in consumption order */
+void orc_shuffle_indices(int n, const double *u, int32_t *indices);
 
 #ifdef __cplusplus
 }

@@ -14,6 +14,7 @@ _SO = os.path.join(_HERE, "liborc.so")
 
 f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
 i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
+f64p = np.ctypeslib.ndpointer(dtype=np.float64, flags="C_CONTIGUOUS")
 u32p = np.ctypeslib.ndpointer(dtype=np.uint32, flags="C_CONTIGUOUS")
 
 
@@ -123,6 +124,7 @@ def load():
         "orc_clamp_log_std": (None, [f32p, C.c_int, C.c_int]),
         "orc_rms_update": (None, [C.POINTER(Rms), f32p, C.c_int]),
         "orc_rms_normalize": (None, [C.POINTER(Rms), f32p, C.c_int]),
+        "orc_shuffle_indices": (None, [C.c_int, f64p, i32p]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)

@@ -329,3 +329,19 @@ void orc_rms_normalize(const orc_rms *r, float *x, int n) {
     double std = sqrt(var + 1e-8);
     for (int i = 0; i < n; ++i) x[i] = (float)(((double)x[i] - r->mean) / (std + 1e-8));
 }
+
+/* Fisher-Yates shuffle of the indices 0 .. n-1 on supplied uniforms (core/utils/shuffle.mojo:21-48;
+ * the same loop inline in deep_agents/ppo/ppo.mojo:2425-2434): for i = n-1 down to 1,
+ * j = Int(u * Float64(i + 1)) with u the next draw of random_float64() -- here u[n-1-i], the draws in
+ * the order the loop consumes them -- clamped to i (shuffle.mojo:42-43; a draw in [0, 1) never needs
+ * it), then indices[i] <-> indices[j]. */
+void orc_shuffle_indices(int n, const double *u, int32_t *indices) {
+    for (int i = 0; i < n; ++i) indices[i] = i;
+    for (int i = n - 1; i > 0; --i) {
+        int j = (int)(u[n - 1 - i] * (double)(i + 1));
+        if (j > i) j = i;
+        const int32_t tmp = indices[i];
+        indices[i] = indices[j];
+        indices[j] = tmp;
+    }
+}

@@ -2,9 +2,9 @@
 (CPU) and against the HIP path through the C ABI (GPU).
 
 The trajectories were produced by this repository's oracle, not by the reference (which cannot
-run here): they are regression anchors.  Observations 1e-5 relative / 1e-6 absolute, rewards and
-done flags exact (LunarLander, CartPole, Pendulum); the walkers' rewards are differences of
-fp32 positions and are compared at the state tolerance."""
+run here): they are regression anchors.  Observations, rewards, done flags and the final state rows
+are compared bit for bit, for every environment, on the CPU (oracle) and on the GPU (HIP path),
+with no resynchronisation between the 64 steps."""
 import json
 import os
 
@@ -81,7 +81,7 @@ def test_oracle_reproduces_golden_trajectories(orc, traj, name):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,cls", [("pendulum", "PendulumV2"), ("lunar", "LunarLanderV2"),
+@pytest.mark.parametrize("name,cls", [("cartpole", "CartPoleEnv"), ("pendulum", "PendulumV2"), ("lunar", "LunarLanderV2"),
                                       ("bipedal", "BipedalWalkerV2"), ("cheetah", "HalfCheetahPlanarV2")])
 def test_hip_path_reproduces_golden_trajectories(mrl, traj, name, cls):
     import torch
@@ -91,6 +91,9 @@ def test_hip_path_reproduces_golden_trajectories(mrl, traj, name, cls):
     T, N = R.shape
     s = torch.from_numpy(traj["%s_state0" % name].copy()).cuda().reshape(-1)
     r, d, o = torch.zeros(N, device="cuda"), torch.zeros(N, device="cuda"), torch.zeros(O[0].size, device="cuda")
+    if name == "cartpole":      # the step counters behind the 500-step truncation, in the caller's hands
+        steps = torch.zeros(N, dtype=torch.int32, device="cuda")
+        E.bind_step_counters(ctx, s, steps)
     for t in range(T):
         print(name, "step", t, flush=True)
         a = torch.from_numpy(np.ascontiguousarray(A[t].reshape(-1))).cuda()
@@ -103,3 +106,7 @@ def test_hip_path_reproduces_golden_trajectories(mrl, traj, name, cls):
         E.selective_reset_kernel_gpu(ctx, s, d, 1000 + t)
     ctx.synchronize()
     np.testing.assert_array_equal(s.cpu().numpy().reshape(N, -1), traj["%s_state_end" % name])
+    if name == "cartpole":
+        # a counter holds the steps since its row's last reset
+        since = np.array([T - 1 - (np.nonzero(D[:, i])[0].max() if D[:, i].any() else -1) for i in range(N)])
+        np.testing.assert_array_equal(steps.cpu().numpy(), since)

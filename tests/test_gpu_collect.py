@@ -105,6 +105,18 @@ def _low_start(E, N, seed, orc):
     b[:, :, 1] -= rng.uniform(7.5, 9.4, N).astype(np.float32)[:, None]
     b[:, :, 0] += rng.uniform(-6, 6, N).astype(np.float32)[:, None]
     b[:, 0, 2] = rng.uniform(-0.4, 0.4, N).astype(np.float32)
+    # Every fourth row hovers over the helipad instead: legs folded to their joint limit with the feet
+    # 3 mm above the pad -- inside the 1 cm band of the leg-contact observation, no solver contact --
+    # and every body moving up at g * dt, which the step's gravity cancels.  A step without engine
+    # power leaves such a row at rest on both legs: the +100 landing branch (:1230-1247).
+    pad, th = np.float32(400 / 30 / 4), np.float32(0.399)
+    leg_y = pad + np.float32(0.2745)
+    hov = b[::4]
+    hov[:, 0, :3] = (10.0, leg_y + np.float32(10 / 30) + np.cos(th) * np.float32(8 / 30), 0.0)
+    for k, sgn in ((1, -1.0), (2, 1.0)):
+        hov[:, k, 0] = np.float32(10 + sgn * 20 / 30) + np.float32(sgn) * np.sin(th) * np.float32(8 / 30)
+        hov[:, k, 1], hov[:, k, 2] = leg_y, np.float32(-sgn) * th
+    hov[:, :, 3:6] = (0.0, 0.2, 0.0)
     return s_h
 
 
@@ -168,7 +180,7 @@ def test_fused_collection_through_contacts(mrl, ctx, orc, env, kind, N):
         np.testing.assert_allclose(fused1.obs.cpu().numpy().reshape(N, 8), s_h[:, :8], rtol=1e-5, atol=1e-6)
         s_h[:] = sg
     print("  crashes", crashes, "landings", landed, "leg-contact observations", leg_obs, "resets", resets, flush=True)
-    assert crashes > N // 40 and leg_obs > N // 4 and resets >= crashes
+    assert crashes > N // 40 and leg_obs > N // 4 and resets >= crashes + landed and landed > N // 64
 
     # (2) the same range as two launches, against single steps
     dsingle, dfused = single.descriptor(), fused.descriptor()

@@ -301,3 +301,40 @@ def test_running_mean_std_chan_merge(orc, orcmod):
     np.testing.assert_allclose(x, (a - allv.mean()) / (math.sqrt(allv.var() + 1e-8) + 1e-8), rtol=1e-5, atol=1e-6)
     r0 = orcmod.Rms(1, 5.0, 0); y = np.array([6.0], np.float32); orc.orc_rms_normalize(C.byref(r0), y, 1)
     assert abs(y[0] - 1.0) < 1e-6                                         # variance defaults to 1 while count < 2
+
+
+def test_shuffle_indices_brute_force(orc):
+    """orc_shuffle_indices (core/utils/shuffle.mojo:21-48) pinned without retyping its loop:
+    (i) over an exhaustive grid of draws for n <= 5 -- one draw per bin of every iteration, at the
+    bin's lower edge, middle and just below its upper edge -- the result equals the product of the
+    transposition MATRICES (i j_i) applied to the identity vector in loop order (n-1 first), and
+    the n! bin choices give n! different permutations (Fisher-Yates is a bijection from bin
+    choices to permutations: a dropped iteration, an off-by-one in the range or a bin computed
+    from i instead of i + 1 breaks this count); (ii) u = 1.0 falls back to j = i (no move) and
+    u = 0.0 swaps with position 0; (iii) draws are consumed in loop order, u[0] by i = n - 1."""
+    import itertools
+    for n in range(1, 6):
+        seen = set()
+        bins = [range(i + 1) for i in range(n - 1, 0, -1)]          # iteration i = n-1 .. 1
+        for choice in itertools.product(*bins):
+            mats = np.eye(n, dtype=np.int64)
+            for i, j in zip(range(n - 1, 0, -1), choice):
+                t = np.eye(n, dtype=np.int64)
+                t[[i, j]] = t[[j, i]]
+                mats = t @ mats
+            want = (mats @ np.arange(n)).astype(np.int32)
+            for frac in (0.0, 0.5, 1.0 - 1e-9):
+                u = np.array([(j + frac) / (i + 1) for i, j in zip(range(n - 1, 0, -1), choice)] + [0.0],
+                             np.float64)
+                got = np.full(n, -1, np.int32)
+                orc.orc_shuffle_indices(n, u, got)
+                np.testing.assert_array_equal(got, want)
+            seen.add(tuple(want.tolist()))
+        assert len(seen) == math.factorial(n)
+    got = np.zeros(4, np.int32)
+    orc.orc_shuffle_indices(4, np.array([1.0, 1.0, 1.0]), got)
+    np.testing.assert_array_equal(got, [0, 1, 2, 3])
+    orc.orc_shuffle_indices(4, np.array([0.0, 0.0, 0.0]), got)
+    np.testing.assert_array_equal(got, [1, 2, 3, 0])           # 0<->3, then 3(at 0)<->2 ..., a rotation
+    orc.orc_shuffle_indices(4, np.array([0.0, 0.99, 0.99]), got)    # only the first draw (i = 3) moves anything
+    np.testing.assert_array_equal(got, [3, 1, 2, 0])
