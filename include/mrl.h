@@ -43,7 +43,13 @@ enum mrl_env_id {
      * (lunar_lander_v2.mojo:1520-1588); rows, reset and selective reset are those of
      * MRL_ENV_LUNARLANDER */
     MRL_ENV_LUNARLANDER_CONTINUOUS = 5,
-    MRL_ENV_CARRACING = 6    /* envs/car_racing/car_racing_v2.mojo:90 CarRacingV2 (GPUContinuousEnv, :947-1150) */
+    /* envs/car_racing/car_racing_v2.mojo:90 CarRacingV2 behind GPUContinuousEnv (:947-1150): the trait's
+     * row, reset and done-row protocol.  NOTE the reward: by default the step pays what the reference's
+     * CPU env pays (-0.1 per step + 100 / tiles per new tile, Float64, :258-287 and :781-846), which is
+     * NOT what the reference's step_kernel_gpu pays (0.5 * forward speed - 0.01 + 100 / tiles in fp32,
+     * :1636-1666): returns of a run trained with the default are not comparable with the reference's
+     * train_gpu.  mrl_car_racing_set_step_form(ctx, MRL_CAR_STEP_GPU_TRAIT) selects the trait's. */
+    MRL_ENV_CARRACING = 6
 };
 
 /* layer kinds of an MLP description; deep_rl/model/{linear,linear_relu,linear_tanh,stochastic_actor}.mojo */
@@ -91,7 +97,11 @@ int mrl_ctx_reserve(mrl_ctx *ctx, uint64_t mlp_floats, uint64_t rollout_floats);
 /* The fused collection kernels let groups of wavefronts of a workgroup meet at barriers of their own
  * (counters in LDS).  Every such wait is bounded: after `polls` polls (MRL_DEFAULT_SPIN_LIMIT unless
  * set here; 0 restores the default) the waiting wavefront gives up, the workgroup stops stepping, the
- * kernel ends normally and the next mrl_ctx_synchronize returns MRL_E_SYNC (once).  No counterpart
+ * kernel ends normally and the next mrl_ctx_synchronize returns MRL_E_SYNC (once).  What the calls since
+ * the last synchronize wrote is void then: a workgroup that gave up stores neither its env rows nor its
+ * observations nor its episode sums (they keep the values from before the launch), the other workgroups'
+ * envs have advanced, and rollout rows and the finished-episode list hold a mixture -- reset the envs
+ * and clear done_count before collecting again.  No counterpart
  * in the reference; a tiny limit is how a test exercises the error path without hanging anything. */
 #define MRL_DEFAULT_SPIN_LIMIT (1u << 22)
 int mrl_ctx_set_spin_limit(mrl_ctx *ctx, unsigned polls);
@@ -147,6 +157,18 @@ int mrl_cartpole_bind_steps(mrl_ctx *ctx, const float *states, int batch, int32_
  * (turbulence), computed in Float64 as _apply_wind does (:983-1023), with t = the row's step
  * count as in the GPU trait (:2041-2105).  Takes effect for steps enqueued after the call. */
 int mrl_lunar_set_wind(mrl_ctx *ctx, int enable, double wind_power, double turbulence_power);
+/* Which of the reference's two CarRacingV2 steps the context's env steps follow (plain and fused).  The
+ * dynamics, the controls, the visited flags and the observation are the same in both; they differ in the
+ * reward and in the precision of the termination tests:
+ *   MRL_CAR_STEP_CPU_ENV (default)  CarRacingV2.step, car_racing_v2.mojo:258-287: reward -0.1 (+ 100 /
+ *       tiles for a new tile) in Float64, -100 off the playfield, tests in Float64, episode total taken
+ *       before the playfield penalty (:781-846);
+ *   MRL_CAR_STEP_GPU_TRAIT          step_kernel_gpu, car_racing_v2.mojo:1556-1716, which the reference's
+ *       train_gpu runs: reward 0.5 * (vx cos(angle) + vy sin(angle)) - 0.01 (+ 100 / tiles) in fp32 from
+ *       the hull state after the physics, fp32 tests, episode total taken after the penalty.
+ * Takes effect for steps enqueued after the call. */
+enum { MRL_CAR_STEP_CPU_ENV = 0, MRL_CAR_STEP_GPU_TRAIT = 1 };
+int mrl_car_racing_set_step_form(mrl_ctx *ctx, int form);
 /* step, then re-initialise rows that finished with the selective-reset protocol, then write
  * obs from the (possibly fresh) row: the sequence step_kernel_gpu -> selective_reset_kernel_gpu
  * -> _extract_obs_from_state_kernel of deep_agents/ppo/ppo.mojo:2148-2285 in one launch.

@@ -83,6 +83,7 @@ SIGNATURES = {
     "mrl_env_step_autoreset": [P, I, I, P, P, P, P, P, U64, U64],
     "mrl_cartpole_bind_steps": [P, P, I, P],
     "mrl_lunar_set_wind": [P, I, D, D],
+    "mrl_car_racing_set_step_form": [P, I],
     "mrl_mlp_param_size": [DP],
     "mrl_mlp_cache_size": [DP],
     "mrl_mlp_out_dim": [DP],

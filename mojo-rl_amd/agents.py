@@ -118,8 +118,10 @@ class _PPOAgentBase:
         :186-222) -> (observation, reward, done).  Per step: one policy launch, the actions to the host,
         the envs stepped one by one in index order, finished envs reset at once, the observations back to
         the device.  The continuous agent hands the envs  clip(action * action_scale + action_bias, -1, 1)
-        and stores the raw action, as the reference does.  The rollout is dropped without an update when
-        the episode target is reached inside it (the reference's early `break`).  GAE, normalisation and
+        and stores the raw action, as the reference does.  When the episode target is reached inside a
+        rollout, the rollout's remaining steps are still taken (and their episodes logged) and the call
+        then returns without an update: the reference tests the target behind its step loop, not inside
+        it (ppo.mojo:3290 and :3454-3456, ppo_continuous.mojo likewise).  GAE, normalisation and
         the epochs are those of train_gpu, on the device."""
         if len(envs) != self.n_envs:
             raise ValueError("expected %d environments, got %d" % (self.n_envs, len(envs)))

@@ -15,6 +15,7 @@ struct CollectArgs {
     Accounting acc;                       // r_rewards / r_dones unused here (set per step)
     unsigned spin_limit;                  // polls before a wait at a wavefront-group barrier gives up
     int *sync_error;                      // raised (host-visible) by a workgroup whose wait gave up
+    int car_trait_form;                   // CarRacingV2: reward / termination arithmetic of the GPU trait's step
 };
 
 // BipedalWalker / HalfCheetah with the agents' 256-wide Gaussian nets: true when `a` was launched

@@ -206,9 +206,13 @@ MRL_DEV void wheel_forces(float wheel_omega, float joint_angle, float hull_angle
 // them: the row itself, or a copy that a kernel holds on chip over many steps; `row` is read for the tile
 // table and takes the visited flags.  Every lane returns the same reward / done and the observation the row
 // now starts with; lane 0 has written `head`.
+// trait_form: false = the CPU env's reward and termination arithmetic (car_racing_v2.mojo:781-846, Float64),
+// true = the GPU trait's step_kernel_gpu (car_racing_v2.mojo:1622-1710: reward 0.5 * forward speed - 0.01
+// (+ 100 / tiles) in fp32 from the hull state after the physics, fp32 playfield and lap tests, the episode
+// total taken after the playfield penalty).  The dynamics and the decoded controls are the same in both.
 template <bool FLAGS_COHERENT = false>
 MRL_DEV void step_wave(float *head, float *row, float *table, const float *action, int sub, float &reward,
-                       float &done, float (&ob)[OBS]) {
+                       float &done, float (&ob)[OBS], bool trait_form = false) {
     float *M = head + META;
     if (M[M_DONE] > 0.5f) {   // car_racing_v2.mojo:1564-1572
 #pragma unroll
@@ -315,25 +319,45 @@ MRL_DEV void step_wave(float *head, float *row, float *table, const float *actio
     const float hpx[1] = {x}, hpy[1] = {y};
     int tile_idx[1];
     tiles.at<1>(hpx, hpy, num_tiles, sub, tile_idx);
-    double step_reward = -0.1;
     float tiles_visited = M[M_VISITED];
     const bool fresh = tile_idx[0] >= 0 && !(tiles.visited(tile_idx[0] >= 0 ? tile_idx[0] : 0) > 0.5f);
-    if (fresh) {
-        tiles_visited = tiles_visited + 1.0f;
-        step_reward += 100.0 / (double)num_tiles;
-    }
-    const float total = (float)((double)M[M_TOTAL] + step_reward);
     const float step_count = M[M_STEP] + 1.0f;
-    bool is_done = false;
-    const double playfield = 2000.0 / SCALE_;
-    const double hx = (double)x, hy = (double)y;
-    const double abs_x = hx >= 0.0 ? hx : -hx, abs_y = hy >= 0.0 ? hy : -hy;
-    if (abs_x > playfield || abs_y > playfield) { is_done = true; step_reward = -100.0; }
-    const double progress = (double)tiles_visited / (double)(num_tiles > 1 ? num_tiles : 1);
-    if (progress >= 0.95) is_done = true;
     const bool truncated = step_count >= (float)500.0;
+    bool is_done = false;
+    float total;
+    if (trait_form) {
+        float sin_h, cos_h;
+        sincos32(angle, sin_h, cos_h);
+        const float forward_vel = vx * cos_h + vy * sin_h;
+        float step_reward = forward_vel * (float)0.5 - (float)0.01;
+        if (fresh) {
+            const float tile_reward = (float)100.0 / (float)num_tiles;
+            step_reward = step_reward + tile_reward;
+            tiles_visited = tiles_visited + 1.0f;
+        }
+        const float playfield = (float)(2000.0 / SCALE_);
+        const float abs_x = x >= 0.0f ? x : -x, abs_y = y >= 0.0f ? y : -y;
+        if (abs_x > playfield || abs_y > playfield) { is_done = true; step_reward = (float)-100.0; }
+        const float progress = tiles_visited / (float)(num_tiles > 1 ? num_tiles : 1);
+        if (progress >= (float)0.95) is_done = true;
+        total = M[M_TOTAL] + step_reward;
+        reward = step_reward;
+    } else {
+        double step_reward = -0.1;
+        if (fresh) {
+            tiles_visited = tiles_visited + 1.0f;
+            step_reward += 100.0 / (double)num_tiles;
+        }
+        total = (float)((double)M[M_TOTAL] + step_reward);
+        const double playfield = 2000.0 / SCALE_;
+        const double hx = (double)x, hy = (double)y;
+        const double abs_x = hx >= 0.0 ? hx : -hx, abs_y = hy >= 0.0 ? hy : -hy;
+        if (abs_x > playfield || abs_y > playfield) { is_done = true; step_reward = -100.0; }
+        const double progress = (double)tiles_visited / (double)(num_tiles > 1 ? num_tiles : 1);
+        if (progress >= 0.95) is_done = true;
+        reward = (float)step_reward;
+    }
     if (truncated) is_done = true;
-    reward = (float)step_reward;
     done = is_done ? 1.0f : 0.0f;
     // observation (update_observation, car_dynamics.mojo:292-350; _update_observation, :848-898)
     ob[0] = x; ob[1] = y; ob[2] = angle; ob[3] = vx; ob[4] = vy; ob[5] = omega;

@@ -84,6 +84,7 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
         sync_detect = 0;
         sync_failed = 0;
     }
+    if (t < PR) ncontacts[t] = 0;   // read by the solver also when the detection's wait gave up
     __syncthreads();
     // wavefront 0, lane = env slot: the env's running episode return and length stay in registers
     const bool owner = t < nenv;
@@ -209,10 +210,15 @@ __global__ __launch_bounds__(E::THREADS) void collect_kernel(CollectArgs a) {
         __syncthreads();   // env step done, values complete
         if (tid < ne) a.r_values[row + tid] = vals[tid];
         // a wait that gave up: the block's results are void from here on; leave the loop (every
-        // thread reads the same word after the barrier), store what there is and end normally
+        // thread reads the same word after the barrier) and end normally
         if (sync_failed != 0u) break;
     }
-    if (t == 0 && sync_failed != 0u) *a.sync_error = 1;
+    if (sync_failed != 0u) {
+        // a wait gave up: the step in progress ran on data that was never produced.  Nothing of it is
+        // stored: rows, observations and episode sums of this block keep the values from before the launch
+        if (t == 0) *a.sync_error = 1;
+        return;
+    }
 
     if (owner) {
         a.acc.ep_return[env0 + t] = ep_return;
@@ -400,10 +406,13 @@ __global__ __launch_bounds__(256, 2) void collect16_kernel(CollectArgs a) {
         __syncthreads();   // env step done, values complete
         if (tid < ne) a.r_values[row + tid] = vals[tid];
         // a wait that gave up: the block's results are void from here on; leave the loop (every
-        // thread reads the same word after the barrier), store what there is and end normally
+        // thread reads the same word after the barrier) and end normally
         if (sync_failed != 0u) break;
     }
-    if (t == 0 && sync_failed != 0u) *a.sync_error = 1;
+    if (sync_failed != 0u) {   // as in collect_kernel: nothing of a block whose wait gave up is stored
+        if (t == 0) *a.sync_error = 1;
+        return;
+    }
 
     if (owner) {
         a.acc.ep_return[env0 + (t & 63)] = ep_return;
@@ -639,6 +648,7 @@ int mrl_rollout_steps(mrl_ctx *ctx, const mrl_rollout *r, int t0, int n_steps, u
                        r->done_count, r->done_cap};
     a.spin_limit = ctx->spin_limit;
     a.sync_error = ctx->sync_error;
+    a.car_trait_form = ctx->car_trait_form;
     // LunarLander: with at most 16 envs per CU the 16-row kernel (a shorter chain per step); beyond that
     // the 32-row kernel, whose single solver wavefront per CU steps twice the envs in the same time
     const bool lander = r->env_id == MRL_ENV_LUNARLANDER || r->env_id == MRL_ENV_LUNARLANDER_CONTINUOUS;

@@ -248,11 +248,15 @@ __global__ __launch_bounds__(512) void collect_walker_kernel(CollectArgs a) {
         }
         __syncthreads();   // env step done: the rows hold the next observation
         if (tid < ne) a.r_values[row + tid] = vals[tid];
-        // a wait that gave up: the block's results are void from here on; leave the loop, store what
-        // there is and end normally
+        // a wait that gave up: the block's results are void from here on; leave the loop and end normally
         if (sync_failed != 0u) break;
     }
-    if (t == 0 && sync_failed != 0u) *a.sync_error = 1;
+    if (sync_failed != 0u) {
+        // a wait gave up: the step in progress ran on data that was never produced; the block's rows and
+        // observations are not stored and keep the values from before the launch
+        if (t == 0) *a.sync_error = 1;
+        return;
+    }
 
     for (int i = t; i < nenv * E::OBS; i += T) {
         const int r = i / E::OBS, c = i - r * E::OBS;
@@ -314,7 +318,8 @@ __global__ __launch_bounds__(512) void collect_car_kernel(CollectArgs a) {
                 float *head = heads + slot * (HEAD + 1);
                 float *grow = a.states + (size_t)env * cr::STATE;
                 float r, d, ob[cr::OBS];
-                cr::step_wave<true>(head, grow, overlay + wave * cr::TABLE, act + slot * AW, sub, r, d, ob);
+                cr::step_wave<true>(head, grow, overlay + wave * cr::TABLE, act + slot * AW, sub, r, d, ob,
+                                    a.car_trait_form != 0);
                 if (sub == 0) account(acc, slot, r, d);
                 if (d > 0.5f) {
                     float sx, sy, sa;

@@ -200,14 +200,14 @@ constexpr int CAR_RESET_GROUP = 16, CAR_RESET_EPB = CAR_THREADS / CAR_RESET_GROU
 template <bool AUTORESET>
 __global__ __launch_bounds__(CAR_THREADS) void car_step_kernel(float *states, const float *actions, float *rewards,
                                                                float *dones, float *obs, int batch,
-                                                               uint64_t reset_seed, Accounting acc) {
+                                                               uint64_t reset_seed, Accounting acc, int trait_form) {
     __shared__ __align__(16) float tables[CAR_EPB][cr::TABLE];   // each wavefront's copy of its env's tile table
     const int sub = threadIdx.x & 63, wave = threadIdx.x / cr::STEP_LANES;
     const int env = blockIdx.x * CAR_EPB + wave;
     if (env >= batch) return;   // whole wavefronts leave together
     float *row = states + (size_t)env * cr::STATE;
     float r, d, ob[cr::OBS];
-    cr::step_wave(row, row, tables[wave], actions + (size_t)env * cr::ACT, sub, r, d, ob);
+    cr::step_wave(row, row, tables[wave], actions + (size_t)env * cr::ACT, sub, r, d, ob, trait_form != 0);
     if (sub == 0) {
         rewards[env] = r;
         dones[env] = d;
@@ -351,6 +351,14 @@ __global__ void lunar_wind_kernel(float *shapes, float on, float wind_power, flo
     }
 }
 
+int mrl_car_racing_set_step_form(mrl_ctx *ctx, int form) {
+    MRL_CHECK_ARG(ctx, "mrl_car_racing_set_step_form: NULL ctx");
+    MRL_CHECK_ARG(form == MRL_CAR_STEP_CPU_ENV || form == MRL_CAR_STEP_GPU_TRAIT,
+                  "mrl_car_racing_set_step_form: form %d is neither MRL_CAR_STEP_CPU_ENV nor MRL_CAR_STEP_GPU_TRAIT", form);
+    ctx->car_trait_form = form;   // a kernel argument of the launches made from now on
+    return MRL_OK;
+}
+
 int mrl_lunar_set_wind(mrl_ctx *ctx, int enable, double wind_power, double turbulence_power) {
     MRL_CHECK_ARG(ctx, "mrl_lunar_set_wind: NULL ctx");
     MRL_CHECK_ARG(std::isfinite(wind_power) && std::isfinite(turbulence_power),
@@ -460,10 +468,10 @@ static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, con
             const dim3 grid(grid_for(batch, CAR_EPB)), block(CAR_THREADS);
             if (autoreset)
                 hipLaunchKernelGGL((car_step_kernel<true>), grid, block, 0, ctx->stream, states, actions, rewards, dones,
-                                   obs, batch, reset_seed, acc);
+                                   obs, batch, reset_seed, acc, ctx->car_trait_form);
             else
                 hipLaunchKernelGGL((car_step_kernel<false>), grid, block, 0, ctx->stream, states, actions, rewards, dones,
-                                   obs, batch, reset_seed, acc);
+                                   obs, batch, reset_seed, acc, ctx->car_trait_form);
             break;
         }
         default:

@@ -39,6 +39,8 @@ struct mrl_ctx {
     // writes directly) and the kernel ends normally.  mrl_ctx_synchronize reports and clears it.
     unsigned spin_limit;
     int *sync_error;
+    // CarRacingV2: 0 = the CPU env's reward / termination arithmetic (default), 1 = the GPU trait's
+    int car_trait_form;
     // phase timing: events recorded on `stream` at phase boundaries while armed
     bool profiling;
     std::vector<hipEvent_t> prof_events;

@@ -720,10 +720,11 @@ int mrl_clip_grad_norm_static(mrl_ctx *ctx, float *grads, int n, float max_norm)
                   "variant (use mrl_clip_grad_norm)", n, MRL_CLIP_STATIC_MAX_N);
     if (n == 0) return MRL_OK;
     MRL_CHECK_ARG(grads, "mrl_clip_grad_norm_static: NULL buffer");
-    int dev = -1;
-    MRL_CHECK_HIP(hipGetDevice(&dev));
-    int rc = mrl::clip_static_setup(dev);          // resolved by mrl_ctx_create; a lookup, no allocation
-    if (rc != MRL_OK) return rc;
+    // the array of the CONTEXT's device (its stream runs there), whatever device is current on this thread;
+    // mrl_ctx_create looked the address up with that device current
+    const int dev = ctx->device;
+    MRL_CHECK_ARG(dev >= 0 && dev < CLIP_STATIC_MAX_DEVICES && g_clip_scratch_ptr[dev] != nullptr,
+                  "mrl_clip_grad_norm_static: the scratch array of device %d was not resolved at context creation", dev);
     float *part = g_clip_scratch_ptr[dev];
     // same kernels and block count as mrl_clip_grad_norm: the results are the same bit for bit.
     // Every partial that the second kernel reads has been written by the first: nothing to clear.

@@ -132,3 +132,12 @@ class CarRacingV2(_GPUEnv):           # envs/car_racing/car_racing_v2.mojo:90
     """State-based CarRacing: 13-float observation (hull pose and velocity, front wheel angles, wheel
     spins, speed), action [steering, gas, brake] in [-1, 1]; every row carries its own random track."""
     ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_CARRACING, 3040, 13, 3
+    STEP_CPU_ENV, STEP_GPU_TRAIT = 0, 1
+
+    @staticmethod
+    def set_step_form(ctx, form):
+        """Which of the reference's two steps the context's CarRacingV2 steps follow from now on:
+        STEP_CPU_ENV (default; CarRacingV2.step, car_racing_v2.mojo:258-287: reward -0.1 + 100 / tiles,
+        Float64) or STEP_GPU_TRAIT (step_kernel_gpu, :1556-1716, what the reference's train_gpu runs:
+        reward 0.5 * forward speed - 0.01 + 100 / tiles, fp32).  Dynamics and observations are the same."""
+        _lib.call("mrl_car_racing_set_step_form", ctx.handle, int(form))

@@ -172,6 +172,8 @@ int orc_cr_tile_at(const float *row, float x, float y, int num_tiles);
 uint64_t orc_cr_combined_seed(uint64_t seed, int env);
 void orc_cr_reset(float *row, uint64_t combined_seed);
 void orc_cr_step(float *row, const float *action, float *reward, float *done);
+/* 0 (default): the CPU env's step, car_racing_v2.mojo:258-287; 1: the GPU trait's step_kernel_gpu, :1556-1716 */
+void orc_cr_set_step_form(int form);
 /* dones == NULL: every row; otherwise rows with dones > 0.5 (their flag is cleared) */
 void orc_cr_reset_batch(float *states, float *dones, int batch, uint64_t seed);
 void orc_cr_step_batch(float *states, const float *actions, float *rewards, float *dones, float *obs, int batch,

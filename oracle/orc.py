@@ -98,6 +98,7 @@ def load():
         "orc_cr_combined_seed": (C.c_uint64, [C.c_uint64, C.c_int]),
         "orc_cr_reset": (None, [f32p, C.c_uint64]),
         "orc_cr_step": (None, [f32p, f32p, f32p, f32p]),
+        "orc_cr_set_step_form": (None, [C.c_int]),
         "orc_cr_reset_batch": (None, [f32p, C.c_void_p, C.c_int, C.c_uint64]),
         "orc_cr_step_batch": (None, [f32p, f32p, f32p, f32p, f32p, C.c_int, C.c_int]),
         "orc_mlp_param_size": (C.c_int, [YP, C.c_int]),

@@ -19,7 +19,8 @@
  * From the GPU trait's protocol: a row whose done flag is set returns (0, done) untouched, and a
  * tile count <= 0 is read as 100 (car_racing_v2.mojo:1564-1581).
  * (The reference's GPU step computes another reward, 0.5 * forward speed - 0.01 + tile reward, in
- * fp32: car_racing_v2.mojo:1636-1666.  The CPU statement is the one followed here.)
+ * fp32: car_racing_v2.mojo:1636-1666.  The CPU statement is the default; orc_cr_set_step_form(1)
+ * selects the trait's.)
  *
  * Reset: the GPU trait's _reset_env_gpu / _generate_random_track_gpu (car_racing_v2.mojo:1155-1485),
  * the only code of the reference that fills the embedded-track row (the CPU env builds its track with
@@ -229,12 +230,20 @@ static void physics_step(float *row, int num_tiles, float dt) {
     update_observation(row);
 }
 
+/* 0: the CPU env's step (car_racing_v2.mojo:258-287, the default); 1: the GPU trait's step_kernel_gpu
+ * (car_racing_v2.mojo:1556-1716): same dynamics, reward 0.5 * forward speed - 0.01 (+ 100 / tiles for a new
+ * tile) in fp32 from the hull state after the physics, fp32 playfield and lap tests, the episode total taken
+ * after the playfield penalty, and the observation left as the dynamics wrote it. */
+static int cr_step_form = 0;
+void orc_cr_set_step_form(int form) { cr_step_form = form; }
+
 void orc_cr_step(float *row, const float *action, float *reward, float *done) {
     float *M = row + CR_META;
     if (M[M_DONE] > 0.5f) { *reward = 0.0f; *done = 1.0f; return; }
     int num_tiles = (int)M[M_NUM_TILES];
     if (num_tiles <= 0) num_tiles = 100;
-    /* car_racing_v2.mojo:262-268: Float64 clamp and remap, stored as fp32 controls */
+    /* car_racing_v2.mojo:262-268: Float64 clamp and remap, stored as fp32 controls.  (The trait's fp32
+     * decoding, :1583-1603, gives the same controls: the halving is exact, so both round a + 1 once.) */
     double steering = (double)action[0];
     steering = steering < -1.0 ? -1.0 : (steering > 1.0 ? 1.0 : steering);
     double gas = ((double)action[1] + 1.0) * 0.5;
@@ -243,8 +252,39 @@ void orc_cr_step(float *row, const float *action, float *reward, float *done) {
     brake = brake < 0.0 ? 0.0 : (brake > 1.0 ? 1.0 : brake);
     row[CR_CTRL + 0] = (float)steering; row[CR_CTRL + 1] = (float)gas; row[CR_CTRL + 2] = (float)brake;
     physics_step(row, num_tiles, (float)0.02);
-    /* _check_tiles_and_reward, :781-809 */
     float hull_x = row[CR_HULL + H_X], hull_y = row[CR_HULL + H_Y];
+    if (cr_step_form == 1) {
+        /* step_kernel_gpu, :1622-1710 */
+        float hull_vx = row[CR_HULL + H_VX], hull_vy = row[CR_HULL + H_VY], hull_angle = row[CR_HULL + H_ANGLE];
+        float cos_angle = f32_cos(hull_angle), sin_angle = f32_sin(hull_angle);
+        float forward_vel = hull_vx * cos_angle + hull_vy * sin_angle;
+        float step_reward = forward_vel * (float)0.5 - (float)0.01;
+        int tile_idx = orc_cr_tile_at(row, hull_x, hull_y, num_tiles);
+        float tiles_visited = M[M_VISITED];
+        if (tile_idx >= 0 && !(row[CR_VISITED + tile_idx] > 0.5f)) {
+            row[CR_VISITED + tile_idx] = 1.0f;
+            float tile_reward = (float)100.0 / (float)num_tiles;
+            step_reward = step_reward + tile_reward;
+            tiles_visited = tiles_visited + 1.0f;
+            M[M_VISITED] = tiles_visited;
+        }
+        float is_done = 0.0f;
+        const float playfield = (float)(2000.0 / SCALE_);
+        float abs_x = hull_x >= 0.0f ? hull_x : -hull_x, abs_y = hull_y >= 0.0f ? hull_y : -hull_y;
+        if (abs_x > playfield || abs_y > playfield) { is_done = 1.0f; step_reward = (float)-100.0; }
+        float num_tiles_f = (float)(num_tiles > 1 ? num_tiles : 1);
+        float progress = tiles_visited / num_tiles_f;
+        if (progress >= (float)0.95) is_done = 1.0f;
+        float step_count = M[M_STEP] + 1.0f;
+        M[M_STEP] = step_count;
+        if (step_count >= (float)500.0) { is_done = 1.0f; M[M_TRUNC] = 1.0f; }
+        M[M_TOTAL] = M[M_TOTAL] + step_reward;
+        M[M_DONE] = is_done;
+        *reward = step_reward;
+        *done = is_done;
+        return;
+    }
+    /* _check_tiles_and_reward, :781-809 */
     int tile_idx = orc_cr_tile_at(row, hull_x, hull_y, num_tiles);
     double step_reward = -0.1;
     float tiles_visited = M[M_VISITED];

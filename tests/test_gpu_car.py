@@ -40,10 +40,24 @@ def driver(rng, s_h, t):
     return a
 
 
-@pytest.mark.parametrize("batch,seed", [(1, 1), (37, 2), (2048, 3)])
-def test_car_racing_reset_and_rollout_parity(mrl, orc, ctx, batch, seed):
-    say("car racing batch", batch)
+@pytest.mark.parametrize("batch,seed,form", [(1, 1, 0), (37, 2, 0), (2048, 3, 0), (37, 4, 1), (2048, 5, 1)])
+def test_car_racing_reset_and_rollout_parity(mrl, orc, batch, seed, form):
+    """form 0: the CPU env's step (the default); form 1: the GPU trait's step_kernel_gpu
+    (car_racing_v2.mojo:1556-1716: reward 0.5 * forward speed - 0.01 + tile reward in fp32), selected per
+    context with CarRacingV2.set_step_form and in the oracle with orc_cr_set_step_form."""
+    say("car racing batch", batch, "step form", form)
     E = mrl.CarRacingV2
+    ctx = mrl.DeviceContext("cuda:0")          # a context of its own: the setting belongs to the context
+    E.set_step_form(ctx, form)
+    orc.orc_cr_set_step_form(form)
+    try:
+        _rollout_parity(mrl, orc, ctx, E, batch, seed, form)
+    finally:
+        orc.orc_cr_set_step_form(0)
+        ctx.close()
+
+
+def _rollout_parity(mrl, orc, ctx, E, batch, seed, form):
     s_h = np.zeros((batch, S), np.float32)
     orc.orc_cr_reset_batch(s_h, None, batch, seed)
     s = torch.full((batch * S,), 7.0, device="cuda")          # garbage: the reset must write every float
@@ -80,6 +94,9 @@ def test_car_racing_reset_and_rollout_parity(mrl, orc, ctx, batch, seed):
     say("  finished rows", n_done, "tiles newly visited", new_tiles)
     if batch > 100:
         assert n_done > batch // 8 and new_tiles > batch
+    if form == 1:
+        with pytest.raises(mrl.MrlError, match="neither"):
+            E.set_step_form(ctx, 2)
 
 
 def test_car_racing_done_rows_stay_untouched(mrl, orc, ctx):

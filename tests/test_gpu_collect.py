@@ -267,8 +267,24 @@ def test_fused_collection_with_wind(mrl, orc, env, N):
 
 
 @pytest.mark.parametrize("env,kind,N", [("bipedal", "tanh", 512), ("cheetah", "tanh", 512), ("car", "relu", 300),
-                                        ("bipedal", "relu", 45)])
-def test_fused_walker_collection_against_the_oracle(mrl, ctx, orc, env, kind, N):
+                                        ("bipedal", "relu", 45), ("car_trait", "tanh", 300)])
+def test_fused_walker_collection_against_the_oracle(mrl, orc, env, kind, N):
+    """car_trait: CarRacingV2 with the reward and termination arithmetic of the GPU trait's step
+    (car_racing_v2.mojo:1556-1716) selected for the context and for the oracle."""
+    ctx = mrl.DeviceContext("cuda:0")           # a context of its own: the step form belongs to the context
+    trait = env == "car_trait"
+    if trait:
+        env = "car"
+        mrl.CarRacingV2.set_step_form(ctx, mrl.CarRacingV2.STEP_GPU_TRAIT)
+        orc.orc_cr_set_step_form(1)
+    try:
+        _walker_collection_against_the_oracle(mrl, ctx, orc, env, kind, N)
+    finally:
+        orc.orc_cr_set_step_form(0)
+        ctx.close()
+
+
+def _walker_collection_against_the_oracle(mrl, ctx, orc, env, kind, N):
     """The fused collection kernels of BipedalWalker, HalfCheetah and CarRacingV2 in launches of one step,
     against the oracle fed the kernel's own actions: rewards and done flags exact, the rows (state after
     the in-launch reset of finished envs) and the observation bit for bit; then the same 64 steps in two
@@ -345,10 +361,18 @@ def test_barrier_wait_gives_up_and_reports(mrl, env):
     one, many = _pair(mrl, ctx, N, T, 256, "relu", env)
     s0, ss = 99, 7919
     ctx.set_spin_limit(1)
+    before, obs_before = many.states.clone(), many.obs.clone()
     mrl.ppo.rollout_steps(ctx, many.descriptor(), 0, T, s0, ss, 0, 0, 5, 1)
     with pytest.raises(mrl.MrlError, match="internal barriers"):
         ctx.synchronize()
     ctx.synchronize()                       # reported once, then cleared
+    # a workgroup that gave up stores nothing: its rows and observations are those from before the launch
+    S = many.env.STATE_SIZE
+    kept = (many.states.view(N, S) == before.view(N, S)).all(1)
+    obs_kept = (many.obs.view(N, -1) == obs_before.view(N, -1)).all(1)
+    print("  rows left as they were:", int(kept.sum()), "of", N, flush=True)
+    assert int(kept.sum()) >= 16 and bool((obs_kept | ~kept).all())
+    assert bool(torch.isfinite(many.states).all())
     ctx.set_spin_limit(0)
     one, many = _pair(mrl, ctx, N, T, 256, "relu", env)
     d1, d2 = one.descriptor(), many.descriptor()

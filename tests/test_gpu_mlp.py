@@ -114,6 +114,36 @@ def test_forward_matches_torch_fp32_at_update_size(mrl, ctx):
     torch.testing.assert_close(grads, want_g, rtol=1e-4, atol=1e-4 * float(want_g.abs().max()))
 
 
+@pytest.mark.parametrize("H", [32, 256])      # 32: the layer-by-layer kernels; 256: the fused tile kernels
+def test_tanh_layer_keeps_relative_accuracy_for_small_arguments(mrl, ctx, H):
+    """The hidden layers' tanh against (float)tanh((double)x) over a log-spaced sweep of both signs,
+    1e-9 .. 12: absolute error below 3e-7 AND relative error below 2e-6 (the exp-based form alone
+    cancels for small |x|: relative error 1e-3 at 1e-4, and 0 instead of x below 3e-8).  Read from the
+    cache of the first LinearTanh layer of an 8 -> H -> H -> 1 net whose first layer passes column 0
+    of the input through unchanged (weights 1, bias 0), for the layer-by-layer and the fused forward."""
+    model = mk(mrl, [(TANH, 8, H), (TANH, H, H), (LIN, H, 1)])
+    mags = np.concatenate([np.logspace(-9, np.log10(12.0), 2040), [0.125, np.nextafter(np.float32(0.125), 0), 0.0, 1.0]])
+    x = np.concatenate([mags, -mags]).astype(np.float32)
+    B = x.size
+    assert B == 4088
+    inp = np.zeros((B, 8), np.float32); inp[:, 0] = x
+    p = np.zeros(model.PARAM_SIZE, np.float32)
+    p[:H] = 1.0                                             # W0[0, :] = 1, every other weight and bias 0
+    out = torch.zeros(B, device="cuda"); cache = torch.zeros(B * model.CACHE_SIZE, device="cuda")
+    model.forward_gpu_ws(ctx, out, torch.from_numpy(inp.reshape(-1)).cuda(), torch.from_numpy(p).cuda(), cache)
+    ctx.synchronize()
+    y = cache[:B * (8 + H)].cpu().numpy().reshape(B, 8 + H)[:, 8:]       # layer 0: [input | tanh output] per row
+    want = np.tanh(x.astype(np.float64)).astype(np.float32)
+    for j in (0, H - 1):
+        err = np.abs(y[:, j].astype(np.float64) - want)
+        assert err.max() < 3e-7
+        nz = want != 0
+        assert (err[nz] / np.abs(want[nz])).max() < 2e-6, float((err[nz] / np.abs(want[nz])).max())
+        assert np.array_equal(y[~nz, j], want[~nz])
+        tiny = np.abs(x) < 1e-4
+        np.testing.assert_array_equal(y[tiny, j], x[tiny])                # tanh x = x to fp32 there
+
+
 def test_mlp_argument_errors(mrl, ctx):
     model = mk(mrl, [(RELU, 8, 16), (LIN, 16, 2)])
     p = torch.zeros(model.PARAM_SIZE, device="cuda")

@@ -177,5 +177,11 @@ def test_train_gpu_cpu_env_steps_host_envs_and_learns(mrl, continuous):
     assert first < 0.7 * L and last > 0.85 * L
     # the episode target inside a rollout ends the call without an update for that rollout
     t_before = agent.actor.optimizer.t
+    seen = [len(e.log) for e in envs]
     m3 = agent.train_gpu_cpu_env(ctx, envs, num_episodes=5)
     assert m3.rollouts == 0 and len(m3.episode_rewards) >= 5 and agent.actor.optimizer.t == t_before
+    # ... after the rollout's steps have all been taken: the reference tests the episode target behind its
+    # `for t in range(rollout_len)` loop, not inside it (ppo.mojo:3290, :3454-3456), so every env has been
+    # stepped T more times and every episode that ended on the way is in the metrics
+    assert [len(e.log) - n for e, n in zip(envs, seen)] == [T] * N and m3.total_steps == N * T
+    assert len(m3.episode_rewards) == N * T // L

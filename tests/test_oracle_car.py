@@ -259,3 +259,70 @@ def test_driving_round_the_track_collects_tiles(orc):
     flags = row[VISITED:VISITED + n]
     assert seen > 20 and flags.sum() == seen and flags[:seen].sum() >= seen - 4      # in order, a tile or two skipped
     np.testing.assert_allclose(total, -0.1 * row[META + 0] + seen * 100.0 / n, rtol=1e-4)
+
+
+def test_trait_step_form_reward_and_termination(orc):
+    """orc_cr_set_step_form(1) = the GPU trait's step_kernel_gpu (car_racing_v2.mojo:1556-1716), pinned
+    against the CPU form and against the formula evaluated independently in float64:
+    the row after a step is the CPU form's except for the episode total (same dynamics, controls,
+    visited flags, observation); reward = 0.5 * (vx cos(angle) + vy sin(angle)) - 0.01 from the hull state
+    AFTER the physics (+ 100 / n on a new tile, once); -100 off the playfield, and there the episode total
+    takes the penalty (the CPU form's takes the step reward it had before); lap and step-limit
+    terminations as in the CPU form."""
+    try:
+        rng = np.random.default_rng(5)
+        a_row, b_row = fresh(orc, 4, 3), fresh(orc, 4, 3)
+        T, n = tiles(a_row)
+        centre = T[:, :8].reshape(n, 4, 2).mean(1)
+        total64, new_tiles = 0.0, 0
+        for t in range(150):
+            x, y, ang = a_row[HULL:HULL + 3]                    # the follow-the-next-tile controller, plus jitter
+            tx, ty = centre[min(int(a_row[META + 4]) + 3, n - 1)]
+            err = (math.atan2(ty - y, tx - x) - math.pi / 2 - ang + math.pi) % (2 * math.pi) - math.pi
+            act = [float(np.clip(err * 2.0, -1, 1)) + float(rng.uniform(-0.05, 0.05)),
+                   0.2 if a_row[12] < 12 else -1.0, -1.0]
+            seen = a_row[META + 4]
+            orc.orc_cr_set_step_form(0)
+            r0, d0 = step(orc, a_row, act)
+            orc.orc_cr_set_step_form(1)
+            r1, d1 = step(orc, b_row, act)
+            same = np.ones(S, bool); same[META + 1] = False
+            np.testing.assert_array_equal(a_row[same], b_row[same])
+            assert d0 == d1 == 0.0
+            x, y, ang, vx, vy = (float(v) for v in b_row[HULL:HULL + 5])
+            fresh_tile = b_row[META + 4] - seen
+            want = 0.5 * (vx * math.cos(ang) + vy * math.sin(ang)) - 0.01 + fresh_tile * 100.0 / n
+            assert abs(r1 - want) < 2e-6 * max(1.0, abs(want)), (t, r1, want)
+            np.testing.assert_allclose(r0, -0.1 + fresh_tile * 100.0 / n, rtol=1e-6)
+            total64 += want; new_tiles += int(fresh_tile)
+            np.testing.assert_allclose(b_row[META + 1], total64, rtol=1e-5, atol=1e-5)
+        assert new_tiles > 5 and b_row[12] > 5.0            # the car drove: the speed term is not a constant
+        # the axis of the speed term is (cos angle, sin angle), as the kernel writes it (the tyres' rolling
+        # direction is (-sin, cos), so this is across the wheels and a step's tyre forces eat into it)
+        for ang, vx, vy, fwd in ((0.0, 7.0, 0.0, 7.0), (math.pi / 2, 0.0, 7.0, 7.0), (0.0, 0.0, 7.0, 0.0)):
+            row = fresh(orc, 3, 0); row[VISITED] = 1.0
+            row[HULL + 2], row[HULL + 3], row[HULL + 4] = ang, vx, vy
+            r1, _ = step(orc, row, [0, -1, -1])
+            v = row[HULL + 3] * math.cos(row[HULL + 2]) + row[HULL + 4] * math.sin(row[HULL + 2])
+            assert abs(r1 - (0.5 * v - 0.01)) < 1e-5 and abs(v - fwd) < 3.0
+        # off the playfield: -100, done, and the total takes the penalty
+        out = fresh(orc, 3, 0); out[HULL] = 334.0; out[META + 1] = 5.0
+        assert step(orc, out, [0, -1, -1]) == (-100.0, 1.0) and out[META + 1] == -95.0 and out[META + 2] == 1
+        before = out.copy()
+        assert step(orc, out, [1, 1, 1]) == (0.0, 1.0) and np.array_equal(out, before)
+        orc.orc_cr_set_step_form(0)
+        out0 = fresh(orc, 3, 0); out0[HULL] = 334.0; out0[META + 1] = 5.0
+        assert step(orc, out0, [0, -1, -1]) == (-100.0, 1.0)
+        np.testing.assert_allclose(out0[META + 1], 5.0 - 0.1, rtol=1e-6)          # no tile under a car out there
+        orc.orc_cr_set_step_form(1)
+        # lap complete and step limit
+        lap = fresh(orc, 3, 0)
+        T, n = tiles(lap)
+        lap[META + 4] = math.ceil(0.95 * n) - 1
+        r, d = step(orc, lap, [0, -1, -1])
+        assert d == 1.0 and lap[META + 3] == 0 and abs(r - (100.0 / n - 0.01)) < 1e-3     # at rest: no speed term to speak of
+        late = fresh(orc, 3, 0); late[META + 0] = 499
+        r, d = step(orc, late, [0, -1, -1])
+        assert d == 1.0 and late[META + 3] == 1 and late[META + 0] == 500
+    finally:
+        orc.orc_cr_set_step_form(0)
