@@ -144,6 +144,9 @@ def cpu_baseline(np, n_envs=2048, steps=120):
         list(pool.map(lambda k: _cpu_update(np, orc, o, mb, k), range(cores)))
     duc = time.perf_counter() - t0
     return {"value": per * cores * steps / dtc, "unit": "env-steps/s", "cores": cores, "kind": "port",
+            # cores = threads used: this job's CPU share of the box (OMP_NUM_THREADS there, at most 16);
+            # host_cores = what the host reports, most of which belongs to other jobs
+            "host_cores": os.cpu_count(),
             "single_thread_value": single,
             "update_samples_per_s": mb * cores / duc, "update_single_thread_samples_per_s": mb / du1,
             "sample": "LunarLander collection steps (env step + actor / critic forward + sampling + reset): "
@@ -188,6 +191,13 @@ def main():
     ap.add_argument("--min-timed-ms", type=float, default=150.0,
                     help="the timed region of `steps` steps is repeated until this much time has been measured; "
                          "the median repeat is reported")
+    ap.add_argument("--full-update", action="store_true",
+                    help="after the rollout, time the whole PPO update of the collected batch as the reference runs "
+                         "it: bootstrap values, reward normalisation (continuous agents), GAE, advantage normalisation, "
+                         "then --epochs epochs of (device permutation + every whole minibatch of 4096).  With "
+                         "--workload halfcheetah --steps 1000 this is the full update of the HalfCheetah configuration: "
+                         "10 epochs x 1000 minibatches on 4 096 000 samples")
+    ap.add_argument("--epochs", type=int, default=10, help="epochs of --full-update")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 64 MiB read + 64 MiB write elementwise kernel 10 times, the "
@@ -348,6 +358,25 @@ def main():
     torch.cuda.synchronize()
     gae_ms = (time.perf_counter() - t2) * 1e3
 
+    full = None
+    if args.full_update:
+        # deep_agents/ppo/ppo_continuous.mojo:2852-3260 (ppo.mojo:2296-2727): phases 2 and 3 of one train_gpu
+        # iteration on the batch just collected, no early stop (target_kl = 0)
+        per_epoch = total // MB
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        ran = upd.update(args.epochs, seed=0x5EED)
+        torch.cuda.synchronize()
+        dtf = time.perf_counter() - t3
+        finite = bool(torch.isfinite(anet.params).all().item() and torch.isfinite(cnet.params).all().item())
+        full = {"epochs": ran, "minibatches_per_epoch": per_epoch, "minibatch": MB, "batch_samples": total,
+                "samples_processed": ran * per_epoch * MB, "ms": 1e3 * dtf,
+                "samples_per_s": ran * per_epoch * MB / dtf, "ms_per_minibatch": 1e3 * dtf / max(1, ran * per_epoch),
+                "includes": "bootstrap value forward, reward normalisation (continuous), GAE, advantage normalisation, "
+                            "per epoch one device permutation and every whole minibatch (forward, loss gradients, "
+                            "backward, clip, Adam)",
+                "adam_steps_taken": anet.optimizer.t, "parameters_finite": finite}
+
     out = {
         "metric": "env-steps/s incl. policy fwd on 1 MI355X; PPO update samples/s",
         "value": env_steps_per_s, "unit": "env-steps/s", "n_gpus": 1, "steps": T, "warmup": args.warmup,
@@ -369,6 +398,9 @@ def main():
                         update_TFLOPs=3.0 * FWD_FLOPS * update_sps / 1e12),
         "roofline": roofline,
     }
+    if full is not None:
+        out["full_update_samples_per_s"] = full["samples_per_s"]
+        out["full_update"] = full
     if two is not None:
         out["two_kernels_per_step"] = two
     if args.copy_calibration:

@@ -116,8 +116,8 @@ MRL_DEV void physics_lanes(float *row, float *contacts, int n, int lane) {
         float *C = contacts + c * CONTACT_SIZE;
         const ContactFixed f = contact_prepare<OneBody>(B1, 0, C[C_PX], C[C_PY], C[C_NX], C[C_NY]);
         C[C_PX] = f.ra_x; C[C_PY] = f.ra_y;
-        contacts[L::MAX_CONTACTS * CONTACT_SIZE + 2 * c] = f.k;
-        contacts[L::MAX_CONTACTS * CONTACT_SIZE + 2 * c + 1] = f.k_t;
+        float *K = contacts + L::MAX_CONTACTS * CONTACT_SIZE + 4 * c;
+        K[0] = f.k; K[1] = f.k_t; K[2] = f.rk; K[3] = f.rk_t;
     }
     // ... and the joint's lever arms, K^-1 and limit angle (joints/revolute.mojo:90-200), by the child
     float sin_a, cos_a;
@@ -137,6 +137,7 @@ MRL_DEV void physics_lanes(float *row, float *contacts, int n, int lane) {
         inv_k11 = k22 * inv_det; inv_k12 = -k12 * inv_det; inv_k22 = k11 * inv_det;
     }
     const float eff = p_ii + ii;
+    const float reff = 1.0f / eff;   // the limit and motor terms of every sweep divide by eff (div_by)
     const float angle_error = (ang - p_ang) - jref;
     const float spring_term = -jstiff * angle_error;
     const float rel_angle = ang - p_ang - jref;
@@ -149,8 +150,8 @@ MRL_DEV void physics_lanes(float *row, float *contacts, int n, int lane) {
             ContactFixed f;
             f.nx = C[C_NX]; f.ny = C[C_NY]; f.ra_x = C[C_PX]; f.ra_y = C[C_PY];
             f.inv_mass_a = im; f.inv_inertia_a = ii;
-            f.k = contacts[L::MAX_CONTACTS * CONTACT_SIZE + 2 * c];
-            f.k_t = contacts[L::MAX_CONTACTS * CONTACT_SIZE + 2 * c + 1];
+            const float *K = contacts + L::MAX_CONTACTS * CONTACT_SIZE + 4 * c;
+            f.k = K[0]; f.k_t = K[1]; f.rk = K[2]; f.rk_t = K[3];
             float jn = C[C_JN], jt = C[C_JT];
             B1.vx[0] = vx; B1.vy[0] = vy; B1.w[0] = w;
             contact_velocity<OneBody>(B1, 0, f, jn, jt, friction, restitution);
@@ -178,18 +179,19 @@ MRL_DEV void physics_lanes(float *row, float *contacts, int n, int lane) {
                 const float spring_torque = spring_term - jdamp * rel_omega;
                 const float angular_impulse = spring_torque * dt;
                 if (e > 1e-10f) {
-                    cur_wa = cur_wa - inv_ia * angular_impulse / e;
-                    cur_wb = cur_wb + inv_ib * angular_impulse / e;
+                    cur_wa = cur_wa - div_by(inv_ia * angular_impulse, e, reff);
+                    cur_wb = cur_wb + div_by(inv_ib * angular_impulse, e, reff);
                 }
             }
             if (jflags & JF_LIMIT) {
                 const float rel_omega = cur_wb - cur_wa;
                 if (e > 1e-10f) {
                     float limit_impulse = 0.0f;
+                    const float stop = div_by(-rel_omega, e, reff);   // the same quotient on both sides of the test
                     if (rel_angle <= jlo) {
-                        if (rel_omega < 0.0f) limit_impulse = -rel_omega / e;
+                        if (rel_omega < 0.0f) limit_impulse = stop;
                     } else if (rel_angle >= jhi) {
-                        if (rel_omega > 0.0f) limit_impulse = -rel_omega / e;
+                        if (rel_omega > 0.0f) limit_impulse = stop;
                     }
                     if (limit_impulse != 0.0f) {
                         cur_wa = cur_wa - inv_ia * limit_impulse;
@@ -201,7 +203,7 @@ MRL_DEV void physics_lanes(float *row, float *contacts, int n, int lane) {
                 const float rel_omega = cur_wb - cur_wa;
                 const float speed_error = motor_speed - rel_omega;
                 if (e > 1e-10f) {
-                    float motor_impulse = speed_error / e;
+                    float motor_impulse = div_by(speed_error, e, reff);
                     const float max_impulse = max_torque * dt;
                     if (motor_impulse > max_impulse) motor_impulse = max_impulse;
                     if (motor_impulse < -max_impulse) motor_impulse = -max_impulse;
@@ -282,8 +284,8 @@ MRL_DEV void physics_lanes(float *row, float *contacts, int n, int lane) {
                         if (relative_angle < jlo) angle_correction = baumgarte * (jlo - relative_angle);
                         else if (relative_angle > jhi) angle_correction = baumgarte * (jhi - relative_angle);
                         if (angle_correction != 0.0f) {
-                            cur_a = cur_a - inv_ia * angle_correction / e;
-                            cur_b = cur_b + inv_ib * angle_correction / e;
+                            cur_a = cur_a - div_by(inv_ia * angle_correction, e, reff);
+                            cur_b = cur_b + div_by(inv_ib * angle_correction, e, reff);
                         }
                     }
                 }

@@ -162,6 +162,8 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
 #pragma unroll
     for (int v = 0; v < 4; ++v) { lvx[v] = S[2 + v * 2]; lvy[v] = S[3 + v * 2]; }
     const float p_im = from_parent(im, b), p_ii = from_parent(ii, b);
+    const float eff = p_ii + ii;
+    const float reff = 1.0f / eff;   // the limit and motor terms of every sweep divide by eff (div_by)
     const double x_before = (double)x;   // meaningful on lane 0 (the torso)
 
     // sine and cosine of my body's angle, kept in step with it (recomputed whenever the angle may have
@@ -229,6 +231,8 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
             k_t = k_t + f.inv_inertia_a * ra_cross_t * ra_cross_t;
             k_t = k_t + inv_inertia_b * rb_cross_t * rb_cross_t;
             f.k_t = k_t;
+            f.rk = 1.0f / k;
+            f.rk_t = 1.0f / k_t;
             cf[q] = f;
         }
         // ... and the joint's lever arms, K^-1 and limit angle (joints/revolute.mojo:90-200), by the child
@@ -247,7 +251,6 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
             const float inv_det = 1.0f / det;
             inv_k11 = k22 * inv_det; inv_k12 = -k12 * inv_det; inv_k22 = k11 * inv_det;
         }
-        const float eff = p_ii + ii;
         const float angle_error = (ang - p_ang) - jref;
         const float spring_term = -jstiff * angle_error;
         const float rel_angle = ang - p_ang - jref;
@@ -266,7 +269,7 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
                 float rel_vel_x = vel_at_a_x - vel_at_b_x, rel_vel_y = vel_at_a_y - vel_at_b_y;
                 const float vel_normal = rel_vel_x * f.nx + rel_vel_y * f.ny;
                 if (!(vel_normal < 0.0f)) continue;
-                float j_normal = -(1.0f + restitution) * vel_normal / f.k;
+                float j_normal = div_by(-(1.0f + restitution) * vel_normal, f.k, f.rk);
                 const float old_impulse = jn[q];
                 float new_impulse = old_impulse + j_normal;
                 if (new_impulse < 0.0f) new_impulse = 0.0f;
@@ -281,7 +284,7 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
                 rel_vel_x = vel_at_a_x - vel_at_b_x; rel_vel_y = vel_at_a_y - vel_at_b_y;
                 const float tangent_x = -f.ny, tangent_y = f.nx;
                 const float vel_tangent = rel_vel_x * tangent_x + rel_vel_y * tangent_y;
-                float j_tangent = -vel_tangent / f.k_t;
+                float j_tangent = div_by(-vel_tangent, f.k_t, f.rk_t);
                 const float max_friction = friction * new_impulse;
                 const float old_tangent = jt[q];
                 float new_tangent = old_tangent + j_tangent;
@@ -315,18 +318,19 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
                     const float spring_torque = spring_term - jdamp * rel_omega;
                     const float angular_impulse = spring_torque * dt;
                     if (e > 1e-10f) {
-                        cur_wa = cur_wa - inv_ia * angular_impulse / e;
-                        cur_wb = cur_wb + inv_ib * angular_impulse / e;
+                        cur_wa = cur_wa - div_by(inv_ia * angular_impulse, e, reff);
+                        cur_wb = cur_wb + div_by(inv_ib * angular_impulse, e, reff);
                     }
                 }
                 if (jflags & JF_LIMIT) {
                     const float rel_omega = cur_wb - cur_wa;
                     if (e > 1e-10f) {
                         float limit_impulse = 0.0f;
+                        const float stop = div_by(-rel_omega, e, reff);   // the same quotient on both sides of the test
                         if (rel_angle <= jlo) {
-                            if (rel_omega < 0.0f) limit_impulse = -rel_omega / e;
+                            if (rel_omega < 0.0f) limit_impulse = stop;
                         } else if (rel_angle >= jhi) {
-                            if (rel_omega > 0.0f) limit_impulse = -rel_omega / e;
+                            if (rel_omega > 0.0f) limit_impulse = stop;
                         }
                         if (limit_impulse != 0.0f) {
                             cur_wa = cur_wa - inv_ia * limit_impulse;
@@ -338,7 +342,7 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
                     const float rel_omega = cur_wb - cur_wa;
                     const float speed_error = motor_speed - rel_omega;
                     if (e > 1e-10f) {
-                        float motor_impulse = speed_error / e;
+                        float motor_impulse = div_by(speed_error, e, reff);
                         const float max_impulse = max_torque * dt;
                         if (motor_impulse > max_impulse) motor_impulse = max_impulse;
                         if (motor_impulse < -max_impulse) motor_impulse = -max_impulse;
@@ -426,8 +430,8 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
                             if (relative_angle < jlo) angle_correction = baumgarte * (jlo - relative_angle);
                             else if (relative_angle > jhi) angle_correction = baumgarte * (jhi - relative_angle);
                             if (angle_correction != 0.0f) {
-                                cur_a = cur_a - inv_ia * angle_correction / e;
-                                cur_b = cur_b + inv_ib * angle_correction / e;
+                                cur_a = cur_a - div_by(inv_ia * angle_correction, e, reff);
+                                cur_b = cur_b + div_by(inv_ib * angle_correction, e, reff);
                             }
                         }
                     }

@@ -27,8 +27,9 @@
 
 namespace mrl {
 
-// floats of LDS scratch per contact: the 9-float record plus two slots for the effective masses
-constexpr int CONTACT_SCRATCH = CONTACT_SIZE + 2;
+// floats of LDS scratch per contact: the 9-float record plus four slots for the two effective masses
+// and their reciprocals
+constexpr int CONTACT_SCRATCH = CONTACT_SIZE + 4;
 
 // Per-body quantities of an env live in short vector values (ext_vector_type), not in arrays:
 // reading or replacing one element of a vector is an operation on the whole value, so the
@@ -134,6 +135,7 @@ MRL_DEV void reg_integrate_positions(RegBodies<L> &B, float dt) {
 // Everything about one contact that stays fixed during the velocity phase.
 struct ContactFixed {
     float nx, ny, ra_x, ra_y, inv_mass_a, inv_inertia_a, k, k_t;
+    float rk, rk_t;   // 1 / k and 1 / k_t: every sweep divides by the effective masses (div_by)
 };
 
 template <class L>
@@ -158,6 +160,8 @@ MRL_DEV ContactFixed contact_prepare(const RegBodies<L> &B, int ia, float point_
     k_t = k_t + f.inv_inertia_a * ra_cross_t * ra_cross_t;
     k_t = k_t + inv_inertia_b * rb_cross_t * rb_cross_t;
     f.k_t = k_t;
+    f.rk = 1.0f / k;
+    f.rk_t = 1.0f / k_t;
     return f;
 }
 
@@ -175,7 +179,7 @@ MRL_DEV void contact_velocity(RegBodies<L> &B, int ia, const ContactFixed &f, fl
     const float vel_normal = rel_vel_x * normal_x + rel_vel_y * normal_y;
     if (!(vel_normal < 0.0f)) return;
 
-    float j_normal = -(1.0f + restitution) * vel_normal / f.k;
+    float j_normal = div_by(-(1.0f + restitution) * vel_normal, f.k, f.rk);
     const float old_impulse = jn;
     float new_impulse = old_impulse + j_normal;
     if (new_impulse < 0.0f) new_impulse = 0.0f;
@@ -191,7 +195,7 @@ MRL_DEV void contact_velocity(RegBodies<L> &B, int ia, const ContactFixed &f, fl
 
     const float tangent_x = -normal_y, tangent_y = normal_x;
     const float vel_tangent = rel_vel_x * tangent_x + rel_vel_y * tangent_y;
-    float j_tangent = -vel_tangent / f.k_t;
+    float j_tangent = div_by(-vel_tangent, f.k_t, f.rk_t);
     const float max_friction = friction * new_impulse;
     const float old_tangent = jt;
     float new_tangent = old_tangent + j_tangent;
@@ -235,7 +239,7 @@ struct RegContacts {
         for (int c = 0; c < MC; ++c) {
             body[c] = 0;
             depth[c] = jn[c] = jt[c] = 0.0f;
-            f[c] = ContactFixed{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 1.0f, 1.0f};
+            f[c] = ContactFixed{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 1.0f, 1.0f, 1.0f, 1.0f};
             if (c < count) {
                 const float *C = contacts + c * CONTACT_SIZE;
                 body[c] = (int)C[C_BODY_A];
@@ -261,15 +265,15 @@ struct RegContacts {
 };
 
 // Contact list left in the lane's LDS scratch (long lists).  After load() the record's contact
-// point slots hold the lever arm (the only way the point enters a sweep) and two slots behind
-// the MAX_CONTACTS records hold each contact's effective masses; body indices, normals, depth
+// point slots hold the lever arm (the only way the point enters a sweep) and four slots behind
+// the MAX_CONTACTS records hold each contact's effective masses and their reciprocals; body indices, normals, depth
 // and accumulated impulses stay where the detector put them.
 template <class L>
 struct LdsContacts {
     int n;
     float *cts;
 
-    MRL_DEV float &k_slot(int c, int which) { return cts[L::MAX_CONTACTS * CONTACT_SIZE + 2 * c + which]; }
+    MRL_DEV float &k_slot(int c, int which) { return cts[L::MAX_CONTACTS * CONTACT_SIZE + 4 * c + which]; }
 
     MRL_DEV void load(const RegBodies<L> &B, float *contacts, int count) {
         n = count;
@@ -280,6 +284,8 @@ struct LdsContacts {
             C[C_PX] = f.ra_x; C[C_PY] = f.ra_y;
             k_slot(c, 0) = f.k;
             k_slot(c, 1) = f.k_t;
+            k_slot(c, 2) = f.rk;
+            k_slot(c, 3) = f.rk_t;
         }
     }
     MRL_DEV void velocity_sweep(RegBodies<L> &B, float friction, float restitution) {
@@ -289,7 +295,7 @@ struct LdsContacts {
             ContactFixed f;
             f.nx = C[C_NX]; f.ny = C[C_NY]; f.ra_x = C[C_PX]; f.ra_y = C[C_PY];
             f.inv_mass_a = sel<L::NUM_BODIES>(B.im, ia); f.inv_inertia_a = sel<L::NUM_BODIES>(B.ii, ia);
-            f.k = k_slot(c, 0); f.k_t = k_slot(c, 1);
+            f.k = k_slot(c, 0); f.k_t = k_slot(c, 1); f.rk = k_slot(c, 2); f.rk_t = k_slot(c, 3);
             float jn = C[C_JN], jt = C[C_JT];
             contact_velocity<L>(B, ia, f, jn, jt, friction, restitution);
             C[C_JN] = jn; C[C_JT] = jt;
@@ -314,8 +320,8 @@ struct RegJoints {
     int ba_[MJ], bb_[MJ], flags[MJ];
     float lo[MJ], hi[MJ], max_torque[MJ], motor_speed[MJ], damp[MJ];
     // fixed during the velocity phase
-    float rax[MJ], ray[MJ], rbx[MJ], rby[MJ], inv_k11[MJ], inv_k12[MJ], inv_k22[MJ], eff[MJ],
-        spring_term[MJ], rel_angle[MJ];
+    float rax[MJ], ray[MJ], rbx[MJ], rby[MJ], inv_k11[MJ], inv_k12[MJ], inv_k22[MJ], eff[MJ], reff[MJ],
+        spring_term[MJ], rel_angle[MJ];   // reff = 1 / eff: the spring, limit and motor terms all divide by eff (div_by)
 
     MRL_DEV int ba(int j) const { return T::STATIC ? T::a(j) : ba_[j]; }
     MRL_DEV int bb(int j) const { return T::STATIC ? T::b(j) : bb_[j]; }
@@ -342,6 +348,7 @@ struct RegJoints {
             max_torque[j] = J[J_MAX_TORQUE]; motor_speed[j] = J[J_MOTOR_SPEED]; damp[j] = J[J_DAMP];
             rax[j] = ray[j] = rbx[j] = rby[j] = inv_k11[j] = inv_k12[j] = inv_k22[j] = 0.0f;
             eff[j] = spring_term[j] = rel_angle[j] = 0.0f;
+            reff[j] = 1.0f;
             if (!active[j]) continue;
             const int a = ba(j), b = bb(j);
             anchor(B, J, a, b, rax[j], ray[j], rbx[j], rby[j]);
@@ -355,6 +362,7 @@ struct RegJoints {
             const float inv_det = 1.0f / det;
             inv_k11[j] = k22 * inv_det; inv_k12[j] = -k12 * inv_det; inv_k22[j] = k11 * inv_det;
             eff[j] = inv_ia + inv_ib;
+            reff[j] = 1.0f / eff[j];
             const float angle_a = sel<L::NUM_BODIES>(B.ang, a), angle_b = sel<L::NUM_BODIES>(B.ang, b);
             const float ref = J[J_REF];
             const float angle_error = (angle_b - angle_a) - ref;
@@ -386,14 +394,14 @@ struct RegJoints {
             float cur_wb = wb + inv_ib * (r_bx * impulse_y - r_by * impulse_x);
 
             const int fl = flags[j];
-            const float e = eff[j];
+            const float e = eff[j], re = reff[j];
             if (fl & JF_SPRING) {
                 const float rel_omega = wb - wa;  // angular velocities from before the point impulse
                 const float spring_torque = spring_term[j] - damp[j] * rel_omega;
                 const float angular_impulse = spring_torque * dt;
                 if (e > 1e-10f) {
-                    cur_wa = cur_wa - inv_ia * angular_impulse / e;
-                    cur_wb = cur_wb + inv_ib * angular_impulse / e;
+                    cur_wa = cur_wa - div_by(inv_ia * angular_impulse, e, re);
+                    cur_wb = cur_wb + div_by(inv_ib * angular_impulse, e, re);
                 }
             }
             if (fl & JF_LIMIT) {
@@ -401,10 +409,12 @@ struct RegJoints {
                 const float rel_omega = cur_wb - cur_wa;
                 if (e > 1e-10f) {
                     float limit_impulse = 0.0f;
+                    // (the same quotient on both sides of the test: taken once, used where the test says)
+                    const float stop = div_by(-rel_omega, e, re);
                     if (relative_angle <= lo[j]) {
-                        if (rel_omega < 0.0f) limit_impulse = -rel_omega / e;
+                        if (rel_omega < 0.0f) limit_impulse = stop;
                     } else if (relative_angle >= hi[j]) {
-                        if (rel_omega > 0.0f) limit_impulse = -rel_omega / e;
+                        if (rel_omega > 0.0f) limit_impulse = stop;
                     }
                     if (limit_impulse != 0.0f) {
                         cur_wa = cur_wa - inv_ia * limit_impulse;
@@ -416,7 +426,7 @@ struct RegJoints {
                 const float rel_omega = cur_wb - cur_wa;
                 const float speed_error = motor_speed[j] - rel_omega;
                 if (e > 1e-10f) {
-                    float motor_impulse = speed_error / e;
+                    float motor_impulse = div_by(speed_error, e, re);
                     const float max_impulse = max_torque[j] * dt;
                     if (motor_impulse > max_impulse) motor_impulse = max_impulse;
                     if (motor_impulse < -max_impulse) motor_impulse = -max_impulse;
@@ -469,8 +479,8 @@ struct RegJoints {
                     if (relative_angle < lo[j]) angle_correction = baumgarte * (lo[j] - relative_angle);
                     else if (relative_angle > hi[j]) angle_correction = baumgarte * (hi[j] - relative_angle);
                     if (angle_correction != 0.0f) {
-                        cur_a = cur_a - inv_ia * angle_correction / e;
-                        cur_b = cur_b + inv_ib * angle_correction / e;
+                        cur_a = cur_a - div_by(inv_ia * angle_correction, e, reff[j]);
+                        cur_b = cur_b + div_by(inv_ib * angle_correction, e, reff[j]);
                     }
                 }
             }
