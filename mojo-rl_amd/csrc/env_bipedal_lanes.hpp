@@ -295,7 +295,9 @@ MRL_DEV void physics_lanes(float *row, float *contacts, int n, int lane) {
             const float g_x = from_kid(s, n_xa, b), g_y = from_kid(s, n_ya, b), g_a = from_kid(s, n_aa, b);
             if ((kidmask >> s) & 1) { x = g_x; y = g_y; ang = g_a; }
             if (myslot == s) { x = n_xb; y = n_yb; ang = n_ab; }
-            if (!(it == 1 && s == 2)) sincos32(ang, sin_a, cos_a);   // (nothing reads them after the last slot)
+            // (the last slot moves leg 2's segments only: the second iteration reads them in its last two slots,
+            // behind another of these, and nothing reads them after the second iteration)
+            if (s != 2) sincos32(ang, sin_a, cos_a);
         }
     }
     // ---- bodies and cleared forces back into the row

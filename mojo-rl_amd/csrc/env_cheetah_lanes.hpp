@@ -83,12 +83,11 @@ MRL_DEV bool lanes_row_ok(const float *row, const float *shapes) {
     return ok;
 }
 
-// everything after the physics of an env step (cheetah_planar_v2.mojo:790-846): reward, metadata,
-// observation; `a` = the clamped action, `penalised` = ground contacts of the last sub-step on
-// bodies other than the two feet
-MRL_DEV void step_tail(float *row, const double *a, double x_before, int penalised, float &reward, float &done) {
-    const float *B = row + L::BODIES_OFF;
-    const double x_after = B[IDX_X], torso_z = B[IDX_Y];
+// everything after the physics of an env step but the observation (cheetah_planar_v2.mojo:790-846): reward
+// and metadata; `a` = the clamped action, (x_after, torso_z) = the torso's position after the physics,
+// `penalised` = ground contacts of the last sub-step on bodies other than the two feet
+MRL_DEV void step_tail(float *row, const double *a, double x_before, double x_after, double torso_z, int penalised,
+                       float &reward, float &done) {
     const double forward_velocity = (x_after - x_before) / (0.01 * (double)5);
     const double forward_reward = 1.0 * forward_velocity;
     double ctrl_cost = 0.0;
@@ -110,7 +109,6 @@ MRL_DEV void step_tail(float *row, const double *a, double x_before, int penalis
     M[META_TOTAL] = (float)((double)M[META_TOTAL] + r);
     const bool d = step_count >= 1000;
     M[META_DONE] = d ? 1.0f : 0.0f;
-    observe(row);
     reward = (float)r;
     done = d ? 1.0f : 0.0f;
 }
@@ -442,7 +440,9 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
                 const float g_a = from_kid_slot(s, n_aa, b);
                 if ((kidmask >> s) & 1) { x = g_x; y = g_y; ang = g_a; }
                 if (myslot == s) { x = n_xb; y = n_yb; ang = n_ab; }
-                sincos32(ang, sin_a, cos_a);
+                // (the last slot moves the front shin and foot only, which the second iteration reads in its
+                // last two slots, behind two more of these; after the second iteration the next sub-step reads all)
+                if (!(it == 0 && s == 3)) sincos32(ang, sin_a, cos_a);
             }
         }
     }
@@ -457,7 +457,18 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
         const int c = group_get(kept, base, o);
         penalised += (o != 3 && o != 6) ? c : 0;
     }
-    wave_sync_lds();
+    // ---- the observation (hc::observe: the same expressions on the same values), every body's lane its own
+    // entries: the torso its height, angle and velocity, a leg segment its angle and angular velocity
+    // against its parent's
+    {
+        const double p_ang = (double)from_parent(ang, b), p_w = (double)from_parent(w, b);
+        if (b == 0) {
+            row[0] = y; row[1] = ang; row[8] = vx; row[9] = vy; row[10] = w;
+        } else if (child) {
+            row[2 + j] = (float)((double)ang - p_ang);
+            row[11 + j] = (float)((double)w - p_w);
+        }
+    }
     if (b == 0) {
         double a[ACT];
 #pragma unroll
@@ -467,8 +478,9 @@ MRL_DEV void step_lanes(float *row, const float *shapes, const float *action, in
             v = v > -1.0f ? v : -1.0f;
             a[k] = (double)v;
         }
-        step_tail(row, a, x_before, penalised, reward, done);
+        step_tail(row, a, x_before, (double)x, (double)y, penalised, reward, done);
     }
+    wave_sync_lds();   // the row is complete for whoever reads it next
 }
 
 }  // namespace hc
