@@ -617,16 +617,41 @@ struct DwSet { DwProblem p[6]; int n; };
 // dW = X^T G of every problem, split over the batch: grid.x = sum of the problems' tiles,
 // grid.y = batch splits; partial[z][P].  The next 32-row chunk is fetched into registers while
 // the matrix cores work on the current one.
+// Workgroups go to the chip's eight XCDs in turn (workgroup n to XCD n % 8), and each XCD has an L2 of its
+// own.  The tiles of one (problem, batch split) read the same rows of X and G -- every 64-column block of X
+// is wanted by all tiles of its tile row, every block of G by all tiles of its tile column --, so the
+// launch is a flat list of workgroups ordered so that those tiles sit on ONE XCD: the group is fetched
+// from memory once and its re-reads are L2 hits (measured: 50 MB -> 17 MB fetched per launch at a
+// minibatch of 4096, which is what X and G hold).  groups = problems x splits, `tiles` workgroups each
+// (every problem of a launch has the same number of tiles); group g runs on XCD g % 8.
+constexpr int XCDS = 8;
+
 __global__ __launch_bounds__(256) void dw3_kernel(DwSet d, int M, int rows_per_split, int P,
-                                                  float *__restrict__ partial) {
+                                                  float *__restrict__ partial, int splits) {
     __shared__ float As[DKC * DLD];
     __shared__ float Bs[DKC * DLD];
-    int tile = blockIdx.x, li = 0;
-    while (li < d.n - 1 && tile >= d.p[li].tiles) { tile -= d.p[li].tiles; ++li; }
+    const int tiles = d.p[0].tiles, groups = d.n * splits;
+    // workgroup n = (round r, XCD x): the r-th workgroup that XCD x receives.  An XCD walks its groups
+    // g = x, x + 8, ... one after the other, `tiles` workgroups each; with a group count that is not a
+    // multiple of 8 the last round is short and its workgroups keep the plain order.
+    int g, tile;
+    {
+        const int n = blockIdx.x, full = (groups / XCDS) * XCDS * tiles;   // workgroups of whole rounds of 8 groups
+        if (n < full) {
+            const int x = n % XCDS, q = n / XCDS;
+            tile = q % tiles;
+            g = (q / tiles) * XCDS + x;
+        } else {
+            const int m = n - full;
+            tile = m % tiles;
+            g = (groups / XCDS) * XCDS + m / tiles;
+        }
+    }
+    const int li = g / splits, z = g % splits;
     const DwProblem &pr = d.p[li];
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wr = w >> 1, wc = w & 1;
     const int half = lane >> 5, l31 = lane & 31;
-    const int j0 = (tile % pr.tiles_n) * DBN, i0 = (tile / pr.tiles_n) * DBM, z = blockIdx.y;
+    const int j0 = (tile % pr.tiles_n) * DBN, i0 = (tile / pr.tiles_n) * DBM;
     const long b_begin = (long)z * rows_per_split;
     long b_end = b_begin + rows_per_split;
     if (b_end > M) b_end = M;
@@ -928,8 +953,9 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
         base += sn.P[i];
     }
     const int Ptot = base;
-    hipLaunchKernelGGL(dw3_kernel, dim3(total_tiles, splits), dim3(256), 0, ctx->stream, dw, batch, rows_per,
-                       Ptot, partial);
+    // (both nets have the same width: every problem has the same number of tiles, see dw3_kernel)
+    hipLaunchKernelGGL(dw3_kernel, dim3(total_tiles * splits), dim3(256), 0, ctx->stream, dw, batch, rows_per,
+                       Ptot, partial, splits);
     const int sum_blocks = grid_for(Ptot, 256);
     if (sum_blocks > 1024) sq_part = nullptr;   // more partials than the caller's buffer holds
     if (sq_blocks) *sq_blocks = sq_part ? sum_blocks : 0;
