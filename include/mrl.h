@@ -49,7 +49,16 @@ enum mrl_env_id {
      * NOT what the reference's step_kernel_gpu pays (0.5 * forward speed - 0.01 + 100 / tiles in fp32,
      * :1636-1666): returns of a run trained with the default are not comparable with the reference's
      * train_gpu.  mrl_car_racing_set_step_form(ctx, MRL_CAR_STEP_GPU_TRAIT) selects the trait's. */
-    MRL_ENV_CARRACING = 6
+    MRL_ENV_CARRACING = 6,
+    /* envs/mujoco_planar/hopper_planar.mojo:162 HopperPlanar and walker_planar.mojo:168 Walker2dPlanar: Float64
+     * CPU structs in the reference (reset() / step(action) on lists of Float64), which has no
+     * GPUContinuousEnv form of them and hence no row layout; here they stand behind the same calls as the
+     * other envs, on rows of this library's own: [obs fp32 (11 / 17) | one float of padding | the struct's
+     * Float64 state, two floats per double: torso x, y, angle, vx, vy, omega; (x, y, angle) of the other
+     * bodies; joint_angles; joint_velocities; step_count, done, total_reward, prev_x] = 62 / 98 floats.
+     * states must be 8-byte aligned.  A row whose done flag is set returns (0, 1) untouched, as elsewhere. */
+    MRL_ENV_HOPPER_PLANAR = 7,
+    MRL_ENV_WALKER2D_PLANAR = 8
 };
 
 /* layer kinds of an MLP description; deep_rl/model/{linear,linear_relu,linear_tanh,stochastic_actor}.mojo */

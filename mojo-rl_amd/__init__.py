@@ -11,7 +11,7 @@ _lib.lib()  # load now: a missing or unloadable HIP library is an import error, 
 
 from .context import DeviceContext  # noqa: E402
 from .envs import (CartPoleEnv, PendulumV2, LunarLanderV2, LunarLanderV2Continuous, BipedalWalkerV2,  # noqa: E402
-                   HalfCheetahPlanarV2, CarRacingV2, VecStepResult)
+                   HalfCheetahPlanarV2, CarRacingV2, HopperPlanar, Walker2dPlanar, VecStepResult)
 from .model import Model, Linear, LinearReLU, LinearTanh, StochasticActor, seq  # noqa: E402
 from .optimizer import Adam  # noqa: E402
 from .training import Network, Xavier, Kaiming, init_params_small  # noqa: E402
@@ -19,7 +19,7 @@ from . import ppo, checkpoint  # noqa: E402
 from .agents import DeepPPOAgent, DeepPPOContinuousAgent, TrainingMetrics  # noqa: E402
 
 __all__ = ["DeviceContext", "CartPoleEnv", "PendulumV2", "LunarLanderV2", "LunarLanderV2Continuous", "BipedalWalkerV2",
-           "HalfCheetahPlanarV2", "CarRacingV2", "VecStepResult", "MrlError", "Model",
+           "HalfCheetahPlanarV2", "CarRacingV2", "HopperPlanar", "Walker2dPlanar", "VecStepResult", "MrlError", "Model",
            "Linear", "LinearReLU", "LinearTanh", "StochasticActor", "seq", "Adam", "ppo",
            "Network", "Xavier", "Kaiming", "init_params_small", "checkpoint",
            "DeepPPOAgent", "DeepPPOContinuousAgent", "TrainingMetrics",

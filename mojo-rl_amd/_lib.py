@@ -19,6 +19,7 @@ LINEAR, LINEAR_RELU, LINEAR_TANH, STOCHASTIC_ACTOR = 0, 1, 2, 3
 ENV_CARTPOLE, ENV_PENDULUM, ENV_LUNARLANDER, ENV_BIPEDAL, ENV_HALFCHEETAH = 0, 1, 2, 3, 4
 ENV_LUNARLANDER_CONTINUOUS = 5
 ENV_CARRACING = 6
+ENV_HOPPER_PLANAR, ENV_WALKER2D_PLANAR = 7, 8
 
 
 class Layer(C.Structure):

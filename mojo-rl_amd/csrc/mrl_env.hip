@@ -13,6 +13,7 @@
 #include "env_block.hpp"
 #include "env_cheetah_lanes.hpp"
 #include "env_car.hpp"
+#include "env_planar.hpp"
 
 namespace mrl {
 
@@ -240,6 +241,49 @@ __global__ __launch_bounds__(CAR_THREADS) void car_reset_kernel(float *states, f
     if (selective && sub == 0) dones[env] = 0.0f;
 }
 
+// HopperPlanar / Walker2dPlanar (env_planar.hpp): one lane per env, the Float64 state in registers for the
+// step; rows are 248 / 392 bytes and are read and written by their lane
+template <class M, bool AUTORESET>
+__global__ __launch_bounds__(256) void planar_step_kernel(float *states, const float *actions, float *rewards,
+                                                          float *dones, float *obs, int batch, uint64_t reset_seed,
+                                                          Accounting acc) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= batch) return;
+    float *row = states + (size_t)i * M::STATE;
+    planar::State<M> s;
+    s.load(row);
+    float a[M::ACT];
+#pragma unroll
+    for (int k = 0; k < M::ACT; ++k) a[k] = actions[(size_t)i * M::ACT + k];
+    const bool was_done = s.meta[1] > 0.5;   // such a row is left as it is
+    float r, d;
+    planar::step<M>(s, a, r, d);
+    const bool fresh = AUTORESET && d > 0.5f;
+    if (fresh) planar::reset<M>(s, planar::combined_seed(reset_seed, i));
+    if (!was_done || fresh) s.store(row);
+    float o[M::OBS];
+    s.observe(o);
+#pragma unroll
+    for (int k = 0; k < M::OBS; ++k) obs[(size_t)i * M::OBS + k] = o[k];
+    rewards[i] = r;
+    dones[i] = d;
+    account(acc, i, r, d);
+}
+
+template <class M>
+__global__ __launch_bounds__(256) void planar_reset_kernel(float *states, float *dones, int batch, uint64_t seed,
+                                                           int selective) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= batch) return;
+    if (selective) {
+        if (!(dones[i] > 0.5f)) return;
+    }
+    planar::State<M> s;
+    planar::reset<M>(s, planar::combined_seed(seed, i));
+    s.store(states + (size_t)i * M::STATE);
+    if (selective) dones[i] = 0.0f;
+}
+
 template <class E>
 __global__ __launch_bounds__(E::THREADS) void phys_reset_kernel(float *states, const float *dones, int batch,
                                                            uint64_t seed, int selective) {
@@ -319,6 +363,8 @@ int mrl_env_dims(int env_id, int *state_size, int *obs_dim, int *num_actions, in
         case MRL_ENV_BIPEDAL: s = bw::STATE; o = bw::OBS; na = 0; ad = bw::ACT; break;
         case MRL_ENV_HALFCHEETAH: s = hc::STATE; o = hc::OBS; na = 0; ad = hc::ACT; break;
         case MRL_ENV_CARRACING: s = cr::STATE; o = cr::OBS; na = 0; ad = cr::ACT; break;
+        case MRL_ENV_HOPPER_PLANAR: s = planar::Hopper::STATE; o = planar::Hopper::OBS; na = 0; ad = planar::Hopper::ACT; break;
+        case MRL_ENV_WALKER2D_PLANAR: s = planar::Walker2d::STATE; o = planar::Walker2d::OBS; na = 0; ad = planar::Walker2d::ACT; break;
         default: return set_error(MRL_E_UNSUPPORTED, "mrl_env_dims: env_id %d is not built", env_id);
     }
     if (state_size) *state_size = s;
@@ -403,6 +449,16 @@ static int env_reset_impl(mrl_ctx *ctx, int env_id, int batch, float *states, fl
             hipLaunchKernelGGL(car_reset_kernel, dim3(grid_for(batch, CAR_RESET_EPB)), dim3(CAR_THREADS), 0, ctx->stream, states,
                                dones, batch, seed, selective);
             break;
+        case MRL_ENV_HOPPER_PLANAR:
+            MRL_CHECK_ARG(reinterpret_cast<uintptr_t>(states) % 8 == 0, "mrl_env_reset: HopperPlanar rows hold doubles: states must be 8-byte aligned");
+            hipLaunchKernelGGL(planar_reset_kernel<planar::Hopper>, dim3(grid_for(batch, 256)), dim3(256), 0, ctx->stream,
+                               states, dones, batch, seed, selective);
+            break;
+        case MRL_ENV_WALKER2D_PLANAR:
+            MRL_CHECK_ARG(reinterpret_cast<uintptr_t>(states) % 8 == 0, "mrl_env_reset: Walker2dPlanar rows hold doubles: states must be 8-byte aligned");
+            hipLaunchKernelGGL(planar_reset_kernel<planar::Walker2d>, dim3(grid_for(batch, 256)), dim3(256), 0, ctx->stream,
+                               states, dones, batch, seed, selective);
+            break;
         default:
             return set_error(MRL_E_UNSUPPORTED, "mrl_env_reset: env_id %d is not built", env_id);
     }
@@ -472,6 +528,25 @@ static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, con
             else
                 hipLaunchKernelGGL((car_step_kernel<false>), grid, block, 0, ctx->stream, states, actions, rewards, dones,
                                    obs, batch, reset_seed, acc, ctx->car_trait_form);
+            break;
+        }
+        case MRL_ENV_HOPPER_PLANAR:
+        case MRL_ENV_WALKER2D_PLANAR: {
+            MRL_CHECK_ARG(reinterpret_cast<uintptr_t>(states) % 8 == 0, "mrl_env_step: the planar envs' rows hold doubles: states must be 8-byte aligned");
+            const dim3 grid(grid_for(batch, 256)), block(256);
+            const bool hopper = env_id == MRL_ENV_HOPPER_PLANAR;
+            if (hopper && autoreset)
+                hipLaunchKernelGGL((planar_step_kernel<planar::Hopper, true>), grid, block, 0, ctx->stream, states, actions,
+                                   rewards, dones, obs, batch, reset_seed, acc);
+            else if (hopper)
+                hipLaunchKernelGGL((planar_step_kernel<planar::Hopper, false>), grid, block, 0, ctx->stream, states, actions,
+                                   rewards, dones, obs, batch, reset_seed, acc);
+            else if (autoreset)
+                hipLaunchKernelGGL((planar_step_kernel<planar::Walker2d, true>), grid, block, 0, ctx->stream, states, actions,
+                                   rewards, dones, obs, batch, reset_seed, acc);
+            else
+                hipLaunchKernelGGL((planar_step_kernel<planar::Walker2d, false>), grid, block, 0, ctx->stream, states, actions,
+                                   rewards, dones, obs, batch, reset_seed, acc);
             break;
         }
         default:

@@ -141,3 +141,16 @@ class CarRacingV2(_GPUEnv):           # envs/car_racing/car_racing_v2.mojo:90
         Float64) or STEP_GPU_TRAIT (step_kernel_gpu, :1556-1716, what the reference's train_gpu runs:
         reward 0.5 * forward speed - 0.01 + 100 / tiles, fp32).  Dynamics and observations are the same."""
         _lib.call("mrl_car_racing_set_step_form", ctx.handle, int(form))
+
+
+class HopperPlanar(_GPUEnv):          # envs/mujoco_planar/hopper_planar.mojo:162
+    """The reference's planar Hopper (a Float64 CPU struct with a simplified physics of its own: 4 bodies,
+    3 joints, observation 11, action 3) behind the batched env calls.  The reference has no GPU form of
+    it; the row is this library's: the fp32 observation, one float of padding, then the struct's Float64
+    state as pairs of floats (include/mrl.h at MRL_ENV_HOPPER_PLANAR)."""
+    ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_HOPPER_PLANAR, 62, 11, 3
+
+
+class Walker2dPlanar(_GPUEnv):        # envs/mujoco_planar/walker_planar.mojo:168
+    """The reference's planar Walker2d (7 bodies, 6 joints, observation 17, action 6), as HopperPlanar."""
+    ENV_ID, STATE_SIZE, OBS_DIM, ACTION_DIM = _lib.ENV_WALKER2D_PLANAR, 98, 17, 6

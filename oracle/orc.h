@@ -179,6 +179,16 @@ void orc_cr_reset_batch(float *states, float *dones, int batch, uint64_t seed);
 void orc_cr_step_batch(float *states, const float *actions, float *rewards, float *dones, float *obs, int batch,
                        int n_threads);
 
+/* ------------------------------------------------- HopperPlanar / Walker2dPlanar ---
+ * envs/mujoco_planar/hopper_planar.mojo, walker_planar.mojo (Float64 CPU structs); which = 0 hopper
+ * (row of 62 floats, obs 11, action 3), 1 walker (98, 17, 6); row layout in orc_planar.c */
+int orc_planar_state_size(int which);
+void orc_planar_reset(int which, float *row, uint64_t combined_seed);
+void orc_planar_step(int which, float *row, const float *action, float *reward, float *done);
+void orc_planar_reset_batch(int which, float *states, const float *dones, int batch, uint64_t seed);
+void orc_planar_step_batch(int which, float *states, const float *actions, float *rewards, float *dones,
+                           float *obs, int batch, int n_threads);
+
 void orc_add_obs_noise(float *obs, int n, int obs_dim, float noise_std, uint32_t seed);
 void orc_gae(int T, int N, const float *rewards, const float *values, const float *dones,
              const float *bootstrap, double gamma, double lam, float *adv, float *ret);

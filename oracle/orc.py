@@ -101,6 +101,11 @@ def load():
         "orc_cr_set_step_form": (None, [C.c_int]),
         "orc_cr_reset_batch": (None, [f32p, C.c_void_p, C.c_int, C.c_uint64]),
         "orc_cr_step_batch": (None, [f32p, f32p, f32p, f32p, f32p, C.c_int, C.c_int]),
+        "orc_planar_state_size": (C.c_int, [C.c_int]),
+        "orc_planar_reset": (None, [C.c_int, f32p, C.c_uint64]),
+        "orc_planar_step": (None, [C.c_int, f32p, f32p, f32p, f32p]),
+        "orc_planar_reset_batch": (None, [C.c_int, f32p, C.c_void_p, C.c_int, C.c_uint64]),
+        "orc_planar_step_batch": (None, [C.c_int, f32p, f32p, f32p, f32p, f32p, C.c_int, C.c_int]),
         "orc_mlp_param_size": (C.c_int, [YP, C.c_int]),
         "orc_mlp_cache_size": (C.c_int, [YP, C.c_int]),
         "orc_mlp_forward": (None, [YP, C.c_int, C.c_int, f32p, f32p, f32p, C.c_void_p]),
