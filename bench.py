@@ -155,10 +155,46 @@ def cpu_baseline(np, n_envs=2048, steps=120):
                       "thread in %.1f s" % (per * cores, steps, cores, dtc, n_envs // 4, steps, dt1, cores, mb, duc, du1)}
 
 
-def measured_traffic():
+# batch at which the stand-alone env-step kernel is timed a second time: large enough that the chip is
+# filled many times over, which is where its rate against the HBM roofline peaks
+ENV_STEP_PEAK_BATCH = {"lunarlander": 524288, "bipedal": 65536, "halfcheetah": 131072, "carracing": 32768,
+                       "cartpole": 4194304, "pendulum": 4194304}
+
+
+def env_step_at_large_batch(mrl, ctx, torch, E, workload, bytes_per_step, steps=40):
+    """The stand-alone step + auto-reset kernel alone (actions fixed, no policy), HIP events around
+    each launch on the launch stream, median launch: us per step, GB/s of algorithmic bytes, fraction
+    of the HBM peak."""
+    n = ENV_STEP_PEAK_BATCH[workload]
+    s = torch.zeros(n * E.STATE_SIZE, device="cuda")
+    E.reset_kernel_gpu(ctx, s, 1)
+    if E.NUM_ACTIONS:
+        a = torch.randint(0, E.NUM_ACTIONS, (n,), device="cuda").float()
+    else:
+        a = torch.rand(n * E.ACTION_DIM, device="cuda") * 2 - 1
+    r, d, o = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda"), torch.zeros(n * E.OBS_DIM, device="cuda")
+    for t in range(60):      # into the mix of flight, contacts and resets
+        E.step_autoreset_kernel_gpu(ctx, s, a, r, d, o, t, 100 + t)
+    ctx.synchronize()
+    with torch.cuda.stream(ctx.stream):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2 * steps)]
+        for t in range(steps):
+            ev[2 * t].record(ctx.stream)
+            E.step_autoreset_kernel_gpu(ctx, s, a, r, d, o, 200 + t, 1000 + t)
+            ev[2 * t + 1].record(ctx.stream)
+    ctx.synchronize()
+    us = sorted(ev[2 * t].elapsed_time(ev[2 * t + 1]) * 1e3 for t in range(steps))
+    med = us[len(us) // 2]
+    gbs = bytes_per_step * n / (med * 1e-6) / 1e9
+    return {"n_envs": n, "us_per_step": med, "env_steps_per_s": n / (med * 1e-6), "GBs": gbs,
+            "frac_hbm": gbs / HBM_PEAK_GBS, "bytes_per_env_step": bytes_per_step}
+
+
+def measured_traffic(steps_per_launch):
     """HBM bytes per launch by kernel name, from the committed counter summary
-    (profiles/bench_lunarlander8192_hbm_traffic.md: FETCH_SIZE / WRITE_SIZE readings of two
-    rocprofv3 --pmc runs of this script, already scaled by the copy-kernel calibration).
+    (profiles/bench_lunarlander8192_hbm_traffic.md: FETCH_SIZE / WRITE_SIZE readings of
+    rocprofv3 --pmc runs of this script, already scaled by the copy-kernel calibration).  A row of
+    the fused collection kernel counts only for launches of the number of steps it was measured at.
     Empty when the file is absent."""
     path = os.path.join(ROOT, "profiles", "bench_lunarlander8192_hbm_traffic.md")
     out = {}
@@ -167,8 +203,8 @@ def measured_traffic():
     with open(path) as f:
         for line in f:
             cells = [c.strip() for c in line.strip().strip("|").split("|")]
-            if len(cells) == 6 and cells[4].isdigit():
-                out[cells[0].replace("void ", "")] = int(cells[4])
+            if len(cells) == 7 and cells[5].isdigit() and cells[1] in ("", str(steps_per_launch)):
+                out[cells[0].replace("void ", "")] = int(cells[5])
     return out
 
 
@@ -278,7 +314,7 @@ def main():
     episodes = int(rb.done_count.item())
 
     ph_us = {k: (1e3 * v[0] / max(v[1], 1)) for k, v in phases.items()}
-    traffic = measured_traffic() if args.workload == "lunarlander" else {}
+    traffic = measured_traffic(SPL) if args.workload == "lunarlander" else {}
     kernels = {}
     if fused:
         # one kernel does everything: its nearest roofline is the fp32 matrix-core peak (the policy
@@ -296,8 +332,8 @@ def main():
         roofline = {"kernel": name + " (policy forward + sampling + env step + auto-reset + rollout stores, %d steps per launch)" % steps_per_launch,
                     "bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
-                    # measured with 250 steps per launch: it describes no other launch shape
-                    "traffic": traffic.get(name) if steps_per_launch == 250 else None,
+                    # the counters were read at 250 and at 20 steps per launch: no figure for other shapes
+                    "traffic": traffic.get(name) if steps_per_launch == SPL else None,
                     "avg_launch_us": launch_us, "steps_per_launch": steps_per_launch,
                     "us_per_step": launch_us / steps_per_launch}
         kernels["collect_TFLOPs"] = tflops
@@ -377,6 +413,10 @@ def main():
                             "backward, clip, Adam)",
                 "adam_steps_taken": anet.optimizer.t, "parameters_finite": finite}
 
+    # the env-step kernel against the HBM roofline where it does best (a batch that fills the chip many
+    # times over), beside the figure at the workload's own batch in env_step_GBs / env_step_frac_hbm
+    env_peak = env_step_at_large_batch(mrl, ctx, torch, E, args.workload, ENV_STEP_BYTES)
+
     out = {
         "metric": "env-steps/s incl. policy fwd on 1 MI355X; PPO update samples/s",
         "value": env_steps_per_s, "unit": "env-steps/s", "n_gpus": 1, "steps": T, "warmup": args.warmup,
@@ -395,7 +435,8 @@ def main():
         "kernels": dict(kernels, policy_fwd_TFLOPs=fwd_tflops, env_step_GBs=env_gbs,
                         env_step_frac_hbm=env_gbs / HBM_PEAK_GBS,
                         policy_fwd_frac_mfma=fwd_tflops / MFMA_FP32_PEAK_TFLOPS,
-                        update_TFLOPs=3.0 * FWD_FLOPS * update_sps / 1e12),
+                        update_TFLOPs=3.0 * FWD_FLOPS * update_sps / 1e12,
+                        env_step_alone_at_large_batch=env_peak),
         "roofline": roofline,
     }
     if full is not None:

@@ -46,6 +46,7 @@ MRL_DEV void account(const Accounting &acc, int i, float r, float d) { account(a
 struct LunarLander {
     using L = ll::L;
     static constexpr int STATE = ll::STATE, OBS = ll::OBS, ACT_W = 1, EPB = 32, THREADS = 512;
+    static constexpr int DENSE_FROM = 24576;   // batch from which the stand-alone step runs 16 rows per workgroup
     static constexpr int DYN_END = L::JOINTS_OFF, NSHAPE = ll::NSHAPE_FLOATS;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
@@ -100,6 +101,7 @@ struct LunarLanderContinuous : LunarLander {
 struct BipedalWalker {
     using L = bw::L;
     static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 16, THREADS = 512;
+    static constexpr int DENSE_FROM = 0;
     static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = bw::NSHAPE_FLOATS;
     // the ten lidar rays of the observation are left out of the step and run afterwards, spread
     // over all wavefronts of the block: task k = part k % 3 of the edges for ray k / 3; the parts of
@@ -168,6 +170,7 @@ struct BipedalWalker {
 struct HalfCheetah {
     using L = hc::L;
     static constexpr int STATE = hc::STATE, OBS = hc::OBS, ACT_W = hc::ACT, EPB = 64, THREADS = 256;
+    static constexpr int DENSE_FROM = 0;
     static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = hc::NSHAPE_FLOATS;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
@@ -421,8 +424,10 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
         // other wavefronts: contacts of one (body, vertex) pair each (read positions only), into
         // lists of their own.  A vertex that fills its list, or a body whose shape the task table
         // does not cover, sends that env back to detection inside step_finish.
-        constexpr int NT = E::DETECT_TASKS, HALF = WAVE / 2;
-        static_assert(E::EPB <= HALF && (NT + 1) / 2 < E::THREADS / WAVE, "two tasks per wavefront besides wavefront 0");
+        // (a wavefront holds WAVE / EPB tasks at a time; a block with fewer such groups than tasks takes turns)
+        constexpr int NT = E::DETECT_TASKS, GROUP = E::EPB, PER_WAVE = WAVE / GROUP;
+        constexpr int AT_ONCE = (E::THREADS / WAVE - 1) * PER_WAVE;
+        static_assert((GROUP == 16 || GROUP == 32) && AT_ONCE > 0, "16 or 32 rows per workgroup, wavefront 0 and at least one more");
         const int wave = tid / WAVE, lane = tid % WAVE;
         typename E::Carry carry{};
         EpisodeSums sums{0.0f, 0.0f};
@@ -431,8 +436,10 @@ MRL_DEV void phys_step_block(float *rows, float *cts, const float *shapes, float
             if (lane < nenv)
                 carry = E::step_begin(rows + lane * S::STRIDE, env0 + lane, actions + (size_t)lane * E::ACT_W, shapes);
         } else {
-            const int task = (wave - 1) * 2 + lane / HALF, e = lane % HALF;
-            if (task < NT && e < nenv) detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
+            const int e = lane % GROUP;
+#pragma unroll 1
+            for (int task = (wave - 1) * PER_WAVE + lane / GROUP; task < NT; task += AT_ONCE)
+                if (e < nenv) detect_vertex_task<E>(rows, shapes, dlist, dcount, task, e);
         }
         __syncthreads();
         if (wave == 0) {

@@ -100,10 +100,9 @@ __global__ __launch_bounds__(256) void pendulum_reset_kernel(float *states, floa
 // AUTORESET = false: step_kernel_gpu of the trait.  AUTORESET = true: step, then rows that
 // finished are re-initialised in place (selective reset) before the observation is copied out.
 template <class E, bool AUTORESET>
-__global__ __launch_bounds__(E::THREADS) void phys_step_kernel(float *states, const float *actions,
-                                                          float *rewards, float *dones, float *obs,
-                                                          const float *shapes_g, int batch,
-                                                          uint64_t reset_seed, Accounting acc) {
+__device__ __forceinline__ void phys_step_body(float *states, const float *actions, float *rewards, float *dones,
+                                               float *obs, const float *shapes_g, int batch, uint64_t reset_seed,
+                                               Accounting acc) {
     using S = Stage<E>;
     __shared__ float rows[E::EPB * S::STRIDE];
     __shared__ float cts[E::EPB * S::CSTRIDE];
@@ -133,6 +132,25 @@ __global__ __launch_bounds__(E::THREADS) void phys_step_kernel(float *states, co
     S::out(rows, gbase, nenv, tid, 0, E::DYN_END);
     S::out(rows, gbase, nenv, tid, E::L::META_OFF, E::STATE);
     if (AUTORESET) S::out_rows(rows, gbase, nenv, was_reset, tid, E::DYN_END, E::L::META_OFF);
+}
+
+template <class E, bool AUTORESET>
+__global__ __launch_bounds__(E::THREADS) void phys_step_kernel(float *states, const float *actions,
+                                                          float *rewards, float *dones, float *obs,
+                                                          const float *shapes_g, int batch,
+                                                          uint64_t reset_seed, Accounting acc) {
+    phys_step_body<E, AUTORESET>(states, actions, rewards, dones, obs, shapes_g, batch, reset_seed, acc);
+}
+
+// The same step for batches that fill the chip several times over: 16 rows per workgroup of four
+// wavefronts and registers bounded for three wavefronts per SIMD, so that a CU holds three workgroups
+// (three solver wavefronts at work instead of one) where the 32-row form holds one.
+template <class E, bool AUTORESET>
+__global__ __launch_bounds__(256, 3) void phys_step_dense_kernel(float *states, const float *actions,
+                                                                 float *rewards, float *dones, float *obs,
+                                                                 const float *shapes_g, int batch,
+                                                                 uint64_t reset_seed, Accounting acc) {
+    phys_step_body<Rows16<E>, AUTORESET>(states, actions, rewards, dones, obs, shapes_g, batch, reset_seed, acc);
 }
 
 // HalfCheetah with one lane per body (env_cheetah_lanes.hpp): a workgroup is one wavefront with
@@ -315,6 +333,18 @@ template <class E>
 static int launch_phys_step(mrl_ctx *ctx, int batch, float *states, const float *actions, float *rewards,
                             float *dones, float *obs, const float *shapes, bool autoreset,
                             uint64_t reset_seed, const Accounting &acc) {
+    if constexpr (E::DENSE_FROM > 0) {
+        if (batch >= E::DENSE_FROM && getenv("MRL_NO_DENSE") == nullptr) {
+            dim3 grid16(grid_for(batch, 16));
+            if (autoreset)
+                hipLaunchKernelGGL((phys_step_dense_kernel<E, true>), grid16, dim3(256), 0, ctx->stream, states, actions,
+                                   rewards, dones, obs, shapes, batch, reset_seed, acc);
+            else
+                hipLaunchKernelGGL((phys_step_dense_kernel<E, false>), grid16, dim3(256), 0, ctx->stream, states, actions,
+                                   rewards, dones, obs, shapes, batch, reset_seed, acc);
+            return MRL_OK;
+        }
+    }
     dim3 grid(grid_for(batch, E::EPB));
     if (autoreset)
         hipLaunchKernelGGL((phys_step_kernel<E, true>), grid, dim3(E::THREADS), 0, ctx->stream, states, actions,

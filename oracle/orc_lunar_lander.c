@@ -357,6 +357,10 @@ void orc_ll_selective_reset_batch(float *states, const float *dones, int batch, 
 
 void orc_ll_step_continuous_batch(float *states, const float *actions, float *rewards, float *dones,
                                   float *obs, int batch) {
+    /* rows are independent; the thread count is the OpenMP default (OMP_NUM_THREADS) */
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
     for (int i = 0; i < batch; ++i) {
         float *row = states + (long)i * ORC_LL_STATE;
         orc_ll_step_continuous(row, i, actions[2 * i], actions[2 * i + 1], rewards + i, dones + i, 0, 0);

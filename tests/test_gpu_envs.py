@@ -287,6 +287,55 @@ def test_lunar_lander_continuous_rollout_parity(mrl, orc, ctx, batch, seed, low)
 
 
 @pytest.mark.parametrize("cont", [False, True])
+def test_lunar_lander_large_batch_form_parity(mrl, orc, ctx, cont):
+    """From 24576 rows on, the stand-alone step runs 16 rows per workgroup of four wavefronts (three
+    workgroups per CU) instead of 32 per workgroup of eight: same results, bit for bit, through steps,
+    contacts, crashes and in-place resets.  The batch has a ragged last workgroup."""
+    batch = 32768 + 5
+    E = mrl.LunarLanderV2Continuous if cont else mrl.LunarLanderV2
+    say("lunar large batch", batch, "continuous", cont)
+    s_h = np.zeros((batch, 192), np.float32)
+    orc.orc_ll_reset_batch(s_h, batch, 31)
+    rng = np.random.default_rng(31)
+    b = s_h[:, 8:47].reshape(batch, 3, 13)
+    b[:, :, 1] -= rng.uniform(7.5, 9.4, batch).astype(np.float32)[:, None]
+    b[:, :, 0] += rng.uniform(-6, 6, batch).astype(np.float32)[:, None]
+    s = dev(s_h.reshape(-1))
+    aw = 2 if cont else 1
+    a = torch.zeros(batch * aw, device="cuda")
+    r, d, o = (torch.zeros(n, device="cuda") for n in (batch, batch, batch * 8))
+    r_h, d_h, o_h = np.zeros(batch, np.float32), np.zeros(batch, np.float32), np.zeros((batch, 8), np.float32)
+    n_done = 0
+    for t in range(12):
+        if cont:
+            act = llc_policy(rng, s_h[:, :8])
+        else:
+            act = rng.integers(0, 4, batch).astype(np.float32)
+        a.copy_(dev(act.reshape(-1)))
+        if t % 2 == 0:      # both entry points take the large-batch form
+            E.step_autoreset_kernel_gpu(ctx, s, a, r, d, o, t, 600 + t)
+        else:
+            E.step_kernel_gpu(ctx, s, a, r, d, o, t)
+            E.selective_reset_kernel_gpu(ctx, s, d.clone(), 600 + t)
+        if cont:
+            orc.orc_ll_step_continuous_batch(s_h, act, r_h, d_h, o_h, batch)
+        else:
+            orc.orc_ll_step_batch(s_h, act, r_h, d_h, o_h, batch, 8)
+        orc.orc_ll_selective_reset_batch(s_h, d_h, batch, 600 + t)
+        ctx.synchronize()
+        sg = s.cpu().numpy().reshape(batch, 192)
+        same_bits(sg, s_h, "state, step %d" % t)
+        np.testing.assert_array_equal(d.cpu().numpy(), d_h)
+        np.testing.assert_array_equal(r.cpu().numpy(), r_h)
+        if t % 2 == 0:      # the observation of the row as it stands after the reset
+            same_bits(o.cpu().numpy().reshape(batch, 8), sg[:, :8], "obs, step %d" % t)
+        n_done += int(d_h.sum())
+        s_h[:] = sg
+    say("  finished rows seen:", n_done)
+    assert n_done > 1000
+
+
+@pytest.mark.parametrize("cont", [False, True])
 def test_lunar_lander_wind_parity(mrl, orc, cont):
     """ENABLE_WIND (lunar_lander_v2.mojo:123-127, :983-1023) as a setting of the context: 64 steps of both
     action forms against the oracle with the same setting, bit for bit; the rows start at different step
