@@ -38,6 +38,11 @@ WORKLOADS = {
     # per env-step: the 300 x 9 tile table read once (10800 B) + 40 floats of car state read and written
     "carracing": ("CarRacingV2", 4096, 256, "tanh", 11120,
                   "CarRacing (state-based) continuous, 4096 envs, Gaussian 13-256-256-3 + value"),
+    # Float64 rows read and written once (248 / 392 B each way) + actions, observation, reward, done
+    "hopper": ("HopperPlanar", 4096, 256, "tanh", 560,
+               "HopperPlanar continuous (Float64 simplified physics), 4096 envs, Gaussian 11-256-256-3 + value"),
+    "walker2d": ("Walker2dPlanar", 4096, 256, "tanh", 884,
+                 "Walker2dPlanar continuous (Float64 simplified physics), 4096 envs, Gaussian 17-256-256-6 + value"),
 }
 
 
@@ -158,7 +163,7 @@ def cpu_baseline(np, n_envs=2048, steps=120):
 # batch at which the stand-alone env-step kernel is timed a second time: large enough that the chip is
 # filled many times over, which is where its rate against the HBM roofline peaks
 ENV_STEP_PEAK_BATCH = {"lunarlander": 524288, "bipedal": 65536, "halfcheetah": 131072, "carracing": 32768,
-                       "cartpole": 4194304, "pendulum": 4194304}
+                       "cartpole": 4194304, "pendulum": 4194304, "hopper": 1048576, "walker2d": 1048576}
 
 
 def env_step_at_large_batch(mrl, ctx, torch, E, workload, bytes_per_step, steps=40):
@@ -367,7 +372,9 @@ def main():
             name = {"lunarlander": "mrl::phys_step_kernel<mrl::LunarLander, true>",
                     "bipedal": "mrl::phys_step_kernel<mrl::BipedalWalker, true>",
                     "halfcheetah": "mrl::hc_lanes_step_kernel<true>", "carracing": "mrl::car_step_kernel<true>",
-                    "cartpole": "mrl::cartpole_step_kernel", "pendulum": "mrl::pendulum_step_kernel"}[args.workload]
+                    "cartpole": "mrl::cartpole_step_kernel", "pendulum": "mrl::pendulum_step_kernel",
+                    "hopper": "mrl::planar_step_kernel<mrl::planar::Hopper, true>",
+                    "walker2d": "mrl::planar_step_kernel<mrl::planar::Walker2d, true>"}[args.workload]
             roofline = {"kernel": name + " (env step + auto-reset + post-step stores)", "bound": "hbm",
                         "achieved": env_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": env_gbs / HBM_PEAK_GBS,
                         "traffic": traffic.get(name), "avg_launch_us": env_us}
