@@ -260,32 +260,58 @@ __global__ __launch_bounds__(CAR_THREADS) void car_reset_kernel(float *states, f
 }
 
 // HopperPlanar / Walker2dPlanar (env_planar.hpp): one lane per env, the Float64 state in registers for the
-// step; rows are 248 / 392 bytes and are read and written by their lane
+// step.  Rows are 248 / 392 bytes: a workgroup's 128 rows are one contiguous range, copied to LDS and back
+// with every lane moving 8 bytes next to its neighbour's; a lane then reads its own row out of LDS (a row is
+// an odd number of doubles, so the lanes' reads of one field fall into different banks).
+constexpr int PLANAR_ROWS = 128;
 template <class M, bool AUTORESET>
-__global__ __launch_bounds__(256) void planar_step_kernel(float *states, const float *actions, float *rewards,
-                                                          float *dones, float *obs, int batch, uint64_t reset_seed,
-                                                          Accounting acc) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= batch) return;
-    float *row = states + (size_t)i * M::STATE;
-    planar::State<M> s;
-    s.load(row);
-    float a[M::ACT];
+__global__ __launch_bounds__(PLANAR_ROWS) void planar_step_kernel(float *states, const float *actions, float *rewards,
+                                                                  float *dones, float *obs, int batch,
+                                                                  uint64_t reset_seed, Accounting acc) {
+    __shared__ __align__(16) float slab[PLANAR_ROWS * M::STATE];
+    static_assert(M::STATE % 2 == 0 && (M::STATE / 2) % 2 == 1, "rows are whole doubles, an odd number of them");
+    const int tid = threadIdx.x;
+    const int env0 = blockIdx.x * PLANAR_ROWS;
+    const int nenv = min(PLANAR_ROWS, batch - env0);
+    float2 *g = reinterpret_cast<float2 *>(states + (size_t)env0 * M::STATE);
+    float2 *l = reinterpret_cast<float2 *>(slab);
+    constexpr int PER_LANE = M::STATE / 2;           // 8-byte pieces of the slab per lane when it is full
+    if (nenv == PLANAR_ROWS) {
 #pragma unroll
-    for (int k = 0; k < M::ACT; ++k) a[k] = actions[(size_t)i * M::ACT + k];
-    const bool was_done = s.meta[1] > 0.5;   // such a row is left as it is
-    float r, d;
-    planar::step<M>(s, a, r, d);
-    const bool fresh = AUTORESET && d > 0.5f;
-    if (fresh) planar::reset<M>(s, planar::combined_seed(reset_seed, i));
-    if (!was_done || fresh) s.store(row);
-    float o[M::OBS];
-    s.observe(o);
+        for (int k = 0; k < PER_LANE; ++k) l[tid + k * PLANAR_ROWS] = g[tid + k * PLANAR_ROWS];
+    } else {
+        for (int i = tid; i < nenv * PER_LANE; i += PLANAR_ROWS) l[i] = g[i];
+    }
+    __syncthreads();
+    if (tid < nenv) {
+        const int i = env0 + tid;
+        float *row = slab + tid * M::STATE;
+        planar::State<M> s;
+        s.load(row);
+        float a[M::ACT];
 #pragma unroll
-    for (int k = 0; k < M::OBS; ++k) obs[(size_t)i * M::OBS + k] = o[k];
-    rewards[i] = r;
-    dones[i] = d;
-    account(acc, i, r, d);
+        for (int k = 0; k < M::ACT; ++k) a[k] = actions[(size_t)i * M::ACT + k];
+        const bool was_done = s.meta[1] > 0.5;       // such a row is left as it is
+        float r, d;
+        planar::step<M>(s, a, r, d);
+        const bool fresh = AUTORESET && d > 0.5f;
+        if (fresh) planar::reset<M>(s, planar::combined_seed(reset_seed, i));
+        if (!was_done || fresh) s.store(row);
+        rewards[i] = r;
+        dones[i] = d;
+        account(acc, i, r, d);
+    }
+    __syncthreads();
+    if (nenv == PLANAR_ROWS) {
+#pragma unroll
+        for (int k = 0; k < PER_LANE; ++k) g[tid + k * PLANAR_ROWS] = l[tid + k * PLANAR_ROWS];
+    } else {
+        for (int i = tid; i < nenv * PER_LANE; i += PLANAR_ROWS) g[i] = l[i];
+    }
+    for (int i = tid; i < nenv * M::OBS; i += PLANAR_ROWS) {   // observation out: [nenv, OBS] contiguous
+        const int r = i / M::OBS, c = i - r * M::OBS;
+        obs[(size_t)env0 * M::OBS + i] = slab[r * M::STATE + c];
+    }
 }
 
 template <class M>
@@ -563,7 +589,7 @@ static int env_step_impl(mrl_ctx *ctx, int env_id, int batch, float *states, con
         case MRL_ENV_HOPPER_PLANAR:
         case MRL_ENV_WALKER2D_PLANAR: {
             MRL_CHECK_ARG(reinterpret_cast<uintptr_t>(states) % 8 == 0, "mrl_env_step: the planar envs' rows hold doubles: states must be 8-byte aligned");
-            const dim3 grid(grid_for(batch, 256)), block(256);
+            const dim3 grid(grid_for(batch, PLANAR_ROWS)), block(PLANAR_ROWS);
             const bool hopper = env_id == MRL_ENV_HOPPER_PLANAR;
             if (hopper && autoreset)
                 hipLaunchKernelGGL((planar_step_kernel<planar::Hopper, true>), grid, block, 0, ctx->stream, states, actions,
