@@ -333,7 +333,9 @@ def main():
                 "pendulum": "mrl::collect_classic_kernel<mrl::PendulumSlot, %d, true>" % act_id,
                 "bipedal": "mrl::collect_walker_kernel<mrl::BipedalWalker, %d, false>" % act_id,
                 "halfcheetah": "mrl::collect_walker_kernel<mrl::HalfCheetah16, %d, true>" % act_id,
-                "carracing": "mrl::collect_car_kernel<%d>" % act_id}[args.workload]
+                "carracing": "mrl::collect_car_kernel<%d>" % act_id,
+                "hopper": "mrl::collect_planar_kernel<mrl::planar::Hopper, %d>" % act_id,
+                "walker2d": "mrl::collect_planar_kernel<mrl::planar::Walker2d, %d>" % act_id}[args.workload]
         roofline = {"kernel": name + " (policy forward + sampling + env step + auto-reset + rollout stores, %d steps per launch)" % steps_per_launch,
                     "bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": tflops / MFMA_FP32_PEAK_TFLOPS,

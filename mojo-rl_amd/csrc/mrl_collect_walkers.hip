@@ -32,6 +32,7 @@
 #include "env_block.hpp"
 #include "env_cheetah_lanes.hpp"
 #include "env_car.hpp"
+#include "env_planar.hpp"
 #include "collect_args.hpp"
 
 namespace mrl {
@@ -351,13 +352,108 @@ __global__ __launch_bounds__(512) void collect_car_kernel(CollectArgs a) {
     }
 }
 
+// HopperPlanar / Walker2dPlanar (env_planar.hpp): the rows (248 / 392 bytes, Float64 state behind the fp32
+// observation) stay in LDS over the whole launch; the actor runs on wavefronts 0 .. 3, then lanes 0 .. 15 of
+// wavefront 0 step one env each (Float64, state in registers for the four sub-steps), account and rebuild
+// finished rows in place, while the critic runs beside them on wavefronts 2, 3, 6 and 7.
+template <class M, int ACT>
+__global__ __launch_bounds__(512) void collect_planar_kernel(CollectArgs a) {
+    constexpr int H = 256, IN = M::OBS, AW = M::ACT, R = PR16, T = 512;
+    static_assert(IN <= PIN_MAX && AW <= PA_MAX && M::STATE % 2 == 0, "tile limits; rows are whole doubles");
+    __shared__ __align__(16) float rows[R * M::STATE];
+    __shared__ float xs[R * XS_LD];
+    __shared__ __align__(16) float w2a[HEAD_LDS(H)];
+    __shared__ float w2c[H + 1];
+    __shared__ float logits[R * (PA_MAX + 1)];
+    __shared__ float vals[R];
+    __shared__ float act[R * PA_MAX];
+    __shared__ float part[R * PA_MAX];
+    __shared__ unsigned sync_actor, sync_critic, sync_failed;
+    __shared__ __align__(16) float tiles[2 * H * HT16_LD];
+
+    const int t = threadIdx.x;
+    const int env0 = blockIdx.x * R;
+    const int nenv = min(R, a.n_envs - env0);
+    const int N = a.n_envs;
+    float2 *g2 = reinterpret_cast<float2 *>(a.states + (size_t)env0 * M::STATE);
+    float2 *l2 = reinterpret_cast<float2 *>(rows);
+    for (int i = t; i < nenv * (M::STATE / 2); i += T) l2[i] = g2[i];
+    stage_head(a.actor_p + IN * H + H + H * H + H, H, a.A, true, w2a, t, T);
+    for (int i = t; i < H + 1; i += T) w2c[i] = a.critic_p[IN * H + H + H * H + H + i];
+    if (t == 0) {
+        sync_actor = 0;
+        sync_critic = 0;
+        sync_failed = 0;
+    }
+    __syncthreads();
+
+    for (int k = 0; k < a.n_steps; ++k) {
+        // nothing but the rows is carried from one step to the next (see collect16_kernel)
+        int tid = t, ne = __builtin_amdgcn_readfirstlane(nenv), A = __builtin_amdgcn_readfirstlane(a.A), zero = 0;
+        asm volatile("" : "+v"(tid), "+s"(zero), "+s"(ne), "+s"(A) : : "memory");
+        const size_t row = (size_t)(a.t0 + k) * N + env0;
+        const uint32_t sseed = a.sample_seed + (uint32_t)k * a.sample_stride;
+        const uint64_t rseed = a.reset_seed + (uint64_t)k * a.reset_stride;
+        const int wave = tid / WAVE, lane = tid % WAVE;
+        for (int i = tid; i < R * IN; i += T) {
+            const int r = i / IN, c = i - r * IN;
+            float v = 0.0f;
+            if (r < ne) {
+                v = rows[r * M::STATE + c];
+                a.r_obs[row * IN + i] = v;
+            }
+            xs[r * XS_LD + c] = v;
+        }
+        __syncthreads();
+        if (wave < 4) {
+            WaveGroupSync actor_sync{&sync_actor, (unsigned)k * ACTOR16_ROUNDS * 4u, 4u, &sync_failed, a.spin_limit};
+            actor16_gauss<IN, AW, ACT>(a, tid, ne, A, zero, row, sseed, env0, xs, tiles, w2a, logits, act, part, actor_sync);
+        }
+        if (wave == 0) {
+            if (lane < ne) {
+                Accounting acc = a.acc;
+                acc.r_rewards = a.r_rewards + (size_t)(a.t0 + k) * N;
+                acc.r_dones = a.r_dones + (size_t)(a.t0 + k) * N;
+                acc = acc.at(env0);
+                float *rowp = rows + lane * M::STATE;
+                planar::State<M> s;
+                s.load(rowp);
+                float r, d;
+                planar::step<M>(s, act + lane * AW, r, d);
+                account(acc, lane, r, d);
+                if (d > 0.5f) planar::reset<M>(s, planar::combined_seed(rseed, env0 + lane));
+                s.store(rowp);
+            }
+        } else {
+            critic16_side<IN, ACT>(a, zero, k, tid, xs, tiles + H * HT16_LD, w2c, vals, &sync_critic, &sync_failed);
+        }
+        __syncthreads();   // env step done: the rows hold the next observation
+        if (tid < ne) a.r_values[row + tid] = vals[tid];
+        if (sync_failed != 0u) break;
+    }
+    if (sync_failed != 0u) {
+        // a wait gave up: the block's rows and observations keep the values from before the launch
+        if (t == 0) *a.sync_error = 1;
+        return;
+    }
+    for (int i = t; i < nenv * IN; i += T) {
+        const int r = i / IN, c = i - r * IN;
+        a.obs[(size_t)env0 * IN + i] = rows[r * M::STATE + c];
+    }
+    for (int i = t; i < nenv * (M::STATE / 2); i += T) g2[i] = l2[i];
+}
+
 bool collect_walker_fusable(const mrl_rollout *r, int *act) {
     if (r->num_actions != 0) return false;
     int obs, aw;
     if (r->env_id == MRL_ENV_BIPEDAL) { obs = BipedalWalker::OBS; aw = BipedalWalker::ACT_W; }
     else if (r->env_id == MRL_ENV_HALFCHEETAH) { obs = HalfCheetah::OBS; aw = HalfCheetah::ACT_W; }
     else if (r->env_id == MRL_ENV_CARRACING) { obs = cr::OBS; aw = cr::ACT; }
+    else if (r->env_id == MRL_ENV_HOPPER_PLANAR) { obs = planar::Hopper::OBS; aw = planar::Hopper::ACT; }
+    else if (r->env_id == MRL_ENV_WALKER2D_PLANAR) { obs = planar::Walker2d::OBS; aw = planar::Walker2d::ACT; }
     else return false;
+    // (the planar rows hold doubles)
+    if (r->env_id >= MRL_ENV_HOPPER_PLANAR && reinterpret_cast<uintptr_t>(r->states) % 8 != 0) return false;
     const mrl_mlp_desc &a = r->actor, &c = r->critic;
     if (a.n_layers != 3 || c.n_layers != 3) return false;
     const int k0 = a.layers[0].kind;
@@ -385,6 +481,12 @@ int launch_collect_walker(mrl_ctx *ctx, const mrl_rollout *r, const CollectArgs 
     } else if (r->env_id == MRL_ENV_CARRACING) {
         if (act == 1) hipLaunchKernelGGL((collect_car_kernel<1>), grid, block, 0, ctx->stream, a);
         else hipLaunchKernelGGL((collect_car_kernel<2>), grid, block, 0, ctx->stream, a);
+    } else if (r->env_id == MRL_ENV_HOPPER_PLANAR) {
+        if (act == 1) hipLaunchKernelGGL((collect_planar_kernel<planar::Hopper, 1>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((collect_planar_kernel<planar::Hopper, 2>), grid, block, 0, ctx->stream, a);
+    } else if (r->env_id == MRL_ENV_WALKER2D_PLANAR) {
+        if (act == 1) hipLaunchKernelGGL((collect_planar_kernel<planar::Walker2d, 1>), grid, block, 0, ctx->stream, a);
+        else hipLaunchKernelGGL((collect_planar_kernel<planar::Walker2d, 2>), grid, block, 0, ctx->stream, a);
     } else {
         a.shapes = ctx->hc_shapes;
         if (act == 1) hipLaunchKernelGGL((collect_walker_kernel<HalfCheetah16, 1, true>), grid, block, 0, ctx->stream, a);

@@ -21,7 +21,7 @@ def ctx(mrl):
 def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
     E = {"lunar": mrl.LunarLanderV2, "lunarc": mrl.LunarLanderV2Continuous, "cartpole": mrl.CartPoleEnv,
          "pendulum": mrl.PendulumV2, "bipedal": mrl.BipedalWalkerV2, "cheetah": mrl.HalfCheetahPlanarV2,
-         "car": mrl.CarRacingV2}[env]
+         "car": mrl.CarRacingV2, "hopper": mrl.HopperPlanar, "walker2d": mrl.Walker2dPlanar}[env]
     lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
     head = mrl.StochasticActor(hidden, E.ACTION_DIM) if E.ACTION_DIM else mrl.Linear(hidden, E.NUM_ACTIONS)
     actor = mrl.seq(lin(E.OBS_DIM, hidden), lin(hidden, hidden), head)
@@ -47,6 +47,16 @@ def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
             rows[::3, 34] = 495.0     # step counter (first metadata float) close to its limit of 500
         elif env == "cheetah":
             rows[::3, 245] = 995.0    # step counter (first metadata float) close to its limit of 1000
+        elif env in ("hopper", "walker2d"):
+            # no step limit in these envs: every third torso starts tilted beyond the health bound (first step
+            # ends the episode), the next third high up with the legs folded, so that it falls through the
+            # height bound some steps later.  The Float64 state begins behind the observation and a padding float.
+            d = rb.states.view(torch.float64).view(N, E.STATE_SIZE // 2)[:, (E.OBS_DIM + 1) // 2:]
+            nj = E.ACTION_DIM
+            d[::3, 2] = 1.5
+            d[1::3, 1] = 1.3
+            d[1::3, 15 + 3 * (nj - 3):15 + 3 * (nj - 3) + nj] = -1.0    # joint angles
+            rows[::3, 1] = 1.5
         else:
             rows[::3, 4] = 197.0      # step counter close to the limit
         rb.obs.copy_(rows[:, :E.OBS_DIM].reshape(-1))
@@ -70,6 +80,10 @@ def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
     # steps of the same launch), truncations rebuild the track inside the launch
     ("car", 4096, 12, 256, "tanh"), ("car", 77, 7, 256, "relu"), ("car", 300, 48, 256, "tanh"),
     ("car", 100, 5, 64, "tanh"),              # not fusable
+    # the Float64 planar envs: unhealthy torsos end episodes from the first step on, resets inside the launch
+    ("hopper", 4096, 12, 256, "tanh"), ("hopper", 77, 7, 256, "relu"), ("hopper", 500, 64, 256, "tanh"),
+    ("walker2d", 4096, 12, 256, "tanh"), ("walker2d", 77, 7, 256, "relu"), ("walker2d", 500, 64, 256, "tanh"),
+    ("hopper", 100, 5, 64, "tanh"),           # not fusable
 ])
 def test_rollout_steps_equals_single_steps(mrl, ctx, env, N, T, hidden, kind):
     print("case", env, N, T, hidden, kind, flush=True)
@@ -86,6 +100,8 @@ def test_rollout_steps_equals_single_steps(mrl, ctx, env, N, T, hidden, kind):
     for name in ("r_obs", "r_actions", "r_log_probs", "r_values", "r_rewards", "r_dones", "states", "obs",
                  "ep_return", "ep_length"):
         a, b = getattr(one, name), getattr(many, name)
+        if name == "states":     # as bit patterns: the halves of the planar envs' doubles include NaN patterns
+            a, b = a.view(torch.int32), b.view(torch.int32)
         assert torch.equal(a, b), "%s differs in %d places" % (name, int((a != b).sum()))
     cnt = int(one.done_count.item())
     assert cnt == int(many.done_count.item()) and cnt > 0
