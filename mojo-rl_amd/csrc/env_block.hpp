@@ -46,7 +46,7 @@ MRL_DEV void account(const Accounting &acc, int i, float r, float d) { account(a
 struct LunarLander {
     using L = ll::L;
     static constexpr int STATE = ll::STATE, OBS = ll::OBS, ACT_W = 1, EPB = 32, THREADS = 512;
-    static constexpr int DENSE_FROM = 24576;   // batch from which the stand-alone step runs 16 rows per workgroup
+    static constexpr int LANE_FROM = 8193;   // batch from which the stand-alone step runs one lane per env
     static constexpr int DYN_END = L::JOINTS_OFF, NSHAPE = ll::NSHAPE_FLOATS;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {
@@ -101,7 +101,7 @@ struct LunarLanderContinuous : LunarLander {
 struct BipedalWalker {
     using L = bw::L;
     static constexpr int STATE = bw::STATE, OBS = bw::OBS, ACT_W = bw::ACT, EPB = 16, THREADS = 512;
-    static constexpr int DENSE_FROM = 0;
+    static constexpr int LANE_FROM = 0;      // (never: the lane form is no faster for this env at any batch)
     static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = bw::NSHAPE_FLOATS;
     // the ten lidar rays of the observation are left out of the step and run afterwards, spread
     // over all wavefronts of the block: task k = part k % 3 of the edges for ray k / 3; the parts of
@@ -170,7 +170,7 @@ struct BipedalWalker {
 struct HalfCheetah {
     using L = hc::L;
     static constexpr int STATE = hc::STATE, OBS = hc::OBS, ACT_W = hc::ACT, EPB = 64, THREADS = 256;
-    static constexpr int DENSE_FROM = 0;
+    static constexpr int LANE_FROM = 0;      // (never: the lane form is no faster for this env at any batch)
     static constexpr int DYN_END = L::EDGES_OFF, NSHAPE = hc::NSHAPE_FLOATS;
     static MRL_DEV void step(float *row, float *cts, const float *shapes, int env, const float *a,
                              float &r, float &d) {

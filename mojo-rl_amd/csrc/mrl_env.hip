@@ -142,15 +142,33 @@ __global__ __launch_bounds__(E::THREADS) void phys_step_kernel(float *states, co
     phys_step_body<E, AUTORESET>(states, actions, rewards, dones, obs, shapes_g, batch, reset_seed, acc);
 }
 
-// The same step for batches that fill the chip several times over: 16 rows per workgroup of four
-// wavefronts and registers bounded for three wavefronts per SIMD, so that a CU holds three workgroups
-// (three solver wavefronts at work instead of one) where the 32-row form holds one.
+// The same step with one lane per ENV and the rows left in global memory (64 envs per single-wavefront
+// workgroup, only the contact scratch in LDS): nothing is shared between lanes, so a batch that fills the
+// chip runs at the rate of the vector units instead of at the latency of one workgroup's phase chain.
+// Used from E::LANE_FROM envs on (LunarLander: one wavefront's step lasts 44 us whatever the batch, the
+// 32-row workgroup's 33 us, but a CU holds five of these wavefronts and one such workgroup).
 template <class E, bool AUTORESET>
-__global__ __launch_bounds__(256, 3) void phys_step_dense_kernel(float *states, const float *actions,
-                                                                 float *rewards, float *dones, float *obs,
-                                                                 const float *shapes_g, int batch,
-                                                                 uint64_t reset_seed, Accounting acc) {
-    phys_step_body<Rows16<E>, AUTORESET>(states, actions, rewards, dones, obs, shapes_g, batch, reset_seed, acc);
+__global__ __launch_bounds__(64) void phys_step_lane_kernel(float *states, const float *actions, float *rewards,
+                                                            float *dones, float *obs, const float *shapes_g, int batch,
+                                                            uint64_t reset_seed, Accounting acc) {
+    using S = Stage<E>;
+    __shared__ float cts[WAVE * S::CSTRIDE];
+    __shared__ float shapes[E::NSHAPE];
+    const int lane = threadIdx.x;
+    const int env = blockIdx.x * WAVE + lane;
+    for (int i = lane; i < E::NSHAPE; i += WAVE) shapes[i] = shapes_g[i];
+    __syncthreads();
+    if (env >= batch) return;
+    float *row = states + (size_t)env * E::STATE;
+    const EpisodeSums sums = account_before(acc, env);
+    float r, d;
+    E::step(row, cts + lane * S::CSTRIDE, shapes, env, actions + (size_t)env * E::ACT_W, r, d);
+    rewards[env] = r;
+    dones[env] = d;
+    account(acc, env, r, d, sums);
+    if (AUTORESET && d > 0.5f) E::reset(row, reset_seed, env);
+#pragma unroll
+    for (int k = 0; k < E::OBS; ++k) obs[(size_t)env * E::OBS + k] = row[k];
 }
 
 // HalfCheetah with one lane per body (env_cheetah_lanes.hpp): a workgroup is one wavefront with
@@ -359,14 +377,14 @@ template <class E>
 static int launch_phys_step(mrl_ctx *ctx, int batch, float *states, const float *actions, float *rewards,
                             float *dones, float *obs, const float *shapes, bool autoreset,
                             uint64_t reset_seed, const Accounting &acc) {
-    if constexpr (E::DENSE_FROM > 0) {
-        if (batch >= E::DENSE_FROM && getenv("MRL_NO_DENSE") == nullptr) {
-            dim3 grid16(grid_for(batch, 16));
+    if constexpr (E::LANE_FROM > 0) {
+        if (batch >= E::LANE_FROM) {
+            dim3 grid64(grid_for(batch, WAVE));
             if (autoreset)
-                hipLaunchKernelGGL((phys_step_dense_kernel<E, true>), grid16, dim3(256), 0, ctx->stream, states, actions,
+                hipLaunchKernelGGL((phys_step_lane_kernel<E, true>), grid64, dim3(WAVE), 0, ctx->stream, states, actions,
                                    rewards, dones, obs, shapes, batch, reset_seed, acc);
             else
-                hipLaunchKernelGGL((phys_step_dense_kernel<E, false>), grid16, dim3(256), 0, ctx->stream, states, actions,
+                hipLaunchKernelGGL((phys_step_lane_kernel<E, false>), grid64, dim3(WAVE), 0, ctx->stream, states, actions,
                                    rewards, dones, obs, shapes, batch, reset_seed, acc);
             return MRL_OK;
         }

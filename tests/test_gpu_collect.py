@@ -67,6 +67,9 @@ def _pair(mrl, ctx, N, T, hidden, kind, env="lunar"):
 @pytest.mark.parametrize("env,N,T,hidden,kind", [
     ("lunar", 8192, 12, 256, "relu"), ("lunar", 1000, 9, 256, "tanh"), ("lunar", 77, 5, 256, "relu"),
     ("lunar", 300, 6, 64, "relu"),            # not fusable: the loop of single steps behind the same call
+    # above 8192 envs the single steps run the one-lane-per-env step kernel (rows in global memory,
+    # detection inline, accounting and reset by the env's lane) against the fused kernel's 32-row workgroups
+    ("lunar", 9001, 8, 256, "relu"), ("lunarc", 9001, 6, 256, "tanh"),
     ("cartpole", 8192, 12, 64, "relu"), ("cartpole", 77, 7, 64, "tanh"),
     ("pendulum", 8192, 12, 64, "tanh"), ("pendulum", 1000, 9, 64, "relu"),
     ("cartpole", 300, 6, 256, "relu"),        # not fusable

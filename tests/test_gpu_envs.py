@@ -288,9 +288,10 @@ def test_lunar_lander_continuous_rollout_parity(mrl, orc, ctx, batch, seed, low)
 
 @pytest.mark.parametrize("cont", [False, True])
 def test_lunar_lander_large_batch_form_parity(mrl, orc, ctx, cont):
-    """From 24576 rows on, the stand-alone step runs 16 rows per workgroup of four wavefronts (three
-    workgroups per CU) instead of 32 per workgroup of eight: same results, bit for bit, through steps,
-    contacts, crashes and in-place resets.  The batch has a ragged last workgroup."""
+    """Above 8192 rows the stand-alone step runs one lane per env on rows left in global memory (contact
+    detection inline on the env's own lane) instead of a 32-row workgroup with the detection spread over
+    seven wavefronts: same results, bit for bit, through steps, contacts, crashes and in-place resets.  The
+    batch has a ragged last wavefront."""
     batch = 32768 + 5
     E = mrl.LunarLanderV2Continuous if cont else mrl.LunarLanderV2
     say("lunar large batch", batch, "continuous", cont)
