@@ -1,5 +1,5 @@
 // Fused collection kernels of the continuous-control envs beyond the classic ones (BipedalWalker,
-// HalfCheetah planar, CarRacingV2) with the agents' 256-wide Gaussian nets: many rollout steps of a
+// HalfCheetah planar, CarRacingV2, HopperPlanar, Walker2dPlanar) with the agents' 256-wide Gaussian nets: many rollout steps of a
 // block's 16 envs in ONE launch, like the kernels of mrl_collect.hip.  The env rows (CarRacing: the 40
 // floats in front of the track) stay in LDS from the first step to the last; per step and block
 //   policy   the actor  OBS -> 256 -> 256 -> A  on wavefronts 0 .. 3 and the critic  OBS -> 256 -> 256 -> 1
@@ -15,7 +15,8 @@
 //            wavefront, wave-cooperative resets); HalfCheetah: one lane per body on wavefronts 0 and 1
 //            (env_cheetah_lanes.hpp); CarRacing: a wavefront per env, two rounds of eight (env_car.hpp);
 //            the tile tables stay in global memory and are staged through LDS every step (16 x 12 KB do
-//            not fit beside the rest);
+//            not fit beside the rest); HopperPlanar / Walker2dPlanar: one lane per env on wavefront 0
+//            (Float64, env_planar.hpp), the critic beside it as for the walkers;
 //   rollout row t of obs, action, log-prob, value, reward, done written on the way.
 // With these envs the step is 70 - 80 % env step, a chain of one or two wavefronts' instructions: what the
 // fusion buys is the launch gaps, the observation / action round trip through HBM, the staging of the rows

@@ -6,7 +6,8 @@
 // (row stride odd => the lanes touch distinct banks for any field) while the other wavefronts
 // detect its contacts where the env splits that off, and the fields that a step can change are
 // copied back with coalesced stores.  HBM sees each row once in and the changed part once out;
-// nothing is re-read.
+// nothing is re-read.  (LunarLander above 8192 envs: one lane per env on rows left in global memory,
+// phys_step_lane_kernel.)
 #include <cmath>
 #include "mrl_host.hpp"
 #include "env_classic.hpp"
