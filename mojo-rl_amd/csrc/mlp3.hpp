@@ -13,6 +13,7 @@ struct Mlp3Net {
     const float *grad_out;   // backward
     float *g1, *g0, *ls_part, *db_part, *thin_part;  // backward workspace (set by the host function)
     int A, gauss;            // set by the host function from the description
+    int thin_stride;         // floats per row tile in thin_part: IN H + H A, + H H where the tiles carry dW1 too
 };
 struct Mlp3Nets { Mlp3Net n[2]; };
 

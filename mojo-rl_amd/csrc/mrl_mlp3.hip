@@ -154,7 +154,7 @@ __global__ __launch_bounds__(2 * H) void mlp3_bwd_dx_kernel(int B, int IN, Mlp3N
     float *__restrict__ db_part = nn.db_part + (size_t)blockIdx.x * (2 * H + PA_MAX);   // this tile's slice
     const int A = nn.A;
     // this tile's share of the two thin weight gradients: [dW0 (IN x H) | dW2 (H x A)]
-    float *__restrict__ thin_part = nn.thin_part + (size_t)blockIdx.x * ((size_t)IN * H + (size_t)H * A);
+    float *__restrict__ thin_part = nn.thin_part + (size_t)blockIdx.x * (size_t)nn.thin_stride;
     const bool GAUSS = nn.gauss != 0;
     constexpr int KCH = 64;                       // k-chunk of W1 staged per round
     __shared__ float g2s[PR * (2 * PA_MAX + 1)];
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
     float *__restrict__ ls_part = nn.ls_part;
     float *__restrict__ db_part = nn.db_part + (size_t)blockIdx.x * (2 * H + PA_MAX);
     const int A = nn.A;
-    float *__restrict__ thin_part = nn.thin_part + (size_t)blockIdx.x * ((size_t)IN * H + (size_t)H * A);
+    float *__restrict__ thin_part = nn.thin_part + (size_t)blockIdx.x * (size_t)nn.thin_stride;
     const bool GAUSS = nn.gauss != 0;
     const int ld = GAUSS ? 2 * A : A;
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, half = lane >> 5, l31 = lane & 31;
@@ -541,6 +541,28 @@ __global__ __launch_bounds__(2 * H) void mlp3_fb_kernel(int B, int IN, Mlp3Nets 
         if (t < A) db_part[2 * H + t] = cs2;
         else ls_part[(long)blockIdx.x * A + (t - A)] = cs2;
     }
+    if constexpr (H == 64) {
+        // Hidden width 64: the hidden layer's weight gradient of the tile, dW1[k][n] = sum_r h1[r][k] g1[r][n],
+        // is four 32 x 32 tiles of 16 k-steps.  It is taken here, from h1 and g1 while both lie in LDS, as one
+        // more per-tile piece for the sum kernel (wavefront w: columns [32w, 32w + 32)), instead of in a launch
+        // of its own that reads h1 and g1 back from global memory: that launch was 10 us of a 37 us minibatch.
+        __syncthreads();   // gT complete
+        float *o1 = thin_part + (size_t)IN * H + (size_t)H * A;
+#pragma unroll
+        for (int kt = 0; kt < H / 32; ++kt) {
+            floatx16 c = {0};
+#pragma unroll
+            for (int kk = 0; kk < PR / 2; ++kk) {
+                const int r = 2 * kk + half;
+                c = __builtin_amdgcn_mfma_f32_32x32x2f32(hT[(32 * kt + l31) * HT_LD + r], gT[col * HT_LD + r], c, 0, 0, 0);
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int k = 32 * kt + 8 * (v >> 2) + 4 * half + (v & 3);
+                o1[(size_t)k * H + col] = c[v];
+            }
+        }
+    }
     // ---- dh1 = g1 W1^T: wavefront w owns input columns [32w, 32w + 32); the next chunk of W1 is
     // fetched into registers while the matrix cores work on the current one
     floatx16 acc = {0};
@@ -719,6 +741,8 @@ struct SumNets {
     const float *ls_part[2], *db_part[2], *thin_part[2];
     int P[2], A[2], gauss[2];
     int n, IN, H;
+    int thin_stride[2];   // floats per row tile in thin_part, per net
+    int hh_in_tiles;   // the H x H block is summed from the row tiles' pieces (behind dW0 and dW2) instead of `partial`
 };
 
 __global__ __launch_bounds__(256) void sum3_kernel(const float *__restrict__ partial, int splits, int Ptot,
@@ -744,10 +768,15 @@ __global__ __launch_bounds__(256) void sum3_kernel(const float *__restrict__ par
         const float *p;
         size_t stride;
         int n;
-        if (bias_layer < 0 && i >= o1 && i < o1 + H * H) { p = partial + gi; stride = (size_t)Ptot; n = splits; }
+        if (bias_layer < 0 && i >= o1 && i < o1 + H * H && sn.hh_in_tiles) {
+            p = sn.thin_part[net] + (size_t)IN * H + (size_t)H * A + (i - o1);
+            stride = (size_t)sn.thin_stride[net];
+            n = tiles;
+        }
+        else if (bias_layer < 0 && i >= o1 && i < o1 + H * H) { p = partial + gi; stride = (size_t)Ptot; n = splits; }
         else if (bias_layer < 0) {   // a weight of layer 0 or of the head: per-tile pieces of the dx kernel
             p = sn.thin_part[net] + (i < o1 ? i : (size_t)IN * H + (i - o2));
-            stride = (size_t)IN * H + (size_t)H * A;
+            stride = (size_t)sn.thin_stride[net];
             n = tiles;
         }
         else if (bias_layer == 3) { p = sn.ls_part[net] + j; stride = (size_t)A; n = tiles; }
@@ -876,7 +905,8 @@ size_t mlp3_backward_ws(const mrl_mlp_desc *const *descs, int n_nets, int batch)
         const int H = descs[i]->layers[0].out_dim;
         const int IN = descs[i]->layers[0].in_dim, A = descs[i]->layers[2].out_dim;
         total += (size_t)2 * batch * H +
-                 (size_t)((batch + PR - 1) / PR) * (2 * PA_MAX + 2 * H + (size_t)IN * H + (size_t)H * A);
+                 (size_t)((batch + PR - 1) / PR) * (2 * PA_MAX + 2 * H + (size_t)IN * H + (size_t)H * A +
+                                                    (H == 64 ? (size_t)H * H : 0));
         P += net_P(*descs[i]);
     }
     return total + (size_t)32 * P;
@@ -903,6 +933,7 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
     int splits = std::max(1, std::min(32, batch / 256));
     int rows_per = ((batch + splits - 1) / splits + DKC - 1) / DKC * DKC;
     splits = (batch + rows_per - 1) / rows_per;
+    const bool hh_in_tiles = fused != nullptr && H == 64;
     // workspace: per net g1 [B, H] | g0 [B, H] | ls_part [tiles, PA_MAX] | db_part [tiles, 2H + PA_MAX] |
     // thin_part [tiles, IN H + H A]; then partial [splits, Ptot]
     float *w = ws;
@@ -911,7 +942,9 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
         io.n[i].g0 = w; w += (size_t)batch * H;
         io.n[i].ls_part = w; w += (size_t)tiles * PA_MAX;
         io.n[i].db_part = w; w += (size_t)tiles * (2 * H + PA_MAX);
-        io.n[i].thin_part = w; w += (size_t)tiles * ((size_t)IN * H + (size_t)H * descs[i]->layers[2].out_dim);
+        // (the fused forward + backward kernel of the 64-wide nets leaves the tile's dW1 there as well)
+        io.n[i].thin_stride = IN * H + H * descs[i]->layers[2].out_dim + (hh_in_tiles ? H * H : 0);
+        io.n[i].thin_part = w; w += (size_t)tiles * (size_t)io.n[i].thin_stride;
     }
     float *partial = w;
     FwdLoss fl{};
@@ -931,6 +964,7 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
     sn.n = n_nets;
     sn.IN = IN;
     sn.H = H;
+    sn.hh_in_tiles = hh_in_tiles ? 1 : 0;
     int base = 0, total_tiles = 0;
     for (int i = 0; i < n_nets; ++i) {
         const Mlp3Net &nn = io.n[i];
@@ -947,6 +981,7 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
         sn.ls_part[i] = nn.ls_part;
         sn.db_part[i] = nn.db_part;
         sn.thin_part[i] = nn.thin_part;
+        sn.thin_stride[i] = nn.thin_stride;
         sn.P[i] = net_P(*descs[i]);
         sn.A[i] = A;
         sn.gauss[i] = nn.gauss;
@@ -954,8 +989,9 @@ int mlp3_backward_n(mrl_ctx *ctx, const mrl_mlp_desc *const *descs, int n_nets, 
     }
     const int Ptot = base;
     // (both nets have the same width: every problem has the same number of tiles, see dw3_kernel)
-    hipLaunchKernelGGL(dw3_kernel, dim3(total_tiles * splits), dim3(256), 0, ctx->stream, dw, batch, rows_per,
-                       Ptot, partial, splits);
+    if (!hh_in_tiles)
+        hipLaunchKernelGGL(dw3_kernel, dim3(total_tiles * splits), dim3(256), 0, ctx->stream, dw, batch, rows_per,
+                           Ptot, partial, splits);
     const int sum_blocks = grid_for(Ptot, 256);
     if (sum_blocks > 1024) sq_part = nullptr;   // more partials than the caller's buffer holds
     if (sq_blocks) *sq_blocks = sq_part ? sum_blocks : 0;

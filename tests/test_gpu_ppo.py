@@ -924,21 +924,25 @@ def test_update_driver_runs_epochs_and_stops_on_kl(mrl, ctx):
     assert torch.equal(frozen, anet.params)
 
 
-@pytest.mark.parametrize("env_name,kind,MB", [("LunarLanderV2", "relu", 4096), ("LunarLanderV2", "tanh", 1000),
-                                              ("HalfCheetahPlanarV2", "tanh", 777)])
-def test_fused_update_minibatch_equals_its_parts(mrl, ctx, env_name, kind, MB):
-    """mrl_ppo_update_minibatch on nets of hidden width 256 (one kernel takes a row tile forward,
+@pytest.mark.parametrize("env_name,kind,MB,HID", [("LunarLanderV2", "relu", 4096, 256), ("LunarLanderV2", "tanh", 1000, 256),
+                                                  ("HalfCheetahPlanarV2", "tanh", 777, 256),
+                                                  # hidden width 64: the fused kernel also leaves the hidden layer's
+                                                  # weight gradient per row tile (no weight-gradient launch)
+                                                  ("CartPoleEnv", "tanh", 4096, 64), ("PendulumV2", "tanh", 1000, 64),
+                                                  ("CartPoleEnv", "relu", 777, 64)])
+def test_fused_update_minibatch_equals_its_parts(mrl, ctx, env_name, kind, MB, HID):
+    """mrl_ppo_update_minibatch on nets of hidden width 256 or 64 (one kernel takes a row tile forward,
     through the loss and back) against the same minibatch issued call by call: gather,
     normalise, forward with cache, loss gradients, backward, clip, Adam.  The fused kernel sums
     in a different order, hence MLP tolerances on the gradients."""
-    say("case", env_name, kind, MB)
+    say("case", env_name, kind, MB, HID)
     E = getattr(mrl, env_name)
     cont = E.NUM_ACTIONS == 0
     lin = mrl.LinearReLU if kind == "relu" else mrl.LinearTanh
     A = E.ACTION_DIM if cont else E.NUM_ACTIONS
-    head = mrl.StochasticActor(256, A) if cont else mrl.Linear(256, A)
-    actor = mrl.seq(lin(E.OBS_DIM, 256), lin(256, 256), head)
-    critic = mrl.seq(lin(E.OBS_DIM, 256), lin(256, 256), mrl.Linear(256, 1))
+    head = mrl.StochasticActor(HID, A) if cont else mrl.Linear(HID, A)
+    actor = mrl.seq(lin(E.OBS_DIM, HID), lin(HID, HID), head)
+    critic = mrl.seq(lin(E.OBS_DIM, HID), lin(HID, HID), mrl.Linear(HID, 1))
     N, T = 512, 8
     g = torch.Generator(device="cuda").manual_seed(11)
     rnd = lambda n, s=1.0: (torch.rand(n, device="cuda", generator=g) - 0.5) * 2 * s
